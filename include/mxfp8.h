@@ -1,0 +1,127 @@
+/*
+ * C ABI of the MI355X (gfx950) MXFP8 linear path.
+ *
+ * Every entry point takes raw device pointers, sizes and a HIP stream (as void*), launches
+ * asynchronously on that stream, allocates nothing, never synchronises, and returns an
+ * mx_status_t (0 = ok).  No exceptions cross this boundary.  Calls are thread-safe as long
+ * as concurrent calls use distinct output buffers.
+ *
+ * The reference has no native interface for this path: its converter hands the arithmetic
+ * to an external Python library.  Each declaration cites the reference statement that the
+ * entry point stands in for.
+ *
+ * Data formats (OCP Microscaling v1.0, "MXFP8"):
+ *   codes   uint8  e4m3fn (S EEEE MMM, bias 7, max 448, 0x7F/0xFF NaN), saturating RNE
+ *   scales  uint8  E8M0, byte b = 2^(b-127), 255 = NaN; one per 32 consecutive elements
+ *   hp      bf16   (uint16 bit patterns), row-major
+ */
+#ifndef MXFP8_H_
+#define MXFP8_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  MX_OK = 0,
+  MX_ERR_INVALID_ARG = 1,   /* null pointer, negative size, bad enum */
+  MX_ERR_ALIGNMENT = 2,     /* a dimension is not a multiple of what the kernel needs */
+  MX_ERR_LAUNCH = 3,        /* hipLaunchKernel reported an error */
+  MX_ERR_UNSUPPORTED = 4    /* shape outside what this build handles */
+} mx_status_t;
+
+/* How the E8M0 scale is derived from the block's max |x| (amax = (1+m) 2^E):
+ *   FLOOR  s = E - 8                         (OCP MX v1.0 section 6.3; may saturate codes)
+ *   RCEIL  s = ceil(log2(amax / 448))        (recipe "mxfp8_rceil",
+ *                                             torchtitan/components/quantization/mx.py:37-42)
+ */
+typedef enum { MX_SCALE_FLOOR = 0, MX_SCALE_RCEIL = 1 } mx_scale_mode_t;
+
+/* Where a cast writes its scale bytes:
+ *   ROWMAJOR  [rows, nblk]
+ *   MFMA      [ceil(rows/64), ceil(nblk/4), 64, 4]: for row tile rt, K-step ks, lane l,
+ *             byte t the entry is scale[rt*64 + t*16 + (l & 15)][ks*4 + (l >> 4)]
+ *             (zero beyond the matrix) -- the order mx_gemm_nt reads.
+ */
+typedef enum { MX_SCALES_ROWMAJOR = 0, MX_SCALES_MFMA = 1 } mx_scale_order_t;
+
+/* Library/ABI version (major*100 + minor). */
+int mx_version(void);
+const char* mx_status_string(int status);
+
+/* Bytes of a scale buffer in MX_SCALES_MFMA order for a [rows, nblk] scale matrix. */
+int64_t mx_scales_mfma_bytes(int64_t rows, int64_t nblk);
+
+/* Row-wise to_mx: x bf16 [rows, cols] (row stride ldx elements) ->
+ * codes u8 [rows, cols] (dense) and scales for blocks of 32 along `cols`.
+ * Requires cols % 32 == 0.  Stands in for the cast of the activation / weight along the
+ * contraction dim that the converted F.linear performs
+ * (torchtitan/components/quantization/mx.py:27-31,119-125; docs/mxfp8.md:35). */
+int mx_cast_dim0(const void* x, int64_t rows, int64_t cols, int64_t ldx, uint8_t* codes,
+                 uint8_t* scales, int scale_mode, int scale_order, void* stream);
+
+/* Column-wise to_mx: x bf16 [rows, cols] -> codes u8 [cols, rows] (transposed, dense) and
+ * scales [cols, rows/32] for blocks of 32 down the rows.  Requires rows % 32 == 0 and
+ * cols % 2 == 0.  Equals mx_cast_dim0 of the transposed tensor.  Feeds dgrad / wgrad
+ * operands (docs/mxfp8.md:61; torchtitan/models/common/moe/utils.py:47-52). */
+int mx_cast_dim1(const void* x, int64_t rows, int64_t cols, int64_t ldx, uint8_t* codes_t,
+                 uint8_t* scales_t, int scale_mode, int scale_order, void* stream);
+
+/* Both casts from one read of x.  Requires rows % 32 == 0 and cols % 32 == 0. */
+int mx_cast_dim0_dim1(const void* x, int64_t rows, int64_t cols, int64_t ldx, uint8_t* codes,
+                      uint8_t* scales, uint8_t* codes_t, uint8_t* scales_t, int scale_mode,
+                      int scale_order, void* stream);
+
+/* Re-order a row-major [rows, nblk] scale matrix into MX_SCALES_MFMA order
+ * (the "blocked layout" step the reference leaves to torch._scaled_mm, docs/mxfp8.md:36). */
+int mx_scale_layout(const uint8_t* scales, int64_t rows, int64_t nblk, uint8_t* out, void* stream);
+/* Inverse permutation. */
+int mx_scale_unlayout(const uint8_t* laid, int64_t rows, int64_t nblk, uint8_t* out, void* stream);
+
+/* D[M,N] (bf16, row stride ldd) = deq(A)[M,K] * deq(B)[N,K]^T, fp32 accumulate.
+ * a_codes [M,K], b_codes [N,K] row-major dense; a_scales / b_scales in MX_SCALES_MFMA order
+ * for [M, K/32] and [N, K/32].  Requires K % 32 == 0.  One primitive serves forward
+ * (X along K, W along K), dgrad (dY along N, W^T along N) and wgrad (dY^T along M, X^T along
+ * M) -- the F.linear on a converted weight and its autograd
+ * (torchtitan/components/quantization/mx.py:27-31; torchtitan/models/common/feed_forward.py:61-62). */
+int mx_gemm_nt(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+               const uint8_t* b_scales, void* d, int64_t M, int64_t N, int64_t K, int64_t ldd,
+               void* stream);
+
+/* Grouped GEMM, 2D x 3D: for group g with rows [offs[g-1], offs[g]) of A:
+ * D[rows, :] = deq(A[rows, :]) * deq(B[g])^T.  a_codes [T,K]; b_codes [G,N,K];
+ * a_scales MFMA order for [T, K/32]; b_scales G consecutive MFMA-order blocks for [N, K/32].
+ * offs int32 [G] inclusive cumulative sizes on the device; rows >= offs[G-1] are written as
+ * zeros.  Group sizes need not be aligned for this entry point.  Stands in for
+ * torch._grouped_mm(x, w^T, offs) in forward and dgrad
+ * (torchtitan/models/common/moe/moe.py:59-76). */
+int mx_grouped_gemm_2d3d(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                         const uint8_t* b_scales, const int32_t* offs, void* d, int64_t T,
+                         int64_t N, int64_t K, int64_t G, int64_t ldd, void* stream);
+
+/* Grouped GEMM, 2D x 2D (wgrad): D[g][N,K] = deq(A^T[:, rows_g]) * deq(B^T[:, rows_g])^T,
+ * contracting over the tokens of group g.  at_codes [N,T] and bt_codes [K,T] are the
+ * column-wise casts; their scales are row-major [N, T/32] and [K, T/32].  Every group size
+ * must be a multiple of 32 (torchtitan/models/common/moe/utils.py:47-52); empty groups give
+ * zeros.  d is [G,N,K] bf16 dense. */
+int mx_grouped_gemm_2d2d(const uint8_t* at_codes, const uint8_t* at_scales,
+                         const uint8_t* bt_codes, const uint8_t* bt_scales, const int32_t* offs,
+                         void* d, int64_t T, int64_t N, int64_t K, int64_t G, void* stream);
+
+/* Token-group padding: from per-(rank, expert) counts build
+ *   m_sizes[e]   = round_up(max(sum_r counts[r*E+e], alignment), alignment)   int32 [E]
+ *   m_offsets    = inclusive cumsum(m_sizes)                                  int32 [E]
+ *   perm[max_len]: perm[write_off[e] + j] = start[r*E+e] + j, -1 in padding   int64
+ * One launch, no host synchronisation.  Stands in for generate_permute_indices and its
+ * Triton fill kernel (torchtitan/models/common/moe/kernels.py:16-63,145-218).
+ * Requires experts_per_rank * num_ranks <= 65536. */
+int mx_group_offsets_pad(const int32_t* counts, int64_t experts_per_rank, int64_t num_ranks,
+                         int64_t max_len, int64_t alignment, int64_t* perm, int32_t* m_sizes,
+                         int32_t* m_offsets, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MXFP8_H_ */

@@ -1,0 +1,366 @@
+"""CPU oracle for the MXFP8 linear path.  TEST INFRASTRUCTURE ONLY.
+
+This module is the checker for the HIP kernels: only tests, the smoke check and the
+benchmark's CPU-baseline leg may import it.  The product never routes through it.
+
+It restates, in NumPy integer/float32 arithmetic, the path that the reference's MXFP8
+converter hands to an external library (reference call site:
+torchtitan/components/quantization/mx.py:100-125; format statement docs/mxfp8.md:31-37;
+block-size constant torchtitan/components/quantization/__init__.py:36).  That library
+(torchao, unpinned: "--pre" nightly in .github/workflows/unit_test_cpu.yaml:33,
+"v0.14.0 or newer" in docs/mxfp8.md:27) is absent from the reference tree, so every
+function here is written from the OCP Microscaling (MX) v1.0 block format:
+
+  * element type  e4m3fn : S EEEE MMM, bias 7, max 448, no inf, 0x7F/0xFF = NaN
+  * scale type    E8M0   : byte b means 2**(b-127), b = 255 means NaN
+  * block         32 consecutive elements along the contraction dim share one scale
+
+Pinning status (what fixes each function independently of its own formula):
+
+  e4m3_encode / e4m3_decode  pinned  -- torch's CPU float8_e4m3fn cast (library routine),
+                                        exhaustive over all bf16 inputs; decode/encode
+                                        round trip over all 256 codes
+  bf16 <-> f32               pinned  -- torch's CPU bfloat16 cast, exhaustive
+  scale byte FLOOR / RCEIL   pinned for finite normal amax by the closed forms
+                                        floor(log2 amax) - 8 and ceil(log2(amax/448))
+                                        evaluated in float64 over every bf16 amax, plus the
+                                        hand-computed known answers in tests/golden
+                             PARITY UNPINNED for: amax = 0 / subnormal / inf / NaN, the
+                                        clamp of the scale byte at 0, and which of
+                                        FLOOR / RCEIL the reference recipe means at a given
+                                        call site (the converter asks for "mxfp8_rceil",
+                                        mx.py:37-42); no reference test holds a vector
+  cast_dim1                  pinned  -- by definition equal to cast_dim0 of the transpose
+  mx_matmul                  pinned  -- textbook: exact dequantize, float64 matmul, special
+                                        cases (unit scales, one-hot operands, K = 32)
+  grouped variants           pinned  -- loop of mx_matmul over groups, the shape of the
+                                        reference's own per-expert loop
+                                        (torchtitan/models/common/moe/moe.py:24-56)
+  generate_permute_indices   pinned  -- the worked example and invariants of
+                                        torchtitan/models/common/moe/kernels.py:145-218
+                                        and tests/unit_tests/test_permute_indices_kernel.py
+
+bf16 tensors are carried as uint16 bit patterns, fp8 codes and scales as uint8.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+BLOCK = 32  # torchtitan/components/quantization/__init__.py:36 (MXFP8_GROUP_ALIGNMENT_SIZE)
+FLOOR = 0
+RCEIL = 1
+E4M3_MAX = 448.0
+E4M3_EMAX = 8  # 448 = 1.75 * 2**8
+
+
+# --------------------------------------------------------------------------- formats
+def bf16_bits_to_f32(bits: np.ndarray) -> np.ndarray:
+    """bf16 is the top half of an IEEE float32."""
+    return (np.ascontiguousarray(bits).astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
+def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:
+    """Round-to-nearest-even narrowing of float32 to bf16 bit patterns (NaN stays NaN)."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    nan = (u & np.uint32(0x7FFFFFFF)) > np.uint32(0x7F800000)
+    lsb = (u >> np.uint32(16)) & np.uint32(1)
+    r = ((u.astype(np.uint64) + np.uint64(0x7FFF) + lsb) >> np.uint64(16)).astype(np.uint16)
+    quiet = ((u >> np.uint32(16)) | np.uint32(0x0040)).astype(np.uint16)
+    return np.where(nan, quiet, r)
+
+
+def e4m3_decode_table() -> np.ndarray:
+    """Value of each of the 256 e4m3fn codes, from the format definition."""
+    t = np.zeros(256, dtype=np.float32)
+    for c in range(256):
+        s = -1.0 if c & 0x80 else 1.0
+        e = (c >> 3) & 0xF
+        m = c & 0x7
+        if e == 0xF and m == 0x7:
+            v = float("nan")
+        elif e == 0:
+            v = s * m * 2.0 ** -9
+        else:
+            v = s * (1.0 + m / 8.0) * 2.0 ** (e - 7)
+        t[c] = v
+    return t
+
+
+_E4M3_TABLE = e4m3_decode_table()
+
+
+def e4m3_decode(codes: np.ndarray) -> np.ndarray:
+    return _E4M3_TABLE[codes]
+
+
+def e4m3_encode(y: np.ndarray) -> np.ndarray:
+    """Saturating round-to-nearest-even narrowing float32 -> e4m3fn code.
+
+    |y| > 448 (inf included) saturates to 0x7E; NaN gives 0x7F; the sign bit is kept,
+    so -0.0 gives 0x80.
+    """
+    y = np.ascontiguousarray(y, dtype=np.float32)
+    u = y.view(np.uint32)
+    sign = ((u >> np.uint32(24)) & np.uint32(0x80)).astype(np.uint8)
+    a = u & np.uint32(0x7FFFFFFF)
+    nan = a > np.uint32(0x7F800000)
+    a = np.minimum(a, np.uint32(0x43E00000))  # 448.0f
+    # normal e4m3 range: keep 3 mantissa bits with ties-to-even, then rebias 127 -> 7
+    lsb = (a >> np.uint32(20)) & np.uint32(1)
+    rn = (a + np.uint32(0x7FFFF) + lsb) >> np.uint32(20)
+    normal = (rn - np.uint32(120 << 3)).astype(np.int64)
+    # below 2**-6 the code is the integer number of 2**-9 steps, ties-to-even
+    mag = a.view(np.float32)
+    sub = np.rint(mag * np.float32(512.0)).astype(np.int64)
+    code = np.where(a < np.uint32(0x3C800000), sub, normal)
+    code = np.where(nan, 0x7F, code).astype(np.uint8)
+    return code | sign
+
+
+# --------------------------------------------------------------------------- scales
+def scale_from_amax_bits(amax_bits: np.ndarray, mode: int) -> np.ndarray:
+    """E8M0 byte for a block whose max |x| has bf16 bit pattern `amax_bits` (sign clear).
+
+    FLOOR: s = floor(log2 amax) - 8, read off the exponent field.
+    RCEIL: s = ceil(log2(amax / 448)) = E - 8 + [mantissa > 0.75] for amax = (1+m) 2**E.
+    Both clamp s to [-127, 127]; byte = s + 127; NaN amax -> 255; amax = 0 -> 0.
+    Unpinned corners, fixed here: a subnormal amax is treated as E = -127 (FLOOR) or by
+    its true log2 (RCEIL, always clamps to byte 0); amax = inf follows the same integer
+    formula as a finite value with exponent field 255.
+    """
+    a = amax_bits.astype(np.int64)
+    expf = a >> 7
+    man = a & 0x7F
+    if mode == FLOOR:
+        s = expf - 127 - E4M3_EMAX
+    elif mode == RCEIL:
+        s = expf - 127 - E4M3_EMAX + (man > 0x60)
+    else:
+        raise ValueError(f"unknown scale mode {mode}")
+    s = np.clip(s, -127, 127)
+    byte = s + 127
+    byte = np.where(a == 0, 0, byte)
+    byte = np.where(a > 0x7F80, 255, byte)
+    return byte.astype(np.uint8)
+
+
+def _multiplier_from_scale(byte: np.ndarray, mode: int) -> np.ndarray:
+    """float32 factor 2**(-s) applied to the block before narrowing.
+
+    For byte 0 the factor is 2**126 in FLOOR mode (the divisor is held at the smallest
+    normal float32) and 1.0 in RCEIL mode; both only reachable for amax <= 2**-119.
+    For byte 255 (NaN block) the factor is 0, so finite lanes become signed zeros and
+    NaN lanes stay NaN.
+    """
+    b = byte.astype(np.int64)
+    e = 127 - b  # -s
+    mult_bits = ((e + 127) << 23).astype(np.uint32)
+    mult = mult_bits.view(np.float32).copy()
+    if mode == FLOOR:
+        mult = np.where(b == 0, np.float32(2.0 ** 126), mult)
+    else:
+        mult = np.where(b == 0, np.float32(1.0), mult)
+    mult = np.where(b == 254, np.float32(2.0 ** -127), mult)  # subnormal factor
+    mult = np.where(b == 255, np.float32(0.0), mult)
+    return mult.astype(np.float32)
+
+
+# --------------------------------------------------------------------------- casts
+def cast_dim0(x_bits: np.ndarray, mode: int = FLOOR):
+    """Row-wise to_mx: bf16 [R, C] -> (codes u8 [R, C], scales u8 [R, C/32]).
+
+    Blocks of 32 run along the last (contiguous) dimension.
+    """
+    x_bits = np.ascontiguousarray(x_bits, dtype=np.uint16)
+    R, C = x_bits.shape
+    if C % BLOCK:
+        raise ValueError("last dim must be a multiple of 32")
+    blk = x_bits.reshape(R, C // BLOCK, BLOCK)
+    amax_bits = (blk & np.uint16(0x7FFF)).max(axis=-1)
+    scales = scale_from_amax_bits(amax_bits, mode)
+    mult = _multiplier_from_scale(scales, mode)
+    with np.errstate(invalid="ignore", over="ignore"):
+        y = bf16_bits_to_f32(blk) * mult[..., None]
+    # inf * 0 above would give NaN for an inf lane in a NaN block; keep it a signed zero
+    inf_lane = (blk & np.uint16(0x7FFF)) == np.uint16(0x7F80)
+    nan_blk = (scales == 255)[..., None]
+    y = np.where(inf_lane & nan_blk, np.copysign(np.float32(0), bf16_bits_to_f32(blk)), y)
+    codes = e4m3_encode(y.astype(np.float32)).reshape(R, C)
+    return codes, scales
+
+
+def cast_dim1(x_bits: np.ndarray, mode: int = FLOOR):
+    """Column-wise to_mx: bf16 [R, C] -> (codes u8 [C, R], scales u8 [C, R/32]).
+
+    Blocks of 32 run down the first dimension; outputs are stored transposed so the
+    quantized axis is contiguous.
+    """
+    return cast_dim0(np.ascontiguousarray(np.asarray(x_bits).T), mode)
+
+
+def dequant(codes: np.ndarray, scales: np.ndarray) -> np.ndarray:
+    """float32 value of MX data: e4m3 value times 2**(scale-127), blocks along last dim."""
+    R, C = codes.shape
+    v = e4m3_decode(codes).reshape(R, C // BLOCK, BLOCK).astype(np.float64)
+    s = np.where(scales == 255, np.nan, np.exp2(scales.astype(np.float64) - 127.0))
+    return (v * s[..., None]).reshape(R, C).astype(np.float32)
+
+
+# --------------------------------------------------------------------------- matmul
+def mx_matmul_q(a_codes, a_scales, b_codes, b_scales, accumulate=np.float32) -> np.ndarray:
+    """bf16 bits of  deq(A)[M,K] @ deq(B)[N,K]^T  with `accumulate`-precision sums."""
+    a = dequant(a_codes, a_scales).astype(accumulate)
+    b = dequant(b_codes, b_scales).astype(accumulate)
+    return f32_to_bf16_bits((a @ b.T).astype(np.float32))
+
+
+def mx_matmul(a_bits: np.ndarray, b_bits: np.ndarray, mode: int = FLOOR, accumulate=np.float32):
+    """Emulated MXFP8 product of bf16 A[M,K] and B[N,K], both quantized along K."""
+    ac, asc = cast_dim0(a_bits, mode)
+    bc, bsc = cast_dim0(b_bits, mode)
+    return mx_matmul_q(ac, asc, bc, bsc, accumulate)
+
+
+def linear_fwd(x_bits, w_bits, mode=FLOOR):
+    """Y[M,N] = X[M,K] W[N,K]^T, both cast along K."""
+    return mx_matmul(x_bits, w_bits, mode)
+
+
+def linear_dgrad(dy_bits, w_bits, mode=FLOOR):
+    """dX[M,K] = dY[M,N] W[N,K]: dY cast along N (dim0), W cast along N (dim1)."""
+    ac, asc = cast_dim0(dy_bits, mode)
+    bc, bsc = cast_dim1(w_bits, mode)
+    return mx_matmul_q(ac, asc, bc, bsc)
+
+
+def linear_wgrad(dy_bits, x_bits, mode=FLOOR):
+    """dW[N,K] = dY[M,N]^T X[M,K]: both cast along M (dim1)."""
+    ac, asc = cast_dim1(dy_bits, mode)
+    bc, bsc = cast_dim1(x_bits, mode)
+    return mx_matmul_q(ac, asc, bc, bsc)
+
+
+# --------------------------------------------------------------------------- grouped
+def _group_bounds(offs):
+    offs = [int(o) for o in offs]
+    return list(zip([0] + offs[:-1], offs))
+
+
+def grouped_fwd(x_bits, w_bits, offs, mode=FLOOR):
+    """Y[rows of group g] = mx_matmul(X[rows of g], W[g]); rows >= offs[-1] give zeros.
+
+    x_bits [T, K], w_bits [E, N, K], offs = int32 inclusive cumulative group sizes
+    (the `offs` argument of torch._grouped_mm at torchtitan/models/common/moe/moe.py:66-74).
+    """
+    T = x_bits.shape[0]
+    E, N, K = w_bits.shape
+    out = np.zeros((T, N), dtype=np.uint16)
+    for g, (lo, hi) in enumerate(_group_bounds(offs)):
+        if hi > lo:
+            out[lo:hi] = mx_matmul(x_bits[lo:hi], w_bits[g], mode)
+    return out
+
+
+def grouped_dgrad(dy_bits, w_bits, offs, mode=FLOOR):
+    """dX[rows of g] = deq(dY_g cast along N) @ deq(W_g cast along N)."""
+    T = dy_bits.shape[0]
+    E, N, K = w_bits.shape
+    out = np.zeros((T, K), dtype=np.uint16)
+    for g, (lo, hi) in enumerate(_group_bounds(offs)):
+        if hi > lo:
+            out[lo:hi] = linear_dgrad(dy_bits[lo:hi], w_bits[g], mode)
+    return out
+
+
+def grouped_wgrad(dy_bits, x_bits, offs, mode=FLOOR):
+    """dW[g][N,K] = deq(dY_g cast along tokens)^T @ deq(X_g cast along tokens).
+
+    Every group size must be a multiple of 32 so no block straddles a group boundary
+    (torchtitan/models/common/moe/utils.py:47-52).  Empty groups give zeros.
+    """
+    N = dy_bits.shape[1]
+    K = x_bits.shape[1]
+    bounds = _group_bounds(offs)
+    out = np.zeros((len(bounds), N, K), dtype=np.uint16)
+    for g, (lo, hi) in enumerate(bounds):
+        if (hi - lo) % BLOCK:
+            raise ValueError("group sizes must be multiples of 32")
+        if hi > lo:
+            out[g] = linear_wgrad(dy_bits[lo:hi], x_bits[lo:hi], mode)
+    return out
+
+
+# --------------------------------------------------------------------------- scale layout
+def scale_layout(scales: np.ndarray) -> np.ndarray:
+    """Permute a [rows, nblk] scale matrix into the order the MFMA loop reads.
+
+    Output is [ceil(rows/64), ceil(nblk/4), 64, 4] bytes: for row-tile rt, K-step ks,
+    lane l and byte t the entry is scales[rt*64 + t*16 + (l & 15)][ks*4 + (l >> 4)],
+    zero where that index is out of range.  One aligned dword per lane then holds the
+    scales of the lane's K-block for four consecutive 16-row sub-tiles.
+    """
+    rows, nblk = scales.shape
+    rt_n = (rows + 63) // 64
+    ks_n = (nblk + 3) // 4
+    padded = np.zeros((rt_n * 64, ks_n * 4), dtype=np.uint8)
+    padded[:rows, :nblk] = scales
+    # [rt, t, i, ks, j] -> [rt, ks, j, i, t]
+    v = padded.reshape(rt_n, 4, 16, ks_n, 4)
+    return np.ascontiguousarray(v.transpose(0, 3, 4, 2, 1)).reshape(rt_n, ks_n, 64, 4)
+
+
+def scale_unlayout(laid: np.ndarray, rows: int, nblk: int) -> np.ndarray:
+    rt_n, ks_n = laid.shape[:2]
+    v = laid.reshape(rt_n, ks_n, 4, 16, 4).transpose(0, 4, 3, 1, 2)
+    return np.ascontiguousarray(v).reshape(rt_n * 64, ks_n * 4)[:rows, :nblk]
+
+
+# --------------------------------------------------------------------------- group padding
+def round_up(x: int, a: int) -> int:
+    return (x + a - 1) // a * a
+
+
+def generate_permute_indices(tokens_per_expert_group, experts_per_rank, num_ranks, max_len, alignment):
+    """Index map from routed-token order to expert-grouped, alignment-padded order.
+
+    Follows torchtitan/models/common/moe/kernels.py:145-218 (sizes/offsets) and :108-142
+    (the fill): returns (permuted_indices int64 [max_len] with -1 in padding slots,
+    m_sizes int32 [experts_per_rank], m_offsets int32 inclusive cumsum).
+    """
+    t = np.asarray(tokens_per_expert_group, dtype=np.int64)
+    start = np.cumsum(t) - t
+    total = t.reshape(num_ranks, -1).sum(0)
+    total = np.maximum(total, alignment)
+    m_sizes = ((total + alignment - 1) // alignment * alignment).astype(np.int32)
+    m_offsets = np.cumsum(m_sizes.astype(np.int64))
+    write = m_offsets - m_sizes
+    perm = np.full(max_len, -1, dtype=np.int64)
+    for e in range(experts_per_rank):
+        ws = int(write[e])
+        for r in range(num_ranks):
+            i = r * experts_per_rank + e
+            n = int(t[i])
+            if n > 0:
+                end = min(ws + n, max_len)
+                if ws < end:
+                    perm[ws:end] = np.arange(start[i], start[i] + (end - ws))
+            ws += n
+    return perm, m_sizes, m_offsets.astype(np.int32)
+
+
+def padded_max_len(num_tokens: int, num_experts: int, alignment: int) -> int:
+    """torchtitan/models/common/moe/utils.py:66-68."""
+    return round_up(num_tokens + num_experts * alignment, alignment)
+
+
+# --------------------------------------------------------------------------- inputs
+def make_cfg1_inputs(seed: int, M: int = 8192, K: int = 4096, N: int = 4096):
+    """Seeded N(0,1) bf16 X[M,K], W[N,K] with 0.1 % of entries scaled by 100."""
+    rng = np.random.default_rng(seed)
+
+    def one(r, c):
+        x = rng.standard_normal((r, c), dtype=np.float32)
+        x = np.where(rng.random((r, c)) < 1e-3, x * np.float32(100.0), x)
+        return f32_to_bf16_bits(x)
+
+    return one(M, K), one(N, K)

@@ -1,0 +1,154 @@
+"""GPU parity: HIP to_mx casts vs the CPU oracle, bit-exact (codes and scale bytes)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import mx_oracle as mo
+from tests.helpers import bf16_from_bits, bits_of, randn_bits, u8
+from torchtitan_amd import ops
+
+pytestmark = pytest.mark.gpu
+
+MODES = [("floor", mo.FLOOR), ("rceil", mo.RCEIL)]
+
+
+def _check_dim0(bits, mode_name, mode, device):
+    x = bf16_from_bits(bits, device)
+    got = ops.to_mx_dim0(x, mode_name)
+    codes, scales = mo.cast_dim0(bits, mode)
+    assert np.array_equal(u8(got.scales), scales), "scale bytes differ"
+    assert np.array_equal(u8(got.codes), codes), "codes differ"
+    laid = ops.to_mx_dim0(x, mode_name, ops.MX_SCALES_MFMA)
+    assert np.array_equal(u8(laid.codes), codes)
+    assert np.array_equal(u8(laid.scales).reshape(-1), mo.scale_layout(scales).reshape(-1))
+
+
+def _check_dim1(bits, mode_name, mode, device):
+    x = bf16_from_bits(bits, device)
+    got = ops.to_mx_dim1(x, mode_name)
+    codes, scales = mo.cast_dim1(bits, mode)
+    assert np.array_equal(u8(got.scales), scales), "scale bytes differ"
+    assert np.array_equal(u8(got.codes), codes), "codes differ"
+    laid = ops.to_mx_dim1(x, mode_name, ops.MX_SCALES_MFMA)
+    assert np.array_equal(u8(laid.codes), codes)
+    assert np.array_equal(u8(laid.scales).reshape(-1), mo.scale_layout(scales).reshape(-1))
+
+
+def _check_fused(bits, mode_name, mode, device):
+    x = bf16_from_bits(bits, device)
+    for order in (ops.MX_SCALES_ROWMAJOR, ops.MX_SCALES_MFMA):
+        r, c = ops.to_mx_dim0_dim1(x, mode_name, order)
+        c0, s0 = mo.cast_dim0(bits, mode)
+        c1, s1 = mo.cast_dim1(bits, mode)
+        if order == ops.MX_SCALES_MFMA:
+            s0, s1 = mo.scale_layout(s0).reshape(-1), mo.scale_layout(s1).reshape(-1)
+        assert np.array_equal(u8(r.codes), c0) and np.array_equal(u8(c.codes), c1)
+        assert np.array_equal(u8(r.scales).reshape(-1), s0.reshape(-1))
+        assert np.array_equal(u8(c.scales).reshape(-1), s1.reshape(-1))
+
+
+@pytest.mark.parametrize("mode_name,mode", MODES)
+def test_every_bf16_value_as_amax_dim0(device, mode_name, mode):
+    """All 65536 bf16 patterns as the first lane of a block, three fill patterns for the rest."""
+    allv = np.arange(65536, dtype=np.uint16)
+    rng = np.random.default_rng(0)
+    for fill in ("zero", "half", "random"):
+        blk = np.zeros((65536, 32), dtype=np.uint16)
+        blk[:, 0] = allv
+        if fill == "half":  # other lanes: amax / 2 with alternating sign (exponent - 1)
+            e = (allv >> 7) & 0xFF
+            half = np.where(e > 1, allv - np.uint16(0x80), np.uint16(0)) & np.uint16(0x7FFF)
+            half = np.where((allv & 0x7FFF) > 0x7F80, np.uint16(0x3F80), half)
+            blk[:, 1:] = half[:, None] ^ (np.arange(31, dtype=np.uint16)[None, :] % 2 * 0x8000)
+        elif fill == "random":
+            blk[:, 1:] = rng.integers(0, 65536, size=(65536, 31), dtype=np.uint16)
+        _check_dim0(blk.reshape(512, 4096), mode_name, mode, device)
+
+
+@pytest.mark.parametrize("mode_name,mode", MODES)
+def test_every_bf16_value_dim1(device, mode_name, mode):
+    """Same sweep through the column-wise kernel: blocks run down 32 rows."""
+    rng = np.random.default_rng(1)
+    blk = rng.integers(0, 65536, size=(65536, 32), dtype=np.uint16)
+    blk[:, 0] = np.arange(65536, dtype=np.uint16)
+    # lay the 65536 blocks out as columns: x[32*g + k, c] = blk[g*512 + c, k]
+    x = np.ascontiguousarray(blk.reshape(128, 512, 32).transpose(0, 2, 1)).reshape(128 * 32, 512)
+    _check_dim1(x, mode_name, mode, device)
+    _check_fused(x, mode_name, mode, device)
+
+
+@pytest.mark.parametrize("mode_name,mode", MODES)
+@pytest.mark.parametrize("shape", [(32, 32), (64, 96), (96, 64), (160, 224), (128, 128),
+                                   (256, 4096), (1024, 768), (416, 2048), (32, 14336)])
+def test_shapes_with_outliers(device, mode_name, mode, shape):
+    rng = np.random.default_rng(hash(shape) & 0xFFFF)
+    bits = randn_bits(rng, shape, outliers=1e-3)
+    _check_dim0(bits, mode_name, mode, device)
+    _check_dim1(bits, mode_name, mode, device)
+    _check_fused(bits, mode_name, mode, device)
+
+
+def test_dim1_equals_dim0_of_transpose(device):
+    rng = np.random.default_rng(7)
+    bits = randn_bits(rng, (512, 1024), outliers=1e-3)
+    x = bf16_from_bits(bits, device)
+    a = ops.to_mx_dim1(x, "rceil")
+    b = ops.to_mx_dim0(x.t().contiguous(), "rceil")
+    assert torch.equal(a.codes, b.codes) and torch.equal(a.scales, b.scales)
+
+
+def test_strided_input_rows(device):
+    rng = np.random.default_rng(8)
+    bits = randn_bits(rng, (128, 512))
+    x = bf16_from_bits(bits, device)
+    view = x[:, :256]  # row stride 512, 256 columns
+    got = ops.to_mx_dim0(view, "floor")
+    codes, scales = mo.cast_dim0(bits[:, :256], mo.FLOOR)
+    assert np.array_equal(u8(got.codes), codes) and np.array_equal(u8(got.scales), scales)
+    got1 = ops.to_mx_dim1(view, "floor")
+    codes1, scales1 = mo.cast_dim1(bits[:, :256], mo.FLOOR)
+    assert np.array_equal(u8(got1.codes), codes1) and np.array_equal(u8(got1.scales), scales1)
+
+
+def test_scale_layout_round_trip(device):
+    rng = np.random.default_rng(9)
+    for rows, nblk in [(64, 4), (100, 7), (256, 128), (4096, 448), (33, 1)]:
+        s = rng.integers(0, 256, size=(rows, nblk), dtype=np.uint8)
+        t = torch.from_numpy(s).to(device)
+        laid = ops.scale_layout(t)
+        assert np.array_equal(u8(laid), mo.scale_layout(s).reshape(-1))
+        back = ops.scale_unlayout(laid, rows, nblk)
+        assert np.array_equal(u8(back), s)
+
+
+def test_empty_and_errors(device):
+    x = torch.empty((0, 64), dtype=torch.bfloat16, device=device)
+    out = ops.to_mx_dim0(x)
+    assert out.codes.shape == (0, 64)
+    with pytest.raises(ValueError):
+        ops.to_mx_dim0(torch.zeros((4, 48), dtype=torch.bfloat16, device=device))
+    with pytest.raises(ValueError):
+        ops.to_mx_dim1(torch.zeros((48, 64), dtype=torch.bfloat16, device=device))
+    with pytest.raises(TypeError):
+        ops.to_mx_dim0(torch.zeros((4, 64), dtype=torch.float32, device=device))
+    with pytest.raises(Exception):
+        ops.to_mx_dim0(torch.zeros((4, 64), dtype=torch.bfloat16))  # CPU tensor: no fallback
+
+
+def test_full_size_properties(device):
+    """BASELINE-size tensor: properties that need no CPU oracle pass over the whole tensor."""
+    torch.manual_seed(0)
+    x = torch.randn((16384, 4096), device=device, dtype=torch.bfloat16)
+    r, c = ops.to_mx_dim0_dim1(x, "floor")
+    r2 = ops.to_mx_dim0(x, "floor")
+    c2 = ops.to_mx_dim1(x, "floor")
+    assert torch.equal(r.codes, r2.codes) and torch.equal(r.scales, r2.scales)
+    assert torch.equal(c.codes, c2.codes) and torch.equal(c.scales, c2.scales)
+    # idempotence under transpose
+    ct = ops.to_mx_dim0(x.t().contiguous(), "floor")
+    assert torch.equal(ct.codes, c.codes) and torch.equal(ct.scales, c.scales)
+    # the oracle on a slice
+    sl = bits_of(x[4096:4096 + 64])
+    codes, scales = mo.cast_dim0(sl, mo.FLOOR)
+    assert np.array_equal(u8(r.codes[4096:4096 + 64]), codes)
+    assert np.array_equal(u8(r.scales[4096:4096 + 64]), scales)

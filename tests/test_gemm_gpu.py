@@ -1,0 +1,124 @@
+"""GPU parity: MXFP8 GEMM vs the oracle's emulated MX matmul (rel-L2 <= 1e-3, bf16 both sides)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import mx_oracle as mo
+from tests.helpers import bf16_from_bits, bits_of, randn_bits, rel_l2, u8
+from torchtitan_amd import ops
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-3  # north-star tolerance: rel-L2, fp32 accumulate, bf16 out on both sides
+
+
+def _gemm_from_codes(ac, asc, bc, bsc, device):
+    a = ops.MXData(torch.from_numpy(ac).to(device), torch.from_numpy(asc).to(device), ops.MX_SCALES_ROWMAJOR)
+    b = ops.MXData(torch.from_numpy(bc).to(device), torch.from_numpy(bsc).to(device), ops.MX_SCALES_ROWMAJOR)
+    return ops.mx_gemm_nt(a, b)
+
+
+def _f32(bits):
+    return mo.bf16_bits_to_f32(bits)
+
+
+@pytest.mark.parametrize("M,N,K", [(16, 16, 32), (16, 16, 128), (64, 64, 128), (128, 128, 256),
+                                   (256, 256, 128), (256, 256, 512), (512, 768, 1024),
+                                   (300, 200, 160), (257, 129, 96), (1000, 1000, 2048),
+                                   (2048, 1024, 4096)])
+def test_gemm_matches_oracle(device, M, N, K):
+    rng = np.random.default_rng(M * 7 + N * 3 + K)
+    a_bits = randn_bits(rng, (M, K), outliers=1e-3)
+    b_bits = randn_bits(rng, (N, K), std=0.02)
+    ac, asc = mo.cast_dim0(a_bits, mo.FLOOR)
+    bc, bsc = mo.cast_dim0(b_bits, mo.FLOOR)
+    ref = mo.mx_matmul_q(ac, asc, bc, bsc)
+    got = _gemm_from_codes(ac, asc, bc, bsc, device)
+    err = rel_l2(_f32(bits_of(got)), _f32(ref))
+    assert err <= TOL, f"rel-L2 {err}"
+
+
+def test_one_hot_picks_single_products(device):
+    """A = one-hot rows: D[m, n] must equal deq(A)[m, k_m] * deq(B)[n, k_m] rounded to bf16."""
+    rng = np.random.default_rng(3)
+    M, N, K = 128, 64, 256
+    a = np.zeros((M, K), dtype=np.float32)
+    ks = rng.integers(0, K, size=M)
+    a[np.arange(M), ks] = rng.choice([1.0, -2.0, 0.5, 3.0], size=M)
+    a_bits = mo.f32_to_bf16_bits(a)
+    b_bits = randn_bits(rng, (N, K))
+    ac, asc = mo.cast_dim0(a_bits, mo.RCEIL)
+    bc, bsc = mo.cast_dim0(b_bits, mo.RCEIL)
+    da, db = mo.dequant(ac, asc), mo.dequant(bc, bsc)
+    expect = mo.f32_to_bf16_bits(da[np.arange(M), ks][:, None] * db[:, ks].T)
+    got = bits_of(_gemm_from_codes(ac, asc, bc, bsc, device))
+    assert np.array_equal(got, expect)
+
+
+def test_unit_scales_reduce_to_plain_fp8(device):
+    """All scale bytes 127: the result is the plain e4m3 x e4m3 product sum (exact in fp32 here)."""
+    rng = np.random.default_rng(4)
+    M, N, K = 64, 64, 128
+    ac = rng.integers(0, 0x40, size=(M, K), dtype=np.uint8)  # small positive codes, exact sums
+    bc = rng.integers(0, 0x40, size=(N, K), dtype=np.uint8)
+    asc = np.full((M, K // 32), 127, dtype=np.uint8)
+    bsc = np.full((N, K // 32), 127, dtype=np.uint8)
+    ref = mo.f32_to_bf16_bits((mo.e4m3_decode(ac).astype(np.float64) @ mo.e4m3_decode(bc).astype(np.float64).T).astype(np.float32))
+    got = bits_of(_gemm_from_codes(ac, asc, bc, bsc, device))
+    assert np.array_equal(got, ref)
+
+
+def test_scale_blocks_map_to_the_right_k(device):
+    """Distinct power-of-two scale per (row, block): any mis-mapped scale changes the result."""
+    M, N, K = 64, 32, 256
+    ac = np.full((M, K), 0x38, dtype=np.uint8)  # 1.0
+    bc = np.full((N, K), 0x38, dtype=np.uint8)
+    asc = (120 + (np.arange(M)[:, None] % 5) + np.arange(K // 32)[None, :]).astype(np.uint8)
+    bsc = (118 + (np.arange(N)[:, None] % 3) * 2 + (np.arange(K // 32)[None, :] % 4)).astype(np.uint8)
+    ref = mo.mx_matmul_q(ac, asc, bc, bsc, accumulate=np.float64)
+    got = bits_of(_gemm_from_codes(ac, asc, bc, bsc, device))
+    assert np.array_equal(got, ref)
+
+
+def test_linear_passes_end_to_end(device):
+    """fwd, dgrad, wgrad built from the HIP casts + GEMM vs the oracle's three passes."""
+    rng = np.random.default_rng(5)
+    M, K, N = 512, 256, 384
+    x_bits = randn_bits(rng, (M, K), outliers=1e-3)
+    w_bits = randn_bits(rng, (N, K), std=0.02)
+    dy_bits = randn_bits(rng, (M, N), std=1e-3)
+    x, w, dy = (bf16_from_bits(b, device) for b in (x_bits, w_bits, dy_bits))
+    L = ops.MX_SCALES_MFMA
+    for mode_name, mode in (("floor", mo.FLOOR), ("rceil", mo.RCEIL)):
+        y = ops.mx_gemm_nt(ops.to_mx_dim0(x, mode_name, L), ops.to_mx_dim0(w, mode_name, L))
+        dx = ops.mx_gemm_nt(ops.to_mx_dim0(dy, mode_name, L), ops.to_mx_dim1(w, mode_name, L))
+        dw = ops.mx_gemm_nt(ops.to_mx_dim1(dy, mode_name, L), ops.to_mx_dim1(x, mode_name, L))
+        assert rel_l2(_f32(bits_of(y)), _f32(mo.linear_fwd(x_bits, w_bits, mode))) <= TOL
+        assert rel_l2(_f32(bits_of(dx)), _f32(mo.linear_dgrad(dy_bits, w_bits, mode))) <= TOL
+        assert rel_l2(_f32(bits_of(dw)), _f32(mo.linear_wgrad(dy_bits, x_bits, mode))) <= TOL
+
+
+def test_full_size_linearity(device):
+    """8B-FFN shape: D(A, B) rows are independent and scale-linear.
+
+    Doubling every A scale byte (+1) must exactly double D (power-of-two scaling commutes with
+    fp32 accumulation and bf16 rounding), and a row slice of the big GEMM must equal the GEMM of
+    the slice -- both hold for any correct kernel at any size, without a CPU pass.
+    """
+    torch.manual_seed(1)
+    M, K, N = 16384, 4096, 14336
+    x = torch.randn((M, K), device=device, dtype=torch.bfloat16)
+    w = torch.randn((N, K), device=device, dtype=torch.bfloat16) * 0.02
+    a = ops.to_mx_dim0(x, "floor")
+    b = ops.to_mx_dim0(w, "floor")
+    d = ops.mx_gemm_nt(a, b)
+    a2 = ops.MXData(a.codes, a.scales + 1, a.scale_order)
+    d2 = ops.mx_gemm_nt(a2, b)
+    assert torch.equal(d2, d * 2)
+    rows = slice(5000, 5000 + 192)
+    ds = ops.mx_gemm_nt(ops.MXData(a.codes[rows].contiguous(), a.scales[rows].contiguous(), a.scale_order), b)
+    assert torch.equal(ds, d[rows])
+    # a 64x96 corner against the oracle
+    ref = mo.mx_matmul_q(u8(a.codes[:64]), u8(a.scales[:64]), u8(b.codes[:96]), u8(b.scales[:96]))
+    err = rel_l2(_f32(bits_of(d[:64, :96])), _f32(ref))
+    assert err <= TOL

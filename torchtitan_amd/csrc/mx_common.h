@@ -1,0 +1,92 @@
+// Shared device helpers for the gfx950 MXFP8 kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "mxfp8.h"
+
+namespace mx {
+
+constexpr int kBlock = 32;  // elements per E8M0 scale
+
+typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+  us2 x = __builtin_bit_cast(us2, a), y = __builtin_bit_cast(us2, b);
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(x, y));
+}
+
+// Lane exchange inside a quad / row through DPP (no LDS traffic).
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, false);
+}
+constexpr int kQuadXor1 = 0xB1;  // quad_perm:[1,0,3,2]
+constexpr int kQuadXor2 = 0x4E;  // quad_perm:[2,3,0,1]
+
+// E8M0 byte from the bf16 bit pattern of the block's max magnitude (sign bit clear).
+//   FLOOR: floor(log2 amax) - 8          RCEIL: ceil(log2(amax / 448))
+// both read off the exponent / mantissa fields, clamped to [0, 254]; amax == 0 -> 0,
+// NaN -> 255.
+template <int MODE>
+__device__ __forceinline__ uint32_t scale_byte(uint32_t amax_bits) {
+  int expf = (int)(amax_bits >> 7);
+  int b = expf - 8;
+  if (MODE == MX_SCALE_RCEIL) b += ((amax_bits & 0x7F) > 0x60) ? 1 : 0;
+  b = b < 0 ? 0 : (b > 254 ? 254 : b);
+  if (amax_bits == 0) b = 0;
+  if (amax_bits > 0x7F80) b = 255;
+  return (uint32_t)b;
+}
+
+// float factor 2^(127 - byte) applied before narrowing; byte 0 -> 2^126 (FLOOR) or 1
+// (RCEIL); byte 255 (NaN block) -> 0.
+template <int MODE>
+__device__ __forceinline__ float scale_multiplier(uint32_t byte) {
+  uint32_t bits = (254u - byte) << 23;
+  if (byte == 0) bits = (MODE == MX_SCALE_FLOOR) ? 0x7E800000u : 0x3F800000u;
+  if (byte >= 254) bits = (byte == 254) ? 0x00400000u : 0u;
+  return __uint_as_float(bits);
+}
+
+// Two bf16 (packed in one dword) -> two saturating e4m3 codes in the low or high half of
+// `old`.  v_med3_f32 clamps to +-448 so the narrowing never overflows; the hardware convert
+// rounds to nearest even, subnormals included.
+template <bool HIGH>
+__device__ __forceinline__ uint32_t cvt2(uint32_t w, float mult, uint32_t old) {
+  float lo = __uint_as_float(w << 16) * mult;
+  float hi = __uint_as_float(w & 0xFFFF0000u) * mult;
+  lo = __builtin_amdgcn_fmed3f(lo, -448.0f, 448.0f);
+  hi = __builtin_amdgcn_fmed3f(hi, -448.0f, 448.0f);
+  return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(lo, hi, (int)old, HIGH);
+}
+
+// Two floats -> two codes (same contract as cvt2, inputs already scaled).
+template <bool HIGH>
+__device__ __forceinline__ uint32_t cvt2f(float lo, float hi, uint32_t old) {
+  lo = __builtin_amdgcn_fmed3f(lo, -448.0f, 448.0f);
+  hi = __builtin_amdgcn_fmed3f(hi, -448.0f, 448.0f);
+  return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(lo, hi, (int)old, HIGH);
+}
+
+// Code of one bf16 lane inside a block whose amax is NaN: NaN lanes keep NaN (0x7F) with
+// their sign, every other lane becomes a signed zero.
+__device__ __forceinline__ uint32_t nan_block_code(uint32_t bf16_bits) {
+  uint32_t sign = (bf16_bits >> 8) & 0x80u;
+  return ((bf16_bits & 0x7FFFu) > 0x7F80u ? 0x7Fu : 0u) | sign;
+}
+__device__ __forceinline__ uint32_t nan_block_codes2(uint32_t w) {
+  return nan_block_code(w & 0xFFFFu) | (nan_block_code(w >> 16) << 8);
+}
+
+// Byte offset of scale (row, blk) in MX_SCALES_MFMA order; ks_n = ceil(nblk / 4).
+__device__ __host__ __forceinline__ int64_t mfma_scale_offset(int64_t row, int64_t blk,
+                                                              int64_t ks_n) {
+  return (((row >> 6) * ks_n + (blk >> 2)) << 8) + ((((blk & 3) << 4) + (row & 15)) << 2) +
+         ((row & 63) >> 4);
+}
+
+}  // namespace mx

@@ -1,0 +1,68 @@
+// Dense MXFP8 GEMM entry point: D[M,N] = deq(A)[M,K] * deq(B)[N,K]^T (bf16 out).
+#include "mx_gemm_tile.h"
+
+namespace mx {
+
+struct DenseArgs {
+  const uint8_t* a_codes;
+  const uint8_t* a_scales;
+  const uint8_t* b_codes;
+  const uint8_t* b_scales;
+  uint16_t* d;
+  int64_t M, N, K, ldd;
+};
+
+template <int BM, int BN>
+__global__ __launch_bounds__(256, 1) void gemm_nt_kernel(DenseArgs p) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  using Tile = GemmTile<BM, BN, false, false>;
+  const int64_t tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+  int64_t tm, tn;
+  if (!map_tile(tiles_m, tiles_n, tm, tn)) return;
+  const int64_t ks_n = (p.K / 32 + 3) / 4;
+  Operand A{p.a_codes + tm * BM * p.K, p.K, p.M - tm * BM,
+            p.a_scales + tm * (BM / 64) * ks_n * 256, ks_n};
+  Operand B{p.b_codes + tn * BN * p.K, p.K, p.N - tn * BN,
+            p.b_scales + tn * (BN / 64) * ks_n * 256, ks_n};
+  Tile::run(smem, A, B, 0, p.K, p.d + tm * BM * p.ldd + tn * BN, p.ldd);
+}
+
+template <int BM, int BN>
+static int launch_dense(const DenseArgs& p, hipStream_t st) {
+  using Tile = GemmTile<BM, BN, false, false>;
+  auto kern = gemm_nt_kernel<BM, BN>;
+  static bool configured = false;  // raising the dynamic-LDS limit is a per-function setting
+  if (!configured) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                            Tile::kLdsBytes) != hipSuccess)
+      return MX_ERR_LAUNCH;
+    configured = true;
+  }
+  const int64_t nb = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+  const int64_t grid = (nb + 7) / 8 * 8;
+  if (grid > 0x7FFFFFFF) return MX_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), Tile::kLdsBytes, st, p);
+  return hipGetLastError() == hipSuccess ? MX_OK : MX_ERR_LAUNCH;
+}
+
+}  // namespace mx
+
+using namespace mx;
+
+extern "C" int mx_gemm_nt(const uint8_t* a_codes, const uint8_t* a_scales,
+                          const uint8_t* b_codes, const uint8_t* b_scales, void* d, int64_t M,
+                          int64_t N, int64_t K, int64_t ldd, void* stream) {
+  if (M < 0 || N < 0 || K < 0 || ldd < N) return MX_ERR_INVALID_ARG;
+  if (M == 0 || N == 0) return MX_OK;
+  if (!a_codes || !a_scales || !b_codes || !b_scales || !d) return MX_ERR_INVALID_ARG;
+  if (K % 32 || K == 0) return MX_ERR_ALIGNMENT;  // K == 0 would need a zero fill: not a linear
+  if (((uintptr_t)a_codes & 15) || ((uintptr_t)b_codes & 15) || ((uintptr_t)a_scales & 3) ||
+      ((uintptr_t)b_scales & 3) || ((uintptr_t)d & 1) || (K % 16))
+    return MX_ERR_ALIGNMENT;
+  if (256 * K > 0x7FFFFFFFll) return MX_ERR_UNSUPPORTED;
+  DenseArgs p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, M, N, K, ldd};
+  hipStream_t st = (hipStream_t)stream;
+  if (M <= 128 || N <= 128) return launch_dense<128, 128>(p, st);
+  return launch_dense<256, 256>(p, st);
+}

@@ -1,0 +1,153 @@
+"""Tensor-level wrappers over the C ABI (include/mxfp8.h).
+
+PyTorch is used for device memory and the current HIP stream only; every computation is a
+call into libmxfp8_gfx950.so.  There is no fallback path: CPU tensors are rejected.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import NamedTuple
+
+import torch
+
+from . import _lib
+from ._lib import MX_SCALE_FLOOR, MX_SCALE_RCEIL, MX_SCALES_MFMA, MX_SCALES_ROWMAJOR
+
+BLOCK = 32  # torchtitan/components/quantization/__init__.py:36
+
+SCALE_MODES = {"floor": MX_SCALE_FLOOR, "rceil": MX_SCALE_RCEIL}
+
+
+class MXData(NamedTuple):
+    """e4m3 codes [rows, cols] (uint8) + E8M0 scales, blocks of 32 along `cols`."""
+
+    codes: torch.Tensor
+    scales: torch.Tensor
+    scale_order: int  # MX_SCALES_ROWMAJOR: [rows, cols/32]; MX_SCALES_MFMA: flat re-laid buffer
+
+
+def _mode(mode) -> int:
+    if isinstance(mode, str):
+        return SCALE_MODES[mode]
+    if mode not in (MX_SCALE_FLOOR, MX_SCALE_RCEIL):
+        raise ValueError(f"unknown scale mode {mode!r}")
+    return int(mode)
+
+
+def _stream(t: torch.Tensor) -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _ptr(t: torch.Tensor) -> ctypes.c_void_p:
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _check_hp(x: torch.Tensor) -> torch.Tensor:
+    if not x.is_cuda:
+        raise _lib.MXLibraryError("the MXFP8 kernels run on the GPU only; got a CPU tensor")
+    if x.dtype != torch.bfloat16:
+        raise TypeError(f"to_mx expects bfloat16, got {x.dtype}")
+    if x.dim() != 2:
+        raise ValueError("to_mx expects a 2-D tensor")
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    return x
+
+
+def mfma_scale_bytes(rows: int, nblk: int) -> int:
+    return ((rows + 63) // 64) * ((nblk + 3) // 4) * 256
+
+
+def _alloc_scales(rows: int, nblk: int, order: int, device) -> torch.Tensor:
+    if order == MX_SCALES_MFMA:
+        return torch.empty(mfma_scale_bytes(rows, nblk), dtype=torch.uint8, device=device)
+    return torch.empty((rows, nblk), dtype=torch.uint8, device=device)
+
+
+def to_mx_dim0(x: torch.Tensor, mode="floor", order: int = MX_SCALES_ROWMAJOR) -> MXData:
+    """Row-wise cast: blocks of 32 along the last dim of x [R, C]."""
+    x = _check_hp(x)
+    R, C = x.shape
+    if C % BLOCK:
+        raise ValueError(f"last dim {C} is not a multiple of {BLOCK}")
+    codes = torch.empty((R, C), dtype=torch.uint8, device=x.device)
+    scales = _alloc_scales(R, C // BLOCK, order, x.device)
+    with torch.cuda.device(x.device):
+        st = _lib.load().mx_cast_dim0(_ptr(x), R, C, x.stride(0), _ptr(codes), _ptr(scales),
+                                      _mode(mode), order, _stream(x))
+    _lib.check(st, "mx_cast_dim0")
+    return MXData(codes, scales, order)
+
+
+def to_mx_dim1(x: torch.Tensor, mode="floor", order: int = MX_SCALES_ROWMAJOR) -> MXData:
+    """Column-wise cast of x [R, C]: codes [C, R], blocks of 32 down the rows of x."""
+    x = _check_hp(x)
+    R, C = x.shape
+    if R % BLOCK:
+        raise ValueError(f"first dim {R} is not a multiple of {BLOCK}")
+    codes = torch.empty((C, R), dtype=torch.uint8, device=x.device)
+    scales = _alloc_scales(C, R // BLOCK, order, x.device)
+    with torch.cuda.device(x.device):
+        st = _lib.load().mx_cast_dim1(_ptr(x), R, C, x.stride(0), _ptr(codes), _ptr(scales),
+                                      _mode(mode), order, _stream(x))
+    _lib.check(st, "mx_cast_dim1")
+    return MXData(codes, scales, order)
+
+
+def to_mx_dim0_dim1(x: torch.Tensor, mode="floor", order: int = MX_SCALES_ROWMAJOR):
+    """Both casts from one read of x; returns (row-wise MXData, column-wise MXData)."""
+    x = _check_hp(x)
+    R, C = x.shape
+    if R % BLOCK or C % BLOCK:
+        raise ValueError(f"both dims of {tuple(x.shape)} must be multiples of {BLOCK}")
+    codes = torch.empty((R, C), dtype=torch.uint8, device=x.device)
+    scales = _alloc_scales(R, C // BLOCK, order, x.device)
+    codes_t = torch.empty((C, R), dtype=torch.uint8, device=x.device)
+    scales_t = _alloc_scales(C, R // BLOCK, order, x.device)
+    with torch.cuda.device(x.device):
+        st = _lib.load().mx_cast_dim0_dim1(_ptr(x), R, C, x.stride(0), _ptr(codes), _ptr(scales),
+                                           _ptr(codes_t), _ptr(scales_t), _mode(mode), order,
+                                           _stream(x))
+    _lib.check(st, "mx_cast_dim0_dim1")
+    return MXData(codes, scales, order), MXData(codes_t, scales_t, order)
+
+
+def scale_layout(scales: torch.Tensor) -> torch.Tensor:
+    """Row-major [rows, nblk] scales -> flat buffer in MFMA order."""
+    rows, nblk = scales.shape
+    scales = scales.contiguous()
+    out = torch.empty(mfma_scale_bytes(rows, nblk), dtype=torch.uint8, device=scales.device)
+    with torch.cuda.device(scales.device):
+        st = _lib.load().mx_scale_layout(_ptr(scales), rows, nblk, _ptr(out), _stream(scales))
+    _lib.check(st, "mx_scale_layout")
+    return out
+
+
+def scale_unlayout(laid: torch.Tensor, rows: int, nblk: int) -> torch.Tensor:
+    out = torch.empty((rows, nblk), dtype=torch.uint8, device=laid.device)
+    with torch.cuda.device(laid.device):
+        st = _lib.load().mx_scale_unlayout(_ptr(laid), rows, nblk, _ptr(out), _stream(laid))
+    _lib.check(st, "mx_scale_unlayout")
+    return out
+
+
+def _as_mfma(d: MXData) -> torch.Tensor:
+    return d.scales if d.scale_order == MX_SCALES_MFMA else scale_layout(d.scales)
+
+
+def mx_gemm_nt(a: MXData, b: MXData, out: torch.Tensor | None = None) -> torch.Tensor:
+    """bf16 D[M,N] = deq(a)[M,K] @ deq(b)[N,K]^T with fp32 accumulation."""
+    M, K = a.codes.shape
+    N, Kb = b.codes.shape
+    if K != Kb:
+        raise ValueError(f"contraction mismatch: {K} vs {Kb}")
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=a.codes.device)
+    elif out.shape != (M, N) or out.dtype != torch.bfloat16 or out.stride(1) != 1:
+        raise ValueError("out must be a bf16 [M, N] tensor with unit inner stride")
+    sa, sb = _as_mfma(a), _as_mfma(b)
+    with torch.cuda.device(out.device):
+        st = _lib.load().mx_gemm_nt(_ptr(a.codes), _ptr(sa), _ptr(b.codes), _ptr(sb), _ptr(out),
+                                    M, N, K, out.stride(0), _stream(out))
+    _lib.check(st, "mx_gemm_nt")
+    return out
