@@ -74,6 +74,18 @@ int mx_cast_dim0_dim1(const void* x, int64_t rows, int64_t cols, int64_t ldx, ui
                       uint8_t* scales, uint8_t* codes_t, uint8_t* scales_t, int scale_mode,
                       int scale_order, void* stream);
 
+/* Batched forms for 3-D expert weights x [batch, rows, cols] (dense, matrix stride rows*ldx):
+ * every matrix is cast on its own; outputs are [batch, cols, rows] codes (and [batch, rows,
+ * cols] for the fused form) with one scale block per matrix, each laid out as for the
+ * unbatched call.  Same alignment rules; with batch > 1 also rows*cols % 16 == 0.
+ * (3-D expert parameters: torchtitan/models/common/moe/moe.py:90-92.) */
+int mx_cast_dim1_batched(const void* x, int64_t batch, int64_t rows, int64_t cols, int64_t ldx,
+                         uint8_t* codes_t, uint8_t* scales_t, int scale_mode, int scale_order,
+                         void* stream);
+int mx_cast_dim0_dim1_batched(const void* x, int64_t batch, int64_t rows, int64_t cols,
+                              int64_t ldx, uint8_t* codes, uint8_t* scales, uint8_t* codes_t,
+                              uint8_t* scales_t, int scale_mode, int scale_order, void* stream);
+
 /* Re-order a row-major [rows, nblk] scale matrix into MX_SCALES_MFMA order
  * (the "blocked layout" step the reference leaves to torch._scaled_mm, docs/mxfp8.md:36). */
 int mx_scale_layout(const uint8_t* scales, int64_t rows, int64_t nblk, uint8_t* out, void* stream);
@@ -92,7 +104,8 @@ int mx_gemm_nt(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b
 
 /* Grouped GEMM, 2D x 3D: for group g with rows [offs[g-1], offs[g]) of A:
  * D[rows, :] = deq(A[rows, :]) * deq(B[g])^T.  a_codes [T,K]; b_codes [G,N,K];
- * a_scales MFMA order for [T, K/32]; b_scales G consecutive MFMA-order blocks for [N, K/32].
+ * a_scales row-major [T, K/32] (group boundaries need not fall on 64-row tiles);
+ * b_scales G consecutive MFMA-order blocks, each for [N, K/32].
  * offs int32 [G] inclusive cumulative sizes on the device; rows >= offs[G-1] are written as
  * zeros.  Group sizes need not be aligned for this entry point.  Stands in for
  * torch._grouped_mm(x, w^T, offs) in forward and dgrad
@@ -116,7 +129,7 @@ int mx_grouped_gemm_2d2d(const uint8_t* at_codes, const uint8_t* at_scales,
  *   perm[max_len]: perm[write_off[e] + j] = start[r*E+e] + j, -1 in padding   int64
  * One launch, no host synchronisation.  Stands in for generate_permute_indices and its
  * Triton fill kernel (torchtitan/models/common/moe/kernels.py:16-63,145-218).
- * Requires experts_per_rank * num_ranks <= 65536. */
+ * Requires experts_per_rank * num_ranks <= 4096. */
 int mx_group_offsets_pad(const int32_t* counts, int64_t experts_per_rank, int64_t num_ranks,
                          int64_t max_len, int64_t alignment, int64_t* perm, int32_t* m_sizes,
                          int32_t* m_offsets, void* stream);

@@ -59,8 +59,9 @@ def test_unit_scales_reduce_to_plain_fp8(device):
     """All scale bytes 127: the result is the plain e4m3 x e4m3 product sum (exact in fp32 here)."""
     rng = np.random.default_rng(4)
     M, N, K = 64, 64, 128
-    ac = rng.integers(0, 0x40, size=(M, K), dtype=np.uint8)  # small positive codes, exact sums
-    bc = rng.integers(0, 0x40, size=(N, K), dtype=np.uint8)
+    # normal codes in [2^-3, 1.875] with random signs: every partial sum is exact in fp32
+    ac = rng.integers(0x20, 0x40, size=(M, K), dtype=np.uint8) | (rng.integers(0, 2, size=(M, K), dtype=np.uint8) << 7)
+    bc = rng.integers(0x20, 0x40, size=(N, K), dtype=np.uint8) | (rng.integers(0, 2, size=(N, K), dtype=np.uint8) << 7)
     asc = np.full((M, K // 32), 127, dtype=np.uint8)
     bsc = np.full((N, K // 32), 127, dtype=np.uint8)
     ref = mo.f32_to_bf16_bits((mo.e4m3_decode(ac).astype(np.float64) @ mo.e4m3_decode(bc).astype(np.float64).T).astype(np.float32))
@@ -78,6 +79,21 @@ def test_scale_blocks_map_to_the_right_k(device):
     ref = mo.mx_matmul_q(ac, asc, bc, bsc, accumulate=np.float64)
     got = bits_of(_gemm_from_codes(ac, asc, bc, bsc, device))
     assert np.array_equal(got, ref)
+
+
+def test_each_scale_block_applies_to_its_own_32_k(device):
+    """One-hot A at column k with per-block scales 127+b: D must be 2^(k // 32)."""
+    M, N, K = 16, 16, 256
+    for k in range(0, K, 8):
+        ac = np.zeros((M, K), dtype=np.uint8)
+        ac[:, k] = 0x38
+        bc = np.full((N, K), 0x38, dtype=np.uint8)
+        asc = np.tile((127 + np.arange(K // 32))[None, :], (M, 1)).astype(np.uint8)
+        bsc = np.full((N, K // 32), 127, dtype=np.uint8)
+        got = _f32(bits_of(_gemm_from_codes(ac, asc, bc, bsc, device)))
+        assert np.all(got == 2.0 ** (k // 32)), k
+        got = _f32(bits_of(_gemm_from_codes(bc, bsc, ac, asc, device)))
+        assert np.all(got == 2.0 ** (k // 32)), k
 
 
 def test_linear_passes_end_to_end(device):

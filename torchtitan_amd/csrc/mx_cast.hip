@@ -160,9 +160,13 @@ __global__ __launch_bounds__(256) void cast_dim1_kernel(const uint16_t* __restri
                                                         int64_t rows, int64_t cols, int64_t ldx,
                                                         uint8_t* __restrict__ codes_t,
                                                         uint8_t* __restrict__ scales_t,
-                                                        int64_t nblk_t, int64_t ks_n_t) {
+                                                        int64_t nblk_t, int64_t ks_n_t,
+                                                        int64_t x_bstride, int64_t st_bstride) {
   __shared__ __attribute__((aligned(16))) uint8_t lds_codes[kT * kPitch];
   __shared__ __attribute__((aligned(16))) uint8_t lds_scales[kT * 4];
+  x += blockIdx.z * x_bstride;  // batch of independent [rows, cols] matrices
+  codes_t += blockIdx.z * rows * cols;
+  scales_t += blockIdx.z * st_bstride;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int64_t r0 = (int64_t)blockIdx.y * kT, c0 = (int64_t)blockIdx.x * kT;
   const int64_t rb = r0 + wave * 32;
@@ -213,9 +217,14 @@ __global__ __launch_bounds__(256) void cast_dim0_dim1_kernel(
     const uint16_t* __restrict__ x, int64_t rows, int64_t cols, int64_t ldx,
     uint8_t* __restrict__ codes, uint8_t* __restrict__ scales, int64_t nblk, int64_t ks_n,
     uint8_t* __restrict__ codes_t, uint8_t* __restrict__ scales_t, int64_t nblk_t,
-    int64_t ks_n_t) {
+    int64_t ks_n_t, int64_t x_bstride, int64_t s_bstride, int64_t st_bstride) {
   __shared__ __attribute__((aligned(16))) uint8_t lds_codes[kT * kPitch];
   __shared__ __attribute__((aligned(16))) uint8_t lds_scales[kT * 4];
+  x += blockIdx.z * x_bstride;  // batch of independent [rows, cols] matrices
+  codes += blockIdx.z * rows * cols;
+  scales += blockIdx.z * s_bstride;
+  codes_t += blockIdx.z * rows * cols;
+  scales_t += blockIdx.z * st_bstride;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int64_t r0 = (int64_t)blockIdx.y * kT, c0 = (int64_t)blockIdx.x * kT;
   const int64_t rb = r0 + wave * 32;
@@ -380,23 +389,68 @@ extern "C" int mx_cast_dim0(const void* x, int64_t rows, int64_t cols, int64_t l
   return launch_status();
 }
 
-extern "C" int mx_cast_dim1(const void* x, int64_t rows, int64_t cols, int64_t ldx,
-                            uint8_t* codes_t, uint8_t* scales_t, int scale_mode,
-                            int scale_order, void* stream) {
-  if (rows < 0 || cols < 0 || ldx < cols || bad_enums(scale_mode, scale_order))
+static inline int64_t scale_bytes(int64_t rows, int64_t nblk, int order) {
+  return order == MX_SCALES_MFMA ? ((rows + 63) / 64) * ((nblk + 3) / 4) * 256 : rows * nblk;
+}
+
+extern "C" int mx_cast_dim1_batched(const void* x, int64_t batch, int64_t rows, int64_t cols,
+                                    int64_t ldx, uint8_t* codes_t, uint8_t* scales_t,
+                                    int scale_mode, int scale_order, void* stream) {
+  if (batch < 0 || rows < 0 || cols < 0 || ldx < cols || bad_enums(scale_mode, scale_order))
     return MX_ERR_INVALID_ARG;
-  if (rows == 0 || cols == 0) return MX_OK;
+  if (batch == 0 || rows == 0 || cols == 0) return MX_OK;
   if (!x || !codes_t || !scales_t) return MX_ERR_INVALID_ARG;
   if (rows % 32 || cols % 2 || ldx % 2 || ((uintptr_t)x & 3) || ((uintptr_t)codes_t & 15) ||
       ((uintptr_t)scales_t & 3))
     return MX_ERR_ALIGNMENT;
   const int64_t nblk_t = rows / 32, ks_n_t = (nblk_t + 3) / 4;
+  const int64_t st_b = scale_bytes(cols, nblk_t, scale_order);
+  if (batch > 1 && ((rows * cols) % 16 || st_b % 4)) return MX_ERR_ALIGNMENT;
   const int64_t gx = (cols + kT - 1) / kT, gy = (rows + kT - 1) / kT;
-  if (gy > 65535 || gx > 0x7FFFFFFF) return MX_ERR_UNSUPPORTED;
-  dim3 grid((unsigned)gx, (unsigned)gy), block(256);
+  if (gy > 65535 || batch > 65535 || gx > 0x7FFFFFFF) return MX_ERR_UNSUPPORTED;
+  dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch), block(256);
   hipStream_t st = (hipStream_t)stream;
   MX_DISPATCH_MODE_ORDER(cast_dim1_kernel, (const uint16_t*)x, rows, cols, ldx, codes_t,
-                         scales_t, nblk_t, ks_n_t);
+                         scales_t, nblk_t, ks_n_t, rows * ldx, st_b);
+  return launch_status();
+}
+
+extern "C" int mx_cast_dim1(const void* x, int64_t rows, int64_t cols, int64_t ldx,
+                            uint8_t* codes_t, uint8_t* scales_t, int scale_mode,
+                            int scale_order, void* stream) {
+  return mx_cast_dim1_batched(x, 1, rows, cols, ldx, codes_t, scales_t, scale_mode,
+                              scale_order, stream);
+}
+
+extern "C" int mx_cast_dim0_dim1_batched(const void* x, int64_t batch, int64_t rows,
+                                         int64_t cols, int64_t ldx, uint8_t* codes,
+                                         uint8_t* scales, uint8_t* codes_t, uint8_t* scales_t,
+                                         int scale_mode, int scale_order, void* stream) {
+  if (batch < 0 || rows < 0 || cols < 0 || ldx < cols || bad_enums(scale_mode, scale_order))
+    return MX_ERR_INVALID_ARG;
+  if (batch == 0 || rows == 0 || cols == 0) return MX_OK;
+  if (!x || !codes || !scales || !codes_t || !scales_t) return MX_ERR_INVALID_ARG;
+  if (rows % 32 || cols % 32 || ldx % 2 || ((uintptr_t)x & 3) || ((uintptr_t)codes & 1) ||
+      ((uintptr_t)codes_t & 15) || ((uintptr_t)scales_t & 3))
+    return MX_ERR_ALIGNMENT;
+  const int64_t nblk = cols / 32, ks_n = (nblk + 3) / 4;
+  const int64_t nblk_t = rows / 32, ks_n_t = (nblk_t + 3) / 4;
+  const int64_t s_b = scale_bytes(rows, nblk, scale_order);
+  const int64_t st_b = scale_bytes(cols, nblk_t, scale_order);
+  const int64_t gx = (cols + kT - 1) / kT, gy = (rows + kT - 1) / kT;
+  if (gy > 65535 || batch > 65535 || gx > 0x7FFFFFFF) return MX_ERR_UNSUPPORTED;
+  dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  if (scale_order == MX_SCALES_MFMA && ((uintptr_t)scales & 3)) return MX_ERR_ALIGNMENT;
+  if (scale_order == MX_SCALES_MFMA && ((rows & 63) || (nblk & 3))) {
+    // padding of every batch entry's row-wise scale block must read as zero
+    const int64_t n = batch * s_b / 4;
+    hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+                       (uint32_t*)scales, n, 0u);
+  }
+  MX_DISPATCH_MODE_ORDER(cast_dim0_dim1_kernel, (const uint16_t*)x, rows, cols, ldx, codes,
+                         scales, nblk, ks_n, codes_t, scales_t, nblk_t, ks_n_t, rows * ldx, s_b,
+                         st_b);
   return launch_status();
 }
 
@@ -404,24 +458,8 @@ extern "C" int mx_cast_dim0_dim1(const void* x, int64_t rows, int64_t cols, int6
                                  uint8_t* codes, uint8_t* scales, uint8_t* codes_t,
                                  uint8_t* scales_t, int scale_mode, int scale_order,
                                  void* stream) {
-  if (rows < 0 || cols < 0 || ldx < cols || bad_enums(scale_mode, scale_order))
-    return MX_ERR_INVALID_ARG;
-  if (rows == 0 || cols == 0) return MX_OK;
-  if (!x || !codes || !scales || !codes_t || !scales_t) return MX_ERR_INVALID_ARG;
-  if (rows % 32 || cols % 32 || ldx % 2 || ((uintptr_t)x & 3) || ((uintptr_t)codes & 1) ||
-      ((uintptr_t)codes_t & 15) || ((uintptr_t)scales_t & 3))
-    return MX_ERR_ALIGNMENT;
-  const int64_t nblk = cols / 32, ks_n = (nblk + 3) / 4;
-  const int64_t nblk_t = rows / 32, ks_n_t = (nblk_t + 3) / 4;
-  const int64_t gx = (cols + kT - 1) / kT, gy = (rows + kT - 1) / kT;
-  if (gy > 65535 || gx > 0x7FFFFFFF) return MX_ERR_UNSUPPORTED;
-  dim3 grid((unsigned)gx, (unsigned)gy), block(256);
-  hipStream_t st = (hipStream_t)stream;
-  if (scale_order == MX_SCALES_MFMA && ((uintptr_t)scales & 3)) return MX_ERR_ALIGNMENT;
-  clear_mfma_padding(scales, rows, nblk, scale_order, st);
-  MX_DISPATCH_MODE_ORDER(cast_dim0_dim1_kernel, (const uint16_t*)x, rows, cols, ldx, codes,
-                         scales, nblk, ks_n, codes_t, scales_t, nblk_t, ks_n_t);
-  return launch_status();
+  return mx_cast_dim0_dim1_batched(x, 1, rows, cols, ldx, codes, scales, codes_t, scales_t,
+                                   scale_mode, scale_order, stream);
 }
 
 extern "C" int64_t mx_scales_mfma_bytes(int64_t rows, int64_t nblk) {

@@ -1,9 +1,9 @@
 // One workgroup's MXFP8 "NT" GEMM tile on gfx950: D[BM,BN] = deq(A)[BM,K] * deq(B)[BN,K]^T.
 //
 // 256 threads = 4 waves in a 2x2 grid, each wave owns a (BM/2)x(BN/2) patch made of 16x16
-// accumulators fed by v_mfma_scale_f32_16x16x128_f8f6f4: per lane 32 consecutive K bytes of
-// one row (= exactly one MX block) plus that block's E8M0 scale, so the block scaling is done
-// by the matrix core and the products are exact.
+// accumulators fed by v_mfma_scale_f32_16x16x128_f8f6f4: per lane 2 x 16 K bytes of one row
+// plus the E8M0 scale of one 32-element MX block, so the block scaling is done by the matrix
+// core and the products are exact.
 //
 // Data movement per 128-deep K step:
 //   * codes: buffer_load_dwordx4 ... lds (global -> LDS without touching VGPRs), two LDS
@@ -90,12 +90,15 @@ struct GemmTile {
     const uint32_t vb_even = lrow * (uint32_t)B.ld + chunk_even * 16;
     const uint32_t vb_odd = lrow * (uint32_t)B.ld + (chunk_even ^ 1) * 16;
 
-    // LDS -> VGPR: lane (li, lj) reads chunks 2*lj, 2*lj+1 of row li of each sub-tile
+    // LDS -> VGPR.  Operand layout of the 16x16x128 f8 MFMA (measured on gfx950): lane
+    // (li, lj) holds row li, K bytes [16*lj, 16*lj+16) in its first four registers and
+    // [64+16*lj, 64+16*lj+16) in the last four, i.e. 16-byte chunks lj and lj+4; the scale
+    // of K-block b (bytes [32b, 32b+32)) is taken from lane group b.
     const uint32_t sw = (li & 7) ^ (li >> 3);
-    const uint32_t fa0 = (wm * WM + li) * kBK + (((2 * lj) ^ sw) << 4);
-    const uint32_t fa1 = (wm * WM + li) * kBK + (((2 * lj + 1) ^ sw) << 4);
-    const uint32_t fb0 = A_BYTES + (wn * WN + li) * kBK + (((2 * lj) ^ sw) << 4);
-    const uint32_t fb1 = A_BYTES + (wn * WN + li) * kBK + (((2 * lj + 1) ^ sw) << 4);
+    const uint32_t fa0 = (wm * WM + li) * kBK + ((lj ^ sw) << 4);
+    const uint32_t fa1 = (wm * WM + li) * kBK + (((lj + 4) ^ sw) << 4);
+    const uint32_t fb0 = A_BYTES + (wn * WN + li) * kBK + ((lj ^ sw) << 4);
+    const uint32_t fb1 = A_BYTES + (wn * WN + li) * kBK + (((lj + 4) ^ sw) << 4);
 
     v4f acc[TM][TN];
 #pragma unroll
@@ -237,6 +240,9 @@ struct GemmTile {
 #pragma unroll
       for (int g = 0; g < SB; ++g) sb_cur[g] = sb_nxt[g];
     }
+
+    // drain the last (out-of-range) prefetch before the wave can retire
+    __builtin_amdgcn_s_waitcnt(0x0F70);
 
     // epilogue: lane holds D[row = m*16 + li][col = n*16 + lj*4 + 0..3]
     const int64_t rows_valid = A.rows_valid, cols_valid = B.rows_valid;
