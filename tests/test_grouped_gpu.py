@@ -1,0 +1,143 @@
+"""GPU parity: grouped MXFP8 GEMMs and the token-group padding kernel vs the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import mx_oracle as mo
+from tests.helpers import bf16_from_bits, bits_of, randn_bits, rel_l2, u8
+from torchtitan_amd import ops
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+R, L = ops.MX_SCALES_ROWMAJOR, ops.MX_SCALES_MFMA
+
+
+def _f32(bits):
+    return mo.bf16_bits_to_f32(bits)
+
+
+def _sizes_to_offs(sizes, device):
+    return torch.tensor(np.cumsum(sizes), dtype=torch.int32, device=device)
+
+
+CASES = [
+    # (group sizes, N, K)
+    ([32, 64, 96], 64, 128),
+    ([0, 128, 0, 32], 128, 256),
+    ([320, 32, 0, 288, 64], 192, 160),
+    ([256, 512, 128], 768, 512),
+    ([1024, 96, 608, 0, 32, 992], 256, 384),
+]
+
+
+@pytest.mark.parametrize("sizes,N,K", CASES)
+@pytest.mark.parametrize("tail_rows", [0, 64])
+def test_grouped_forward_and_dgrad(device, sizes, N, K, tail_rows):
+    """2D x 3D: fwd contracts K with W cast along K; dgrad contracts N with W cast along N."""
+    rng = np.random.default_rng(sum(sizes) + N + K)
+    T = sum(sizes) + tail_rows
+    G = len(sizes)
+    x_bits = randn_bits(rng, (T, K), outliers=1e-3)
+    w_bits = randn_bits(rng, (G, N, K), std=0.02)
+    dy_bits = randn_bits(rng, (T, N), std=1e-3)
+    offs = _sizes_to_offs(sizes, device)
+    x, w, dy = (bf16_from_bits(b, device) for b in (x_bits, w_bits, dy_bits))
+    pad64 = N % 64 == 0
+    for mode_name, mode in (("floor", mo.FLOOR), ("rceil", mo.RCEIL)):
+        wq0, wq1 = ops.to_mx_dim0_dim1_batched(w, mode_name, L)
+        if pad64:
+            assert torch.equal(wq0.codes, ops.to_mx_dim0_batched(w, mode_name, L).codes)
+        y = ops.mx_grouped_gemm_2d3d(ops.to_mx_dim0(x, mode_name, R), wq0, offs)
+        ref = mo.grouped_fwd(x_bits, w_bits, np.cumsum(sizes), mode)
+        assert rel_l2(_f32(bits_of(y)), _f32(ref)) <= TOL
+        assert np.all(bits_of(y)[sum(sizes):] == 0), "padding rows must be zero"
+        dx = ops.mx_grouped_gemm_2d3d(ops.to_mx_dim0(dy, mode_name, R), wq1, offs)
+        ref = mo.grouped_dgrad(dy_bits, w_bits, np.cumsum(sizes), mode)
+        assert rel_l2(_f32(bits_of(dx)), _f32(ref)) <= TOL
+
+
+@pytest.mark.parametrize("sizes,N,K", CASES)
+def test_grouped_wgrad(device, sizes, N, K):
+    """2D x 2D: dW[g] contracts the tokens of group g; blocks of 32 run down the tokens."""
+    rng = np.random.default_rng(sum(sizes) * 3 + N + K)
+    T = sum(sizes) + 32
+    x_bits = randn_bits(rng, (T, K), outliers=1e-3)
+    dy_bits = randn_bits(rng, (T, N), std=1e-3)
+    offs = _sizes_to_offs(sizes, device)
+    x, dy = bf16_from_bits(x_bits, device), bf16_from_bits(dy_bits, device)
+    for mode_name, mode in (("floor", mo.FLOOR), ("rceil", mo.RCEIL)):
+        dw = ops.mx_grouped_gemm_2d2d(ops.to_mx_dim1(dy, mode_name, R), ops.to_mx_dim1(x, mode_name, R), offs)
+        ref = mo.grouped_wgrad(dy_bits, x_bits, np.cumsum(sizes), mode)
+        got = bits_of(dw)
+        for g, s in enumerate(sizes):
+            if s == 0:
+                assert np.all(got[g] == 0)
+            else:
+                assert rel_l2(_f32(got[g]), _f32(ref[g])) <= TOL, g
+
+
+def test_batched_weight_casts_match_per_matrix(device):
+    rng = np.random.default_rng(11)
+    w_bits = randn_bits(rng, (5, 96, 160), std=0.02, outliers=1e-3)
+    w = bf16_from_bits(w_bits, device)
+    for order in (R, L):
+        q0, q1 = ops.to_mx_dim0_dim1_batched(w, "rceil", order)
+        q1b = ops.to_mx_dim1_batched(w, "rceil", order)
+        assert torch.equal(q1.codes, q1b.codes) and torch.equal(q1.scales.reshape(-1), q1b.scales.reshape(-1))
+        for g in range(5):
+            c0, s0 = mo.cast_dim0(w_bits[g], mo.RCEIL)
+            c1, s1 = mo.cast_dim1(w_bits[g], mo.RCEIL)
+            assert np.array_equal(u8(q0.codes[g]), c0) and np.array_equal(u8(q1.codes[g]), c1)
+            if order == L:
+                s0, s1 = mo.scale_layout(s0).reshape(-1), mo.scale_layout(s1).reshape(-1)
+                n0, n1 = s0.size, s1.size
+                assert np.array_equal(u8(q0.scales)[g * n0:(g + 1) * n0], s0)
+                assert np.array_equal(u8(q1.scales)[g * n1:(g + 1) * n1], s1)
+            else:
+                assert np.array_equal(u8(q0.scales[g]), s0) and np.array_equal(u8(q1.scales[g]), s1)
+
+
+# ---------------------------------------------------------------- padding / permutation
+def _check_pad(device, counts, experts, ranks, alignment, max_len):
+    perm, m_sizes, m_offsets = ops.group_offsets_pad(torch.tensor(counts, device=device), experts, ranks, max_len, alignment)
+    rp, rs, ro = mo.generate_permute_indices(np.asarray(counts), experts, ranks, max_len, alignment)
+    assert np.array_equal(perm.cpu().numpy(), rp)
+    assert np.array_equal(m_sizes.cpu().numpy(), rs) and m_sizes.dtype == torch.int32
+    assert np.array_equal(m_offsets.cpu().numpy(), ro) and m_offsets.dtype == torch.int32
+
+
+def test_pad_docstring_example(device):
+    # the worked example of generate_permute_indices: 2 ranks x 4 experts
+    _check_pad(device, [4, 2, 1, 3, 1, 2, 3, 4], 4, 2, 8, mo.padded_max_len(20, 4, 8))
+
+
+@pytest.mark.parametrize("ranks", [1, 2, 4, 8, 16])
+@pytest.mark.parametrize("token_range", [(1, 16), (0, 5), (0, 0), (100, 2000)])
+def test_pad_matches_reference_fill(device, ranks, token_range):
+    rng = np.random.default_rng(2020 + ranks)
+    total_experts = 256
+    experts = total_experts // ranks
+    counts = rng.integers(token_range[0], token_range[1] + 1, size=total_experts).tolist()
+    for alignment in (8, 16, 32):
+        max_len = mo.padded_max_len(sum(counts), experts, alignment)
+        _check_pad(device, counts, experts, ranks, alignment, max_len)
+        _check_pad(device, counts, experts, ranks, alignment, max(sum(counts) // 2, 1))  # truncated
+
+
+def test_pad_then_grouped_gemm_moe_like(device):
+    """Routed tokens -> padded groups -> grouped GEMM, against the per-expert oracle loop."""
+    rng = np.random.default_rng(5)
+    E, dim, hidden, A = 8, 256, 192, 32
+    counts = np.array([37, 0, 130, 64, 1, 95, 0, 200])
+    T = int(counts.sum())
+    x_bits = randn_bits(rng, (T, dim))
+    w_bits = randn_bits(rng, (E, hidden, dim), std=0.02)
+    max_len = mo.padded_max_len(T, E, A)
+    perm, m_sizes, m_offsets = ops.group_offsets_pad(torch.tensor(counts, device=device), E, 1, max_len, A)
+    x = bf16_from_bits(x_bits, device)
+    xp = torch.vstack((x, x.new_zeros((1, dim))))[perm]
+    y = ops.mx_grouped_gemm_2d3d(ops.to_mx_dim0(xp, "rceil", R), ops.to_mx_dim0_batched(bf16_from_bits(w_bits, device), "rceil", L), m_offsets)
+    rp, rs, ro = mo.generate_permute_indices(counts, E, 1, max_len, A)
+    xp_bits = np.vstack((x_bits, np.zeros((1, dim), np.uint16)))[rp]
+    ref = mo.grouped_fwd(xp_bits, w_bits, ro, mo.RCEIL)
+    assert rel_l2(_f32(bits_of(y)), _f32(ref)) <= TOL

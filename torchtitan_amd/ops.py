@@ -151,3 +151,130 @@ def mx_gemm_nt(a: MXData, b: MXData, out: torch.Tensor | None = None) -> torch.T
                                     M, N, K, out.stride(0), _stream(out))
     _lib.check(st, "mx_gemm_nt")
     return out
+
+
+# --------------------------------------------------------------------------- 3-D weights
+def to_mx_dim0_batched(w: torch.Tensor, mode="floor", order: int = MX_SCALES_MFMA) -> MXData:
+    """Row-wise cast of every matrix of w [G, R, C]: codes [G, R, C], one scale block each.
+
+    A 3-D weight is G stacked matrices, so this is one row-wise cast of the [G*R, C] view;
+    in MFMA order that equals G per-matrix blocks only when R is a multiple of 64.
+    """
+    G, R, C = w.shape
+    if order == MX_SCALES_MFMA and R % 64:
+        raise ValueError("MFMA-order scales of stacked matrices need rows % 64 == 0")
+    d = to_mx_dim0(w.reshape(G * R, C), mode, order)
+    scales = d.scales if order == MX_SCALES_MFMA else d.scales.view(G, R, C // BLOCK)
+    return MXData(d.codes.view(G, R, C), scales, order)
+
+
+def to_mx_dim1_batched(w: torch.Tensor, mode="floor", order: int = MX_SCALES_MFMA) -> MXData:
+    """Column-wise cast of every matrix of w [G, R, C]: codes [G, C, R]."""
+    if w.dim() != 3 or w.dtype != torch.bfloat16 or not w.is_cuda:
+        raise TypeError("expected a 3-D bf16 GPU tensor")
+    w = w.contiguous()
+    G, R, C = w.shape
+    if R % BLOCK:
+        raise ValueError(f"dim 1 ({R}) is not a multiple of {BLOCK}")
+    codes = torch.empty((G, C, R), dtype=torch.uint8, device=w.device)
+    per = mfma_scale_bytes(C, R // BLOCK) if order == MX_SCALES_MFMA else C * (R // BLOCK)
+    scales = torch.empty(G * per, dtype=torch.uint8, device=w.device)
+    with torch.cuda.device(w.device):
+        st = _lib.load().mx_cast_dim1_batched(_ptr(w), G, R, C, C, _ptr(codes), _ptr(scales),
+                                              _mode(mode), order, _stream(w))
+    _lib.check(st, "mx_cast_dim1_batched")
+    if order == MX_SCALES_ROWMAJOR:
+        scales = scales.view(G, C, R // BLOCK)
+    return MXData(codes, scales, order)
+
+
+def to_mx_dim0_dim1_batched(w: torch.Tensor, mode="floor", order: int = MX_SCALES_MFMA):
+    """Both casts of every matrix of w [G, R, C] from one read."""
+    if w.dim() != 3 or w.dtype != torch.bfloat16 or not w.is_cuda:
+        raise TypeError("expected a 3-D bf16 GPU tensor")
+    w = w.contiguous()
+    G, R, C = w.shape
+    if R % BLOCK or C % BLOCK:
+        raise ValueError(f"dims {R}, {C} must be multiples of {BLOCK}")
+    codes = torch.empty((G, R, C), dtype=torch.uint8, device=w.device)
+    codes_t = torch.empty((G, C, R), dtype=torch.uint8, device=w.device)
+    if order == MX_SCALES_MFMA:
+        per, per_t = mfma_scale_bytes(R, C // BLOCK), mfma_scale_bytes(C, R // BLOCK)
+    else:
+        per, per_t = R * (C // BLOCK), C * (R // BLOCK)
+    scales = torch.empty(G * per, dtype=torch.uint8, device=w.device)
+    scales_t = torch.empty(G * per_t, dtype=torch.uint8, device=w.device)
+    with torch.cuda.device(w.device):
+        st = _lib.load().mx_cast_dim0_dim1_batched(_ptr(w), G, R, C, C, _ptr(codes), _ptr(scales),
+                                                   _ptr(codes_t), _ptr(scales_t), _mode(mode),
+                                                   order, _stream(w))
+    _lib.check(st, "mx_cast_dim0_dim1_batched")
+    if order == MX_SCALES_ROWMAJOR:
+        scales, scales_t = scales.view(G, R, C // BLOCK), scales_t.view(G, C, R // BLOCK)
+    return MXData(codes, scales, order), MXData(codes_t, scales_t, order)
+
+
+# --------------------------------------------------------------------------- grouped GEMMs
+def mx_grouped_gemm_2d3d(a: MXData, b: MXData, offs: torch.Tensor,
+                         out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[rows of group g] = deq(a[rows of g]) @ deq(b[g])^T; rows past offs[-1] are zero.
+
+    a: codes [T, K] with row-major scales [T, K/32]; b: codes [G, N, K] with MFMA-order scales
+    (G per-matrix blocks); offs: int32 [G] inclusive cumulative group sizes on the device.
+    """
+    T, K = a.codes.shape
+    G, N, Kb = b.codes.shape
+    if K != Kb:
+        raise ValueError(f"contraction mismatch: {K} vs {Kb}")
+    if a.scale_order != MX_SCALES_ROWMAJOR or b.scale_order != MX_SCALES_MFMA:
+        raise ValueError("2d3d expects row-major scales for a and MFMA-order scales for b")
+    if offs.dtype != torch.int32 or offs.numel() != G:
+        raise ValueError("offs must be int32 with one entry per group")
+    if out is None:
+        out = torch.empty((T, N), dtype=torch.bfloat16, device=a.codes.device)
+    with torch.cuda.device(out.device):
+        st = _lib.load().mx_grouped_gemm_2d3d(_ptr(a.codes), _ptr(a.scales), _ptr(b.codes),
+                                              _ptr(b.scales), _ptr(offs), _ptr(out), T, N, K, G,
+                                              out.stride(0), _stream(out))
+    _lib.check(st, "mx_grouped_gemm_2d3d")
+    return out
+
+
+def mx_grouped_gemm_2d2d(at: MXData, bt: MXData, offs: torch.Tensor,
+                         out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[g] = deq(at[:, tokens of g]) @ deq(bt[:, tokens of g])^T  ->  [G, N, K] bf16.
+
+    at: codes [N, T], bt: codes [K, T] (column-wise casts), both with row-major scales.
+    """
+    N, T = at.codes.shape
+    K, Tb = bt.codes.shape
+    if T != Tb:
+        raise ValueError(f"token count mismatch: {T} vs {Tb}")
+    if at.scale_order != MX_SCALES_ROWMAJOR or bt.scale_order != MX_SCALES_ROWMAJOR:
+        raise ValueError("2d2d expects row-major scales")
+    G = offs.numel()
+    if out is None:
+        out = torch.empty((G, N, K), dtype=torch.bfloat16, device=at.codes.device)
+    with torch.cuda.device(out.device):
+        st = _lib.load().mx_grouped_gemm_2d2d(_ptr(at.codes), _ptr(at.scales), _ptr(bt.codes),
+                                              _ptr(bt.scales), _ptr(offs), _ptr(out), T, N, K, G,
+                                              _stream(out))
+    _lib.check(st, "mx_grouped_gemm_2d2d")
+    return out
+
+
+def group_offsets_pad(counts: torch.Tensor, experts_per_rank: int, num_ranks: int, max_len: int,
+                      alignment: int):
+    """(permuted_indices int64 [max_len], m_sizes int32 [E], m_offsets int32 [E]); one launch."""
+    if not counts.is_cuda:
+        raise _lib.MXLibraryError("group_offsets_pad runs on the GPU only")
+    c32 = counts.to(torch.int32).contiguous()
+    perm = torch.empty(max_len, dtype=torch.int64, device=counts.device)
+    m_sizes = torch.empty(experts_per_rank, dtype=torch.int32, device=counts.device)
+    m_offsets = torch.empty(experts_per_rank, dtype=torch.int32, device=counts.device)
+    with torch.cuda.device(counts.device):
+        st = _lib.load().mx_group_offsets_pad(_ptr(c32), experts_per_rank, num_ranks, max_len,
+                                              alignment, _ptr(perm), _ptr(m_sizes),
+                                              _ptr(m_offsets), _stream(counts))
+    _lib.check(st, "mx_group_offsets_pad")
+    return perm, m_sizes, m_offsets
