@@ -1,0 +1,407 @@
+"""Weight wrapper that re-routes ``F.linear`` and ``torch._grouped_mm`` to the MXFP8 kernels.
+
+After conversion a target weight is still an ordinary trainable high-precision parameter
+(optimizer, ``init_weights``, ``to_empty`` and checkpointing keep working on it), but it is an
+instance of ``MXFP8TrainingWeight``; its ``__torch_function__`` sends the two GEMM entry points
+to autograd functions that quantize dynamically and call the HIP library in forward and
+backward.  This is the role the reference gives to the external tensor subclass installed by
+its converter (torchtitan/components/quantization/mx.py:27-31,93-96,119-125).
+
+Passes of one linear with W [N, K], X [M, K], dY [M, N]  (every GEMM is "NT"):
+    forward  Y  = cast_dim0(X)  x cast_dim0(W)        contraction K
+    dgrad    dX = cast_dim0(dY) x cast_dim1(W)        contraction N
+    wgrad    dW = cast_dim1(dY) x cast_dim1(X)        contraction M
+X and W are read once in forward (fused row+column cast) and their column-wise forms are what
+is saved for backward; dY is read once in backward.
+"""
+from __future__ import annotations
+
+import weakref
+
+import torch
+import torch.nn.functional as F
+
+from . import ops
+from .ops import MX_SCALES_MFMA, MX_SCALES_ROWMAJOR, MXData
+
+
+class MXFP8Config:
+    """Per-weight recipe: scale mode and whether grouped GEMMs pad token groups to 32."""
+
+    __slots__ = ("scale_mode", "pad_token_groups_for_grouped_mm")
+
+    def __init__(self, scale_mode: str = "rceil", pad_token_groups_for_grouped_mm: bool = True):
+        if scale_mode not in ops.SCALE_MODES:
+            raise ValueError(f"unknown scale mode {scale_mode!r}")
+        self.scale_mode = scale_mode
+        self.pad_token_groups_for_grouped_mm = pad_token_groups_for_grouped_mm
+
+    def __repr__(self):
+        return (f"MXFP8Config(scale_mode={self.scale_mode!r}, "
+                f"pad_token_groups_for_grouped_mm={self.pad_token_groups_for_grouped_mm})")
+
+
+# ----------------------------------------------------------------------------- cast reuse
+class _ActivationCastCache:
+    """Remembers the fused cast of the last activation tensor.
+
+    w1(x) and w3(x) of a SwiGLU block, or wq/wk/wv of attention, receive the same tensor object;
+    the second and third linear reuse the codes instead of re-reading x.  The entry is keyed on
+    object identity and the tensor's version counter and holds only a weak reference.
+    """
+
+    def __init__(self):
+        self._ref = None
+        self._key = None
+        self._value = None
+
+    def get(self, x: torch.Tensor, mode: str):
+        if self._ref is not None and self._ref() is x and self._key == (x._version, mode, x.data_ptr()):
+            return self._value
+        return None
+
+    def put(self, x: torch.Tensor, mode: str, value):
+        self._ref = weakref.ref(x)
+        self._key = (x._version, mode, x.data_ptr())
+        self._value = value
+
+    def clear(self):
+        self._ref = self._key = self._value = None
+
+
+_cast_cache = _ActivationCastCache()
+
+
+def _cast_activation(x2: torch.Tensor, src: torch.Tensor, mode: str, need_cols: bool):
+    """(row-wise, column-wise or None) MXFP8 forms of the 2-D bf16 activation `x2`."""
+    hit = _cast_cache.get(src, mode)
+    if hit is not None and (hit[1] is not None or not need_cols):
+        return hit
+    if need_cols and x2.shape[0] % ops.BLOCK == 0:
+        rows, cols = ops.to_mx_dim0_dim1(x2, mode, MX_SCALES_MFMA)
+    else:
+        rows, cols = ops.to_mx_dim0(x2, mode, MX_SCALES_MFMA), None
+    _cast_cache.put(src, mode, (rows, cols))
+    return rows, cols
+
+
+# ----------------------------------------------------------------------------- dense linear
+class _MXLinear(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, cfg: MXFP8Config):
+        mode = cfg.scale_mode
+        K = x.shape[-1]
+        N = weight.shape[0]
+        x2 = x.reshape(-1, K)
+        if x2.dtype != torch.bfloat16:
+            x2 = x2.to(torch.bfloat16)
+        w = weight if weight.dtype == torch.bfloat16 else weight.to(torch.bfloat16)
+        needs_bwd = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
+        M = x2.shape[0]
+        xq0, xq1 = _cast_activation(x2, x, mode, need_cols=ctx.needs_input_grad[1])
+        if needs_bwd and ctx.needs_input_grad[0] and N % ops.BLOCK == 0:
+            wq0, wq1 = ops.to_mx_dim0_dim1(w, mode, MX_SCALES_MFMA)
+        else:
+            wq0, wq1 = ops.to_mx_dim0(w, mode, MX_SCALES_MFMA), None
+        y = ops.mx_gemm_nt(xq0, wq0)
+        ctx.cfg = cfg
+        ctx.x_shape = x.shape
+        ctx.x_dtype = x.dtype
+        ctx.w_dtype = weight.dtype
+        ctx.have_xq1 = xq1 is not None
+        ctx.have_wq1 = wq1 is not None
+        saved = []
+        if ctx.needs_input_grad[1]:
+            saved += [xq1.codes, xq1.scales] if xq1 is not None else [x2]
+        if ctx.needs_input_grad[0]:
+            saved += [wq1.codes, wq1.scales] if wq1 is not None else [w]
+        ctx.save_for_backward(*saved)
+        return y.view(*x.shape[:-1], N)
+
+    @staticmethod
+    def backward(ctx, dy):
+        mode = ctx.cfg.scale_mode
+        need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        saved = list(ctx.saved_tensors)
+        N = dy.shape[-1]
+        dy2 = dy.reshape(-1, N)
+        if dy2.dtype != torch.bfloat16:
+            dy2 = dy2.to(torch.bfloat16)
+        dy2 = dy2.contiguous()
+        M = dy2.shape[0]
+        xq1 = wq1 = None
+        if need_dw:
+            if ctx.have_xq1:
+                xq1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
+            else:  # M not a multiple of 32: pad the token dim with zero rows for the column cast
+                xq1 = _cast_cols_padded(saved.pop(0), mode)
+        if need_dx:
+            if ctx.have_wq1:
+                wq1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
+            else:
+                wq1 = _cast_cols_padded(saved.pop(0), mode)
+        dyq0 = dyq1 = None
+        if need_dx and need_dw and M % ops.BLOCK == 0 and N % ops.BLOCK == 0:
+            dyq0, dyq1 = ops.to_mx_dim0_dim1(dy2, mode, MX_SCALES_MFMA)
+        else:
+            if need_dx:
+                dyq0 = _cast_rows_padded(dy2, mode)
+            if need_dw:
+                dyq1 = _cast_cols_padded(dy2, mode)
+        dx = dw = None
+        if need_dx:
+            dx = ops.mx_gemm_nt(dyq0, wq1).view(ctx.x_shape)
+            if dx.dtype != ctx.x_dtype:
+                dx = dx.to(ctx.x_dtype)
+        if need_dw:
+            dw = ops.mx_gemm_nt(dyq1, xq1)
+            if dw.dtype != ctx.w_dtype:
+                dw = dw.to(ctx.w_dtype)
+        return dx, dw, None
+
+
+def _cast_cols_padded(t: torch.Tensor, mode: str) -> MXData:
+    """Column-wise cast of t [R, C]; R is zero-padded up to a multiple of 32 (zeros add nothing
+    to a contraction over R)."""
+    R = t.shape[0]
+    pad = -R % ops.BLOCK
+    if pad:
+        t = torch.cat((t, t.new_zeros((pad, t.shape[1]))), dim=0)
+    return ops.to_mx_dim1(t.contiguous(), mode, MX_SCALES_MFMA)
+
+
+def _cast_rows_padded(t: torch.Tensor, mode: str) -> MXData:
+    """Row-wise cast of t [R, C]; C is zero-padded up to a multiple of 32."""
+    C = t.shape[1]
+    pad = -C % ops.BLOCK
+    if pad:
+        t = torch.cat((t, t.new_zeros((t.shape[0], pad))), dim=1)
+    return ops.to_mx_dim0(t.contiguous(), mode, MX_SCALES_MFMA)
+
+
+def mx_linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, cfg: MXFP8Config):
+    """``F.linear`` with the matmul in MXFP8; the bias add stays in high precision."""
+    if x.shape[-1] % ops.BLOCK:
+        raise ValueError(f"MXFP8 linear needs in_features % 32 == 0, got {x.shape[-1]}")
+    out_dtype = x.dtype
+    if torch.is_autocast_enabled(x.device.type):
+        out_dtype = torch.get_autocast_dtype(x.device.type)
+    y = _MXLinear.apply(x, weight, cfg)
+    if y.dtype != out_dtype:
+        y = y.to(out_dtype)
+    if bias is not None:
+        y = y + bias.to(y.dtype)
+    return y
+
+
+# ----------------------------------------------------------------------------- grouped GEMM
+def _pad_plan(offs: torch.Tensor, T: int):
+    """Device-side plan that moves rows of variable-size groups into 32-aligned groups.
+
+    Returns (gather indices into [x; 0-row] for the padded layout, padded inclusive offsets,
+    for every original row its row in the padded layout or the index of an appended zero row).
+    No host synchronisation: the padded length is the static bound round_up(T + 32 G, 32).
+    """
+    G = offs.numel()
+    sizes = torch.diff(offs, prepend=offs.new_zeros(1))
+    max_len = -(-(T + ops.BLOCK * G) // ops.BLOCK) * ops.BLOCK
+    perm, _, m_offsets = ops.group_offsets_pad(sizes, G, 1, max_len, ops.BLOCK)
+    back = torch.full((T + 1,), max_len, dtype=torch.int64, device=offs.device)
+    back[perm] = torch.arange(max_len, device=offs.device)  # perm == -1 writes the spare slot T
+    return perm, m_offsets, back[:T]
+
+
+class _MXGroupedMM(torch.autograd.Function):
+    """out[rows of g] = x[rows of g] @ w[g]^T with w [G, N, K]; offs = inclusive cumsum, int32."""
+
+    @staticmethod
+    def forward(ctx, x, weight, offs, cfg: MXFP8Config):
+        mode = cfg.scale_mode
+        T, K = x.shape
+        G, N, _ = weight.shape
+        xb = x if x.dtype == torch.bfloat16 else x.to(torch.bfloat16)
+        w = weight if weight.dtype == torch.bfloat16 else weight.to(torch.bfloat16)
+        w = w.contiguous()
+        plan = None
+        if cfg.pad_token_groups_for_grouped_mm:
+            plan = _pad_plan(offs, T)
+            perm, offs_p, back = plan
+            xb = torch.cat((xb, xb.new_zeros((1, K))), dim=0)[perm]
+        else:
+            offs_p = offs
+            if T % ops.BLOCK:
+                raise ValueError("without padding the token dimension must be a multiple of 32")
+        xb = xb.contiguous()
+        need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        if need_dw:
+            xq0, xq1 = ops.to_mx_dim0_dim1(xb, mode, MX_SCALES_ROWMAJOR)
+        else:
+            xq0, xq1 = ops.to_mx_dim0(xb, mode, MX_SCALES_ROWMAJOR), None
+        if need_dx and N % ops.BLOCK == 0:
+            wq0, wq1 = ops.to_mx_dim0_dim1_batched(w, mode, MX_SCALES_MFMA)
+        else:
+            wq0 = _cast_w_rows(w, mode)
+            wq1 = None
+        y = ops.mx_grouped_gemm_2d3d(xq0, wq0, offs_p)
+        if plan is not None:
+            y = torch.cat((y, y.new_zeros((1, N))), dim=0)[back]
+        ctx.cfg = cfg
+        ctx.dims = (T, K, N, G)
+        ctx.dtypes = (x.dtype, weight.dtype)
+        ctx.padded = plan is not None
+        saved = [offs_p]
+        if plan is not None:
+            saved += [plan[0], plan[2]]
+        if need_dw:
+            saved += [xq1.codes, xq1.scales]
+        if need_dx:
+            ctx.have_wq1 = wq1 is not None
+            saved += [wq1.codes, wq1.scales] if wq1 is not None else [w]
+        ctx.save_for_backward(*saved)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        mode = ctx.cfg.scale_mode
+        T, K, N, G = ctx.dims
+        need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        saved = list(ctx.saved_tensors)
+        offs_p = saved.pop(0)
+        dyb = dy if dy.dtype == torch.bfloat16 else dy.to(torch.bfloat16)
+        if ctx.padded:
+            perm, back = saved.pop(0), saved.pop(0)
+            dyb = torch.cat((dyb, dyb.new_zeros((1, N))), dim=0)[perm]
+        dyb = dyb.contiguous()
+        dx = dw = None
+        if need_dw:
+            xq1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_ROWMAJOR)
+        if need_dx and need_dw and N % ops.BLOCK == 0:
+            dyq0, dyq1 = ops.to_mx_dim0_dim1(dyb, mode, MX_SCALES_ROWMAJOR)
+        else:
+            dyq0 = ops.to_mx_dim0(dyb, mode, MX_SCALES_ROWMAJOR) if need_dx else None
+            dyq1 = ops.to_mx_dim1(dyb, mode, MX_SCALES_ROWMAJOR) if need_dw else None
+        if need_dx:
+            if ctx.have_wq1:
+                wq1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
+            else:
+                wq1 = ops.to_mx_dim1_batched(saved.pop(0), mode, MX_SCALES_MFMA)
+            dx = ops.mx_grouped_gemm_2d3d(dyq0, wq1, offs_p)
+            if ctx.padded:
+                dx = torch.cat((dx, dx.new_zeros((1, K))), dim=0)[back]
+            if dx.dtype != ctx.dtypes[0]:
+                dx = dx.to(ctx.dtypes[0])
+        if need_dw:
+            dw = ops.mx_grouped_gemm_2d2d(dyq1, xq1, offs_p)
+            if dw.dtype != ctx.dtypes[1]:
+                dw = dw.to(ctx.dtypes[1])
+        return dx, dw, None, None
+
+
+def _cast_w_rows(w: torch.Tensor, mode: str) -> MXData:
+    """Row-wise cast of stacked matrices w [G, N, K] with one MFMA-order scale block each."""
+    G, N, K = w.shape
+    if N % 64 == 0:
+        return ops.to_mx_dim0_batched(w, mode, MX_SCALES_MFMA)
+    parts = [ops.to_mx_dim0(w[g], mode, MX_SCALES_MFMA) for g in range(G)]
+    return MXData(torch.stack([p.codes for p in parts]), torch.cat([p.scales for p in parts]),
+                  MX_SCALES_MFMA)
+
+
+def mx_grouped_mm(x: torch.Tensor, w_t: torch.Tensor, offs: torch.Tensor, cfg: MXFP8Config):
+    """``torch._grouped_mm(x, w_t, offs=offs)`` for x [T, K], w_t [G, K, N] = weight^T."""
+    if x.dim() != 2 or w_t.dim() != 3 or offs is None:
+        raise NotImplementedError("MXFP8 grouped_mm supports the 2D x 3D form with offsets only")
+    weight = w_t.transpose(-2, -1)  # back to the parameter's [G, N, K] layout
+    if x.shape[-1] % ops.BLOCK:
+        raise ValueError(f"MXFP8 grouped_mm needs K % 32 == 0, got {x.shape[-1]}")
+    return _MXGroupedMM.apply(x, weight, offs.to(torch.int32), cfg)
+
+
+# ----------------------------------------------------------------------------- the wrapper
+_LINEAR_FUNCS = {F.linear}
+_GROUPED_FUNCS = {torch._grouped_mm}
+
+
+def _unwrap(t):
+    return t.as_subclass(torch.Tensor) if isinstance(t, MXFP8TrainingWeight) else t
+
+
+class MXFP8TrainingWeight(torch.Tensor):
+    """A high-precision weight whose GEMMs run in MXFP8.
+
+    Shares storage with the tensor it was made from (like ``nn.Parameter``), so in-place
+    initialisation and optimizer updates act on the real weight.  Every op other than
+    ``F.linear`` / ``torch._grouped_mm`` behaves as for a plain tensor, and results that are
+    views or casts of the weight stay wrapped so that ``w.bfloat16().transpose(-2, -1)`` still
+    reaches the grouped kernel.
+    """
+
+    mx_config: MXFP8Config = MXFP8Config()
+
+    @staticmethod
+    def __new__(cls, data: torch.Tensor, config: MXFP8Config | None = None):
+        t = torch.Tensor._make_subclass(cls, data, data.requires_grad)
+        t.mx_config = config or MXFP8Config()
+        return t
+
+    def __repr__(self):
+        return f"MXFP8TrainingWeight({self.as_subclass(torch.Tensor)!r}, config={self.mx_config!r})"
+
+    @classmethod
+    def __torch_function__(cls, func, types, args=(), kwargs=None):
+        kwargs = kwargs or {}
+        if func in _LINEAR_FUNCS:
+            x = args[0]
+            w = args[1] if len(args) > 1 else kwargs["weight"]
+            b = args[2] if len(args) > 2 else kwargs.get("bias")
+            if isinstance(w, cls) and not isinstance(x, cls):
+                return mx_linear(x, _unwrap(w), _unwrap(b), w.mx_config)
+        elif func in _GROUPED_FUNCS:
+            a, b = args[0], args[1]
+            offs = kwargs.get("offs", args[2] if len(args) > 2 else None)
+            if isinstance(b, cls) and not isinstance(a, cls):
+                return mx_grouped_mm(a, _unwrap(b), offs, b.mx_config)
+        cfg = next((a.mx_config for a in _flatten(args) if isinstance(a, cls)), None)
+        with torch._C.DisableTorchFunctionSubclass():
+            out = func(*args, **kwargs)
+        return _rewrap(out, cls, cfg, func)
+
+    # plain-tensor semantics for pickling / deepcopy of the storage
+    def __reduce_ex__(self, proto):
+        return (MXFP8TrainingWeight, (self.as_subclass(torch.Tensor), self.mx_config))
+
+
+_KEEP_WRAPPED = {
+    torch.Tensor.transpose, torch.Tensor.t, torch.Tensor.bfloat16, torch.Tensor.to,
+    torch.Tensor.detach, torch.Tensor.requires_grad_, torch.Tensor.contiguous,
+    torch.Tensor.view, torch.Tensor.reshape, torch.Tensor.float, torch.Tensor.half,
+    torch.transpose, torch.empty_like, torch.zeros_like, torch.Tensor.clone, torch.clone,
+    torch.Tensor.cuda, torch.Tensor.cpu, torch.Tensor.type,
+}
+
+
+def _flatten(args):
+    for a in args:
+        if isinstance(a, (list, tuple)):
+            yield from _flatten(a)
+        else:
+            yield a
+
+
+def _rewrap(out, cls, cfg, func):
+    """Results of view / cast / clone style ops on a wrapped weight stay wrapped; in-place ops
+    return their (already wrapped) input; everything else is a plain tensor."""
+    if cfg is None or func not in _KEEP_WRAPPED:
+        return out
+    if isinstance(out, torch.Tensor) and not isinstance(out, cls):
+        wrapped = out.as_subclass(cls)
+        wrapped.mx_config = cfg
+        return wrapped
+    return out
+
+
+def wrap_parameter(param: torch.nn.Parameter, cfg: MXFP8Config) -> torch.nn.Parameter:
+    """A Parameter of type MXFP8TrainingWeight sharing `param`'s storage."""
+    if isinstance(param.data, MXFP8TrainingWeight) or isinstance(param, MXFP8TrainingWeight):
+        return param
+    return torch.nn.Parameter(MXFP8TrainingWeight(param.data, cfg), requires_grad=param.requires_grad)

@@ -1,0 +1,118 @@
+"""``MXFP8Converter``: the model-converter plugin that switches target linears and 3-D expert
+parameters to MXFP8 GEMMs on MI355X.
+
+Same surface as the reference's converter (torchtitan/components/quantization/mx.py:26-140):
+``Config(recipe_name, fqns, pad_token_groups_for_grouped_mm)``, ``_quantization_type = "mxfp8"``,
+constructor kwargs ``parallel_dims`` and ``model_compile_enabled``, ``convert(model)`` mutating in
+place, ``post_optimizer_hook`` a no-op.  Where the reference hands the work to an external
+library and asserts an SM100 GPU, this converter wraps the weights in ``MXFP8TrainingWeight``
+(backed by the in-tree HIP library) and asserts a gfx950 GPU.
+"""
+from __future__ import annotations
+
+import logging
+from dataclasses import dataclass, field
+from typing import Any, ClassVar, Literal
+
+import torch
+import torch.nn as nn
+
+from .. import _lib
+from ..modules.linear import Linear
+from ..mx_tensor import MXFP8Config, MXFP8TrainingWeight, wrap_parameter
+from . import QuantizationConverter
+from .module_utils import capture_module_attrs, inject_module_protocol, verify_module_protocol
+
+logger = logging.getLogger("torchtitan_amd")
+
+_RECIPES = {"mxfp8_rceil": "rceil", "mxfp8_floor": "floor"}
+
+
+def has_rocm_capability(major: int, minor: int) -> bool:
+    """True on an AMD GPU of at least gfx<major><minor>x (9, 5 -> gfx950 = MI350X / MI355X)."""
+    if not torch.cuda.is_available() or torch.version.hip is None:
+        return False
+    arch = torch.cuda.get_device_properties(0).gcnArchName.split(":")[0]
+    digits = arch.removeprefix("gfx")
+    try:
+        got = (int(digits[:-2]), int(digits[-2], 16))
+    except ValueError:
+        return False
+    return got >= (major, minor)
+
+
+class MXFP8Converter(QuantizationConverter):
+    """Wraps the weights of target ``nn.Linear`` modules and 3-D ``nn.Parameter`` experts in a
+    tensor subclass that overrides ``F.linear`` and ``torch._grouped_mm`` with dynamically
+    quantized MXFP8 GEMMs."""
+
+    @dataclass(kw_only=True, slots=True)
+    class Config(QuantizationConverter.Config):
+        _quantization_type: ClassVar[str] = "mxfp8"
+
+        recipe_name: Literal["mxfp8_rceil", "mxfp8_floor"] = "mxfp8_rceil"
+        """mxfp8_rceil: E8M0 scale = ceil(log2(amax / 448)) (the reference's recipe);
+        mxfp8_floor: scale = floor(log2 amax) - 8 (OCP MX v1.0 default, codes may saturate)."""
+
+        fqns: list[str] = field(default_factory=list)
+        """Modules whose fully qualified name contains any of these strings are converted.
+        The default (empty) converts nothing."""
+
+        pad_token_groups_for_grouped_mm: bool = True
+        """Pad token groups to multiples of 32 inside the grouped GEMM.  Set to false when the
+        dispatcher already delivers 32-aligned groups."""
+
+    def __init__(self, config: Config, *, parallel_dims: Any, model_compile_enabled: bool):
+        self.enabled = False
+        if not _lib.LIB_PATH.exists():
+            raise ImportError(
+                f"{_lib.LIB_PATH.name} is not built. Run `python -m torchtitan_amd._build` "
+                "to use MXFP8 linear layers."
+            )
+        assert has_rocm_capability(9, 5), "MXFP8 is only supported on gfx950 (MI350X/MI355X) GPUs"
+        if config.recipe_name not in _RECIPES:
+            raise ValueError(f"unknown recipe {config.recipe_name!r}; options: {sorted(_RECIPES)}")
+        if model_compile_enabled:
+            logger.warning("the MXFP8 path runs eager HIP kernels; torch.compile adds nothing to it")
+        self.config = config
+        self.enabled = True
+        logger.info("MXFP8 training enabled")
+
+    def _matches(self, fqn: str) -> bool:
+        return any(target in fqn for target in self.config.fqns)
+
+    def convert(self, model: nn.Module):
+        """Replace, in place, the weight of every matching ``nn.Linear`` and every matching
+        module's 3-D parameters by an ``MXFP8TrainingWeight`` sharing the same storage."""
+        if not self.enabled:
+            return
+        verify_module_protocol(model, nn.Linear, Linear)
+        saved = capture_module_attrs(model, ["_init_mean", "_init_std"], nn_module_cls=nn.Linear)
+        cfg = MXFP8Config(_RECIPES[self.config.recipe_name],
+                          self.config.pad_token_groups_for_grouped_mm)
+        n_linear = n_grouped = 0
+        for fqn, mod in model.named_modules():
+            if not self._matches(fqn):
+                continue
+            if isinstance(mod, nn.Linear):
+                if mod.in_features % 32:
+                    logger.warning("skipping %s: in_features %d is not a multiple of 32", fqn, mod.in_features)
+                    continue
+                mod.weight = wrap_parameter(mod.weight, cfg)
+                n_linear += 1
+                continue
+            for name, p in list(mod.named_parameters(recurse=False)):
+                if p.dim() == 3 and not isinstance(p, MXFP8TrainingWeight):
+                    setattr(mod, name, wrap_parameter(p, cfg))
+                    n_grouped += 1
+        inject_module_protocol(model, Linear, saved)
+        verify_module_protocol(model, nn.Linear, Linear)
+        logger.info(
+            "Converted %d linear weights and %d grouped expert weights matching FQNs %s "
+            "to dynamic %s quantization for grouped_mm and linear ops",
+            n_linear, n_grouped, self.config.fqns, self.config.recipe_name,
+        )
+
+    def post_optimizer_hook(self, model: nn.Module | list[nn.Module]):
+        """MXFP8 training needs no post-optimizer work: weights are re-quantized every forward."""
+        return
