@@ -1,0 +1,238 @@
+#!/usr/bin/env python3
+"""Benchmark of the MXFP8 linear path on one MI355X.
+
+Workload (BASELINE.json configs[1]): dense MXFP8 linear forward + dgrad + wgrad at the
+Llama-3-8B FFN shapes, M = 16384 tokens; w1 and w3 are [14336, 4096], w2 is [4096, 14336];
+activations N(0,1), weights N(0,0.02), upstream grads N(0,1e-3), all bf16, seeded, resident in
+HBM before the timed region.  One step = the three linears, each through the converted module
+(product path): 2 fused casts + GEMM in forward, 1 fused cast + 2 GEMMs in backward.
+
+Prints ONE JSON line.  `value` counts only GEMM flops (2 M N K each) over the whole step time,
+casts included in the time.  `roofline` is for the dominant kernel (the 256x256 MXFP8 GEMM
+tile kernel), timed per launch with HIP events on the launch stream inside the timed steps.
+`casts` gives the to_mx GB/s on inputs rotated through more memory than the 256 MB last-level
+cache.  `cpu_baseline` times the CPU oracle (emulated MX linear forward) on a bounded sample.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+METRIC = "MXFP8 linear TFLOP/s fwd+bwd at 8B FFN shape; to_mx cast GB/s"
+M, DIM, HIDDEN = 16384, 4096, 14336
+PEAK_MXFP8_TFLOPS = 5000.0  # MI355X dense fp8 / MXFP8 MFMA peak
+PEAK_HBM_GBPS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--recipe", default="mxfp8_rceil", choices=["mxfp8_rceil", "mxfp8_floor"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-casts", action="store_true")
+    return ap.parse_args()
+
+
+def build_linears(dev, recipe):
+    import torch
+    import torch.nn as nn
+
+    from torchtitan_amd.modules import Linear
+    from torchtitan_amd.protocols import ModelConvertersContainer
+    from torchtitan_amd.quantization.mx import MXFP8Converter
+
+    g = torch.Generator(device=dev).manual_seed(0)
+    ffn = nn.Module()
+    ffn.w1 = Linear.Config().build(in_features=DIM, out_features=HIDDEN)
+    ffn.w3 = Linear.Config().build(in_features=DIM, out_features=HIDDEN)
+    ffn.w2 = Linear.Config().build(in_features=HIDDEN, out_features=DIM)
+    holder = nn.Module()
+    holder.feed_forward = ffn
+    ModelConvertersContainer.Config(
+        converters=[MXFP8Converter.Config(fqns=["feed_forward"], recipe_name=recipe)]
+    ).build(parallel_dims=None, model_compile_enabled=False).convert(holder)
+    holder.to(dev).to(torch.bfloat16)
+    with torch.no_grad():
+        for lin in (ffn.w1, ffn.w3, ffn.w2):
+            lin.weight.copy_(torch.randn(lin.weight.shape, generator=g, device=dev, dtype=torch.float32) * 0.02)
+    x = torch.randn((M, DIM), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    h = torch.randn((M, HIDDEN), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    dy_h = (torch.randn((M, HIDDEN), generator=g, device=dev, dtype=torch.float32) * 1e-3).to(torch.bfloat16)
+    dy_o = (torch.randn((M, DIM), generator=g, device=dev, dtype=torch.float32) * 1e-3).to(torch.bfloat16)
+    return ffn, x, h, dy_h, dy_o
+
+
+def one_step(ffn, x, h, dy_h, dy_o):
+    from torchtitan_amd import mx_tensor
+
+    mx_tensor._cast_cache.clear()  # a new step has new activations: nothing carries over
+    x.grad = None
+    h.grad = None
+    for lin, inp, dy in ((ffn.w1, x, dy_h), (ffn.w3, x, dy_h), (ffn.w2, h, dy_o)):
+        lin.weight.grad = None
+        y = lin(inp)
+        y.backward(dy)
+
+
+def time_casts(dev, recipe_mode):
+    """to_mx GB/s per direction on cold inputs (rotating buffers > last-level cache)."""
+    import torch
+
+    from torchtitan_amd import ops
+
+    out = {}
+    L = ops.MX_SCALES_MFMA
+    for name, shape, nbuf in (("x_16384x4096", (M, DIM), 6), ("dy_16384x14336", (M, HIDDEN), 3),
+                              ("w_14336x4096", (HIDDEN, DIM), 6)):
+        bufs = [torch.randn(shape, device=dev, dtype=torch.bfloat16) for _ in range(nbuf)]
+        el = shape[0] * shape[1]
+        for kind, fn, bpe in (("dim0", ops.to_mx_dim0, 3.03125), ("dim1", ops.to_mx_dim1, 3.03125),
+                              ("dim0_dim1", ops.to_mx_dim0_dim1, 4.0625)):
+            for b in bufs[:2]:
+                fn(b, recipe_mode, L)
+            torch.cuda.synchronize()
+            reps = 3 * nbuf
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            for i in range(reps):
+                fn(bufs[i % nbuf], recipe_mode, L)
+            e.record()
+            torch.cuda.synchronize()
+            sec = s.elapsed_time(e) * 1e-3 / reps
+            out[f"{kind}:{name}"] = {"us": round(sec * 1e6, 1), "GB/s": round(el * bpe / sec / 1e9, 1),
+                                     "frac_hbm": round(el * bpe / sec / 1e9 / PEAK_HBM_GBPS, 3)}
+        del bufs
+    return out
+
+
+def cpu_baseline(recipe_mode_int):
+    """CPU oracle (emulated MX linear forward: cast X, cast W along K, dequantize, fp32 matmul,
+    bf16 out) on a bounded sample of BASELINE config 1."""
+    import numpy as np
+
+    from oracle import c_oracle as co
+    from oracle import mx_oracle as mo
+
+    cores = min(16, os.cpu_count() or 1)
+    os.environ.setdefault("OMP_NUM_THREADS", str(cores))
+    Ms, K, N = 2048, 4096, 4096
+    xb, wb = mo.make_cfg1_inputs(0, Ms, K, N)
+    t0 = time.perf_counter()
+    xc, xs = co.cast_dim0(xb, recipe_mode_int)
+    wc, ws = co.cast_dim0(wb, recipe_mode_int)
+    t1 = time.perf_counter()
+    a = co.dequant(xc, xs)
+    b = co.dequant(wc, ws)
+    y = mo.f32_to_bf16_bits(a @ b.T)
+    t2 = time.perf_counter()
+    # the C casts must agree with the NumPy oracle on a slice (checker sanity, not a measurement)
+    assert np.array_equal(mo.cast_dim0(xb[:64], recipe_mode_int)[0], xc[:64])
+    flops = 2.0 * Ms * K * N
+    cast_bytes = (Ms * K + N * K) * 3.03125
+    return {
+        "value": round(flops / (t2 - t0) / 1e12, 4),
+        "unit": "TFLOP/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"config 1 at M={Ms} (X[{Ms},{K}], W[{N},{K}], 0.1% x100 outliers): to_mx dim0 of X and W "
+                  f"(C oracle, OpenMP) + dequantize + fp32 matmul (NumPy BLAS) + bf16 round; "
+                  f"casts {cast_bytes / (t1 - t0) / 1e9:.2f} GB/s, matmul part {flops / (t2 - t1) / 1e12:.3f} TFLOP/s, "
+                  f"wall {t2 - t0:.2f} s",
+        "checksum": int(y.astype(np.uint64).sum() % (1 << 32)),
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (no collectives on this path); "
+              f"--gpus {args.gpus} is not supported", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    from torchtitan_amd import _lib, ops
+
+    _lib.load()  # fail loudly if the HIP library is missing
+    dev = torch.device("cuda:0")
+    recipe_mode = {"mxfp8_rceil": "rceil", "mxfp8_floor": "floor"}[args.recipe]
+    ffn, x, h, dy_h, dy_o = build_linears(dev, args.recipe)
+    x.requires_grad_(True)
+    h.requires_grad_(True)
+
+    for _ in range(args.warmup):
+        one_step(ffn, x, h, dy_h, dy_o)
+    torch.cuda.synchronize()
+    timer = ops.KernelTimer()
+    ops.set_kernel_timer(timer)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        one_step(ffn, x, h, dy_h, dy_o)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ops.set_kernel_timer(None)
+    per_kernel = timer.summary()
+
+    step_s = (t1 - t0) / args.steps
+    gemm_flops = 2.0 * M * DIM * HIDDEN  # per GEMM; 9 GEMMs per step
+    value = 9 * gemm_flops / step_s / 1e12
+    n_gemm, gemm_ms = per_kernel["gemm_nt"]
+    achieved = gemm_flops / (gemm_ms * 1e-3) / 1e12
+    cast_ms = sum(ms * n for k, (n, ms) in per_kernel.items() if k.startswith("cast")) / args.steps
+    line = {
+        "metric": METRIC,
+        "value": round(value, 1),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 3),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "mxfp8 (e4m3 codes x e8m0 block scales, fp32 accumulate, bf16 out)",
+        "data": "synthetic",
+        "config": {
+            "workload": "configs[1]: dense MXFP8 linear fwd+dgrad+wgrad, Llama-3-8B FFN shapes "
+                        "(w1,w3: K=4096,N=14336; w2: K=14336,N=4096), M=16384 tokens",
+            "recipe": args.recipe,
+            "gemms_per_step": 9,
+            "casts_per_step": 8,
+        },
+        "roofline": {
+            "kernel": "gemm_nt_kernel<256,256> (v_mfma_scale_f32_16x16x128_f8f6f4)",
+            "bound": "mfma",
+            "achieved": round(achieved, 1),
+            "peak": PEAK_MXFP8_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(achieved / PEAK_MXFP8_TFLOPS, 4),
+            "traffic": None,
+            "launches_timed": n_gemm,
+            "avg_launch_ms": round(gemm_ms, 4),
+        },
+        "step_breakdown_ms": {
+            "gemm": round(gemm_ms * n_gemm / args.steps, 3),
+            "casts": round(cast_ms, 3),
+            "total": round(step_s * 1e3, 3),
+        },
+        "kernels_ms": {k: {"launches": n, "avg_ms": round(ms, 4)} for k, (n, ms) in sorted(per_kernel.items())},
+    }
+    if not args.no_casts:
+        line["casts"] = time_casts(dev, recipe_mode)
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(0 if recipe_mode == "floor" else 1)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

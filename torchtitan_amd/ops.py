@@ -26,6 +26,53 @@ class MXData(NamedTuple):
     scale_order: int  # MX_SCALES_ROWMAJOR: [rows, cols/32]; MX_SCALES_MFMA: flat re-laid buffer
 
 
+class KernelTimer:
+    """Optional per-launch timing with HIP events on the launch stream (used by bench.py).
+
+    While a timer is installed with ``set_kernel_timer`` every library call is bracketed by two
+    events recorded on the stream it is launched on; ``summary()`` synchronises once and
+    returns {kernel name: (launches, mean milliseconds)}.
+    """
+
+    def __init__(self):
+        self.records = []
+
+    def bracket(self, name: str, device):
+        start = torch.cuda.Event(enable_timing=True)
+        stop = torch.cuda.Event(enable_timing=True)
+        self.records.append((name, start, stop))
+        return start, stop
+
+    def summary(self):
+        torch.cuda.synchronize()
+        acc: dict[str, list[float]] = {}
+        for name, a, b in self.records:
+            acc.setdefault(name, []).append(a.elapsed_time(b))
+        return {k: (len(v), sum(v) / len(v)) for k, v in acc.items()}
+
+
+_timer: KernelTimer | None = None
+
+
+def set_kernel_timer(timer: KernelTimer | None) -> None:
+    global _timer
+    _timer = timer
+
+
+def _call(name: str, tag: str, device, *args) -> None:
+    """Run one C-ABI entry point on `device`'s current stream and raise on a non-zero status."""
+    fn = getattr(_lib.load(), name)
+    with torch.cuda.device(device):
+        if _timer is None:
+            st = fn(*args)
+        else:
+            start, stop = _timer.bracket(tag, device)
+            start.record()
+            st = fn(*args)
+            stop.record()
+    _lib.check(st, name)
+
+
 def _mode(mode) -> int:
     if isinstance(mode, str):
         return SCALE_MODES[mode]
@@ -72,10 +119,7 @@ def to_mx_dim0(x: torch.Tensor, mode="floor", order: int = MX_SCALES_ROWMAJOR) -
         raise ValueError(f"last dim {C} is not a multiple of {BLOCK}")
     codes = torch.empty((R, C), dtype=torch.uint8, device=x.device)
     scales = _alloc_scales(R, C // BLOCK, order, x.device)
-    with torch.cuda.device(x.device):
-        st = _lib.load().mx_cast_dim0(_ptr(x), R, C, x.stride(0), _ptr(codes), _ptr(scales),
-                                      _mode(mode), order, _stream(x))
-    _lib.check(st, "mx_cast_dim0")
+    _call("mx_cast_dim0", "cast_dim0", x.device, _ptr(x), R, C, x.stride(0), _ptr(codes), _ptr(scales), _mode(mode), order, _stream(x))
     return MXData(codes, scales, order)
 
 
@@ -87,10 +131,7 @@ def to_mx_dim1(x: torch.Tensor, mode="floor", order: int = MX_SCALES_ROWMAJOR) -
         raise ValueError(f"first dim {R} is not a multiple of {BLOCK}")
     codes = torch.empty((C, R), dtype=torch.uint8, device=x.device)
     scales = _alloc_scales(C, R // BLOCK, order, x.device)
-    with torch.cuda.device(x.device):
-        st = _lib.load().mx_cast_dim1(_ptr(x), R, C, x.stride(0), _ptr(codes), _ptr(scales),
-                                      _mode(mode), order, _stream(x))
-    _lib.check(st, "mx_cast_dim1")
+    _call("mx_cast_dim1", "cast_dim1", x.device, _ptr(x), R, C, x.stride(0), _ptr(codes), _ptr(scales), _mode(mode), order, _stream(x))
     return MXData(codes, scales, order)
 
 
@@ -104,11 +145,7 @@ def to_mx_dim0_dim1(x: torch.Tensor, mode="floor", order: int = MX_SCALES_ROWMAJ
     scales = _alloc_scales(R, C // BLOCK, order, x.device)
     codes_t = torch.empty((C, R), dtype=torch.uint8, device=x.device)
     scales_t = _alloc_scales(C, R // BLOCK, order, x.device)
-    with torch.cuda.device(x.device):
-        st = _lib.load().mx_cast_dim0_dim1(_ptr(x), R, C, x.stride(0), _ptr(codes), _ptr(scales),
-                                           _ptr(codes_t), _ptr(scales_t), _mode(mode), order,
-                                           _stream(x))
-    _lib.check(st, "mx_cast_dim0_dim1")
+    _call("mx_cast_dim0_dim1", "cast_dim0_dim1", x.device, _ptr(x), R, C, x.stride(0), _ptr(codes), _ptr(scales), _ptr(codes_t), _ptr(scales_t), _mode(mode), order, _stream(x))
     return MXData(codes, scales, order), MXData(codes_t, scales_t, order)
 
 
@@ -117,17 +154,13 @@ def scale_layout(scales: torch.Tensor) -> torch.Tensor:
     rows, nblk = scales.shape
     scales = scales.contiguous()
     out = torch.empty(mfma_scale_bytes(rows, nblk), dtype=torch.uint8, device=scales.device)
-    with torch.cuda.device(scales.device):
-        st = _lib.load().mx_scale_layout(_ptr(scales), rows, nblk, _ptr(out), _stream(scales))
-    _lib.check(st, "mx_scale_layout")
+    _call("mx_scale_layout", "scale_layout", scales.device, _ptr(scales), rows, nblk, _ptr(out), _stream(scales))
     return out
 
 
 def scale_unlayout(laid: torch.Tensor, rows: int, nblk: int) -> torch.Tensor:
     out = torch.empty((rows, nblk), dtype=torch.uint8, device=laid.device)
-    with torch.cuda.device(laid.device):
-        st = _lib.load().mx_scale_unlayout(_ptr(laid), rows, nblk, _ptr(out), _stream(laid))
-    _lib.check(st, "mx_scale_unlayout")
+    _call("mx_scale_unlayout", "scale_unlayout", laid.device, _ptr(laid), rows, nblk, _ptr(out), _stream(laid))
     return out
 
 
@@ -146,10 +179,7 @@ def mx_gemm_nt(a: MXData, b: MXData, out: torch.Tensor | None = None) -> torch.T
     elif out.shape != (M, N) or out.dtype != torch.bfloat16 or out.stride(1) != 1:
         raise ValueError("out must be a bf16 [M, N] tensor with unit inner stride")
     sa, sb = _as_mfma(a), _as_mfma(b)
-    with torch.cuda.device(out.device):
-        st = _lib.load().mx_gemm_nt(_ptr(a.codes), _ptr(sa), _ptr(b.codes), _ptr(sb), _ptr(out),
-                                    M, N, K, out.stride(0), _stream(out))
-    _lib.check(st, "mx_gemm_nt")
+    _call("mx_gemm_nt", f"gemm_nt", out.device, _ptr(a.codes), _ptr(sa), _ptr(b.codes), _ptr(sb), _ptr(out), M, N, K, out.stride(0), _stream(out))
     return out
 
 
@@ -179,10 +209,7 @@ def to_mx_dim1_batched(w: torch.Tensor, mode="floor", order: int = MX_SCALES_MFM
     codes = torch.empty((G, C, R), dtype=torch.uint8, device=w.device)
     per = mfma_scale_bytes(C, R // BLOCK) if order == MX_SCALES_MFMA else C * (R // BLOCK)
     scales = torch.empty(G * per, dtype=torch.uint8, device=w.device)
-    with torch.cuda.device(w.device):
-        st = _lib.load().mx_cast_dim1_batched(_ptr(w), G, R, C, C, _ptr(codes), _ptr(scales),
-                                              _mode(mode), order, _stream(w))
-    _lib.check(st, "mx_cast_dim1_batched")
+    _call("mx_cast_dim1_batched", "cast_dim1_batched", w.device, _ptr(w), G, R, C, C, _ptr(codes), _ptr(scales), _mode(mode), order, _stream(w))
     if order == MX_SCALES_ROWMAJOR:
         scales = scales.view(G, C, R // BLOCK)
     return MXData(codes, scales, order)
@@ -204,11 +231,7 @@ def to_mx_dim0_dim1_batched(w: torch.Tensor, mode="floor", order: int = MX_SCALE
         per, per_t = R * (C // BLOCK), C * (R // BLOCK)
     scales = torch.empty(G * per, dtype=torch.uint8, device=w.device)
     scales_t = torch.empty(G * per_t, dtype=torch.uint8, device=w.device)
-    with torch.cuda.device(w.device):
-        st = _lib.load().mx_cast_dim0_dim1_batched(_ptr(w), G, R, C, C, _ptr(codes), _ptr(scales),
-                                                   _ptr(codes_t), _ptr(scales_t), _mode(mode),
-                                                   order, _stream(w))
-    _lib.check(st, "mx_cast_dim0_dim1_batched")
+    _call("mx_cast_dim0_dim1_batched", "cast_dim0_dim1_batched", w.device, _ptr(w), G, R, C, C, _ptr(codes), _ptr(scales), _ptr(codes_t), _ptr(scales_t), _mode(mode), order, _stream(w))
     if order == MX_SCALES_ROWMAJOR:
         scales, scales_t = scales.view(G, R, C // BLOCK), scales_t.view(G, C, R // BLOCK)
     return MXData(codes, scales, order), MXData(codes_t, scales_t, order)
@@ -232,11 +255,7 @@ def mx_grouped_gemm_2d3d(a: MXData, b: MXData, offs: torch.Tensor,
         raise ValueError("offs must be int32 with one entry per group")
     if out is None:
         out = torch.empty((T, N), dtype=torch.bfloat16, device=a.codes.device)
-    with torch.cuda.device(out.device):
-        st = _lib.load().mx_grouped_gemm_2d3d(_ptr(a.codes), _ptr(a.scales), _ptr(b.codes),
-                                              _ptr(b.scales), _ptr(offs), _ptr(out), T, N, K, G,
-                                              out.stride(0), _stream(out))
-    _lib.check(st, "mx_grouped_gemm_2d3d")
+    _call("mx_grouped_gemm_2d3d", "grouped_gemm_2d3d", out.device, _ptr(a.codes), _ptr(a.scales), _ptr(b.codes), _ptr(b.scales), _ptr(offs), _ptr(out), T, N, K, G, out.stride(0), _stream(out))
     return out
 
 
@@ -255,11 +274,7 @@ def mx_grouped_gemm_2d2d(at: MXData, bt: MXData, offs: torch.Tensor,
     G = offs.numel()
     if out is None:
         out = torch.empty((G, N, K), dtype=torch.bfloat16, device=at.codes.device)
-    with torch.cuda.device(out.device):
-        st = _lib.load().mx_grouped_gemm_2d2d(_ptr(at.codes), _ptr(at.scales), _ptr(bt.codes),
-                                              _ptr(bt.scales), _ptr(offs), _ptr(out), T, N, K, G,
-                                              _stream(out))
-    _lib.check(st, "mx_grouped_gemm_2d2d")
+    _call("mx_grouped_gemm_2d2d", "grouped_gemm_2d2d", out.device, _ptr(at.codes), _ptr(at.scales), _ptr(bt.codes), _ptr(bt.scales), _ptr(offs), _ptr(out), T, N, K, G, _stream(out))
     return out
 
 
@@ -272,9 +287,5 @@ def group_offsets_pad(counts: torch.Tensor, experts_per_rank: int, num_ranks: in
     perm = torch.empty(max_len, dtype=torch.int64, device=counts.device)
     m_sizes = torch.empty(experts_per_rank, dtype=torch.int32, device=counts.device)
     m_offsets = torch.empty(experts_per_rank, dtype=torch.int32, device=counts.device)
-    with torch.cuda.device(counts.device):
-        st = _lib.load().mx_group_offsets_pad(_ptr(c32), experts_per_rank, num_ranks, max_len,
-                                              alignment, _ptr(perm), _ptr(m_sizes),
-                                              _ptr(m_offsets), _stream(counts))
-    _lib.check(st, "mx_group_offsets_pad")
+    _call("mx_group_offsets_pad", "group_offsets_pad", counts.device, _ptr(c32), experts_per_rank, num_ranks, max_len, alignment, _ptr(perm), _ptr(m_sizes), _ptr(m_offsets), _stream(counts))
     return perm, m_sizes, m_offsets
