@@ -41,9 +41,10 @@ typedef enum { MX_SCALE_FLOOR = 0, MX_SCALE_RCEIL = 1 } mx_scale_mode_t;
 
 /* Where a cast writes its scale bytes:
  *   ROWMAJOR  [rows, nblk]
- *   MFMA      [ceil(rows/64), ceil(nblk/4), 64, 4]: for row tile rt, K-step ks, lane l,
- *             byte t the entry is scale[rt*64 + t*16 + (l & 15)][ks*4 + (l >> 4)]
- *             (zero beyond the matrix) -- the order mx_gemm_nt reads.
+ *   MFMA      [ceil(rows/128), ceil(nblk/2), 64, 4]: for row group rt, 64-deep K step ks,
+ *             lane l, byte t the entry is scale[rt*128 + t*32 + (l & 31)][ks*2 + (l >> 5)]
+ *             (zero beyond the matrix) -- one dword per lane feeds four 32-row sub-tiles of
+ *             v_mfma_scale_f32_32x32x64_f8f6f4; the order mx_gemm_nt reads.
  */
 typedef enum { MX_SCALES_ROWMAJOR = 0, MX_SCALES_MFMA = 1 } mx_scale_order_t;
 

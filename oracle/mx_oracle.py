@@ -294,25 +294,25 @@ def grouped_wgrad(dy_bits, x_bits, offs, mode=FLOOR):
 def scale_layout(scales: np.ndarray) -> np.ndarray:
     """Permute a [rows, nblk] scale matrix into the order the MFMA loop reads.
 
-    Output is [ceil(rows/64), ceil(nblk/4), 64, 4] bytes: for row-tile rt, K-step ks,
-    lane l and byte t the entry is scales[rt*64 + t*16 + (l & 15)][ks*4 + (l >> 4)],
-    zero where that index is out of range.  One aligned dword per lane then holds the
-    scales of the lane's K-block for four consecutive 16-row sub-tiles.
+    Output is [ceil(rows/128), ceil(nblk/2), 64, 4] bytes: for row group rt, K step ks (64
+    deep = 2 blocks), lane l and byte t the entry is scales[rt*128 + t*32 + (l & 31)][ks*2 + (l >> 5)],
+    zero where that index is out of range.  One aligned dword per lane then holds the scales a
+    32x32x64 MFMA lane needs for four consecutive 32-row sub-tiles.
     """
     rows, nblk = scales.shape
-    rt_n = (rows + 63) // 64
-    ks_n = (nblk + 3) // 4
-    padded = np.zeros((rt_n * 64, ks_n * 4), dtype=np.uint8)
+    rt_n = (rows + 127) // 128
+    ks_n = (nblk + 1) // 2
+    padded = np.zeros((rt_n * 128, ks_n * 2), dtype=np.uint8)
     padded[:rows, :nblk] = scales
     # [rt, t, i, ks, j] -> [rt, ks, j, i, t]
-    v = padded.reshape(rt_n, 4, 16, ks_n, 4)
+    v = padded.reshape(rt_n, 4, 32, ks_n, 2)
     return np.ascontiguousarray(v.transpose(0, 3, 4, 2, 1)).reshape(rt_n, ks_n, 64, 4)
 
 
 def scale_unlayout(laid: np.ndarray, rows: int, nblk: int) -> np.ndarray:
     rt_n, ks_n = laid.shape[:2]
-    v = laid.reshape(rt_n, ks_n, 4, 16, 4).transpose(0, 4, 3, 1, 2)
-    return np.ascontiguousarray(v).reshape(rt_n * 64, ks_n * 4)[:rows, :nblk]
+    v = laid.reshape(rt_n, ks_n, 2, 32, 4).transpose(0, 4, 3, 1, 2)
+    return np.ascontiguousarray(v).reshape(rt_n * 128, ks_n * 2)[:rows, :nblk]
 
 
 # --------------------------------------------------------------------------- group padding

@@ -42,7 +42,7 @@ def test_grouped_forward_and_dgrad(device, sizes, N, K, tail_rows):
     dy_bits = randn_bits(rng, (T, N), std=1e-3)
     offs = _sizes_to_offs(sizes, device)
     x, w, dy = (bf16_from_bits(b, device) for b in (x_bits, w_bits, dy_bits))
-    pad64 = N % 64 == 0
+    pad64 = N % 128 == 0
     for mode_name, mode in (("floor", mo.FLOOR), ("rceil", mo.RCEIL)):
         wq0, wq1 = ops.to_mx_dim0_dim1_batched(w, mode_name, L)
         if pad64:

@@ -255,10 +255,10 @@ def test_scale_layout_index_formula_and_round_trip():
     for rows, nblk in [(64, 4), (100, 7), (200, 13), (16, 1)]:
         s = rng.integers(1, 255, size=(rows, nblk), dtype=np.uint8)
         laid = mo.scale_layout(s)
-        assert laid.shape == ((rows + 63) // 64, (nblk + 3) // 4, 64, 4)
+        assert laid.shape == ((rows + 127) // 128, (nblk + 1) // 2, 64, 4)
         for _ in range(200):
             rt, ks, lane, t = (int(rng.integers(0, n)) for n in laid.shape)
-            r, b = rt * 64 + t * 16 + (lane & 15), ks * 4 + (lane >> 4)
+            r, b = rt * 128 + t * 32 + (lane & 31), ks * 2 + (lane >> 5)
             assert laid[rt, ks, lane, t] == (s[r, b] if r < rows and b < nblk else 0)
         assert np.array_equal(mo.scale_unlayout(laid, rows, nblk), s)
 

@@ -138,10 +138,10 @@ __device__ __forceinline__ void store_transposed_tile(const uint8_t* lds_codes,
   if (tid < kT) {
     const uint32_t s4 = *reinterpret_cast<const uint32_t*>(lds_scales + tid * 4);
     if (ORDER == MX_SCALES_MFMA) {
-      // the 512 staged bytes are two complete 256-byte (64-row, K-step) groups
-      const int64_t rt = (c0 >> 6) + (tid >> 6);
-      if (rt * 64 < ((cols + 63) & ~int64_t(63)))
-        *reinterpret_cast<uint32_t*>(scales_t + ((rt * ks_n_t + (r0 >> 7)) << 8) +
+      // the 512 staged bytes are two complete 256-byte (128-row, 64-deep K step) groups
+      const int64_t ks = (r0 >> 6) + (tid >> 6);
+      if (ks < ks_n_t)
+        *reinterpret_cast<uint32_t*>(scales_t + (((c0 >> 7) * ks_n_t + ks) << 8) +
                                      (tid & 63) * 4) = s4;
     } else if (c0 + tid < cols) {
       const int64_t b0 = r0 >> 5;
@@ -191,8 +191,8 @@ __global__ __launch_bounds__(256) void cast_dim1_kernel(const uint16_t* __restri
   if (!live) sa = sb = 0;
   if (ORDER == MX_SCALES_MFMA) {
     const int ca_ = 2 * lane, cb_ = 2 * lane + 1;
-    lds_scales[(ca_ >> 6) * 256 + (wave * 16 + (ca_ & 15)) * 4 + ((ca_ & 63) >> 4)] = (uint8_t)sa;
-    lds_scales[(cb_ >> 6) * 256 + (wave * 16 + (cb_ & 15)) * 4 + ((cb_ & 63) >> 4)] = (uint8_t)sb;
+    lds_scales[(wave >> 1) * 256 + (((wave & 1) << 5) + (ca_ & 31)) * 4 + (ca_ >> 5)] = (uint8_t)sa;
+    lds_scales[(wave >> 1) * 256 + (((wave & 1) << 5) + (cb_ & 31)) * 4 + (cb_ >> 5)] = (uint8_t)sb;
   } else {
     lds_scales[(2 * lane) * 4 + wave] = (uint8_t)sa;
     lds_scales[(2 * lane + 1) * 4 + wave] = (uint8_t)sb;
@@ -273,8 +273,8 @@ __global__ __launch_bounds__(256) void cast_dim0_dim1_kernel(
   if (!live) sa = sb = 0;
   if (ORDER == MX_SCALES_MFMA) {
     const int ca_ = 2 * lane, cb_ = 2 * lane + 1;
-    lds_scales[(ca_ >> 6) * 256 + (wave * 16 + (ca_ & 15)) * 4 + ((ca_ & 63) >> 4)] = (uint8_t)sa;
-    lds_scales[(cb_ >> 6) * 256 + (wave * 16 + (cb_ & 15)) * 4 + ((cb_ & 63) >> 4)] = (uint8_t)sb;
+    lds_scales[(wave >> 1) * 256 + (((wave & 1) << 5) + (ca_ & 31)) * 4 + (ca_ >> 5)] = (uint8_t)sa;
+    lds_scales[(wave >> 1) * 256 + (((wave & 1) << 5) + (cb_ & 31)) * 4 + (cb_ >> 5)] = (uint8_t)sb;
   } else {
     lds_scales[(2 * lane) * 4 + wave] = (uint8_t)sa;
     lds_scales[(2 * lane + 1) * 4 + wave] = (uint8_t)sb;
@@ -296,11 +296,11 @@ __global__ __launch_bounds__(256) void scale_layout_kernel(const uint8_t* __rest
   const int lane = (int)(d & 63);
   const int64_t g = d >> 6;
   const int64_t ks = g % ks_n, rt = g / ks_n;
-  const int64_t blk = ks * 4 + (lane >> 4);
+  const int64_t blk = ks * 2 + (lane >> 5);
   uint32_t w = 0;
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
-    const int64_t r = rt * 64 + t * 16 + (lane & 15);
+    const int64_t r = rt * 128 + t * 32 + (lane & 31);
     if (r < rows && blk < nblk) w |= (uint32_t)in[r * nblk + blk] << (8 * t);
   }
   out[d] = w;
@@ -353,13 +353,13 @@ static inline int launch_status() {
   return hipGetLastError() == hipSuccess ? MX_OK : MX_ERR_LAUNCH;
 }
 // The row-wise kernels write one scale byte per block and never touch the padding of an
-// MFMA-order buffer; when the matrix does not fill whole (64-row, 4-block) groups the buffer
+// MFMA-order buffer; when the matrix does not fill whole (128-row, 2-block) groups the buffer
 // is cleared first so the padding reads as 2^-127 and never as NaN.  (A fill kernel, not a
 // memset node, so the call stays safe under stream capture.)
 static inline void clear_mfma_padding(uint8_t* scales, int64_t rows, int64_t nblk, int order,
                                       hipStream_t st) {
-  if (order != MX_SCALES_MFMA || ((rows & 63) == 0 && (nblk & 3) == 0)) return;
-  const int64_t n = ((rows + 63) / 64) * ((nblk + 3) / 4) * 64;
+  if (order != MX_SCALES_MFMA || ((rows & 127) == 0 && (nblk & 1) == 0)) return;
+  const int64_t n = mfma_scale_bytes(rows, nblk) / 4;
   hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
                      (uint32_t*)scales, n, 0u);
 }
@@ -376,7 +376,7 @@ extern "C" int mx_cast_dim0(const void* x, int64_t rows, int64_t cols, int64_t l
   const int64_t cpr = cols / 8;
   if (cpr > 0x7FFFFFFF) return MX_ERR_UNSUPPORTED;
   const int64_t total = rows * cpr;
-  const int64_t nblk = cols / 32, ks_n = (nblk + 3) / 4;
+  const int64_t nblk = cols / 32, ks_n = (nblk + 1) / 2;
   const int64_t per_block = kDim0Threads * kDim0Unroll;
   const int64_t nblocks = (total + per_block - 1) / per_block;
   if (nblocks > 0x7FFFFFFF) return MX_ERR_UNSUPPORTED;
@@ -390,7 +390,7 @@ extern "C" int mx_cast_dim0(const void* x, int64_t rows, int64_t cols, int64_t l
 }
 
 static inline int64_t scale_bytes(int64_t rows, int64_t nblk, int order) {
-  return order == MX_SCALES_MFMA ? ((rows + 63) / 64) * ((nblk + 3) / 4) * 256 : rows * nblk;
+  return order == MX_SCALES_MFMA ? mfma_scale_bytes(rows, nblk) : rows * nblk;
 }
 
 extern "C" int mx_cast_dim1_batched(const void* x, int64_t batch, int64_t rows, int64_t cols,
@@ -403,7 +403,7 @@ extern "C" int mx_cast_dim1_batched(const void* x, int64_t batch, int64_t rows, 
   if (rows % 32 || cols % 2 || ldx % 2 || ((uintptr_t)x & 3) || ((uintptr_t)codes_t & 15) ||
       ((uintptr_t)scales_t & 3))
     return MX_ERR_ALIGNMENT;
-  const int64_t nblk_t = rows / 32, ks_n_t = (nblk_t + 3) / 4;
+  const int64_t nblk_t = rows / 32, ks_n_t = (nblk_t + 1) / 2;
   const int64_t st_b = scale_bytes(cols, nblk_t, scale_order);
   if (batch > 1 && ((rows * cols) % 16 || st_b % 4)) return MX_ERR_ALIGNMENT;
   const int64_t gx = (cols + kT - 1) / kT, gy = (rows + kT - 1) / kT;
@@ -433,8 +433,8 @@ extern "C" int mx_cast_dim0_dim1_batched(const void* x, int64_t batch, int64_t r
   if (rows % 32 || cols % 32 || ldx % 2 || ((uintptr_t)x & 3) || ((uintptr_t)codes & 1) ||
       ((uintptr_t)codes_t & 15) || ((uintptr_t)scales_t & 3))
     return MX_ERR_ALIGNMENT;
-  const int64_t nblk = cols / 32, ks_n = (nblk + 3) / 4;
-  const int64_t nblk_t = rows / 32, ks_n_t = (nblk_t + 3) / 4;
+  const int64_t nblk = cols / 32, ks_n = (nblk + 1) / 2;
+  const int64_t nblk_t = rows / 32, ks_n_t = (nblk_t + 1) / 2;
   const int64_t s_b = scale_bytes(rows, nblk, scale_order);
   const int64_t st_b = scale_bytes(cols, nblk_t, scale_order);
   const int64_t gx = (cols + kT - 1) / kT, gy = (rows + kT - 1) / kT;
@@ -442,7 +442,7 @@ extern "C" int mx_cast_dim0_dim1_batched(const void* x, int64_t batch, int64_t r
   dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch), block(256);
   hipStream_t st = (hipStream_t)stream;
   if (scale_order == MX_SCALES_MFMA && ((uintptr_t)scales & 3)) return MX_ERR_ALIGNMENT;
-  if (scale_order == MX_SCALES_MFMA && ((rows & 63) || (nblk & 3))) {
+  if (scale_order == MX_SCALES_MFMA && ((rows & 127) || (nblk & 1))) {
     // padding of every batch entry's row-wise scale block must read as zero
     const int64_t n = batch * s_b / 4;
     hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
@@ -464,7 +464,7 @@ extern "C" int mx_cast_dim0_dim1(const void* x, int64_t rows, int64_t cols, int6
 
 extern "C" int64_t mx_scales_mfma_bytes(int64_t rows, int64_t nblk) {
   if (rows < 0 || nblk < 0) return -1;
-  return ((rows + 63) / 64) * ((nblk + 3) / 4) * 256;
+  return mfma_scale_bytes(rows, nblk);
 }
 
 extern "C" int mx_scale_layout(const uint8_t* scales, int64_t rows, int64_t nblk, uint8_t* out,
@@ -473,7 +473,7 @@ extern "C" int mx_scale_layout(const uint8_t* scales, int64_t rows, int64_t nblk
   if (rows == 0 || nblk == 0) return MX_OK;
   if (!scales || !out) return MX_ERR_INVALID_ARG;
   if ((uintptr_t)out & 3) return MX_ERR_ALIGNMENT;
-  const int64_t ks_n = (nblk + 3) / 4;
+  const int64_t ks_n = (nblk + 1) / 2;
   const int64_t dwords = mx_scales_mfma_bytes(rows, nblk) / 4;
   hipLaunchKernelGGL(scale_layout_kernel, dim3((unsigned)((dwords + 255) / 256)), dim3(256), 0,
                      (hipStream_t)stream, scales, rows, nblk, ks_n, dwords, (uint32_t*)out);
@@ -485,7 +485,7 @@ extern "C" int mx_scale_unlayout(const uint8_t* laid, int64_t rows, int64_t nblk
   if (rows < 0 || nblk < 0) return MX_ERR_INVALID_ARG;
   if (rows == 0 || nblk == 0) return MX_OK;
   if (!laid || !out) return MX_ERR_INVALID_ARG;
-  const int64_t ks_n = (nblk + 3) / 4;
+  const int64_t ks_n = (nblk + 1) / 2;
   const int64_t n = rows * nblk;
   hipLaunchKernelGGL(scale_unlayout_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
                      (hipStream_t)stream, laid, rows, nblk, ks_n, out);

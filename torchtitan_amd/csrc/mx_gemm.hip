@@ -19,11 +19,11 @@ __global__ __launch_bounds__(256, 1) void gemm_nt_kernel(DenseArgs p) {
   const int64_t tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
   int64_t tm, tn;
   if (!map_tile(tiles_m, tiles_n, tm, tn)) return;
-  const int64_t ks_n = (p.K / 32 + 3) / 4;
+  const int64_t ks_n = (p.K / 32 + 1) / 2;
   Operand A{p.a_codes + tm * BM * p.K, p.K, p.M - tm * BM,
-            p.a_scales + tm * (BM / 64) * ks_n * 256, ks_n};
+            p.a_scales + tm * (BM / 128) * ks_n * 256, ks_n};
   Operand B{p.b_codes + tn * BN * p.K, p.K, p.N - tn * BN,
-            p.b_scales + tn * (BN / 64) * ks_n * 256, ks_n};
+            p.b_scales + tn * (BN / 128) * ks_n * 256, ks_n};
   Tile::run(smem, A, B, 0, p.K, p.d + tm * BM * p.ldd + tn * BN, p.ldd);
 }
 
@@ -50,6 +50,20 @@ static int launch_dense(const DenseArgs& p, hipStream_t st) {
 
 using namespace mx;
 
+namespace mx {
+int launch_gemm_nt32(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                     const uint8_t* b_scales, void* d, int64_t M, int64_t N, int64_t K,
+                     int64_t ldd, hipStream_t st);
+}
+// 0: pick by shape; 1: the 16x16x128 tile kernel for every shape (kept for comparison runs)
+static int force_kernel = 0;
+extern "C" void mx_debug_force_kernel(int which) { force_kernel = which; }
+namespace mx { void set_debug_grid(int g); }
+extern "C" void mx_debug_set_grid(int g) { mx::set_debug_grid(g); }
+namespace mx { void set_debug_prof(uint64_t* buf); }
+// device buffer of 256*4*4 uint64 receiving per-wave cycle counts; nullptr switches timing off
+extern "C" void mx_debug_set_prof(void* buf) { mx::set_debug_prof((uint64_t*)buf); }
+
 extern "C" int mx_gemm_nt(const uint8_t* a_codes, const uint8_t* a_scales,
                           const uint8_t* b_codes, const uint8_t* b_scales, void* d, int64_t M,
                           int64_t N, int64_t K, int64_t ldd, void* stream) {
@@ -64,5 +78,7 @@ extern "C" int mx_gemm_nt(const uint8_t* a_codes, const uint8_t* a_scales,
   DenseArgs p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, M, N, K, ldd};
   hipStream_t st = (hipStream_t)stream;
   if (M <= 128 || N <= 128) return launch_dense<128, 128>(p, st);
-  return launch_dense<256, 256>(p, st);
+  if (force_kernel == 1 || K % 128 || (uint64_t)K * 256 > 0x7FFFFFFFull || N % 8 || ldd % 8 ||
+      ((uintptr_t)d & 15) || (uint64_t)ldd * 512 > 0x7FFFFFFFull) return launch_dense<256, 256>(p, st);
+  return launch_gemm_nt32(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd, st);
 }

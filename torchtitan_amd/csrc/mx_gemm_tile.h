@@ -8,9 +8,9 @@
 // Data movement per 128-deep K step:
 //   * codes: buffer_load_dwordx4 ... lds (global -> LDS without touching VGPRs), two LDS
 //     stages, one barrier per step.  A load instruction moves 8 rows x 128 B; inside LDS the
-//     16-byte chunk c of row r sits at chunk position c ^ (r & 7) ^ ((r >> 3) & 1) so the 16
-//     lanes that read one K-block column of a 16-row sub-tile hit 16 different bank groups.
-//   * scales: straight from global into VGPRs, either one dword per lane per 64 rows from a
+//     16-byte chunk c of row r sits at chunk position c ^ ((r & 2) | ((r & 8) >> 1)) so every
+//     16-lane pass of a fragment read hits 16 different bank groups.
+//   * scales: straight from global into VGPRs, either two dwords per lane per 128 rows from a
 //     buffer in MFMA order, or one byte per lane per 16 rows from a row-major matrix.
 //   * out-of-range rows and K tails read as zero through the buffer descriptor's bounds.
 #pragma once
@@ -41,9 +41,9 @@ struct Operand {
   const uint8_t* codes;    // first row of this tile, column 0
   int64_t ld;              // row stride in bytes (= elements)
   int64_t rows_valid;      // rows of the tile that exist (may exceed the tile height)
-  const uint8_t* scales;   // MFMA order: group of the tile's first 64 rows, K-step 0
+  const uint8_t* scales;   // MFMA order: group of the tile's first 128 rows, K-step 0
                            // row-major:  scale of (tile's first row, block 0)
-  int64_t scale_stride;    // MFMA order: ks_n (K-steps per 64-row group); row-major: nblk
+  int64_t scale_stride;    // MFMA order: 64-deep K-steps per 128-row group; row-major: nblk
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, int64_t bytes) {
@@ -51,11 +51,12 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, int64
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, n, 0x00020000);
 }
 
-__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40);
-  u += 0x7FFFu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+
+// two floats -> two bf16 (round to nearest even) in one dword: v_cvt_pk_bf16_f32
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{lo, hi}, v2bf));
 }
 
 template <int BM, int BN, bool A_ROWMAJOR, bool B_ROWMAJOR>
@@ -64,10 +65,10 @@ struct GemmTile {
   static constexpr int TM = WM / 16, TN = WN / 16;
   static constexpr int A_BYTES = BM * kBK, B_BYTES = BN * kBK, STAGE = A_BYTES + B_BYTES;
   static constexpr int A_UNITS = BM / 32, B_UNITS = BN / 32;  // 1 KB load units per wave
-  static constexpr int SA = A_ROWMAJOR ? TM : TM / 4;          // scale registers per step
-  static constexpr int SB = B_ROWMAJOR ? TN : TN / 4;
+  static constexpr int SA = A_ROWMAJOR ? TM : 2;  // scale registers per step (MFMA order:
+  static constexpr int SB = B_ROWMAJOR ? TN : 2;  // one dword for even, one for odd sub-tiles)
   static constexpr int kLdsBytes = 2 * STAGE;
-  static_assert(WM % 64 == 0 && WN % 64 == 0, "wave tile must be a multiple of 64");
+  static_assert((WM == 64 || WM == 128) && (WN == 64 || WN == 128), "wave tile is 64 or 128");
 
   // k_begin/k_end: contraction range in elements (multiples of 32); for MFMA-order scales
   // k_begin must be 0.  d points at the tile's first output element.
@@ -82,19 +83,23 @@ struct GemmTile {
     const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(A.codes, A.rows_valid * A.ld);
     const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(B.codes, B.rows_valid * B.ld);
 
-    // global -> LDS: lane l of a load unit fetches row l/8, logical chunk (l%8)^(l/8)^(unit&1)
+    // global -> LDS: lane l of a load unit (8 rows) fetches row l/8 and the logical chunk that
+    // belongs at physical chunk l%8 of that row: c = (l%8) ^ swz(row), swz(r) = (r&2) | ((r&8)>>1)
     const uint32_t lrow = lane >> 3;
-    const uint32_t chunk_even = (lane & 7) ^ lrow;  // unit parity 0; parity 1 flips bit 0
+    const uint32_t chunk_even = (lane & 7) ^ (lrow & 2);  // even units; odd units flip bit 2
     const uint32_t va_even = lrow * (uint32_t)A.ld + chunk_even * 16;
-    const uint32_t va_odd = lrow * (uint32_t)A.ld + (chunk_even ^ 1) * 16;
+    const uint32_t va_odd = lrow * (uint32_t)A.ld + (chunk_even ^ 4) * 16;
     const uint32_t vb_even = lrow * (uint32_t)B.ld + chunk_even * 16;
-    const uint32_t vb_odd = lrow * (uint32_t)B.ld + (chunk_even ^ 1) * 16;
+    const uint32_t vb_odd = lrow * (uint32_t)B.ld + (chunk_even ^ 4) * 16;
 
     // LDS -> VGPR.  Operand layout of the 16x16x128 f8 MFMA (measured on gfx950): lane
     // (li, lj) holds row li, K bytes [16*lj, 16*lj+16) in its first four registers and
     // [64+16*lj, 64+16*lj+16) in the last four, i.e. 16-byte chunks lj and lj+4; the scale
     // of K-block b (bytes [32b, 32b+32)) is taken from lane group b.
-    const uint32_t sw = (li & 7) ^ (li >> 3);
+    // The swizzle makes ds_read_b128 conflict-free: the LDS serves a b128 read in four passes
+    // of 16 lanes, and (measured) the lanes of a pass are {0-3, 12-15, 20-23, 24-27} and
+    // {4-11, 16-19, 28-31} of each half-wave, not 16 consecutive lanes.
+    const uint32_t sw = (li & 2) | ((li & 8) >> 1);
     const uint32_t fa0 = (wm * WM + li) * kBK + ((lj ^ sw) << 4);
     const uint32_t fa1 = (wm * WM + li) * kBK + (((lj + 4) ^ sw) << 4);
     const uint32_t fb0 = A_BYTES + (wn * WN + li) * kBK + ((lj ^ sw) << 4);
@@ -118,7 +123,7 @@ struct GemmTile {
         const int unit = wave * A_UNITS + q;
         uint32_t v = (q & 1) ? va_odd : va_even;
         if (tail) {
-          const uint32_t c = (q & 1) ? (chunk_even ^ 1) : chunk_even;
+          const uint32_t c = (q & 1) ? (chunk_even ^ 4) : chunk_even;
           if (k0 + c * 16 >= k_end) v = 0x80000000u;
         }
         __builtin_amdgcn_raw_ptr_buffer_load_lds(
@@ -130,7 +135,7 @@ struct GemmTile {
         const int unit = wave * B_UNITS + q;
         uint32_t v = (q & 1) ? vb_odd : vb_even;
         if (tail) {
-          const uint32_t c = (q & 1) ? (chunk_even ^ 1) : chunk_even;
+          const uint32_t c = (q & 1) ? (chunk_even ^ 4) : chunk_even;
           if (k0 + c * 16 >= k_end) v = 0x80000000u;
         }
         __builtin_amdgcn_raw_ptr_buffer_load_lds(
@@ -144,17 +149,24 @@ struct GemmTile {
     // past the end of the operand read as zero through the descriptor's bounds
     const __amdgpu_buffer_rsrc_t rsrc_sa = make_rsrc(
         A.scales, A_ROWMAJOR ? A.rows_valid * A.scale_stride
-                             : ((A.rows_valid + 63) >> 6) * A.scale_stride * 256);
+                             : ((A.rows_valid + 127) >> 7) * A.scale_stride * 256);
     const __amdgpu_buffer_rsrc_t rsrc_sb = make_rsrc(
         B.scales, B_ROWMAJOR ? B.rows_valid * B.scale_stride
-                             : ((B.rows_valid + 63) >> 6) * B.scale_stride * 256);
-    const uint32_t vsa = A_ROWMAJOR ? (uint32_t)li * (uint32_t)A.scale_stride + lj : lane * 4;
-    const uint32_t vsb = B_ROWMAJOR ? (uint32_t)li * (uint32_t)B.scale_stride + lj : lane * 4;
+                             : ((B.rows_valid + 127) >> 7) * B.scale_stride * 256);
+    // MFMA order (groups of 128 rows x 2 blocks, lane = 32 * (block & 1) + (row & 31), byte =
+    // (row & 127) / 32): lane (li, lj) of 16-row sub-tile m needs row m*16 + li, block lj of
+    // the 128-deep step, i.e. group step 2*ks + (lj >> 1), lane 32*(lj & 1) + 16*(m & 1) + li,
+    // byte (m >> 1) -- one dword for the even sub-tiles and one for the odd ones.
+    const uint32_t v_mfma = (uint32_t)(((lj & 1) * 32 + li) * 4 + (lj >> 1) * 256);
+    const uint32_t vsa = A_ROWMAJOR ? (uint32_t)li * (uint32_t)A.scale_stride + lj : v_mfma;
+    const uint32_t vsb = B_ROWMAJOR ? (uint32_t)li * (uint32_t)B.scale_stride + lj : v_mfma;
     const uint32_t sa_stride = (uint32_t)A.scale_stride, sb_stride = (uint32_t)B.scale_stride;
+    // a 64-row wave tile sits in one half of its 128-row group: bring its bytes down
+    const uint32_t sh_a = (WM == 64) ? 16u * wm : 0u, sh_b = (WN == 64) ? 16u * wn : 0u;
 
     auto load_scales_a = [&](uint32_t (&s)[SA], int64_t k0) {
+      const bool valid = k0 + 32 * lj < k_end;
       if constexpr (A_ROWMAJOR) {
-        const bool valid = k0 + 32 * lj < k_end;
 #pragma unroll
         for (int m = 0; m < TM; ++m) {
           const uint32_t so = (uint32_t)(wm * WM + m * 16) * sa_stride + (uint32_t)(k0 >> 5);
@@ -162,16 +174,15 @@ struct GemmTile {
           s[m] = b;
         }
       } else {
+        const uint32_t so = ((uint32_t)(wm * WM / 128) * sa_stride + (uint32_t)(k0 >> 6)) * 256;
 #pragma unroll
-        for (int g = 0; g < SA; ++g) {
-          const uint32_t so = ((uint32_t)(wm * (WM / 64) + g) * sa_stride + (uint32_t)(k0 >> 7)) * 256;
-          s[g] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_sa, vsa, so, 0);
-        }
+        for (int g = 0; g < 2; ++g)
+          s[g] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_sa, valid ? vsa + g * 64 : 0x80000000u, so, 0) >> sh_a;
       }
     };
     auto load_scales_b = [&](uint32_t (&s)[SB], int64_t k0) {
+      const bool valid = k0 + 32 * lj < k_end;
       if constexpr (B_ROWMAJOR) {
-        const bool valid = k0 + 32 * lj < k_end;
 #pragma unroll
         for (int n = 0; n < TN; ++n) {
           const uint32_t so = (uint32_t)(wn * WN + n * 16) * sb_stride + (uint32_t)(k0 >> 5);
@@ -179,11 +190,10 @@ struct GemmTile {
           s[n] = b;
         }
       } else {
+        const uint32_t so = ((uint32_t)(wn * WN / 128) * sb_stride + (uint32_t)(k0 >> 6)) * 256;
 #pragma unroll
-        for (int g = 0; g < SB; ++g) {
-          const uint32_t so = ((uint32_t)(wn * (WN / 64) + g) * sb_stride + (uint32_t)(k0 >> 7)) * 256;
-          s[g] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_sb, vsb, so, 0);
-        }
+        for (int g = 0; g < 2; ++g)
+          s[g] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_sb, valid ? vsb + g * 64 : 0x80000000u, so, 0) >> sh_b;
       }
     };
 
@@ -219,12 +229,12 @@ struct GemmTile {
         const v4i lo = *reinterpret_cast<const v4i*>(sbase + fb0 + n * 2048);
         const v4i hi = *reinterpret_cast<const v4i*>(sbase + fb1 + n * 2048);
         const v8i bf = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-        constexpr int ob = B_ROWMAJOR ? 0 : (n & 3);
-        const uint32_t sbv = sb_cur[B_ROWMAJOR ? n : (n >> 2)];
+        constexpr int ob = B_ROWMAJOR ? 0 : (n >> 1);
+        const uint32_t sbv = sb_cur[B_ROWMAJOR ? n : (n & 1)];
         static_for<0, TM>([&](auto m_) {
           constexpr int m = decltype(m_)::value;
-          constexpr int oa = A_ROWMAJOR ? 0 : (m & 3);
-          const uint32_t sav = sa_cur[A_ROWMAJOR ? m : (m >> 2)];
+          constexpr int oa = A_ROWMAJOR ? 0 : (m >> 1);
+          const uint32_t sav = sa_cur[A_ROWMAJOR ? m : (m & 1)];
           // first MFMA operand = B rows (N), second = A rows (M): the lane then holds four
           // consecutive N of one M row, which stores as 8 contiguous bytes
           acc[m][n] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
@@ -257,12 +267,12 @@ struct GemmTile {
         if (c >= cols_valid) continue;
         const v4f a = acc[m][n];
         uint16_t* dst = d + r * ldd + c;
-        const uint16_t h0 = f32_to_bf16_rne(a.x), h1 = f32_to_bf16_rne(a.y),
-                       h2 = f32_to_bf16_rne(a.z), h3 = f32_to_bf16_rne(a.w);
+        const u32x2 w = {pack_bf16(a.x, a.y), pack_bf16(a.z, a.w)};
         if (vec_ok && c + 3 < cols_valid) {
-          u32x2 w = {(uint32_t)h0 | ((uint32_t)h1 << 16), (uint32_t)h2 | ((uint32_t)h3 << 16)};
           *reinterpret_cast<u32x2*>(dst) = w;
         } else {
+          const uint16_t h0 = (uint16_t)w.x, h1 = (uint16_t)(w.x >> 16), h2 = (uint16_t)w.y,
+                         h3 = (uint16_t)(w.y >> 16);
           dst[0] = h0;
           if (c + 1 < cols_valid) dst[1] = h1;
           if (c + 2 < cols_valid) dst[2] = h2;

@@ -49,11 +49,11 @@ __global__ __launch_bounds__(256, 1) void grouped_2d3d_kernel(G2d3dArgs p) {
     return;
   }
   const int64_t row0 = lo + (mt - first) * BM;
-  const int64_t nblk = p.K / 32, ks_n = (nblk + 3) / 4;
-  const int64_t b_scale_block = ((p.N + 63) / 64) * ks_n * 256;
+  const int64_t nblk = p.K / 32, ks_n = (nblk + 1) / 2;
+  const int64_t b_scale_block = ((p.N + 127) / 128) * ks_n * 256;
   Operand A{p.a_codes + row0 * p.K, p.K, hi - row0, p.a_scales + row0 * nblk, nblk};
   Operand B{p.b_codes + (g * p.N + col0) * p.K, p.K, p.N - col0,
-            p.b_scales + g * b_scale_block + tn * (BN / 64) * ks_n * 256, ks_n};
+            p.b_scales + g * b_scale_block + tn * (BN / 128) * ks_n * 256, ks_n};
   Tile::run(smem, A, B, 0, p.K, p.d + row0 * p.ldd + col0, p.ldd);
 }
 

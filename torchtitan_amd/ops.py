@@ -102,7 +102,7 @@ def _check_hp(x: torch.Tensor) -> torch.Tensor:
 
 
 def mfma_scale_bytes(rows: int, nblk: int) -> int:
-    return ((rows + 63) // 64) * ((nblk + 3) // 4) * 256
+    return ((rows + 127) // 128) * ((nblk + 1) // 2) * 256
 
 
 def _alloc_scales(rows: int, nblk: int, order: int, device) -> torch.Tensor:
@@ -188,11 +188,11 @@ def to_mx_dim0_batched(w: torch.Tensor, mode="floor", order: int = MX_SCALES_MFM
     """Row-wise cast of every matrix of w [G, R, C]: codes [G, R, C], one scale block each.
 
     A 3-D weight is G stacked matrices, so this is one row-wise cast of the [G*R, C] view;
-    in MFMA order that equals G per-matrix blocks only when R is a multiple of 64.
+    in MFMA order that equals G per-matrix blocks only when R is a multiple of 128.
     """
     G, R, C = w.shape
-    if order == MX_SCALES_MFMA and R % 64:
-        raise ValueError("MFMA-order scales of stacked matrices need rows % 64 == 0")
+    if order == MX_SCALES_MFMA and R % 128:
+        raise ValueError("MFMA-order scales of stacked matrices need rows % 128 == 0")
     d = to_mx_dim0(w.reshape(G * R, C), mode, order)
     scales = d.scales if order == MX_SCALES_MFMA else d.scales.view(G, R, C // BLOCK)
     return MXData(d.codes.view(G, R, C), scales, order)
