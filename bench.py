@@ -210,7 +210,7 @@ def main():
             "casts_per_step": 8,
         },
         "roofline": {
-            "kernel": "gemm_nt_kernel<256,256> (v_mfma_scale_f32_16x16x128_f8f6f4)",
+            "kernel": "gemm_nt32_kernel (persistent 256x256 tiles, v_mfma_scale_f32_32x32x64_f8f6f4)",
             "bound": "mfma",
             "achieved": round(achieved, 1),
             "peak": PEAK_MXFP8_TFLOPS,

@@ -3,14 +3,16 @@
 //   D[M,N] (bf16) = deq(A)[M,K] * deq(B)[N,K]^T, fp32 accumulate.
 //
 // One workgroup (4 waves, 2x2, 128x128 each = 256 accumulator registers per lane) per CU walks
-// a list of output tiles; the K loop of all its tiles is one flat stream of 64-deep steps, so
-// the loads of the next tile's first steps are already in flight while a tile is written out.
+// a list of output tiles; the K loop of all its tiles is one flat stream, so the loads of the
+// next tile's first steps are already in flight while a tile is written out.
 //
-// Per step and per CU: 32 KB of codes + 1 KB of scales go global -> LDS with
-// buffer_load ... lds into a ring of NSTAGE stages (issued NSTAGE steps ahead), 64 KB of
-// fragments go LDS -> VGPR (double-buffered in registers, read one step ahead, conflict-free
-// under the b128 pass grouping), and 16 MFMAs per wave (1024 MFMA cycles) consume them.
-// One barrier per step.
+// Global -> LDS moves whole 128-byte rows (buffer_load_dwordx4 ... lds, 8 rows per instruction:
+// full cache lines, which the texture path delivers about twice as fast as 64-byte pieces), so
+// the ring holds two 128-deep "blocks" of 64 KB codes + 2 KB scales.  Compute runs in 64-deep
+// steps (two per block): 16 MFMAs per wave per step (1024 MFMA cycles), fragments LDS -> VGPR
+// double-buffered in registers and read one step ahead, conflict-free under the b128 pass
+// grouping.  The block that was just consumed is refilled two steps before it is needed
+// again; one barrier per block.
 //
 // Operand layout of the 32x32x64 f8 MFMA (measured): lane (i = l & 31, j = l >> 5) holds row i,
 // K bytes [16j, 16j+16) in registers 0-3 and [32+16j, 32+16j+16) in registers 4-7; the scale
@@ -22,11 +24,13 @@ namespace mx {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-constexpr int kT32 = 256;                       // tile edge (M and N)
-constexpr int kK32 = 64;                        // K per step
-constexpr int kCodes32 = 2 * kT32 * kK32;       // 32 KB: A rows then B rows, 64 B per row
-constexpr int kStage32 = kCodes32 + 1024;       // + 4 x 256 B of scales (A group 0,1, B group 0,1)
-constexpr int kVmPerStep = 9;                   // VM instructions per wave per step (8 + 1)
+constexpr int kT32 = 256;                        // tile edge (M and N)
+constexpr int kK32 = 64;                         // K per compute step
+constexpr int kKB = 128;                         // K per ring block (= one cache line per row)
+constexpr int kOperand32 = kT32 * kKB;           // 32 KB: 256 rows x 128 B
+constexpr int kCodes32 = 2 * kOperand32;         // A rows then B rows
+constexpr int kBlock32 = kCodes32 + 2048;        // + scales: 4 groups (A0, A1, B0, B1) x 2 steps x 256 B
+constexpr int kRing32 = 2 * kBlock32;            // 132 KB
 
 struct Dense32Args {
   const uint8_t* a_codes;
@@ -52,13 +56,29 @@ __device__ __forceinline__ void tile_coords(uint32_t t, uint32_t tiles_m, uint32
   tm = first_m + (in - tn * gsz);
 }
 
+// LDS accesses the compiler must not see (see read_piece in the kernel)
+template <int OFF>
+__device__ __forceinline__ void lds_write_b128_hidden(uint32_t addr, v4i v) {
+  asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(addr), "v"(v), "n"(OFF) : "memory");
+}
+template <int OFF>
+__device__ __forceinline__ v4i lds_read_b128_hidden(uint32_t addr) {
+  v4i v;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+  return v;
+}
+__device__ __forceinline__ v4i pin(v4i v) {
+  asm volatile("" : "+v"(v));
+  return v;
+}
+
 struct Frags32 {
   v8i a[4];
   v8i b[4];
   uint32_t sa, sb;
 };
 
-template <int NSTAGE, bool PROF>
+template <bool PROF>
 __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   const int tid = threadIdx.x;
@@ -79,29 +99,30 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
   const uint32_t n_my = t_lo < t_hi ? (t_hi - t_lo + wgs_per_xcd - 1) / wgs_per_xcd : 0;
   if (n_my == 0) return;
   const uint32_t K = (uint32_t)p.K;          // a multiple of 128 for this kernel
-  const uint32_t nsteps = K / kK32;          // even, >= 2
-  const uint32_t ks_n = nsteps;              // 64-deep steps per 128-row scale group
+  const uint32_t nblocks = K / kKB;          // 128-deep ring blocks per tile, >= 1
+  const uint32_t ks_n = K / kK32;            // 64-deep steps per 128-row scale group
 
   // ---- per-lane constants
-  // global -> LDS: a load unit is 16 rows x 64 B; lane l fetches row l/4 and the logical chunk
-  // that belongs at physical chunk l%4: c = (l%4) ^ ((row >> 3) & 3)
-  const uint32_t c_even = (lane & 3) ^ (lane >> 5);  // units 0,2 of a wave; units 1,3 flip bit 1
-  const uint32_t v_even = (uint32_t)(lane >> 2) * K + c_even * 16;
-  const uint32_t v_odd = (uint32_t)(lane >> 2) * K + (c_even ^ 2) * 16;
-  // LDS -> VGPR: lane (li, lj) reads chunks lj and 2+lj of row li of each 32-row sub-tile
-  const uint32_t sw = (li >> 3) & 3;
-  const uint32_t fa0 = (wm * 128 + li) * kK32 + ((lj ^ sw) << 4);
-  const uint32_t fa1 = (wm * 128 + li) * kK32 + (((2 + lj) ^ sw) << 4);
-  const uint32_t fb0 = kT32 * kK32 + (wn * 128 + li) * kK32 + ((lj ^ sw) << 4);
-  const uint32_t fb1 = kT32 * kK32 + (wn * 128 + li) * kK32 + (((2 + lj) ^ sw) << 4);
-  const uint32_t fsa = kCodes32 + wm * 256 + lane * 4;
-  const uint32_t fsb = kCodes32 + 512 + wn * 256 + lane * 4;
-
+  // global -> LDS: a load unit is 8 rows x 128 B; lane l fetches row l/8 and the logical 16-byte
+  // chunk that belongs at physical chunk l%8 of that row: c = (l%8) ^ ((row >> 1) & 7)
+  const uint32_t c_even = (lane & 7) ^ (lane >> 4);  // even units; odd units flip bit 2
+  const uint32_t v_even = (uint32_t)(lane >> 3) * K + c_even * 16;
+  // (odd units: v_even ^ 64 -- K is a multiple of 128, so bit 6 belongs to the chunk alone)
+  // LDS -> VGPR: for K half h of a block, lane (li, lj) reads chunks 4h+lj and 4h+2+lj of row li
+  // of each 32-row sub-tile; physical chunk = logical ^ ((row >> 1) & 7), so the second chunk is
+  // address ^ 32 and h flips address bit 6.  Only the A address is kept per lane; B's differs by
+  // a wave-uniform amount, as do the scale addresses (group g = A0, A1, B0, B1, K half h at
+  // kCodes32 + (g*2 + h) * 256).
+  const uint32_t sw = (li >> 1) & 7;
+  const uint32_t fa0 = (wm * 128 + li) * kKB + ((lj ^ sw) << 4);
+  const uint32_t fb_delta = kOperand32 + (wn - wm) * 128 * kKB;
+  const uint32_t lane4 = lane * 4;
+  const uint32_t fsa_s = kCodes32 + wm * 512, fsb_s = kCodes32 + 1024 + wn * 512;
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void_t*)smem;  // LDS byte address of the ring
 
-  // ---- loader stream (runs NSTAGE steps ahead of the compute stream)
-  uint32_t ld_tile = 0, ld_ks = 0;
-  int ld_stage = 0;
+  // ---- loader stream: fills ring block `ld_slot` with K block `ld_kb` of tile `ld_tile`
+  uint32_t ld_tile = 0, ld_kb = 0;
+  int ld_slot = 0;
   __amdgpu_buffer_rsrc_t ra, rb, rs;  // codes of A, codes of B, scales this wave copies
   auto loader_open_tile = [&]() {
     if (ld_tile < n_my) {
@@ -122,29 +143,43 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
       rs = ra;
     }
   };
-  auto issue_step = [&]() {
-    const uint32_t k0 = ld_ks * kK32;
-    const uint32_t sbase = lds_base + ld_stage * kStage32;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int unit = wave * 4 + q;
-      const uint32_t v = (q & 1) ? v_odd : v_even;
-      const uint32_t so = (uint32_t)(unit * 16) * K + k0;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void_t*)(uintptr_t)(sbase + unit * 1024), 16, v, so, 0, 0);
+  // The 18 copies of a block are issued one at a time, between MFMAs (see block_steps):
+  // piece 0..15 = unit pairs (A unit, B unit alternating), 16,17 = scales, then advance.
+  auto issue_piece = [&](auto i_) {
+    constexpr int i = decltype(i_)::value;
+    const uint32_t sbase = lds_base + ld_slot * kBlock32;
+    if constexpr (i < 16) {
+      constexpr int q = i >> 1;
+      const int unit = wave * 8 + q;
+      const uint32_t v = (q & 1) ? (v_even ^ 64) : v_even;
+      const uint32_t so = (uint32_t)(unit * 8) * K + ld_kb * kKB;
+      if constexpr ((i & 1) == 0)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void_t*)(uintptr_t)(sbase + unit * 1024), 16, v, so, 0, 0);
+      else
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            rb, (lds_void_t*)(uintptr_t)(sbase + kOperand32 + unit * 1024), 16, v, so, 0, 0);
+    } else {
+      // this wave's scale group: the block's two 64-deep steps are 512 contiguous bytes
+      constexpr int h = i - 16;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          rb, (lds_void_t*)(uintptr_t)(sbase + kT32 * kK32 + unit * 1024), 16, v, so, 0, 0);
+          rs, (lds_void_t*)(uintptr_t)(sbase + kCodes32 + wave * 512 + h * 256), 4,
+          lane4, ld_kb * 512 + h * 256, 0, 0);
     }
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void_t*)(uintptr_t)(sbase + kCodes32 + wave * 256), 4,
-                                             (uint32_t)lane * 4, ld_ks * 256, 0, 0);
-    if (++ld_ks == nsteps) {
-      ld_ks = 0;
+  };
+  auto issue_advance = [&]() {
+    if (++ld_kb == nblocks) {
+      ld_kb = 0;
       ++ld_tile;
       loader_open_tile();
     }
-    if (++ld_stage == NSTAGE) ld_stage = 0;
+    ld_slot ^= 1;
+  };
+  auto issue_block = [&]() {
+    static_for<0, 18>([&](auto i_) { issue_piece(i_); });
+    issue_advance();
   };
 
-  // Fragment reads are issued as inline assembly: the compiler cannot tell which ring stage a
+  // Fragment reads are issued as inline assembly: the compiler cannot tell which ring block a
   // ds_read touches, so for reads it can see it waits until every global->LDS copy in flight
   // has landed (vmcnt(0)) and the prefetch distance collapses.  The reads are therefore
   // invisible to its wait-count tracking; `pin_frags` (after the explicit lgkmcnt(0) at the top
@@ -155,23 +190,32 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(off));
     return v;
   };
-  auto read_frags = [&](Frags32& f, int stage) {
-    const uint32_t sbase = lds_base + stage * kStage32;
-    const uint32_t pa0 = sbase + fa0, pa1 = sbase + fa1, pb0 = sbase + fb0, pb1 = sbase + fb1;
-    static_for<0, 4>([&](auto m_) {
-      constexpr int m = decltype(m_)::value;
-      const v4i lo = lds_b128(pa0, std::integral_constant<int, m * 2048>{});
-      const v4i hi = lds_b128(pa1, std::integral_constant<int, m * 2048>{});
-      f.a[m] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-    });
-    static_for<0, 4>([&](auto n_) {
-      constexpr int n = decltype(n_)::value;
-      const v4i lo = lds_b128(pb0, std::integral_constant<int, n * 2048>{});
-      const v4i hi = lds_b128(pb1, std::integral_constant<int, n * 2048>{});
-      f.b[n] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-    });
-    asm volatile("ds_read_b32 %0, %1" : "=v"(f.sa) : "v"(sbase + fsa));
-    asm volatile("ds_read_b32 %0, %1" : "=v"(f.sb) : "v"(sbase + fsb));
+  // piece 0..7: A sub-tile m = piece/2, low/high 16 bytes; 8..15: same for B; 16,17: scales
+  auto read_piece = [&](Frags32& f, uint32_t sbase, auto half_, auto i_) {
+    constexpr int h = decltype(half_)::value;
+    constexpr int i = decltype(i_)::value;
+    if constexpr (i < 16) {
+      constexpr int t = (i & 7) >> 1;       // sub-tile
+      constexpr bool hi = i & 1;
+      const uint32_t base = (fa0 ^ (h * 64 + (hi ? 32 : 0))) + (i < 8 ? 0u : fb_delta);
+      const v4i v = lds_b128(sbase + base, std::integral_constant<int, t * 4096>{});
+      v8i& dst = i < 8 ? f.a[t] : f.b[t];
+      if constexpr (hi) {
+        dst[4] = v.x; dst[5] = v.y; dst[6] = v.z; dst[7] = v.w;
+      } else {
+        dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
+      }
+    } else if constexpr (i == 16) {
+      const uint32_t psa = sbase + fsa_s + h * 256 + lane4;
+      asm volatile("ds_read_b32 %0, %1" : "=v"(f.sa) : "v"(psa));
+    } else {
+      const uint32_t psb = sbase + fsb_s + h * 256 + lane4;
+      asm volatile("ds_read_b32 %0, %1" : "=v"(f.sb) : "v"(psb));
+    }
+  };
+  auto read_frags = [&](Frags32& f, int slot, auto half_) {
+    const uint32_t sbase = lds_base + slot * kBlock32;
+    static_for<0, 18>([&](auto i_) { read_piece(f, sbase, half_, i_); });
   };
   auto pin_frags = [&](Frags32& f) {
 #pragma unroll
@@ -183,50 +227,60 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
 
   // ---- compute stream
   v16f acc[4][4];
-  int c_stage = 0;
-  uint64_t prof_vm = 0, prof_bar = 0, prof_body = 0, prof_last = 0, prof_epi = 0, prof_issue = 0, prof_read = 0;
+  int c_slot = 0;  // ring block holding the K block being computed
+  uint64_t prof_vm = 0, prof_bar = 0, prof_body = 0, prof_last = 0, prof_epi = 0;
 
-  auto mfma_step = [&](const Frags32& f, auto first_) {
+  auto mfma_one = [&](const Frags32& f, auto first_, auto i_) {
     constexpr bool kFirst = decltype(first_)::value;  // first step of a tile starts from zero
-    static_for<0, 4>([&](auto n_) {
-      constexpr int n = decltype(n_)::value;
-      static_for<0, 4>([&](auto m_) {
-        constexpr int m = decltype(m_)::value;
-        if constexpr (kFirst) {
-          acc[m][n] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-              f.b[n], f.a[m], v16f{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, 0, 0, n,
-              (int)f.sb, m, (int)f.sa);
-        } else {
-          acc[m][n] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-              f.b[n], f.a[m], acc[m][n], 0, 0, n, (int)f.sb, m, (int)f.sa);
-        }
-      });
-    });
+    constexpr int n = decltype(i_)::value >> 2, m = decltype(i_)::value & 3;
+    if constexpr (kFirst) {
+      acc[m][n] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+          f.b[n], f.a[m], v16f{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, 0, 0, n, (int)f.sb,
+          m, (int)f.sa);
+    } else {
+      acc[m][n] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.b[n], f.a[m], acc[m][n], 0, 0, n,
+                                                                  (int)f.sb, m, (int)f.sa);
+    }
   };
 
-  // One step: `cur` holds the fragments of step g (read during step g-1), `nxt` receives g+1.
-  // The first step of a tile follows the previous tile's output stores, which sit in the same
-  // counter as the loads, so it waits for everything outstanding.
-  auto step = [&](Frags32& cur, Frags32& nxt, auto first_) {
-    constexpr bool kFirst = decltype(first_)::value;
-    // stage c_stage is free once every wave holds its fragments of this step in registers;
-    // stage c_stage+1 must have landed for everyone before it is read
-    // (waits written as assembly: the compiler rewrites the immediates of s_waitcnt builtins
-    // from its own, here too pessimistic, model of what is outstanding)
+  // A K block is two steps.  Entering step A, f0 holds the fragments of the block's first half
+  // (read during the previous step); ring block c_slot holds the block, c_slot^1 the next one
+  // (still landing).
+  //   step A: read the second half into f1, MFMAs on f0.
+  //   step B: every wave now holds all fragments of this block in registers, and the next
+  //           block must have landed: wait, barrier, refill c_slot with the block after next,
+  //           read the next block's first half into f0, MFMAs on f1.
+  // A wave issues in order and an MFMA occupies the matrix pipe for 64 cycles, so every other
+  // instruction is placed in the shadow of an MFMA: the sequence below is pinned with
+  // scheduling fences (one MFMA, then one or two copies / fragment reads).
+  // (waits written as assembly: the compiler rewrites the immediates of s_waitcnt builtins
+  // from its own, here too pessimistic, model of what is outstanding)
+  auto block_steps = [&](Frags32& f0, Frags32& f1, auto first_, auto last_) {
+    constexpr bool kLast = decltype(last_)::value;  // last block of a tile: see the tile loop
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    pin_frags(cur);
+    pin_frags(f0);
+    {
+      const uint32_t sbase = lds_base + c_slot * kBlock32;
+      static_for<0, 16>([&](auto i_) {
+        constexpr int i = decltype(i_)::value;
+        mfma_one(f0, first_, i_);
+        // the last two copies of the block being fetched (its scales) trail into this step
+        if constexpr (i < 2) issue_piece(std::integral_constant<int, 16 + i>{});
+        if constexpr (i == 2) issue_advance();
+        read_piece(f1, sbase, std::integral_constant<int, 1>{}, i_);
+        if constexpr (i >= 14) read_piece(f1, sbase, std::integral_constant<int, 1>{}, std::integral_constant<int, i + 2>{});
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    }
+
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    pin_frags(f1);
     uint64_t t0 = 0, t1 = 0;
     if constexpr (PROF) {
       t0 = __builtin_readcyclecounter();
       prof_body += t0 - prof_last;
     }
-    if constexpr (kFirst) {
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    } else {
-      // groups in flight: g+1 .. g+NSTAGE-1; all but the first may stay outstanding
-      static_assert(NSTAGE == 4 && kVmPerStep == 9, "update the immediate below");
-      asm volatile("s_waitcnt vmcnt(18)" ::: "memory");
-    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the next block (and any output stores)
     if constexpr (PROF) {
       t1 = __builtin_readcyclecounter();
       prof_vm += t1 - t0;
@@ -236,27 +290,38 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
       prof_last = __builtin_readcyclecounter();
       prof_bar += prof_last - t1;
     }
-    issue_step();  // step g+NSTAGE into the stage just freed
-    const int next_stage = c_stage + 1 == NSTAGE ? 0 : c_stage + 1;
-    if constexpr (PROF) {
-      const uint64_t t3 = __builtin_readcyclecounter();
-      prof_issue += t3 - prof_last;
-      read_frags(nxt, next_stage);
-      const uint64_t t4 = __builtin_readcyclecounter();
-      prof_read += t4 - t3;
-    } else {
-      read_frags(nxt, next_stage);
+    {
+      // One copy of the block after next per MFMA (the texture path takes 16 cycles per copy
+      // and serves all four waves, so one per 64-cycle slot per wave is its full rate), into
+      // the ring block just drained; the fragment reads of the next block's first half go last.
+      const uint32_t sbase = lds_base + (c_slot ^ 1) * kBlock32;
+      static_for<0, 16>([&](auto i_) {
+        constexpr int i = decltype(i_)::value;
+        mfma_one(f1, std::false_type{}, i_);
+        issue_piece(i_);
+        if constexpr (i >= 10 && !kLast) {
+          read_piece(f0, sbase, std::integral_constant<int, 0>{}, std::integral_constant<int, 3 * (i - 10)>{});
+          read_piece(f0, sbase, std::integral_constant<int, 0>{}, std::integral_constant<int, 3 * (i - 10) + 1>{});
+          read_piece(f0, sbase, std::integral_constant<int, 0>{}, std::integral_constant<int, 3 * (i - 10) + 2>{});
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      c_slot ^= 1;
     }
-    mfma_step(cur, first_);
-    c_stage = next_stage;
   };
 
   // Output: a lane holds, per 32x32 sub-tile, row li and columns 8q + 4lj + 0..3.  The two
-  // lanes of a row (lj = 0, 1) trade halves with v_permlane32_swap so that each stores 8
-  // consecutive bf16 (16 bytes); ordinary (cached) stores let L2 merge the pieces of a line.
-  // Buffer stores: one descriptor per tile bounds the rows, one 32-bit offset per lane and
-  // sub-tile row, immediates for the columns -- no 64-bit address arithmetic, no branches.
-  // Requires N % 8 == 0 and ldd % 8 == 0 (checked on the host).
+  // lanes of a row (lj = 0, 1) trade halves with v_permlane32_swap so that each owns 8
+  // consecutive bf16; a 32-row x 64-column piece is then turned around in this wave's private
+  // LDS patch (the 28 KB the ring leaves free) so that 8 lanes store one full 128-byte line of
+  // a row -- stores that scatter 32-byte pieces over 32 rows back up the write path.
+  // Buffer stores: one descriptor per tile bounds the rows, a 32-bit offset per lane, scalar
+  // offsets per piece.  Requires N % 8 == 0 and ldd % 8 == 0 (checked on the host).
+  // (LDS accesses as assembly, for the reason given at read_piece.)
+  constexpr int kPatchPitch = 144;  // bytes per staged row: 128 + 16, keeps b128 accesses spread
+  const uint32_t patch = lds_base + kRing32 + wave * 7168;
+  const uint32_t patch_w = patch + li * kPatchPitch + lj * 16;                 // + (n&1)*64 + h*32
+  const uint32_t patch_r = patch + (lane >> 3) * kPatchPitch + (lane & 7) * 16;  // + pass*8 rows
   auto epilogue = [&](uint32_t tile) {
     uint32_t tm, tn;
     tile_coords(t_lo + tile * wgs_per_xcd, tiles_m, tiles_n, tm, tn);
@@ -265,46 +330,64 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
     const uint32_t ldd_b = (uint32_t)p.ldd * 2;
     const __amdgpu_buffer_rsrc_t rd =
         make_rsrc(p.d + (int64_t)tm * kT32 * p.ldd + (int64_t)tn * kT32, rows_valid * ldd_b);
-    // byte offset of (row wm*128 + li, column wn*128 + lj*8); out of range if the column is
-    const uint32_t col0 = wn * 128 + lj * 8;
-    const uint32_t v0 = (wm * 128 + li) * ldd_b + col0 * 2;
+    // lane's place in a stored piece: row (lane >> 3) + 8*pass, columns (lane & 7)*8 .. +7
+    const uint32_t colp = wn * 128 + (lane & 7) * 8;
+    const uint32_t vrow = (wm * 128 + (lane >> 3)) * ldd_b + colp * 2;
     static_for<0, 4>([&](auto m_) {
       constexpr int m = decltype(m_)::value;
-      static_for<0, 4>([&](auto n_) {
-        constexpr int n = decltype(n_)::value;
-        const v16f a = acc[m][n];
-        static_for<0, 2>([&](auto h_) {
-          constexpr int h = decltype(h_)::value;
+      static_for<0, 2>([&](auto np_) {
+        constexpr int np = decltype(np_)::value;  // column pair: sub-tiles n = 2np, 2np+1
+        static_for<0, 4>([&](auto k_) {
+          constexpr int n = 2 * np + (decltype(k_)::value >> 1), h = decltype(k_)::value & 1;
+          const v16f a = acc[m][n];
           const uint32_t x0 = pack_bf16(a[8 * h + 0], a[8 * h + 1]), y0 = pack_bf16(a[8 * h + 2], a[8 * h + 3]);
           const uint32_t x1 = pack_bf16(a[8 * h + 4], a[8 * h + 5]), y1 = pack_bf16(a[8 * h + 6], a[8 * h + 7]);
           const u32x2 sx = __builtin_amdgcn_permlane32_swap(x0, x1, false, false);
           const u32x2 sy = __builtin_amdgcn_permlane32_swap(y0, y1, false, false);
-          const u32x4 w = {sx.x, sy.x, sx.y, sy.y};
-          const uint32_t v = (col0 + n * 32 + h * 16 < cols_valid) ? v0 : 0x80000000u;
-          __builtin_amdgcn_raw_buffer_store_b128(w, rd, v + (n * 32 + h * 16) * 2, m * 32 * ldd_b, 0);
+          const v4i w = {(int)sx.x, (int)sy.x, (int)sx.y, (int)sy.y};
+          lds_write_b128_hidden<(n & 1) * 64 + h * 32>(patch_w, w);
         });
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        v4i r[4];
+        static_for<0, 4>([&](auto q_) {
+          constexpr int q = decltype(q_)::value;
+          r[q] = lds_read_b128_hidden<q * 8 * kPatchPitch>(patch_r);
+        });
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        const uint32_t v = (colp + np * 64 < cols_valid) ? vrow + np * 128 : 0x80000000u;
+        static_for<0, 4>([&](auto q_) {
+          constexpr int q = decltype(q_)::value;
+          const v4i rq = pin(r[q]);
+          const u32x4 w = {(uint32_t)rq.x, (uint32_t)rq.y, (uint32_t)rq.z, (uint32_t)rq.w};
+          __builtin_amdgcn_raw_buffer_store_b128(w, rd, v, (m * 32 + q * 8) * ldd_b, 0);
+        });
+        // keep the pieces apart: hoisting the accumulator reads of later pieces over this
+        // point only costs registers
+        __builtin_amdgcn_sched_barrier(0);
       });
     });
   };
 
   // ---- prologue: fill the ring, fetch the first fragments
   loader_open_tile();
-#pragma unroll
-  for (int s = 0; s < NSTAGE; ++s) issue_step();
-  asm volatile("s_waitcnt vmcnt(27)" ::: "memory");  // (NSTAGE - 1) groups may stay in flight
+  issue_block();
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __builtin_amdgcn_s_barrier();
+  static_for<0, 16>([&](auto i_) { issue_piece(i_); });  // scales + advance follow in the first step
   Frags32 f0, f1;
-  read_frags(f0, 0);
+  read_frags(f0, 0, std::integral_constant<int, 0>{});
   if constexpr (PROF) prof_last = __builtin_readcyclecounter();
 
-  // ---- tiles; at the top of every tile f0 holds the fragments of its step 0 (nsteps is even)
-  const uint32_t pairs = nsteps / 2 - 1;
+  // ---- tiles; at the top of every tile f0 holds the fragments of its first half block.  The
+  // last block of a tile leaves the next tile's first fragments unread until the tile has been
+  // written out, so that no fragment register is live across the epilogue.
   for (uint32_t tile = 0; tile < n_my; ++tile) {
-    step(f0, f1, std::true_type{});
-    step(f1, f0, std::false_type{});
-    for (uint32_t i = 0; i < pairs; ++i) {
-      step(f0, f1, std::false_type{});
-      step(f1, f0, std::false_type{});
+    if (nblocks == 1) {
+      block_steps(f0, f1, std::true_type{}, std::true_type{});
+    } else {
+      block_steps(f0, f1, std::true_type{}, std::false_type{});
+      for (uint32_t i = 2; i < nblocks; ++i) block_steps(f0, f1, std::false_type{}, std::false_type{});
+      block_steps(f0, f1, std::false_type{}, std::true_type{});
     }
     if constexpr (PROF) {
       const uint64_t e0 = __builtin_readcyclecounter();
@@ -315,6 +398,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
     } else {
       epilogue(tile);
     }
+    read_frags(f0, c_slot, std::integral_constant<int, 0>{});
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the over-issued prefetches before retiring
   if constexpr (PROF) {
@@ -324,8 +408,6 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
       o[1] = prof_bar;
       o[2] = prof_body;
       o[3] = prof_epi;
-      o[4] = prof_issue;
-      o[5] = prof_read;
     }
   }
 }
@@ -333,10 +415,10 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
 static int debug_grid = 0;
 static uint64_t* debug_prof = nullptr;  // > 0: number of persistent workgroups (experiments only)
 
-template <int NSTAGE, bool PROF>
+template <bool PROF>
 static int launch_dense32(const Dense32Args& p, hipStream_t st) {
-  auto kern = gemm_nt32_kernel<NSTAGE, PROF>;
-  constexpr int lds = NSTAGE * kStage32;
+  auto kern = gemm_nt32_kernel<PROF>;
+  constexpr int lds = kRing32 + 4 * 7168;  // ring + one output patch per wave = all 160 KB
   static int num_cus = 0;
   if (num_cus == 0) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -365,8 +447,8 @@ int launch_gemm_nt32(const uint8_t* a_codes, const uint8_t* a_scales, const uint
                      const uint8_t* b_scales, void* d, int64_t M, int64_t N, int64_t K,
                      int64_t ldd, hipStream_t st) {
   Dense32Args p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, M, N, K, ldd, debug_prof};
-  if (debug_prof) return launch_dense32<4, true>(p, st);
-  return launch_dense32<4, false>(p, st);
+  if (debug_prof) return launch_dense32<true>(p, st);
+  return launch_dense32<false>(p, st);
 }
 
 }  // namespace mx

@@ -299,12 +299,7 @@ class _MXGroupedMM(torch.autograd.Function):
 
 def _cast_w_rows(w: torch.Tensor, mode: str) -> MXData:
     """Row-wise cast of stacked matrices w [G, N, K] with one MFMA-order scale block each."""
-    G, N, K = w.shape
-    if N % 128 == 0:
-        return ops.to_mx_dim0_batched(w, mode, MX_SCALES_MFMA)
-    parts = [ops.to_mx_dim0(w[g], mode, MX_SCALES_MFMA) for g in range(G)]
-    return MXData(torch.stack([p.codes for p in parts]), torch.cat([p.scales for p in parts]),
-                  MX_SCALES_MFMA)
+    return ops.to_mx_dim0_batched(w, mode, MX_SCALES_MFMA)
 
 
 def mx_grouped_mm(x: torch.Tensor, w_t: torch.Tensor, offs: torch.Tensor, cfg: MXFP8Config):

@@ -187,12 +187,14 @@ def mx_gemm_nt(a: MXData, b: MXData, out: torch.Tensor | None = None) -> torch.T
 def to_mx_dim0_batched(w: torch.Tensor, mode="floor", order: int = MX_SCALES_MFMA) -> MXData:
     """Row-wise cast of every matrix of w [G, R, C]: codes [G, R, C], one scale block each.
 
-    A 3-D weight is G stacked matrices, so this is one row-wise cast of the [G*R, C] view;
-    in MFMA order that equals G per-matrix blocks only when R is a multiple of 128.
+    A 3-D weight is G stacked matrices, so this is one row-wise cast of the [G*R, C] view; in
+    MFMA order that equals G per-matrix blocks only when R is a multiple of 128, otherwise the
+    matrices are cast one by one.
     """
     G, R, C = w.shape
     if order == MX_SCALES_MFMA and R % 128:
-        raise ValueError("MFMA-order scales of stacked matrices need rows % 128 == 0")
+        parts = [to_mx_dim0(w[g], mode, order) for g in range(G)]
+        return MXData(torch.stack([p.codes for p in parts]), torch.cat([p.scales for p in parts]), order)
     d = to_mx_dim0(w.reshape(G * R, C), mode, order)
     scales = d.scales if order == MX_SCALES_MFMA else d.scales.view(G, R, C // BLOCK)
     return MXData(d.codes.view(G, R, C), scales, order)
