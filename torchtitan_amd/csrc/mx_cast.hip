@@ -285,6 +285,287 @@ __global__ __launch_bounds__(256) void cast_dim0_dim1_kernel(
 }
 
 // ------------------------------------------------------------------------------------
+// Tile kernel with 16-byte loads: row-wise, column-wise or both casts of one tile.
+// Workgroup tile = 32*WAVES rows x 128 columns.  Wave w owns rows [32w, 32w+32); lane l owns
+// columns 8(l&15)..+8 of the eight rows 8(l>>4)+k, so one load instruction fetches four
+// 256-byte row segments and a lane keeps an 8x8 patch in 32 registers.
+//   row-wise:    the 4 lanes of a DPP quad share a 32-column block (two quad_perm steps);
+//                codes leave as 8-byte stores (128 B per row segment).
+//   column-wise: the patch gives 8 per-column maxima, completed over the 4 lane groups with
+//                two lane exchanges; a column's 8 codes are one 8-byte LDS write into the
+//                transposed tile, which leaves as 32*WAVES-byte rows.
+// All scale bytes of the tile are staged in LDS in their final order and leave as dwords
+// (whole 256-byte groups in MFMA order, padding entries included as zeros).
+// ------------------------------------------------------------------------------------
+__device__ __forceinline__ uint32_t lane_xor(uint32_t v, int lane, int mask) {
+  return (uint32_t)__builtin_amdgcn_ds_bpermute((lane ^ mask) << 2, (int)v);
+}
+
+// Scale byte and narrowing factor of a block whose amax is finite (bits < 0x7F80): the
+// general formulas without the NaN / byte-254 cases, which cannot occur here.
+template <int MODE>
+__device__ __forceinline__ void finite_scale(uint32_t amax_bits, uint32_t& sb, float& mult) {
+  const uint32_t e = (MODE == MX_SCALE_RCEIL ? amax_bits + 0x1Fu : amax_bits) >> 7;
+  sb = max(e, 8u) - 8u;
+  uint32_t bits = (254u - sb) << 23;
+  if (sb == 0) bits = (MODE == MX_SCALE_FLOOR) ? 0x7E800000u : 0x3F800000u;
+  mult = __uint_as_float(bits);
+}
+
+// Two scaled floats -> two codes.  With RCEIL scales of a finite block every |value| is at
+// most 448 already, so the clamp is only needed for FLOOR scales.
+template <int MODE, bool HIGH>
+__device__ __forceinline__ uint32_t cvt2_finite(float lo, float hi, uint32_t old) {
+  if (MODE == MX_SCALE_FLOOR) {
+    lo = __builtin_amdgcn_fmed3f(lo, -448.0f, 448.0f);
+    hi = __builtin_amdgcn_fmed3f(hi, -448.0f, 448.0f);
+  }
+  return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(lo, hi, (int)old, HIGH);
+}
+
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xFFFF0000u); }
+
+// Quantize one lane's 8x8 patch.  FINITE = no Inf / NaN anywhere in the wave's patches: the
+// straight-line path; otherwise the general path with per-block NaN handling and clamps.
+template <int MODE, int ORDER, bool ROW, bool COL, int WAVES, bool FINITE>
+__device__ __forceinline__ void quantize_patch(u32x4 (&v)[8], const uint32_t (&mr)[8],
+                                               const uint32_t (&mc)[4], uint8_t* codes_row,
+                                               int64_t cols, int rows_left, bool col_ok,
+                                               uint8_t* lds_codes, uint8_t* lds_st,
+                                               uint8_t* lds_sr, int wave, int lane, int rl0) {
+  constexpr int PITCH = 32 * WAVES + 16;
+  const int g = lane >> 4, q = lane & 15;
+  if (ROW) {
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const u32x4 w = v[k];
+      uint32_t sb;
+      float mult;
+      u32x2 out;
+      if (FINITE) {
+        finite_scale<MODE>(mr[k], sb, mult);
+        out.x = cvt2_finite<MODE, true>(bf16_lo(w.y) * mult, bf16_hi(w.y) * mult,
+                                        cvt2_finite<MODE, false>(bf16_lo(w.x) * mult,
+                                                                 bf16_hi(w.x) * mult, 0));
+        out.y = cvt2_finite<MODE, true>(bf16_lo(w.w) * mult, bf16_hi(w.w) * mult,
+                                        cvt2_finite<MODE, false>(bf16_lo(w.z) * mult,
+                                                                 bf16_hi(w.z) * mult, 0));
+      } else {
+        sb = scale_byte<MODE>(mr[k]);
+        mult = scale_multiplier<MODE>(sb);
+        if (sb != 255) {
+          out.x = cvt2<true>(w.y, mult, cvt2<false>(w.x, mult, 0));
+          out.y = cvt2<true>(w.w, mult, cvt2<false>(w.z, mult, 0));
+        } else {
+          out.x = nan_block_codes2(w.x) | (nan_block_codes2(w.y) << 16);
+          out.y = nan_block_codes2(w.z) | (nan_block_codes2(w.w) << 16);
+        }
+      }
+      if (col_ok && k < rows_left)
+        __builtin_nontemporal_store(out, reinterpret_cast<u32x2*>(codes_row + k * cols));
+      if ((lane & 3) == 0) {  // rows / columns beyond the matrix were loaded as zeros: byte 0
+        const int rl = rl0 + k, bl = q >> 2;
+        if (ORDER == MX_SCALES_MFMA)
+          lds_sr[(((rl >> 7) * 2 + (bl >> 1)) << 8) + ((((bl & 1) << 5) + (rl & 31)) << 2) +
+                 ((rl & 127) >> 5)] = (uint8_t)sb;
+        else
+          lds_sr[rl * 4 + bl] = (uint8_t)sb;
+      }
+    }
+  }
+  if (COL) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const uint32_t amax = (j & 1) ? (mc[j >> 1] >> 16) : (mc[j >> 1] & 0xFFFFu);
+      uint32_t sb;
+      float mu;
+      u32x2 d;
+      if (FINITE) {
+        finite_scale<MODE>(amax, sb, mu);
+        float f[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+          f[k] = ((j & 1) ? bf16_hi(v[k][j >> 1]) : bf16_lo(v[k][j >> 1])) * mu;
+        d.x = cvt2_finite<MODE, true>(f[2], f[3], cvt2_finite<MODE, false>(f[0], f[1], 0));
+        d.y = cvt2_finite<MODE, true>(f[6], f[7], cvt2_finite<MODE, false>(f[4], f[5], 0));
+      } else {
+        sb = scale_byte<MODE>(amax);
+        mu = scale_multiplier<MODE>(sb);
+        uint32_t e[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+          e[k] = (j & 1) ? (v[k][j >> 1] >> 16) : (v[k][j >> 1] & 0xFFFFu);
+        if (sb != 255) {
+          float f[8];
+#pragma unroll
+          for (int k = 0; k < 8; ++k) f[k] = __uint_as_float(e[k] << 16) * mu;
+          d.x = cvt2f<true>(f[2], f[3], cvt2f<false>(f[0], f[1], 0));
+          d.y = cvt2f<true>(f[6], f[7], cvt2f<false>(f[4], f[5], 0));
+        } else {
+          d.x = nan_block_code(e[0]) | (nan_block_code(e[1]) << 8) |
+                (nan_block_code(e[2]) << 16) | (nan_block_code(e[3]) << 24);
+          d.y = nan_block_code(e[4]) | (nan_block_code(e[5]) << 8) |
+                (nan_block_code(e[6]) << 16) | (nan_block_code(e[7]) << 24);
+        }
+      }
+      const int cl = 8 * q + j;
+      *reinterpret_cast<u32x2*>(lds_codes + cl * PITCH + wave * 32 + 8 * g) = d;
+      if (g == 0) {
+        if (ORDER == MX_SCALES_MFMA)
+          lds_st[((wave >> 1) << 8) + ((((wave & 1) << 5) + (cl & 31)) << 2) + (cl >> 5)] =
+              (uint8_t)sb;
+        else
+          lds_st[cl * WAVES + wave] = (uint8_t)sb;
+      }
+    }
+  }
+}
+
+template <int MODE, int ORDER, bool ROW, bool COL, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void cast_tile_kernel(
+    const uint16_t* __restrict__ x, int64_t rows, int64_t cols, int64_t ldx,
+    uint8_t* __restrict__ codes, uint8_t* __restrict__ scales, int64_t nblk, int64_t ks_n,
+    uint8_t* __restrict__ codes_t, uint8_t* __restrict__ scales_t, int64_t nblk_t,
+    int64_t ks_n_t, int64_t x_bstride, int64_t s_bstride, int64_t st_bstride, uint32_t gx,
+    uint32_t gy) {
+  constexpr int TR = 32 * WAVES, TC = 128, PITCH = TR + 16;
+  __shared__ __attribute__((aligned(16))) uint8_t lds_codes[COL ? TC * PITCH : 16];
+  __shared__ __attribute__((aligned(16))) uint8_t lds_st[COL ? TC * WAVES : 16];
+  __shared__ __attribute__((aligned(16))) uint8_t lds_sr[ROW ? TR * 4 : 16];
+  x += blockIdx.z * x_bstride;  // batch of independent [rows, cols] matrices
+  if (ROW) {
+    codes += blockIdx.z * rows * cols;
+    scales += blockIdx.z * s_bstride;
+  }
+  if (COL) {
+    codes_t += blockIdx.z * rows * cols;
+    scales_t += blockIdx.z * st_bstride;
+  }
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 4, q = lane & 15;
+  const int rl0 = wave * 32 + 8 * g;  // first tile-local row of this lane
+
+  // Tiles are numbered so that workgroups running together cover compact regions of both
+  // the input and the transposed output: 8x8 blocks of tiles, walked down the rows first.
+  const uint32_t spr = (gx + 7) / 8, sup = blockIdx.x >> 6, in = blockIdx.x & 63;
+  const uint32_t bx = (sup % spr) * 8 + (in >> 3), by = (sup / spr) * 8 + (in & 7);
+  if (bx >= gx || by >= gy) return;
+
+  const int64_t r0 = (int64_t)by * TR, c0 = (int64_t)bx * TC;
+  const int64_t c = c0 + 8 * q;
+  const bool col_ok = c < cols;
+  const int64_t left64 = rows - (r0 + rl0);
+  const int rows_left = left64 > 8 ? 8 : (left64 < 0 ? 0 : (int)left64);
+
+  u32x4 v[8];
+  {
+    const uint16_t* src = x + (r0 + rl0) * ldx + c;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      v[k] = u32x4{0, 0, 0, 0};
+      if (col_ok && k < rows_left)
+        v[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + k * ldx));
+    }
+  }
+
+  // block maxima first: they also tell whether the wave holds any Inf / NaN
+  uint32_t mr[8] = {0, 0, 0, 0, 0, 0, 0, 0}, mc[4] = {0, 0, 0, 0};
+  uint32_t top = 0;
+  if (ROW) {
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const u32x4 w = v[k];
+      uint32_t m = pk_max_u16(pk_max_u16(w.x & 0x7FFF7FFFu, w.y & 0x7FFF7FFFu),
+                              pk_max_u16(w.z & 0x7FFF7FFFu, w.w & 0x7FFF7FFFu));
+      m = max(m & 0xFFFFu, m >> 16);
+      m = max(m, dpp<kQuadXor1>(m));
+      m = max(m, dpp<kQuadXor2>(m));
+      mr[k] = m;
+      top = max(top, m);
+    }
+  }
+  if (COL) {
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      mc[0] = pk_max_u16(mc[0], v[k].x & 0x7FFF7FFFu);
+      mc[1] = pk_max_u16(mc[1], v[k].y & 0x7FFF7FFFu);
+      mc[2] = pk_max_u16(mc[2], v[k].z & 0x7FFF7FFFu);
+      mc[3] = pk_max_u16(mc[3], v[k].w & 0x7FFF7FFFu);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      mc[i] = pk_max_u16(mc[i], lane_xor(mc[i], lane, 16));
+      mc[i] = pk_max_u16(mc[i], lane_xor(mc[i], lane, 32));
+    }
+    if (!ROW) {
+      const uint32_t t = pk_max_u16(pk_max_u16(mc[0], mc[1]), pk_max_u16(mc[2], mc[3]));
+      top = max(t & 0xFFFFu, t >> 16);
+    }
+  }
+  uint8_t* codes_row = ROW ? codes + (r0 + rl0) * cols + c : nullptr;
+  if (__builtin_amdgcn_ballot_w64(top >= 0x7F80u) == 0)
+    quantize_patch<MODE, ORDER, ROW, COL, WAVES, true>(v, mr, mc, codes_row, cols, rows_left,
+                                                       col_ok, lds_codes, lds_st, lds_sr, wave,
+                                                       lane, rl0);
+  else
+    quantize_patch<MODE, ORDER, ROW, COL, WAVES, false>(v, mr, mc, codes_row, cols, rows_left,
+                                                        col_ok, lds_codes, lds_st, lds_sr, wave,
+                                                        lane, rl0);
+  __syncthreads();
+
+  if (ROW && tid < TR) {
+    const uint32_t s4 = *reinterpret_cast<const uint32_t*>(lds_sr + tid * 4);
+    if (ORDER == MX_SCALES_MFMA) {
+      const int grp = tid >> 6;
+      const int64_t rt = (r0 >> 7) + (grp >> 1), ks = (c0 >> 6) + (grp & 1);
+      if (rt * 128 < rows && ks < ks_n)
+        *reinterpret_cast<uint32_t*>(scales + ((rt * ks_n + ks) << 8) + (tid & 63) * 4) = s4;
+    } else if (r0 + tid < rows) {
+      const int64_t b0 = c0 >> 5;
+      uint8_t* dst = scales + (r0 + tid) * nblk + b0;
+      if ((nblk & 3) == 0) {
+        if (b0 < nblk) *reinterpret_cast<uint32_t*>(dst) = s4;
+      } else {
+        for (int w = 0; w < 4 && b0 + w < nblk; ++w) dst[w] = (uint8_t)(s4 >> (8 * w));
+      }
+    }
+  }
+  if (COL) {
+    constexpr int SEGS = TR / 16;  // 16-byte pieces of one transposed row
+    const int seg = tid % SEGS;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const int o = p * 32 + tid / SEGS;
+      if (c0 + o < cols && r0 + seg * 16 < rows) {
+        const u32x4 t = *reinterpret_cast<const u32x4*>(lds_codes + o * PITCH + seg * 16);
+        __builtin_nontemporal_store(
+            t, reinterpret_cast<u32x4*>(codes_t + (c0 + o) * rows + r0 + seg * 16));
+      }
+    }
+    if (ORDER == MX_SCALES_MFMA) {
+      if (tid < TR) {  // WAVES/2 complete 256-byte groups
+        const int64_t ks = (r0 >> 6) + (tid >> 6);
+        if (ks < ks_n_t)
+          *reinterpret_cast<uint32_t*>(scales_t + (((c0 >> 7) * ks_n_t + ks) << 8) +
+                                       (tid & 63) * 4) =
+              *reinterpret_cast<const uint32_t*>(lds_st + tid * 4);
+      }
+    } else if (tid < TC && c0 + tid < cols) {
+      const int64_t b0 = r0 >> 5;
+      uint8_t* dst = scales_t + (c0 + tid) * nblk_t + b0;
+      if ((nblk_t & 3) == 0 && b0 + WAVES <= nblk_t) {
+#pragma unroll
+        for (int w = 0; w < WAVES / 4; ++w)
+          reinterpret_cast<uint32_t*>(dst)[w] =
+              *reinterpret_cast<const uint32_t*>(lds_st + tid * WAVES + 4 * w);
+      } else {
+        for (int w = 0; w < WAVES && b0 + w < nblk_t; ++w) dst[w] = lds_st[tid * WAVES + w];
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------
 // Scale re-layout (pure byte permutation) and its inverse.
 // ------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void scale_layout_kernel(const uint8_t* __restrict__ in,
@@ -345,6 +626,41 @@ using namespace mx;
                          __VA_ARGS__);                                                          \
   } while (0)
 
+#ifndef MX_CAST_WAVES
+#define MX_CAST_WAVES 4
+#endif
+#define MX_DISPATCH_TILE(ROW, COL, ...)                                                          \
+  do {                                                                                           \
+    if (scale_mode == MX_SCALE_FLOOR && scale_order == MX_SCALES_ROWMAJOR)                       \
+      hipLaunchKernelGGL(                                                                        \
+          (cast_tile_kernel<MX_SCALE_FLOOR, MX_SCALES_ROWMAJOR, ROW, COL, MX_CAST_WAVES>), grid, \
+          block, 0, st, __VA_ARGS__);                                                            \
+    else if (scale_mode == MX_SCALE_FLOOR)                                                       \
+      hipLaunchKernelGGL(                                                                        \
+          (cast_tile_kernel<MX_SCALE_FLOOR, MX_SCALES_MFMA, ROW, COL, MX_CAST_WAVES>), grid,     \
+          block, 0, st, __VA_ARGS__);                                                            \
+    else if (scale_order == MX_SCALES_ROWMAJOR)                                                  \
+      hipLaunchKernelGGL(                                                                        \
+          (cast_tile_kernel<MX_SCALE_RCEIL, MX_SCALES_ROWMAJOR, ROW, COL, MX_CAST_WAVES>), grid, \
+          block, 0, st, __VA_ARGS__);                                                            \
+    else                                                                                         \
+      hipLaunchKernelGGL(                                                                        \
+          (cast_tile_kernel<MX_SCALE_RCEIL, MX_SCALES_MFMA, ROW, COL, MX_CAST_WAVES>), grid,     \
+          block, 0, st, __VA_ARGS__);                                                            \
+  } while (0)
+
+// The tile kernel loads 16 bytes (8 columns) per lane.
+static inline bool tile_ok(const void* x, int64_t cols, int64_t ldx) {
+  return ((uintptr_t)x & 15) == 0 && (ldx & 7) == 0 && (cols & 7) == 0;
+}
+constexpr int kTileRows = 32 * MX_CAST_WAVES;
+static inline int64_t tile_grid_x(int64_t gx, int64_t gy) {
+  return ((gx + 7) / 8) * ((gy + 7) / 8) * 64;
+}
+static inline dim3 tile_grid(int64_t gx, int64_t gy, int64_t batch) {
+  return dim3((unsigned)tile_grid_x(gx, gy), 1, (unsigned)batch);
+}
+
 static inline bool bad_enums(int scale_mode, int scale_order) {
   return (scale_mode != MX_SCALE_FLOOR && scale_mode != MX_SCALE_RCEIL) ||
          (scale_order != MX_SCALES_ROWMAJOR && scale_order != MX_SCALES_MFMA);
@@ -383,6 +699,15 @@ extern "C" int mx_cast_dim0(const void* x, int64_t rows, int64_t cols, int64_t l
   dim3 grid((unsigned)nblocks), block(kDim0Threads);
   hipStream_t st = (hipStream_t)stream;
   if (scale_order == MX_SCALES_MFMA && ((uintptr_t)scales & 3)) return MX_ERR_ALIGNMENT;
+  const int64_t tgx = (cols + kT - 1) / kT, tgy = (rows + kTileRows - 1) / kTileRows;
+  if (scale_order == MX_SCALES_MFMA && tile_grid_x(tgx, tgy) <= 0x7FFFFFFF) {
+    // scattered scale bytes cost more than the tiled read: stage them through LDS
+    dim3 grid = tile_grid(tgx, tgy, 1), block(64 * MX_CAST_WAVES);
+    MX_DISPATCH_TILE(true, false, (const uint16_t*)x, rows, cols, ldx, codes, scales, nblk, ks_n,
+                     (uint8_t*)nullptr, (uint8_t*)nullptr, (int64_t)0, (int64_t)0, (int64_t)0,
+                     (int64_t)0, (int64_t)0, (uint32_t)tgx, (uint32_t)tgy);
+    return launch_status();
+  }
   clear_mfma_padding(scales, rows, nblk, scale_order, st);
   MX_DISPATCH_MODE_ORDER(cast_dim0_kernel, (const uint16_t*)x, ldx, (uint32_t)cpr, total, codes,
                          scales, nblk, ks_n);
@@ -408,8 +733,16 @@ extern "C" int mx_cast_dim1_batched(const void* x, int64_t batch, int64_t rows, 
   if (batch > 1 && ((rows * cols) % 16 || st_b % 4)) return MX_ERR_ALIGNMENT;
   const int64_t gx = (cols + kT - 1) / kT, gy = (rows + kT - 1) / kT;
   if (gy > 65535 || batch > 65535 || gx > 0x7FFFFFFF) return MX_ERR_UNSUPPORTED;
-  dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch), block(256);
   hipStream_t st = (hipStream_t)stream;
+  const int64_t tgy = (rows + kTileRows - 1) / kTileRows;
+  if (tile_ok(x, cols, ldx) && tile_grid_x(gx, tgy) <= 0x7FFFFFFF) {
+    dim3 grid = tile_grid(gx, tgy, batch), block(64 * MX_CAST_WAVES);
+    MX_DISPATCH_TILE(false, true, (const uint16_t*)x, rows, cols, ldx, (uint8_t*)nullptr,
+                     (uint8_t*)nullptr, (int64_t)0, (int64_t)0, codes_t, scales_t, nblk_t, ks_n_t,
+                     rows * ldx, (int64_t)0, st_b, (uint32_t)gx, (uint32_t)tgy);
+    return launch_status();
+  }
+  dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch), block(256);
   MX_DISPATCH_MODE_ORDER(cast_dim1_kernel, (const uint16_t*)x, rows, cols, ldx, codes_t,
                          scales_t, nblk_t, ks_n_t, rows * ldx, st_b);
   return launch_status();
@@ -439,9 +772,18 @@ extern "C" int mx_cast_dim0_dim1_batched(const void* x, int64_t batch, int64_t r
   const int64_t st_b = scale_bytes(cols, nblk_t, scale_order);
   const int64_t gx = (cols + kT - 1) / kT, gy = (rows + kT - 1) / kT;
   if (gy > 65535 || batch > 65535 || gx > 0x7FFFFFFF) return MX_ERR_UNSUPPORTED;
-  dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch), block(256);
   hipStream_t st = (hipStream_t)stream;
   if (scale_order == MX_SCALES_MFMA && ((uintptr_t)scales & 3)) return MX_ERR_ALIGNMENT;
+  const int64_t tgy = (rows + kTileRows - 1) / kTileRows;
+  if (tile_ok(x, cols, ldx) && ((uintptr_t)codes & 7) == 0 && ((uintptr_t)scales & 3) == 0 &&
+      tile_grid_x(gx, tgy) <= 0x7FFFFFFF) {
+    dim3 grid = tile_grid(gx, tgy, batch), block(64 * MX_CAST_WAVES);
+    MX_DISPATCH_TILE(true, true, (const uint16_t*)x, rows, cols, ldx, codes, scales, nblk, ks_n,
+                     codes_t, scales_t, nblk_t, ks_n_t, rows * ldx, s_b, st_b, (uint32_t)gx,
+                     (uint32_t)tgy);
+    return launch_status();
+  }
+  dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch), block(256);
   if (scale_order == MX_SCALES_MFMA && ((rows & 127) || (nblk & 1))) {
     // padding of every batch entry's row-wise scale block must read as zero
     const int64_t n = batch * s_b / 4;
