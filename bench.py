@@ -8,10 +8,11 @@ HBM before the timed region.  One step = the three linears, each through the con
 (product path): 2 fused casts + GEMM in forward, 1 fused cast + 2 GEMMs in backward.
 
 Prints ONE JSON line.  `value` counts only GEMM flops (2 M N K each) over the whole step time,
-casts included in the time.  `roofline` is for the dominant kernel (the 256x256 MXFP8 GEMM
-tile kernel), timed per launch with HIP events on the launch stream inside the timed steps.
+casts included in the time.  `roofline` is for the dominant kernel (the persistent 256x256-tile
+MXFP8 GEMM), timed per launch with HIP events on the launch stream inside the timed steps.
 `casts` gives the to_mx GB/s on inputs rotated through more memory than the 256 MB last-level
-cache.  `cpu_baseline` times the CPU oracle (emulated MX linear forward) on a bounded sample.
+cache.  `cpu_baseline` times the CPU oracle (emulated MX linear forward plus the column-wise
+casts) on a bounded sample of about 15 s.
 """
 from __future__ import annotations
 
@@ -30,6 +31,12 @@ METRIC = "MXFP8 linear TFLOP/s fwd+bwd at 8B FFN shape; to_mx cast GB/s"
 M, DIM, HIDDEN = 16384, 4096, 14336
 PEAK_MXFP8_TFLOPS = 5000.0  # MI355X dense fp8 / MXFP8 MFMA peak
 PEAK_HBM_GBPS = 8000.0
+# Bytes the GEMM kernel moves between L2 and the memory fabric per launch, mean over the step's
+# nine GEMMs: rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the same counter reads for a
+# known-size elementwise kernel (profiles/bench_ffn_M16384__hbm_traffic_pmc.txt).  Counters cannot
+# be read from inside this process, so the figure is carried here and re-measured when the kernel
+# changes.
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 1835155593
 
 
 def parse():
@@ -40,6 +47,9 @@ def parse():
     ap.add_argument("--recipe", default="mxfp8_rceil", choices=["mxfp8_rceil", "mxfp8_floor"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-casts", action="store_true")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="also run 4 elementwise passes over a 512 MiB tensor (reads 512 MiB, writes 512 MiB "
+                         "each): the known-size kernel that scales FETCH_SIZE / WRITE_SIZE counter readings")
     return ap.parse_args()
 
 
@@ -115,9 +125,11 @@ def time_casts(dev, recipe_mode):
     return out
 
 
-def cpu_baseline(recipe_mode_int):
-    """CPU oracle (emulated MX linear forward: cast X, cast W along K, dequantize, fp32 matmul,
-    bf16 out) on a bounded sample of BASELINE config 1."""
+def cpu_baseline(recipe_mode_int, target_s=15.0):
+    """CPU oracle on a bounded sample of BASELINE config 1: the emulated MX linear forward
+    (to_mx of X and W along K, dequantize, fp32 matmul, bf16 round) plus the column-wise casts
+    the backward needs, at N=14336, K=4096 and as many rows M as fit about `target_s` seconds
+    (calibrated on M=1024 first)."""
     import numpy as np
 
     from oracle import c_oracle as co
@@ -125,29 +137,44 @@ def cpu_baseline(recipe_mode_int):
 
     cores = min(16, os.cpu_count() or 1)
     os.environ.setdefault("OMP_NUM_THREADS", str(cores))
-    Ms, K, N = 2048, 4096, 4096
-    xb, wb = mo.make_cfg1_inputs(0, Ms, K, N)
-    t0 = time.perf_counter()
-    xc, xs = co.cast_dim0(xb, recipe_mode_int)
-    wc, ws = co.cast_dim0(wb, recipe_mode_int)
-    t1 = time.perf_counter()
-    a = co.dequant(xc, xs)
-    b = co.dequant(wc, ws)
-    y = mo.f32_to_bf16_bits(a @ b.T)
-    t2 = time.perf_counter()
+    K, N = DIM, HIDDEN
+
+    def run(Ms):
+        xb, wb = mo.make_cfg1_inputs(0, Ms, K, N)
+        t0 = time.perf_counter()
+        xc, xs = co.cast_dim0(xb, recipe_mode_int)
+        wc, ws = co.cast_dim0(wb, recipe_mode_int)
+        co.cast_dim1(xb, recipe_mode_int)
+        co.cast_dim1(wb, recipe_mode_int)
+        t1 = time.perf_counter()
+        y = mo.f32_to_bf16_bits(co.dequant(xc, xs) @ co.dequant(wc, ws).T)
+        t2 = time.perf_counter()
+        return xb, xc, y, t1 - t0, t2 - t1
+
+    _, _, _, c_s, m_s = run(1024)
+    # W's casts do not shrink with M: estimate them from the element counts
+    per_row = (c_s * 1024 / (1024 + N) + m_s) / 1024
+    fixed = c_s * N / (1024 + N)
+    Ms = int(max(1024, min(M, (target_s - fixed) / per_row // 1024 * 1024)))
+    xb, xc, y, c_s, m_s = run(Ms)
+    reps = 1
+    while c_s + m_s < 0.8 * target_s and reps < 16:  # fast host: repeat the full-size sample
+        _, _, _, c2, m2 = run(Ms)
+        c_s, m_s, reps = c_s + c2, m_s + m2, reps + 1
+    c_s, m_s = c_s / reps, m_s / reps
     # the C casts must agree with the NumPy oracle on a slice (checker sanity, not a measurement)
     assert np.array_equal(mo.cast_dim0(xb[:64], recipe_mode_int)[0], xc[:64])
     flops = 2.0 * Ms * K * N
-    cast_bytes = (Ms * K + N * K) * 3.03125
+    cast_bytes = 2 * (Ms * K + N * K) * 3.03125
     return {
-        "value": round(flops / (t2 - t0) / 1e12, 4),
+        "value": round(flops / (c_s + m_s) / 1e12, 4),
         "unit": "TFLOP/s",
         "cores": cores,
         "kind": "port",
-        "sample": f"config 1 at M={Ms} (X[{Ms},{K}], W[{N},{K}], 0.1% x100 outliers): to_mx dim0 of X and W "
-                  f"(C oracle, OpenMP) + dequantize + fp32 matmul (NumPy BLAS) + bf16 round; "
-                  f"casts {cast_bytes / (t1 - t0) / 1e9:.2f} GB/s, matmul part {flops / (t2 - t1) / 1e12:.3f} TFLOP/s, "
-                  f"wall {t2 - t0:.2f} s",
+        "sample": f"config 1 at M={Ms} of {M} rows (X[{Ms},{K}], W[{N},{K}], 0.1% x100 outliers): to_mx dim0 and "
+                  f"dim1 of X and W (C oracle, OpenMP) + dequantize + fp32 matmul (NumPy BLAS) + bf16 round; "
+                  f"casts {cast_bytes / c_s / 1e9:.2f} GB/s in {c_s:.2f} s, matmul part "
+                  f"{flops / m_s / 1e12:.3f} TFLOP/s in {m_s:.2f} s; mean of {reps} run(s)",
         "checksum": int(y.astype(np.uint64).sum() % (1 << 32)),
     }
 
@@ -169,6 +196,13 @@ def main():
     x.requires_grad_(True)
     h.requires_grad_(True)
 
+    if args.pmc_calibration:
+        src = torch.ones(256 * 1024 * 1024, device=dev, dtype=torch.bfloat16)
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            torch.mul(src, 2.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         one_step(ffn, x, h, dy_h, dy_o)
     torch.cuda.synchronize()
@@ -216,7 +250,9 @@ def main():
             "peak": PEAK_MXFP8_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_MXFP8_TFLOPS, 4),
-            "traffic": None,
+            "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH,
+            "traffic_note": "bytes per launch between L2 and fabric (rocprofv3 FETCH_SIZE + WRITE_SIZE, offline); "
+                            "operands and output once would be 488.5e6",
             "launches_timed": n_gemm,
             "avg_launch_ms": round(gemm_ms, 4),
         },
@@ -230,7 +266,7 @@ def main():
     if not args.no_casts:
         line["casts"] = time_casts(dev, recipe_mode)
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(0 if recipe_mode == "floor" else 1)
+        line["cpu_baseline"] = cpu_baseline(0 if recipe_mode == "floor" else 1, target_s=12.0)
     print(json.dumps(line))
 
 
