@@ -229,6 +229,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
   v16f acc[4][4];
   int c_slot = 0;  // ring block holding the K block being computed
   uint64_t prof_vm = 0, prof_bar = 0, prof_body = 0, prof_last = 0, prof_epi = 0;
+  uint64_t prof_e_stage = 0, prof_e_wait = 0, prof_e_store = 0;
 
   auto mfma_one = [&](const Frags32& f, auto first_, auto i_) {
     constexpr bool kFirst = decltype(first_)::value;  // first step of a tile starts from zero
@@ -243,32 +244,60 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
     }
   };
 
-  // A K block is two steps.  Entering step A, f0 holds the fragments of the block's first half
-  // (read during the previous step); ring block c_slot holds the block, c_slot^1 the next one
-  // (still landing).
-  //   step A: read the second half into f1, MFMAs on f0.
-  //   step B: every wave now holds all fragments of this block in registers, and the next
-  //           block must have landed: wait, barrier, refill c_slot with the block after next,
-  //           read the next block's first half into f0, MFMAs on f1.
-  // A wave issues in order and an MFMA occupies the matrix pipe for 64 cycles, so every other
-  // instruction is placed in the shadow of an MFMA: the sequence below is pinned with
-  // scheduling fences (one MFMA, then one or two copies / fragment reads).
-  // (waits written as assembly: the compiler rewrites the immediates of s_waitcnt builtins
-  // from its own, here too pessimistic, model of what is outstanding)
-  auto block_steps = [&](Frags32& f0, Frags32& f1, auto first_, auto last_) {
-    constexpr bool kLast = decltype(last_)::value;  // last block of a tile: see the tile loop
+  // A K block is two steps of 16 MFMAs.  Entering step A of block b, f0 holds the fragments of
+  // its first K half, ring block c_slot holds block b and c_slot^1 holds block b+1 (all of its
+  // copies issued, still landing).
+  //   step A: MFMAs on f0; the second half is read into f1 in slots 0-8.  Once every wave has
+  //           done so (barrier before slot kMidA) ring block c_slot is free, and the copies of
+  //           block b+2 into it start: kCopiesA of them in the rest of the step.
+  //   step B: block b+1 must have landed (all but the kCopiesA youngest copies: wait,
+  //           barrier); MFMAs on f1; the remaining copies of block b+2, three every four
+  //           slots; the first half of block b+1 is read into f0 in slots 0-8.
+  // The copy unit serves all four waves at about 20 cycles per copy, so four waves issuing
+  // one copy per 64-cycle slot keep it saturated and the MFMAs start to wait behind them:
+  // spreading the block's 18 copies over 22 slots instead of 16 is what the second barrier
+  // buys.  A wave issues in order and an MFMA occupies the matrix pipe for 64 cycles, so every
+  // other instruction is placed in the shadow of an MFMA; the sequence is pinned with
+  // scheduling fences.  (Waits are written as assembly: the compiler rewrites the immediates
+  // of s_waitcnt builtins from its own, here too pessimistic, model of what is outstanding.)
+  constexpr int kReadSlots = 9;  // 18 fragment reads, two per MFMA slot
+#ifndef MX_MID_A
+#define MX_MID_A 10
+#endif
+#ifndef MX_B_SKIP
+#define MX_B_SKIP 4
+#endif
+  constexpr int kMidA = MX_MID_A;  // slot of step A in front of which the ring block is released
+  constexpr int kSkipB = MX_B_SKIP;  // step B leaves every kSkipB-th slot without a copy (0: none)
+  constexpr int kCopiesA = 16 - kMidA;
+  auto block_steps = [&](Frags32& f0, Frags32& f1, auto first_) {
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     pin_frags(f0);
     {
       const uint32_t sbase = lds_base + c_slot * kBlock32;
       static_for<0, 16>([&](auto i_) {
         constexpr int i = decltype(i_)::value;
+        if constexpr (i == kMidA) {
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave's reads of the block are done
+          uint64_t t0 = 0;
+          if constexpr (PROF) t0 = __builtin_readcyclecounter();
+          __builtin_amdgcn_s_barrier();
+          if constexpr (PROF) {
+            const uint64_t t1 = __builtin_readcyclecounter();
+            prof_bar += t1 - t0;
+            prof_last += t1 - t0;  // keep the barrier out of the body figure
+          }
+        }
         mfma_one(f0, first_, i_);
-        // the last two copies of the block being fetched (its scales) trail into this step
-        if constexpr (i < 2) issue_piece(std::integral_constant<int, 16 + i>{});
-        if constexpr (i == 2) issue_advance();
-        read_piece(f1, sbase, std::integral_constant<int, 1>{}, i_);
-        if constexpr (i >= 14) read_piece(f1, sbase, std::integral_constant<int, 1>{}, std::integral_constant<int, i + 2>{});
+#ifndef MX_ABL_NO_READ
+        if constexpr (i < kReadSlots) {
+          read_piece(f1, sbase, std::integral_constant<int, 1>{}, std::integral_constant<int, 2 * i>{});
+          read_piece(f1, sbase, std::integral_constant<int, 1>{}, std::integral_constant<int, 2 * i + 1>{});
+        }
+#endif
+#ifndef MX_ABL_NO_DMA
+        if constexpr (i >= kMidA) issue_piece(std::integral_constant<int, i - kMidA>{});
+#endif
         __builtin_amdgcn_sched_barrier(0);
       });
     }
@@ -280,7 +309,8 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
       t0 = __builtin_readcyclecounter();
       prof_body += t0 - prof_last;
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the next block (and any output stores)
+    // block b+1 (and any output stores): everything but the copies issued in step A
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kCopiesA) : "memory");
     if constexpr (PROF) {
       t1 = __builtin_readcyclecounter();
       prof_vm += t1 - t0;
@@ -291,19 +321,23 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
       prof_bar += prof_last - t1;
     }
     {
-      // One copy of the block after next per MFMA (the texture path takes 16 cycles per copy
-      // and serves all four waves, so one per 64-cycle slot per wave is its full rate), into
-      // the ring block just drained; the fragment reads of the next block's first half go last.
       const uint32_t sbase = lds_base + (c_slot ^ 1) * kBlock32;
       static_for<0, 16>([&](auto i_) {
         constexpr int i = decltype(i_)::value;
         mfma_one(f1, std::false_type{}, i_);
-        issue_piece(i_);
-        if constexpr (i >= 10 && !kLast) {
-          read_piece(f0, sbase, std::integral_constant<int, 0>{}, std::integral_constant<int, 3 * (i - 10)>{});
-          read_piece(f0, sbase, std::integral_constant<int, 0>{}, std::integral_constant<int, 3 * (i - 10) + 1>{});
-          read_piece(f0, sbase, std::integral_constant<int, 0>{}, std::integral_constant<int, 3 * (i - 10) + 2>{});
+#ifndef MX_ABL_NO_DMA
+        // copies kCopiesA .. 17, one per slot, every kSkipB-th slot left free
+        constexpr int j = kSkipB ? i - i / kSkipB : i;
+        constexpr bool skip = kSkipB && (i % kSkipB) == kSkipB - 1;
+        if constexpr (!skip && kCopiesA + j < 18) issue_piece(std::integral_constant<int, kCopiesA + j>{});
+#endif
+        if constexpr (i == 15) issue_advance();
+#ifndef MX_ABL_NO_READ
+        if constexpr (i < kReadSlots) {
+          read_piece(f0, sbase, std::integral_constant<int, 0>{}, std::integral_constant<int, 2 * i>{});
+          read_piece(f0, sbase, std::integral_constant<int, 0>{}, std::integral_constant<int, 2 * i + 1>{});
         }
+#endif
         __builtin_amdgcn_sched_barrier(0);
       });
       c_slot ^= 1;
@@ -333,38 +367,57 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
     // lane's place in a stored piece: row (lane >> 3) + 8*pass, columns (lane & 7)*8 .. +7
     const uint32_t colp = wn * 128 + (lane & 7) * 8;
     const uint32_t vrow = (wm * 128 + (lane >> 3)) * ldd_b + colp * 2;
-    static_for<0, 4>([&](auto m_) {
-      constexpr int m = decltype(m_)::value;
-      static_for<0, 2>([&](auto np_) {
-        constexpr int np = decltype(np_)::value;  // column pair: sub-tiles n = 2np, 2np+1
-        static_for<0, 4>([&](auto k_) {
-          constexpr int n = 2 * np + (decltype(k_)::value >> 1), h = decltype(k_)::value & 1;
-          const v16f a = acc[m][n];
-          const uint32_t x0 = pack_bf16(a[8 * h + 0], a[8 * h + 1]), y0 = pack_bf16(a[8 * h + 2], a[8 * h + 3]);
-          const uint32_t x1 = pack_bf16(a[8 * h + 4], a[8 * h + 5]), y1 = pack_bf16(a[8 * h + 6], a[8 * h + 7]);
-          const u32x2 sx = __builtin_amdgcn_permlane32_swap(x0, x1, false, false);
-          const u32x2 sy = __builtin_amdgcn_permlane32_swap(y0, y1, false, false);
-          const v4i w = {(int)sx.x, (int)sy.x, (int)sx.y, (int)sy.y};
-          lds_write_b128_hidden<(n & 1) * 64 + h * 32>(patch_w, w);
-        });
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        v4i r[4];
-        static_for<0, 4>([&](auto q_) {
-          constexpr int q = decltype(q_)::value;
-          r[q] = lds_read_b128_hidden<q * 8 * kPatchPitch>(patch_r);
-        });
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        const uint32_t v = (colp + np * 64 < cols_valid) ? vrow + np * 128 : 0x80000000u;
-        static_for<0, 4>([&](auto q_) {
-          constexpr int q = decltype(q_)::value;
-          const v4i rq = pin(r[q]);
-          const u32x4 w = {(uint32_t)rq.x, (uint32_t)rq.y, (uint32_t)rq.z, (uint32_t)rq.w};
-          __builtin_amdgcn_raw_buffer_store_b128(w, rd, v, (m * 32 + q * 8) * ldd_b, 0);
-        });
-        // keep the pieces apart: hoisting the accumulator reads of later pieces over this
-        // point only costs registers
-        __builtin_amdgcn_sched_barrier(0);
+    // Pieces p = 0..7: 32 rows (sub-tile row m = p/2) x 64 columns (sub-tiles n = 2(p%2), +1).
+    // A wave's LDS instructions execute in order, so a piece's reads may follow its writes
+    // without a wait, and the next piece's writes may follow those reads: the only waits are
+    // for the read data, with the next piece's conversion and writes already under way.
+    auto stage = [&](auto p_) {  // accumulators -> bf16 -> patch
+      constexpr int m = decltype(p_)::value >> 1, np = decltype(p_)::value & 1;
+      static_for<0, 4>([&](auto k_) {
+        constexpr int n = 2 * np + (decltype(k_)::value >> 1), h = decltype(k_)::value & 1;
+        const v16f a = acc[m][n];
+        const uint32_t x0 = pack_bf16(a[8 * h + 0], a[8 * h + 1]), y0 = pack_bf16(a[8 * h + 2], a[8 * h + 3]);
+        const uint32_t x1 = pack_bf16(a[8 * h + 4], a[8 * h + 5]), y1 = pack_bf16(a[8 * h + 6], a[8 * h + 7]);
+        const u32x2 sx = __builtin_amdgcn_permlane32_swap(x0, x1, false, false);
+        const u32x2 sy = __builtin_amdgcn_permlane32_swap(y0, y1, false, false);
+        const v4i w = {(int)sx.x, (int)sy.x, (int)sx.y, (int)sy.y};
+        lds_write_b128_hidden<(n & 1) * 64 + h * 32>(patch_w, w);
       });
+    };
+    v4i r[2][4];
+    stage(std::integral_constant<int, 0>{});
+    static_for<0, 8>([&](auto p_) {
+      constexpr int pc = decltype(p_)::value, m = pc >> 1, np = pc & 1;
+      static_for<0, 4>([&](auto q_) {
+        constexpr int q = decltype(q_)::value;
+        r[pc & 1][q] = lds_read_b128_hidden<q * 8 * kPatchPitch>(patch_r);
+      });
+      uint64_t e0 = 0, e1 = 0, e2 = 0;
+      if constexpr (PROF) e0 = __builtin_readcyclecounter();
+      if constexpr (pc < 7) {
+        stage(std::integral_constant<int, pc + 1>{});
+        if constexpr (PROF) e1 = __builtin_readcyclecounter();
+        asm volatile("s_waitcnt lgkmcnt(4)" ::: "memory");  // the reads; the 4 younger writes may trail
+      } else {
+        if constexpr (PROF) e1 = __builtin_readcyclecounter();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      }
+      if constexpr (PROF) e2 = __builtin_readcyclecounter();
+      const uint32_t v = (colp + np * 64 < cols_valid) ? vrow + np * 128 : 0x80000000u;
+      static_for<0, 4>([&](auto q_) {
+        constexpr int q = decltype(q_)::value;
+        const v4i rq = pin(r[pc & 1][q]);
+        const u32x4 w = {(uint32_t)rq.x, (uint32_t)rq.y, (uint32_t)rq.z, (uint32_t)rq.w};
+        __builtin_amdgcn_raw_buffer_store_b128(w, rd, v, (m * 32 + q * 8) * ldd_b, 0);
+      });
+      if constexpr (PROF) {
+        prof_e_stage += e1 - e0;
+        prof_e_wait += e2 - e1;
+        prof_e_store += __builtin_readcyclecounter() - e2;
+      }
+      // keep the pieces apart: hoisting the accumulator reads of later pieces over this
+      // point only costs registers
+      __builtin_amdgcn_sched_barrier(0);
     });
   };
 
@@ -373,22 +426,17 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
   issue_block();
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __builtin_amdgcn_s_barrier();
-  static_for<0, 16>([&](auto i_) { issue_piece(i_); });  // scales + advance follow in the first step
+  issue_block();  // block 1: in flight when the first step starts
   Frags32 f0, f1;
   read_frags(f0, 0, std::integral_constant<int, 0>{});
   if constexpr (PROF) prof_last = __builtin_readcyclecounter();
 
-  // ---- tiles; at the top of every tile f0 holds the fragments of its first half block.  The
-  // last block of a tile leaves the next tile's first fragments unread until the tile has been
-  // written out, so that no fragment register is live across the epilogue.
+  // ---- tiles; at the top of every tile f0 holds the fragments of its first half block (the
+  // last step of a tile has already read them from the next tile's first block, which the
+  // loader fetched like any other block).
   for (uint32_t tile = 0; tile < n_my; ++tile) {
-    if (nblocks == 1) {
-      block_steps(f0, f1, std::true_type{}, std::true_type{});
-    } else {
-      block_steps(f0, f1, std::true_type{}, std::false_type{});
-      for (uint32_t i = 2; i < nblocks; ++i) block_steps(f0, f1, std::false_type{}, std::false_type{});
-      block_steps(f0, f1, std::false_type{}, std::true_type{});
-    }
+    block_steps(f0, f1, std::true_type{});
+    for (uint32_t i = 1; i < nblocks; ++i) block_steps(f0, f1, std::false_type{});
     if constexpr (PROF) {
       const uint64_t e0 = __builtin_readcyclecounter();
       prof_body += e0 - prof_last;
@@ -398,7 +446,6 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
     } else {
       epilogue(tile);
     }
-    read_frags(f0, c_slot, std::integral_constant<int, 0>{});
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the over-issued prefetches before retiring
   if constexpr (PROF) {
@@ -408,6 +455,9 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
       o[1] = prof_bar;
       o[2] = prof_body;
       o[3] = prof_epi;
+      o[4] = prof_e_stage;
+      o[5] = prof_e_wait;
+      o[6] = prof_e_store;
     }
   }
 }
