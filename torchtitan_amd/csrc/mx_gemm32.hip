@@ -261,6 +261,12 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
   // scheduling fences.  (Waits are written as assembly: the compiler rewrites the immediates
   // of s_waitcnt builtins from its own, here too pessimistic, model of what is outstanding.)
   constexpr int kReadSlots = 9;  // 18 fragment reads, two per MFMA slot
+// Output stores carry the nontemporal policy bit: written once, never re-read by this kernel,
+// and without it the output lines displace operand panels in L2 and the copies of the next
+// tile's first blocks queue behind the draining stores.
+#ifndef MX_STORE_AUX
+#define MX_STORE_AUX 2
+#endif
 #ifndef MX_MID_A
 #define MX_MID_A 10
 #endif
@@ -371,56 +377,58 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
     // A wave's LDS instructions execute in order, so a piece's reads may follow its writes
     // without a wait, and the next piece's writes may follow those reads: the only waits are
     // for the read data, with the next piece's conversion and writes already under way.
-    auto stage = [&](auto p_) {  // accumulators -> bf16 -> patch
+    auto stage_part = [&](auto p_, auto k_) {  // 32 rows x 16 columns: accumulators -> bf16 -> patch
       constexpr int m = decltype(p_)::value >> 1, np = decltype(p_)::value & 1;
-      static_for<0, 4>([&](auto k_) {
-        constexpr int n = 2 * np + (decltype(k_)::value >> 1), h = decltype(k_)::value & 1;
-        const v16f a = acc[m][n];
-        const uint32_t x0 = pack_bf16(a[8 * h + 0], a[8 * h + 1]), y0 = pack_bf16(a[8 * h + 2], a[8 * h + 3]);
-        const uint32_t x1 = pack_bf16(a[8 * h + 4], a[8 * h + 5]), y1 = pack_bf16(a[8 * h + 6], a[8 * h + 7]);
-        const u32x2 sx = __builtin_amdgcn_permlane32_swap(x0, x1, false, false);
-        const u32x2 sy = __builtin_amdgcn_permlane32_swap(y0, y1, false, false);
-        const v4i w = {(int)sx.x, (int)sy.x, (int)sx.y, (int)sy.y};
-        lds_write_b128_hidden<(n & 1) * 64 + h * 32>(patch_w, w);
-      });
+      constexpr int n = 2 * np + (decltype(k_)::value >> 1), h = decltype(k_)::value & 1;
+      const v16f a = acc[m][n];
+      const uint32_t x0 = pack_bf16(a[8 * h + 0], a[8 * h + 1]), y0 = pack_bf16(a[8 * h + 2], a[8 * h + 3]);
+      const uint32_t x1 = pack_bf16(a[8 * h + 4], a[8 * h + 5]), y1 = pack_bf16(a[8 * h + 6], a[8 * h + 7]);
+      const u32x2 sx = __builtin_amdgcn_permlane32_swap(x0, x1, false, false);
+      const u32x2 sy = __builtin_amdgcn_permlane32_swap(y0, y1, false, false);
+      const v4i w = {(int)sx.x, (int)sy.x, (int)sx.y, (int)sy.y};
+      lds_write_b128_hidden<(n & 1) * 64 + h * 32>(patch_w, w);
     };
     v4i r[2][4];
-    stage(std::integral_constant<int, 0>{});
+    static_for<0, 4>([&](auto k_) { stage_part(std::integral_constant<int, 0>{}, k_); });
     static_for<0, 8>([&](auto p_) {
       constexpr int pc = decltype(p_)::value, m = pc >> 1, np = pc & 1;
+      uint64_t e0 = 0;
+      if constexpr (PROF) e0 = __builtin_readcyclecounter();
       static_for<0, 4>([&](auto q_) {
         constexpr int q = decltype(q_)::value;
         r[pc & 1][q] = lds_read_b128_hidden<q * 8 * kPatchPitch>(patch_r);
       });
-      uint64_t e0 = 0, e1 = 0, e2 = 0;
-      if constexpr (PROF) e0 = __builtin_readcyclecounter();
-      if constexpr (pc < 7) {
-        stage(std::integral_constant<int, pc + 1>{});
-        if constexpr (PROF) e1 = __builtin_readcyclecounter();
-        asm volatile("s_waitcnt lgkmcnt(4)" ::: "memory");  // the reads; the 4 younger writes may trail
-      } else {
-        if constexpr (PROF) e1 = __builtin_readcyclecounter();
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-      }
-      if constexpr (PROF) e2 = __builtin_readcyclecounter();
       const uint32_t v = (colp + np * 64 < cols_valid) ? vrow + np * 128 : 0x80000000u;
+      // the next piece's conversion runs between this piece's stores, which drain at the
+      // write path's pace
       static_for<0, 4>([&](auto q_) {
         constexpr int q = decltype(q_)::value;
+#ifndef MX_ABL_NO_STAGE
+        if constexpr (pc < 7) stage_part(std::integral_constant<int, pc + 1>{}, q_);
+#else
+        if constexpr (pc < 7) lds_write_b128_hidden<q * 32>(patch_w, v4i{1, 2, 3, 4});
+#endif
+        if constexpr (q == 0) {
+          // the four reads are done once at most the one younger write is outstanding
+          if constexpr (pc < 7) asm volatile("s_waitcnt lgkmcnt(1)" ::: "memory");
+          else asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        }
         const v4i rq = pin(r[pc & 1][q]);
         const u32x4 w = {(uint32_t)rq.x, (uint32_t)rq.y, (uint32_t)rq.z, (uint32_t)rq.w};
-        __builtin_amdgcn_raw_buffer_store_b128(w, rd, v, (m * 32 + q * 8) * ldd_b, 0);
+#ifndef MX_ABL_NO_STORE
+        __builtin_amdgcn_raw_buffer_store_b128(w, rd, v, (m * 32 + q * 8) * ldd_b, MX_STORE_AUX);
+#else
+        asm volatile("" ::"v"(w));
+#endif
+        __builtin_amdgcn_sched_barrier(0);
       });
-      if constexpr (PROF) {
-        prof_e_stage += e1 - e0;
-        prof_e_wait += e2 - e1;
-        prof_e_store += __builtin_readcyclecounter() - e2;
-      }
-      // keep the pieces apart: hoisting the accumulator reads of later pieces over this
-      // point only costs registers
-      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (PROF) prof_e_stage += __builtin_readcyclecounter() - e0;
     });
   };
 
+#ifdef MX_XCD_STAGGER
+  for (uint32_t i = 0, n = xcd * MX_XCD_STAGGER; i < n; ++i) __builtin_amdgcn_s_sleep(1);
+#endif
   // ---- prologue: fill the ring, fetch the first fragments
   loader_open_tile();
   issue_block();
