@@ -105,24 +105,35 @@ int mx_gemm_nt(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b
 
 /* Grouped GEMM, 2D x 3D: for group g with rows [offs[g-1], offs[g]) of A:
  * D[rows, :] = deq(A[rows, :]) * deq(B[g])^T.  a_codes [T,K]; b_codes [G,N,K];
- * a_scales row-major [T, K/32] (group boundaries need not fall on 64-row tiles);
  * b_scales G consecutive MFMA-order blocks, each for [N, K/32].
  * offs int32 [G] inclusive cumulative sizes on the device; rows >= offs[G-1] are written as
- * zeros.  Group sizes need not be aligned for this entry point.  Stands in for
- * torch._grouped_mm(x, w^T, offs) in forward and dgrad
+ * zeros.  a_scale_order says how a_scales is laid out:
+ *   MX_SCALES_ROWMAJOR  [T, K/32]; groups may end anywhere (tile kernel);
+ *   MX_SCALES_MFMA      MFMA order over the whole [T, K/32] matrix; every group must end at a
+ *                       multiple of 128 rows, T % 128 == 0, K % 128 == 0, N % 8 == 0,
+ *                       G <= 638: the persistent 32x32x64 kernel (several times faster).  The
+ *                       group ends live on the device, so they are checked there: a violation
+ *                       fills D with NaN.
+ * Stands in for torch._grouped_mm(x, w^T, offs) in forward and dgrad
  * (torchtitan/models/common/moe/moe.py:59-76). */
 int mx_grouped_gemm_2d3d(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                          const uint8_t* b_scales, const int32_t* offs, void* d, int64_t T,
-                         int64_t N, int64_t K, int64_t G, int64_t ldd, void* stream);
+                         int64_t N, int64_t K, int64_t G, int64_t ldd, int a_scale_order,
+                         void* stream);
 
 /* Grouped GEMM, 2D x 2D (wgrad): D[g][N,K] = deq(A^T[:, rows_g]) * deq(B^T[:, rows_g])^T,
  * contracting over the tokens of group g.  at_codes [N,T] and bt_codes [K,T] are the
- * column-wise casts; their scales are row-major [N, T/32] and [K, T/32].  Every group size
- * must be a multiple of 32 (torchtitan/models/common/moe/utils.py:47-52); empty groups give
- * zeros.  d is [G,N,K] bf16 dense. */
+ * column-wise casts; scale_order says how both scale buffers are laid out:
+ *   MX_SCALES_ROWMAJOR  [N, T/32] and [K, T/32]; every group size a multiple of 32
+ *                       (torchtitan/models/common/moe/utils.py:47-52);
+ *   MX_SCALES_MFMA      MFMA order; every group must end at a multiple of 128 tokens,
+ *                       T % 128 == 0, K % 8 == 0: the persistent kernel; checked on the
+ *                       device, a violation fills D with NaN.
+ * Empty groups give zeros.  d is [G,N,K] bf16 dense. */
 int mx_grouped_gemm_2d2d(const uint8_t* at_codes, const uint8_t* at_scales,
                          const uint8_t* bt_codes, const uint8_t* bt_scales, const int32_t* offs,
-                         void* d, int64_t T, int64_t N, int64_t K, int64_t G, void* stream);
+                         void* d, int64_t T, int64_t N, int64_t K, int64_t G, int scale_order,
+                         void* stream);
 
 /* Token-group padding: from per-(rank, expert) counts build
  *   m_sizes[e]   = round_up(max(sum_r counts[r*E+e], alignment), alignment)   int32 [E]

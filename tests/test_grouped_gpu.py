@@ -76,6 +76,78 @@ def test_grouped_wgrad(device, sizes, N, K):
                 assert rel_l2(_f32(got[g]), _f32(ref[g])) <= TOL, g
 
 
+FAST_CASES = [
+    # (group sizes, all multiples of 128; N; K) -- the persistent-kernel forms (MFMA-order scales)
+    ([128, 256, 384], 256, 128),
+    ([0, 128, 0, 640, 0], 128, 256),
+    ([512, 128, 0, 1024, 256], 768, 384),
+    ([1280, 384], 264, 512),
+]
+
+
+@pytest.mark.parametrize("sizes,N,K", FAST_CASES)
+@pytest.mark.parametrize("tail_rows", [0, 128, 384])
+def test_grouped_forward_and_dgrad_aligned_groups(device, sizes, N, K, tail_rows):
+    """2D x 3D through the persistent kernel: groups end at multiples of 128, MFMA-order scales."""
+    rng = np.random.default_rng(sum(sizes) + N + K + 7)
+    T = sum(sizes) + tail_rows
+    G = len(sizes)
+    x_bits = randn_bits(rng, (T, K), outliers=1e-3)
+    w_bits = randn_bits(rng, (G, N, K), std=0.02)
+    offs = _sizes_to_offs(sizes, device)
+    x, w = bf16_from_bits(x_bits, device), bf16_from_bits(w_bits, device)
+    for mode_name, mode in (("floor", mo.FLOOR), ("rceil", mo.RCEIL)):
+        wq0 = ops.to_mx_dim0_batched(w, mode_name, L)
+        y = ops.mx_grouped_gemm_2d3d(ops.to_mx_dim0(x, mode_name, L), wq0, offs)
+        ref = mo.grouped_fwd(x_bits, w_bits, np.cumsum(sizes), mode)
+        assert rel_l2(_f32(bits_of(y)), _f32(ref)) <= TOL
+        assert np.all(bits_of(y)[sum(sizes):] == 0), "rows behind the last group must be zero"
+        # the general kernel (row-major scales) must agree to the last bit on the same operands
+        y2 = ops.mx_grouped_gemm_2d3d(ops.to_mx_dim0(x, mode_name, R), wq0, offs)
+        assert rel_l2(_f32(bits_of(y)), _f32(bits_of(y2))) <= 2e-3
+    if N % 128 == 0:
+        dy_bits = randn_bits(rng, (T, N), std=1e-3)
+        dy = bf16_from_bits(dy_bits, device)
+        wq1 = ops.to_mx_dim1_batched(w, "rceil", L)
+        dx = ops.mx_grouped_gemm_2d3d(ops.to_mx_dim0(dy, "rceil", L), wq1, offs)
+        ref = mo.grouped_dgrad(dy_bits, w_bits, np.cumsum(sizes), mo.RCEIL)
+        assert rel_l2(_f32(bits_of(dx)), _f32(ref)) <= TOL
+
+
+@pytest.mark.parametrize("sizes,N,K", FAST_CASES)
+def test_grouped_wgrad_aligned_groups(device, sizes, N, K):
+    """2D x 2D through the persistent kernel: token groups end at multiples of 128."""
+    rng = np.random.default_rng(sum(sizes) * 5 + N + K)
+    T = sum(sizes) + 128
+    x_bits = randn_bits(rng, (T, K), outliers=1e-3)
+    dy_bits = randn_bits(rng, (T, N), std=1e-3)
+    offs = _sizes_to_offs(sizes, device)
+    x, dy = bf16_from_bits(x_bits, device), bf16_from_bits(dy_bits, device)
+    for mode_name, mode in (("floor", mo.FLOOR), ("rceil", mo.RCEIL)):
+        dw = ops.mx_grouped_gemm_2d2d(ops.to_mx_dim1(dy, mode_name, L), ops.to_mx_dim1(x, mode_name, L), offs)
+        ref = mo.grouped_wgrad(dy_bits, x_bits, np.cumsum(sizes), mode)
+        got = bits_of(dw)
+        for g, s_ in enumerate(sizes):
+            if s_ == 0:
+                assert np.all(got[g] == 0)
+            else:
+                assert rel_l2(_f32(got[g]), _f32(ref[g])) <= TOL, g
+
+
+def test_aligned_group_forms_poison_the_output_when_a_group_end_is_not_a_multiple_of_128(device):
+    rng = np.random.default_rng(5)
+    sizes, N, K = [128, 160, 96], 128, 128
+    T = sum(sizes)
+    x = bf16_from_bits(randn_bits(rng, (T, K)), device)
+    w = bf16_from_bits(randn_bits(rng, (len(sizes), N, K), std=0.02), device)
+    offs = _sizes_to_offs(sizes, device)
+    y = ops.mx_grouped_gemm_2d3d(ops.to_mx_dim0(x, "rceil", L), ops.to_mx_dim0_batched(w, "rceil", L), offs)
+    assert torch.isnan(y).all()
+    dy = bf16_from_bits(randn_bits(rng, (T, N), std=1e-3), device)
+    dw = ops.mx_grouped_gemm_2d2d(ops.to_mx_dim1(dy, "rceil", L), ops.to_mx_dim1(x, "rceil", L), offs)
+    assert torch.isnan(dw).all()
+
+
 def test_batched_weight_casts_match_per_matrix(device):
     rng = np.random.default_rng(11)
     w_bits = randn_bits(rng, (5, 96, 160), std=0.02, outliers=1e-3)

@@ -32,14 +32,34 @@ constexpr int kCodes32 = 2 * kOperand32;         // A rows then B rows
 constexpr int kBlock32 = kCodes32 + 2048;        // + scales: 4 groups (A0, A1, B0, B1) x 2 steps x 256 B
 constexpr int kRing32 = 2 * kBlock32;            // 132 KB
 
-struct Dense32Args {
+// What a launch works on.  One kernel serves three problems that differ only in how a linear
+// tile number maps to operand rows, K range and output address:
+//   kDense        D[M,N] = A[M,K] B[N,K]^T
+//   kGrouped2d3d  rows of A in groups (inclusive ends offs[g], all multiples of 128), group g
+//                 against B[g][N,K]; rows from offs[G-1] to M are written as zeros
+//   kGrouped2d2d  D[g][M,N] = A[M, lo_g:hi_g] B[N, lo_g:hi_g]^T, K = row length of A and B
+enum Gemm32Mode { kDense = 0, kGrouped2d3d = 1, kGrouped2d2d = 2 };
+struct Gemm32Args {
   const uint8_t* a_codes;
   const uint8_t* a_scales;
   const uint8_t* b_codes;
   const uint8_t* b_scales;
   uint16_t* d;
   int64_t M, N, K, ldd;
+  const int32_t* offs;  // grouped modes: inclusive cumulative group sizes, on the device
+  int64_t G;
   uint64_t* prof;  // timing build only: per wave {vmcnt wait, barrier wait, step body} cycles
+};
+
+// Where one 256x256 tile lives.
+struct Tile32 {
+  const uint8_t *a, *b;    // first operand row of the tile, at the first K byte of its range
+  const uint8_t *sa, *sb;  // scales of the tile's first 128-row group at its first 64-deep step
+  uint16_t* d;
+  int64_t rows_a, rows_b;  // valid rows from the tile's origin (may exceed 256; <= 0: none)
+  uint32_t koff;           // first K byte of the range inside an operand row (kGrouped2d2d)
+  uint32_t nblocks;        // 128-deep K blocks (0: the tile is written as zeros)
+  bool poison;             // grouped modes: the group ends break the alignment contract
 };
 
 // Tile order: 8-tall column-major panels, so tiles that run together share A and B panels.
@@ -72,25 +92,96 @@ __device__ __forceinline__ v4i pin(v4i v) {
   return v;
 }
 
+// One scaled MFMA, C = 0 (FIRST) or accumulate.  Written as assembly: left as builtins, the
+// compiler gathers all 32 MFMAs of a tile's first block behind the block's copies, reads and
+// barriers instead of leaving them interleaved.  op_sel / op_sel_hi pick the scale byte of
+// the lane's scale dword: N for the first operand, M for the second.
+template <int N, int M, bool FIRST>
+__device__ __forceinline__ void mfma_asm(v16f& c, const v8i& b, const v8i& a, uint32_t sb,
+                                         uint32_t sa) {
+  if constexpr (FIRST)
+    asm volatile(
+        "v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, 0, %3, %4 op_sel:[%5,%6,0] op_sel_hi:[%7,%8,0]"
+        : "=a"(c)
+        : "v"(b), "v"(a), "v"(sb), "v"(sa), "n"(N & 1), "n"(M & 1), "n"(N >> 1), "n"(M >> 1));
+  else
+    asm volatile(
+        "v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[%5,%6,0] op_sel_hi:[%7,%8,0]"
+        : "+a"(c)
+        : "v"(b), "v"(a), "v"(sb), "v"(sa), "n"(N & 1), "n"(M & 1), "n"(N >> 1), "n"(M >> 1));
+}
+
 struct Frags32 {
   v8i a[4];
   v8i b[4];
   uint32_t sa, sb;
 };
 
-template <bool PROF>
-__global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
+template <int MODE, bool PROF>
+__global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
   const int li = lane & 31, lj = lane >> 5;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void_t*)smem;  // LDS byte address of the ring
+  const uint32_t K = (uint32_t)p.K;  // bytes per operand row; a multiple of 128 for this kernel
+  const uint32_t ks_n = K / kK32;    // 64-deep steps per 128-row scale group
+  const uint32_t tiles_n = (uint32_t)((p.N + kT32 - 1) / kT32);
+  const uint32_t G = (uint32_t)p.G;
+
+  // ---- tile count.  kGrouped2d3d: group g has ceil(rows_g / 256) x tiles_n tiles; the first
+  //      tile number of every group (G + 2 entries, the last group being the zero rows behind
+  //      offs[G-1]) is kept in the 2.5 KB that wave 0's output patch leaves unused.
+  const uint32_t lds_first = lds_base + kRing32 + 4608;
+  bool poison = false;
+  uint32_t nb;
+  // "any thread saw a bad group end", through a word of wave 1's spare patch bytes (the
+  // kernel's whole 160 KB are dynamic LDS: a library reduction would ask for more)
+  auto any_bad = [&](int bad) -> bool {
+    uint32_t* flag = reinterpret_cast<uint32_t*>(smem + kRing32 + 7168 + 4608);
+    if (tid == 0) *flag = 0;
+    __syncthreads();
+    if (bad) atomicOr(flag, 1u);
+    __syncthreads();
+    return *flag != 0;
+  };
+  if constexpr (MODE == kDense) {
+    nb = (uint32_t)((p.M + kT32 - 1) / kT32) * tiles_n;
+  } else if constexpr (MODE == kGrouped2d2d) {
+    nb = G * (uint32_t)((p.M + kT32 - 1) / kT32) * tiles_n;
+    int bad = 0;
+    for (uint32_t g = tid; g < G; g += 256) {
+      const int32_t hi = p.offs[g], lo = g ? p.offs[g - 1] : 0;
+      bad |= (hi & 127) | (hi < lo) | (hi > (int64_t)K) | (lo < 0);
+    }
+    poison = any_bad(bad);
+  } else {
+    uint32_t* first = reinterpret_cast<uint32_t*>(smem + kRing32 + 4608);
+    int bad = 0;
+    for (uint32_t g = tid; g <= G; g += 256) {
+      const int64_t lo = g ? p.offs[g - 1] : 0, hi = g < G ? (int64_t)p.offs[g] : p.M;
+      bad |= (g < G && (hi & 127)) | (hi < lo) | (hi > p.M) | (lo < 0);
+      const int64_t rows = hi > lo ? hi - lo : 0;
+      first[g + 1] = (uint32_t)((rows + kT32 - 1) / kT32) * tiles_n;
+    }
+    poison = any_bad(bad);
+    if (tid == 0) {
+      uint32_t acc_t = 0;
+      first[0] = 0;
+      for (uint32_t g = 1; g <= G + 1; ++g) {
+        acc_t += first[g];
+        first[g] = acc_t;
+      }
+    }
+    __syncthreads();
+    nb = first[G + 1];
+    if (poison) nb = (uint32_t)((p.M + kT32 - 1) / kT32) * tiles_n;  // then: NaN over all of D
+  }
 
   // ---- this workgroup's tile list: XCD x (= blockIdx % 8) owns one contiguous run of tiles,
   //      its workgroups take them round-robin, so the XCD's CUs work on neighbouring tiles
-  const uint32_t tiles_m = (uint32_t)((p.M + kT32 - 1) / kT32), tiles_n = (uint32_t)((p.N + kT32 - 1) / kT32);
-  const uint32_t nb = tiles_m * tiles_n;
   const uint32_t wgs_per_xcd = gridDim.x / 8;
   const uint32_t xcd = blockIdx.x % 8, idx = blockIdx.x / 8;
   const uint32_t per_xcd = (nb + 7) / 8;
@@ -98,9 +189,64 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
   const uint32_t t_hi = (xcd + 1) * per_xcd < nb ? (xcd + 1) * per_xcd : nb;
   const uint32_t n_my = t_lo < t_hi ? (t_hi - t_lo + wgs_per_xcd - 1) / wgs_per_xcd : 0;
   if (n_my == 0) return;
-  const uint32_t K = (uint32_t)p.K;          // a multiple of 128 for this kernel
-  const uint32_t nblocks = K / kKB;          // 128-deep ring blocks per tile, >= 1
-  const uint32_t ks_n = K / kK32;            // 64-deep steps per 128-row scale group
+
+  // first tile number of group g (kGrouped2d3d), read so that the compiler's wait-count
+  // model does not see an LDS read (see read_piece)
+  auto group_first = [&](uint32_t g) -> uint32_t {
+    uint32_t v;
+    const uint32_t addr = lds_first + g * 4;
+    asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(addr) : "memory");
+    return __builtin_amdgcn_readfirstlane(v);
+  };
+  // Tile number -> operands.  `g` is the caller's cursor into the groups: a stream visits
+  // tiles in increasing order, so the group is found by walking forward from the last one.
+  auto describe = [&](uint32_t t, uint32_t& g) -> Tile32 {
+    Tile32 r;
+    r.poison = poison;
+    r.koff = 0;
+    uint32_t tm, tn;
+    if (MODE == kDense || (MODE == kGrouped2d3d && poison)) {
+      tile_coords(t, (uint32_t)((p.M + kT32 - 1) / kT32), tiles_n, tm, tn);
+      r.a = p.a_codes + (int64_t)tm * kT32 * K;
+      r.b = p.b_codes + (int64_t)tn * kT32 * K;
+      r.sa = p.a_scales + (int64_t)(tm * 2) * ks_n * 256;
+      r.sb = p.b_scales + (int64_t)(tn * 2) * ks_n * 256;
+      r.d = p.d + (int64_t)tm * kT32 * p.ldd + (int64_t)tn * kT32;
+      r.rows_a = p.M - (int64_t)tm * kT32;
+      r.rows_b = p.N - (int64_t)tn * kT32;
+      r.nblocks = poison ? 0 : K / kKB;
+    } else if (MODE == kGrouped2d3d) {
+      while (t >= group_first(g + 1)) ++g;
+      const int64_t lo = g ? p.offs[g - 1] : 0, hi = g < G ? (int64_t)p.offs[g] : p.M;
+      const uint32_t tiles_mg = (uint32_t)((hi - lo + kT32 - 1) / kT32);
+      tile_coords(t - group_first(g), tiles_mg, tiles_n, tm, tn);
+      const int64_t row0 = lo + (int64_t)tm * kT32;
+      const uint32_t gb = g < G ? g : 0;  // the zero rows have no expert: any valid address
+      r.a = p.a_codes + row0 * K;
+      r.b = p.b_codes + ((int64_t)gb * p.N + (int64_t)tn * kT32) * K;
+      r.sa = p.a_scales + (row0 >> 7) * ks_n * 256;
+      r.sb = p.b_scales + ((int64_t)gb * ((p.N + 127) >> 7) + tn * 2) * ks_n * 256;
+      r.d = p.d + row0 * p.ldd + (int64_t)tn * kT32;
+      r.rows_a = hi - row0;
+      r.rows_b = p.N - (int64_t)tn * kT32;
+      r.nblocks = g < G ? K / kKB : 0;
+    } else {
+      const uint32_t tiles_m = (uint32_t)((p.M + kT32 - 1) / kT32), per_g = tiles_m * tiles_n;
+      g = t / per_g;
+      tile_coords(t - g * per_g, tiles_m, tiles_n, tm, tn);
+      const int64_t lo = poison ? 0 : (g ? p.offs[g - 1] : 0), hi = poison ? 0 : p.offs[g];
+      r.a = p.a_codes + (int64_t)tm * kT32 * K + lo;
+      r.b = p.b_codes + (int64_t)tn * kT32 * K + lo;
+      r.sa = p.a_scales + ((int64_t)(tm * 2) * ks_n + (lo >> 6)) * 256;
+      r.sb = p.b_scales + ((int64_t)(tn * 2) * ks_n + (lo >> 6)) * 256;
+      r.d = p.d + ((int64_t)g * p.M + (int64_t)tm * kT32) * p.ldd + (int64_t)tn * kT32;
+      r.rows_a = p.M - (int64_t)tm * kT32;
+      r.rows_b = p.N - (int64_t)tn * kT32;
+      r.koff = (uint32_t)lo;
+      r.nblocks = (uint32_t)((hi - lo) >> 7);
+    }
+    return r;
+  };
 
   // ---- per-lane constants
   // global -> LDS: a load unit is 8 rows x 128 B; lane l fetches row l/8 and the logical 16-byte
@@ -118,26 +264,32 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
   const uint32_t fb_delta = kOperand32 + (wn - wm) * 128 * kKB;
   const uint32_t lane4 = lane * 4;
   const uint32_t fsa_s = kCodes32 + wm * 512, fsb_s = kCodes32 + 1024 + wn * 512;
-  const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void_t*)smem;  // LDS byte address of the ring
 
   // ---- loader stream: fills ring block `ld_slot` with K block `ld_kb` of tile `ld_tile`
-  uint32_t ld_tile = 0, ld_kb = 0;
+  uint32_t ld_tile = 0, ld_kb = 0, ld_nb = 1, ld_g = 0;
   int ld_slot = 0;
   __amdgpu_buffer_rsrc_t ra, rb, rs;  // codes of A, codes of B, scales this wave copies
   auto loader_open_tile = [&]() {
+    Tile32 t;
+    t.nblocks = 0;
+    while (ld_tile < n_my) {  // tiles without K blocks add nothing to the stream
+      t = describe(t_lo + ld_tile * wgs_per_xcd, ld_g);
+      if (MODE == kDense || t.nblocks) break;
+      ++ld_tile;
+    }
     if (ld_tile < n_my) {
-      uint32_t tm, tn;
-      tile_coords(t_lo + ld_tile * wgs_per_xcd, tiles_m, tiles_n, tm, tn);
-      const int64_t rows_a = p.M - (int64_t)tm * kT32, rows_b = p.N - (int64_t)tn * kT32;
-      ra = make_rsrc(p.a_codes + (int64_t)tm * kT32 * K, rows_a * K);
-      rb = make_rsrc(p.b_codes + (int64_t)tn * kT32 * K, rows_b * K);
+      ld_nb = t.nblocks;
+      // (kGrouped2d2d: the range stops at the end of the operand rows, not of the K range;
+      //  the K range is exact because nblocks is)
+      ra = make_rsrc(t.a, t.rows_a * K - t.koff);
+      rb = make_rsrc(t.b, t.rows_b * K - t.koff);
       // wave 0,1 copy A's two 128-row scale groups, wave 2,3 copy B's
-      const int64_t rows = wave < 2 ? rows_a : rows_b;
-      const uint8_t* sbase = wave < 2 ? p.a_scales + (int64_t)(tm * 2 + wave) * ks_n * 256
-                                      : p.b_scales + (int64_t)(tn * 2 + wave - 2) * ks_n * 256;
+      const int64_t rows = wave < 2 ? t.rows_a : t.rows_b;
+      const uint8_t* sbase = (wave < 2 ? t.sa : t.sb) + (int64_t)(wave & 1) * ks_n * 256;
       const int64_t groups_left = ((rows + 127) >> 7) - (wave & 1);
-      rs = make_rsrc(sbase, groups_left > 0 ? (int64_t)ks_n * 256 : 0);
+      rs = make_rsrc(sbase, groups_left > 0 ? (int64_t)ld_nb * 512 : 0);
     } else {  // past the last tile: every lane reads out of range (zeros, no traffic)
+      ld_nb = 1;
       ra = make_rsrc(p.a_codes, 0);
       rb = ra;
       rs = ra;
@@ -167,7 +319,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
     }
   };
   auto issue_advance = [&]() {
-    if (++ld_kb == nblocks) {
+    if (++ld_kb == ld_nb) {
       ld_kb = 0;
       ++ld_tile;
       loader_open_tile();
@@ -234,14 +386,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
   auto mfma_one = [&](const Frags32& f, auto first_, auto i_) {
     constexpr bool kFirst = decltype(first_)::value;  // first step of a tile starts from zero
     constexpr int n = decltype(i_)::value >> 2, m = decltype(i_)::value & 3;
-    if constexpr (kFirst) {
-      acc[m][n] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-          f.b[n], f.a[m], v16f{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, 0, 0, n, (int)f.sb,
-          m, (int)f.sa);
-    } else {
-      acc[m][n] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.b[n], f.a[m], acc[m][n], 0, 0, n,
-                                                                  (int)f.sb, m, (int)f.sa);
-    }
+    mfma_asm<n, m, kFirst>(acc[m][n], f.b[n], f.a[m], f.sb, f.sa);
   };
 
   // A K block is two steps of 16 MFMAs.  Entering step A of block b, f0 holds the fragments of
@@ -337,7 +482,6 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
         constexpr bool skip = kSkipB && (i % kSkipB) == kSkipB - 1;
         if constexpr (!skip && kCopiesA + j < 18) issue_piece(std::integral_constant<int, kCopiesA + j>{});
 #endif
-        if constexpr (i == 15) issue_advance();
 #ifndef MX_ABL_NO_READ
         if constexpr (i < kReadSlots) {
           read_piece(f0, sbase, std::integral_constant<int, 0>{}, std::integral_constant<int, 2 * i>{});
@@ -348,6 +492,12 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
       });
       c_slot ^= 1;
     }
+    // the fragments read in this step become ordinary values before the loader may open a
+    // new tile (a register the compiler moved or spilled while its read was still in
+    // flight would lose the data)
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    pin_frags(f0);
+    issue_advance();
   };
 
   // Output: a lane holds, per 32x32 sub-tile, row li and columns 8q + 4lj + 0..3.  The two
@@ -362,14 +512,12 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
   const uint32_t patch = lds_base + kRing32 + wave * 7168;
   const uint32_t patch_w = patch + li * kPatchPitch + lj * 16;                 // + (n&1)*64 + h*32
   const uint32_t patch_r = patch + (lane >> 3) * kPatchPitch + (lane & 7) * 16;  // + pass*8 rows
-  auto epilogue = [&](uint32_t tile) {
-    uint32_t tm, tn;
-    tile_coords(t_lo + tile * wgs_per_xcd, tiles_m, tiles_n, tm, tn);
-    const int64_t rows_valid = p.M - (int64_t)tm * kT32;
-    const uint32_t cols_valid = (uint32_t)(p.N - (int64_t)tn * kT32);
+  uint32_t ep_g = 0;
+  auto epilogue = [&](const Tile32& t) {
+    const int64_t rows_valid = t.rows_a;
+    const uint32_t cols_valid = (uint32_t)(t.rows_b < kT32 ? t.rows_b : kT32);
     const uint32_t ldd_b = (uint32_t)p.ldd * 2;
-    const __amdgpu_buffer_rsrc_t rd =
-        make_rsrc(p.d + (int64_t)tm * kT32 * p.ldd + (int64_t)tn * kT32, rows_valid * ldd_b);
+    const __amdgpu_buffer_rsrc_t rd = make_rsrc(t.d, rows_valid * ldd_b);
     // lane's place in a stored piece: row (lane >> 3) + 8*pass, columns (lane & 7)*8 .. +7
     const uint32_t colp = wn * 128 + (lane & 7) * 8;
     const uint32_t vrow = (wm * 128 + (lane >> 3)) * ldd_b + colp * 2;
@@ -437,22 +585,49 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
   issue_block();  // block 1: in flight when the first step starts
   Frags32 f0, f1;
   read_frags(f0, 0, std::integral_constant<int, 0>{});
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  pin_frags(f0);
   if constexpr (PROF) prof_last = __builtin_readcyclecounter();
 
   // ---- tiles; at the top of every tile f0 holds the fragments of its first half block (the
   // last step of a tile has already read them from the next tile's first block, which the
   // loader fetched like any other block).
   for (uint32_t tile = 0; tile < n_my; ++tile) {
-    block_steps(f0, f1, std::true_type{});
-    for (uint32_t i = 1; i < nblocks; ++i) block_steps(f0, f1, std::false_type{});
-    if constexpr (PROF) {
-      const uint64_t e0 = __builtin_readcyclecounter();
-      prof_body += e0 - prof_last;
-      epilogue(tile);
-      prof_last = __builtin_readcyclecounter();
-      prof_epi += prof_last - e0;
+    const Tile32 t = describe(t_lo + tile * wgs_per_xcd, ep_g);
+    if (MODE == kDense || t.nblocks) {
+      block_steps(f0, f1, std::true_type{});
+      for (uint32_t i = 1; i < t.nblocks; ++i) block_steps(f0, f1, std::false_type{});
+      // the next tile's first fragments were read in the last step: make them ordinary
+      // values before anything else runs (a register the compiler moved or spilled while
+      // its read was still in flight would lose the data)
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      pin_frags(f0);
+      if constexpr (PROF) {
+        const uint64_t e0 = __builtin_readcyclecounter();
+        prof_body += e0 - prof_last;
+        epilogue(t);
+        prof_last = __builtin_readcyclecounter();
+        prof_epi += prof_last - e0;
+      } else {
+        epilogue(t);
+      }
     } else {
-      epilogue(tile);
+      // no K blocks: zeros (an empty group, the rows behind the last group), or NaN when the
+      // group ends break the contract, so that the mistake cannot pass unnoticed.  Written
+      // straight from registers: wave (wm, wn) owns rows 128 wm.., columns 128 wn..
+      const uint32_t fill = t.poison ? 0x7FC07FC0u : 0u;
+      const u32x4 w = {fill, fill, fill, fill};
+      const uint32_t ldd_b = (uint32_t)p.ldd * 2;
+      const __amdgpu_buffer_rsrc_t rd = make_rsrc(t.d, t.rows_a * ldd_b);
+      const uint32_t cols_valid = (uint32_t)(t.rows_b < kT32 ? t.rows_b : kT32);
+      const uint32_t colp = wn * 128 + (lane & 7) * 8;
+      const uint32_t vrow = (wm * 128 + (lane >> 3)) * ldd_b + colp * 2;
+      for (uint32_t r8 = 0; r8 < 16; ++r8) {
+        const uint32_t v0 = colp < cols_valid ? vrow : 0x80000000u;
+        const uint32_t v1 = colp + 64 < cols_valid ? vrow + 128 : 0x80000000u;
+        __builtin_amdgcn_raw_buffer_store_b128(w, rd, v0, r8 * 8 * ldd_b, 0);
+        __builtin_amdgcn_raw_buffer_store_b128(w, rd, v1, r8 * 8 * ldd_b, 0);
+      }
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the over-issued prefetches before retiring
@@ -473,9 +648,9 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Dense32Args p) {
 static int debug_grid = 0;
 static uint64_t* debug_prof = nullptr;  // > 0: number of persistent workgroups (experiments only)
 
-template <bool PROF>
-static int launch_dense32(const Dense32Args& p, hipStream_t st) {
-  auto kern = gemm_nt32_kernel<PROF>;
+template <int MODE, bool PROF>
+static int launch32(const Gemm32Args& p, int64_t nb, hipStream_t st) {
+  auto kern = gemm_nt32_kernel<MODE, PROF>;
   constexpr int lds = kRing32 + 4 * 7168;  // ring + one output patch per wave = all 160 KB
   static int num_cus = 0;
   if (num_cus == 0) {
@@ -488,10 +663,9 @@ static int launch_dense32(const Dense32Args& p, hipStream_t st) {
       return MX_ERR_LAUNCH;
     num_cus = n;
   }
-  const int64_t nb = ((p.M + kT32 - 1) / kT32) * ((p.N + kT32 - 1) / kT32);
   int64_t grid = (num_cus / 8) * 8;  // one persistent workgroup per CU, a multiple of the 8 XCDs
   if (grid < 8) grid = 8;
-  const int64_t need = (nb + 7) / 8 * 8;
+  const int64_t need = (nb + 7) / 8 * 8;  // nb: the tile count, or an upper bound of it
   if (need < grid) grid = need;
   if (debug_grid > 0) grid = (debug_grid + 7) / 8 * 8;
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, st, p);
@@ -504,9 +678,29 @@ void set_debug_prof(uint64_t* buf) { debug_prof = buf; }
 int launch_gemm_nt32(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                      const uint8_t* b_scales, void* d, int64_t M, int64_t N, int64_t K,
                      int64_t ldd, hipStream_t st) {
-  Dense32Args p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, M, N, K, ldd, debug_prof};
-  if (debug_prof) return launch_dense32<true>(p, st);
-  return launch_dense32<false>(p, st);
+  Gemm32Args p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, M, N, K, ldd, nullptr, 0, debug_prof};
+  const int64_t nb = ((M + kT32 - 1) / kT32) * ((N + kT32 - 1) / kT32);
+  if (debug_prof) return launch32<kDense, true>(p, nb, st);
+  return launch32<kDense, false>(p, nb, st);
+}
+
+// Grouped forms with every group end a multiple of 128 and all scales in MFMA order
+// (a_scales over the whole [T, K/32] matrix, b_scales one block per expert).
+int launch_grouped32_2d3d(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                          const uint8_t* b_scales, const int32_t* offs, void* d, int64_t T,
+                          int64_t N, int64_t K, int64_t G, int64_t ldd, hipStream_t st) {
+  Gemm32Args p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, T, N, K, ldd, offs, G, nullptr};
+  const int64_t nb = ((T + kT32 - 1) / kT32 + G + 1) * ((N + kT32 - 1) / kT32);
+  return launch32<kGrouped2d3d, false>(p, nb, st);
+}
+
+// D[g][N, K] = A^T[N, lo:hi] B^T[K, lo:hi]^T; operand rows are T long.
+int launch_grouped32_2d2d(const uint8_t* at_codes, const uint8_t* at_scales,
+                          const uint8_t* bt_codes, const uint8_t* bt_scales, const int32_t* offs,
+                          void* d, int64_t T, int64_t N, int64_t K, int64_t G, hipStream_t st) {
+  Gemm32Args p{at_codes, at_scales, bt_codes, bt_scales, (uint16_t*)d, N, K, T, K, offs, G, nullptr};
+  const int64_t nb = G * ((N + kT32 - 1) / kT32) * ((K + kT32 - 1) / kT32);
+  return launch32<kGrouped2d2d, false>(p, nb, st);
 }
 
 }  // namespace mx

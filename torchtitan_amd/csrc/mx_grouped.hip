@@ -123,19 +123,39 @@ static int launch_2d2d(const G2d2dArgs& p, hipStream_t st) {
 
 using namespace mx;
 
+namespace mx {
+int launch_grouped32_2d3d(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                          const uint8_t* b_scales, const int32_t* offs, void* d, int64_t T,
+                          int64_t N, int64_t K, int64_t G, int64_t ldd, hipStream_t st);
+int launch_grouped32_2d2d(const uint8_t* at_codes, const uint8_t* at_scales,
+                          const uint8_t* bt_codes, const uint8_t* bt_scales, const int32_t* offs,
+                          void* d, int64_t T, int64_t N, int64_t K, int64_t G, hipStream_t st);
+}  // namespace mx
+
 extern "C" int mx_grouped_gemm_2d3d(const uint8_t* a_codes, const uint8_t* a_scales,
                                     const uint8_t* b_codes, const uint8_t* b_scales,
                                     const int32_t* offs, void* d, int64_t T, int64_t N, int64_t K,
-                                    int64_t G, int64_t ldd, void* stream) {
+                                    int64_t G, int64_t ldd, int a_scale_order, void* stream) {
   if (T < 0 || N < 0 || K < 0 || G <= 0 || ldd < N) return MX_ERR_INVALID_ARG;
+  if (a_scale_order != MX_SCALES_ROWMAJOR && a_scale_order != MX_SCALES_MFMA)
+    return MX_ERR_INVALID_ARG;
   if (T == 0 || N == 0) return MX_OK;
   if (!a_codes || !a_scales || !b_codes || !b_scales || !offs || !d) return MX_ERR_INVALID_ARG;
   if (K == 0 || K % 32) return MX_ERR_ALIGNMENT;
   if (((uintptr_t)a_codes & 15) || ((uintptr_t)b_codes & 15) || ((uintptr_t)b_scales & 3))
     return MX_ERR_ALIGNMENT;
   if (256 * K > 0x7FFFFFFFll) return MX_ERR_UNSUPPORTED;
-  G2d3dArgs p{a_codes, a_scales, b_codes, b_scales, offs, (uint16_t*)d, T, N, K, G, ldd, 0};
   hipStream_t st = (hipStream_t)stream;
+  if (a_scale_order == MX_SCALES_MFMA) {
+    // group ends at multiples of 128 (checked on the device): the persistent 32x32x64 kernel
+    if (K % 128 || N % 8 || ldd % 8 || ((uintptr_t)d & 15) || ((uintptr_t)a_scales & 3) ||
+        T % 128)
+      return MX_ERR_ALIGNMENT;
+    if (G > 638 || ldd * 512 > 0x7FFFFFFFll) return MX_ERR_UNSUPPORTED;
+    return launch_grouped32_2d3d(a_codes, a_scales, b_codes, b_scales, offs, d, T, N, K, G, ldd,
+                                 st);
+  }
+  G2d3dArgs p{a_codes, a_scales, b_codes, b_scales, offs, (uint16_t*)d, T, N, K, G, ldd, 0};
   if (T / G < 192 || N <= 128) return launch_2d3d<128, 128>(p, st);
   return launch_2d3d<256, 256>(p, st);
 }
@@ -143,8 +163,10 @@ extern "C" int mx_grouped_gemm_2d3d(const uint8_t* a_codes, const uint8_t* a_sca
 extern "C" int mx_grouped_gemm_2d2d(const uint8_t* at_codes, const uint8_t* at_scales,
                                     const uint8_t* bt_codes, const uint8_t* bt_scales,
                                     const int32_t* offs, void* d, int64_t T, int64_t N, int64_t K,
-                                    int64_t G, void* stream) {
+                                    int64_t G, int scale_order, void* stream) {
   if (T < 0 || N < 0 || K < 0 || G <= 0) return MX_ERR_INVALID_ARG;
+  if (scale_order != MX_SCALES_ROWMAJOR && scale_order != MX_SCALES_MFMA)
+    return MX_ERR_INVALID_ARG;
   if (N == 0 || K == 0) return MX_OK;
   if (!d || !offs) return MX_ERR_INVALID_ARG;
   if (T % 32) return MX_ERR_ALIGNMENT;
@@ -152,8 +174,16 @@ extern "C" int mx_grouped_gemm_2d2d(const uint8_t* at_codes, const uint8_t* at_s
   if (((uintptr_t)at_codes & 15) || ((uintptr_t)bt_codes & 15) || (T % 16))
     return MX_ERR_ALIGNMENT;
   if (256 * T > 0x7FFFFFFFll) return MX_ERR_UNSUPPORTED;
-  G2d2dArgs p{at_codes, at_scales, bt_codes, bt_scales, offs, (uint16_t*)d, T, N, K, G};
   hipStream_t st = (hipStream_t)stream;
+  if (scale_order == MX_SCALES_MFMA) {
+    if (T % 128 || K % 8 || ((uintptr_t)d & 15) || ((uintptr_t)at_scales & 3) ||
+        ((uintptr_t)bt_scales & 3))
+      return MX_ERR_ALIGNMENT;
+    if (K * 512 > 0x7FFFFFFFll) return MX_ERR_UNSUPPORTED;
+    if (T == 0) return MX_ERR_UNSUPPORTED;  // nothing to contract: the general kernel writes the zeros
+    return launch_grouped32_2d2d(at_codes, at_scales, bt_codes, bt_scales, offs, d, T, N, K, G, st);
+  }
+  G2d2dArgs p{at_codes, at_scales, bt_codes, bt_scales, offs, (uint16_t*)d, T, N, K, G};
   if (N <= 128 || K <= 128) return launch_2d2d<128, 128>(p, st);
   return launch_2d2d<256, 256>(p, st);
 }

@@ -195,17 +195,17 @@ def mx_linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, 
 
 
 # ----------------------------------------------------------------------------- grouped GEMM
-def _pad_plan(offs: torch.Tensor, T: int):
-    """Device-side plan that moves rows of variable-size groups into 32-aligned groups.
+def _pad_plan(offs: torch.Tensor, T: int, align: int = 32):
+    """Device-side plan that moves rows of variable-size groups into `align`-aligned groups.
 
     Returns (gather indices into [x; 0-row] for the padded layout, padded inclusive offsets,
     for every original row its row in the padded layout or the index of an appended zero row).
-    No host synchronisation: the padded length is the static bound round_up(T + 32 G, 32).
+    No host synchronisation: the padded length is the static bound round_up(T + align G, align).
     """
     G = offs.numel()
     sizes = torch.diff(offs, prepend=offs.new_zeros(1))
-    max_len = -(-(T + ops.BLOCK * G) // ops.BLOCK) * ops.BLOCK
-    perm, _, m_offsets = ops.group_offsets_pad(sizes, G, 1, max_len, ops.BLOCK)
+    max_len = -(-(T + align * G) // align) * align
+    perm, _, m_offsets = ops.group_offsets_pad(sizes, G, 1, max_len, align)
     back = torch.full((T + 1,), max_len, dtype=torch.int64, device=offs.device)
     back[perm] = torch.arange(max_len, device=offs.device)  # perm == -1 writes the spare slot T
     return perm, m_offsets, back[:T]
@@ -223,8 +223,12 @@ class _MXGroupedMM(torch.autograd.Function):
         w = weight if weight.dtype == torch.bfloat16 else weight.to(torch.bfloat16)
         w = w.contiguous()
         plan = None
+        # Padding to 128-row groups (instead of the 32 the format needs) lets all three GEMMs
+        # run on the persistent kernel, which wants whole 128-row scale groups per expert.
+        fast = (cfg.pad_token_groups_for_grouped_mm and K % 128 == 0 and N % 128 == 0 and G <= 638)
+        order = MX_SCALES_MFMA if fast else MX_SCALES_ROWMAJOR
         if cfg.pad_token_groups_for_grouped_mm:
-            plan = _pad_plan(offs, T)
+            plan = _pad_plan(offs, T, 128 if fast else ops.BLOCK)
             perm, offs_p, back = plan
             xb = torch.cat((xb, xb.new_zeros((1, K))), dim=0)[perm]
         else:
@@ -234,9 +238,9 @@ class _MXGroupedMM(torch.autograd.Function):
         xb = xb.contiguous()
         need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         if need_dw:
-            xq0, xq1 = ops.to_mx_dim0_dim1(xb, mode, MX_SCALES_ROWMAJOR)
+            xq0, xq1 = ops.to_mx_dim0_dim1(xb, mode, order)
         else:
-            xq0, xq1 = ops.to_mx_dim0(xb, mode, MX_SCALES_ROWMAJOR), None
+            xq0, xq1 = ops.to_mx_dim0(xb, mode, order), None
         if need_dx and N % ops.BLOCK == 0:
             wq0, wq1 = ops.to_mx_dim0_dim1_batched(w, mode, MX_SCALES_MFMA)
         else:
@@ -249,6 +253,7 @@ class _MXGroupedMM(torch.autograd.Function):
         ctx.dims = (T, K, N, G)
         ctx.dtypes = (x.dtype, weight.dtype)
         ctx.padded = plan is not None
+        ctx.order = order
         saved = [offs_p]
         if plan is not None:
             saved += [plan[0], plan[2]]
@@ -274,12 +279,12 @@ class _MXGroupedMM(torch.autograd.Function):
         dyb = dyb.contiguous()
         dx = dw = None
         if need_dw:
-            xq1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_ROWMAJOR)
+            xq1 = MXData(saved.pop(0), saved.pop(0), ctx.order)
         if need_dx and need_dw and N % ops.BLOCK == 0:
-            dyq0, dyq1 = ops.to_mx_dim0_dim1(dyb, mode, MX_SCALES_ROWMAJOR)
+            dyq0, dyq1 = ops.to_mx_dim0_dim1(dyb, mode, ctx.order)
         else:
-            dyq0 = ops.to_mx_dim0(dyb, mode, MX_SCALES_ROWMAJOR) if need_dx else None
-            dyq1 = ops.to_mx_dim1(dyb, mode, MX_SCALES_ROWMAJOR) if need_dw else None
+            dyq0 = ops.to_mx_dim0(dyb, mode, ctx.order) if need_dx else None
+            dyq1 = ops.to_mx_dim1(dyb, mode, ctx.order) if need_dw else None
         if need_dx:
             if ctx.have_wq1:
                 wq1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)

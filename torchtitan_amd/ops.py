@@ -244,20 +244,23 @@ def mx_grouped_gemm_2d3d(a: MXData, b: MXData, offs: torch.Tensor,
                          out: torch.Tensor | None = None) -> torch.Tensor:
     """out[rows of group g] = deq(a[rows of g]) @ deq(b[g])^T; rows past offs[-1] are zero.
 
-    a: codes [T, K] with row-major scales [T, K/32]; b: codes [G, N, K] with MFMA-order scales
-    (G per-matrix blocks); offs: int32 [G] inclusive cumulative group sizes on the device.
+    a: codes [T, K]; b: codes [G, N, K] with MFMA-order scales (G per-matrix blocks); offs:
+    int32 [G] inclusive cumulative group sizes on the device.  With row-major scales for a the
+    groups may end anywhere; with MFMA-order scales for a every group must end at a multiple
+    of 128 rows (checked on the device: a violation fills the output with NaN) and the
+    persistent 32x32x64 kernel runs.
     """
     T, K = a.codes.shape
     G, N, Kb = b.codes.shape
     if K != Kb:
         raise ValueError(f"contraction mismatch: {K} vs {Kb}")
-    if a.scale_order != MX_SCALES_ROWMAJOR or b.scale_order != MX_SCALES_MFMA:
-        raise ValueError("2d3d expects row-major scales for a and MFMA-order scales for b")
+    if b.scale_order != MX_SCALES_MFMA:
+        raise ValueError("2d3d expects MFMA-order scales for b")
     if offs.dtype != torch.int32 or offs.numel() != G:
         raise ValueError("offs must be int32 with one entry per group")
     if out is None:
         out = torch.empty((T, N), dtype=torch.bfloat16, device=a.codes.device)
-    _call("mx_grouped_gemm_2d3d", "grouped_gemm_2d3d", out.device, _ptr(a.codes), _ptr(a.scales), _ptr(b.codes), _ptr(b.scales), _ptr(offs), _ptr(out), T, N, K, G, out.stride(0), _stream(out))
+    _call("mx_grouped_gemm_2d3d", "grouped_gemm_2d3d", out.device, _ptr(a.codes), _ptr(a.scales), _ptr(b.codes), _ptr(b.scales), _ptr(offs), _ptr(out), T, N, K, G, out.stride(0), a.scale_order, _stream(out))
     return out
 
 
@@ -265,18 +268,21 @@ def mx_grouped_gemm_2d2d(at: MXData, bt: MXData, offs: torch.Tensor,
                          out: torch.Tensor | None = None) -> torch.Tensor:
     """out[g] = deq(at[:, tokens of g]) @ deq(bt[:, tokens of g])^T  ->  [G, N, K] bf16.
 
-    at: codes [N, T], bt: codes [K, T] (column-wise casts), both with row-major scales.
+    at: codes [N, T], bt: codes [K, T] (column-wise casts), scales of both in the same order.
+    Row-major: groups may be any multiple of 32.  MFMA order: every group must end at a
+    multiple of 128 tokens (checked on the device: a violation fills the output with NaN) and
+    the persistent 32x32x64 kernel runs.
     """
     N, T = at.codes.shape
     K, Tb = bt.codes.shape
     if T != Tb:
         raise ValueError(f"token count mismatch: {T} vs {Tb}")
-    if at.scale_order != MX_SCALES_ROWMAJOR or bt.scale_order != MX_SCALES_ROWMAJOR:
-        raise ValueError("2d2d expects row-major scales")
+    if at.scale_order != bt.scale_order:
+        raise ValueError("2d2d expects both scale buffers in the same order")
     G = offs.numel()
     if out is None:
         out = torch.empty((G, N, K), dtype=torch.bfloat16, device=at.codes.device)
-    _call("mx_grouped_gemm_2d2d", "grouped_gemm_2d2d", out.device, _ptr(at.codes), _ptr(at.scales), _ptr(bt.codes), _ptr(bt.scales), _ptr(offs), _ptr(out), T, N, K, G, _stream(out))
+    _call("mx_grouped_gemm_2d2d", "grouped_gemm_2d2d", out.device, _ptr(at.codes), _ptr(at.scales), _ptr(bt.codes), _ptr(bt.scales), _ptr(offs), _ptr(out), T, N, K, G, at.scale_order, _stream(out))
     return out
 
 
