@@ -422,6 +422,24 @@ __device__ __forceinline__ void quantize_patch(u32x4 (&v)[8], const uint32_t (&m
   }
 }
 
+// Tiles are walked in blocks of BX x BY tiles, down the rows first inside a block, so that
+// workgroups running together cover compact regions of the input and of the transposed
+// output.  Measured best: wide, flat blocks for the row-wise cast (long contiguous reads and
+// writes), narrow, tall ones as soon as the transposed output is written.
+#ifndef MX_CAST_ROW_BX
+#define MX_CAST_ROW_BX 32
+#define MX_CAST_ROW_BY 2
+#endif
+#ifndef MX_CAST_COL_BX
+#define MX_CAST_COL_BX 2
+#define MX_CAST_COL_BY 32
+#endif
+template <bool COL>
+struct TileWalk {
+  static constexpr uint32_t BX = COL ? MX_CAST_COL_BX : MX_CAST_ROW_BX;
+  static constexpr uint32_t BY = COL ? MX_CAST_COL_BY : MX_CAST_ROW_BY;
+};
+
 template <int MODE, int ORDER, bool ROW, bool COL, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void cast_tile_kernel(
     const uint16_t* __restrict__ x, int64_t rows, int64_t cols, int64_t ldx,
@@ -445,10 +463,11 @@ __global__ __launch_bounds__(64 * WAVES) void cast_tile_kernel(
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 4, q = lane & 15;
   const int rl0 = wave * 32 + 8 * g;  // first tile-local row of this lane
 
-  // Tiles are numbered so that workgroups running together cover compact regions of both
-  // the input and the transposed output: 8x8 blocks of tiles, walked down the rows first.
-  const uint32_t spr = (gx + 7) / 8, sup = blockIdx.x >> 6, in = blockIdx.x & 63;
-  const uint32_t bx = (sup % spr) * 8 + (in >> 3), by = (sup / spr) * 8 + (in & 7);
+  constexpr uint32_t BX = TileWalk<COL>::BX, BY = TileWalk<COL>::BY;
+  const uint32_t spr = (gx + BX - 1) / BX;
+  const uint32_t sup = blockIdx.x / (BX * BY), in = blockIdx.x % (BX * BY);
+  const uint32_t bx = (sup % spr) * BX + in / BY;
+  const uint32_t by = (sup / spr) * BY + in % BY;
   if (bx >= gx || by >= gy) return;
 
   const int64_t r0 = (int64_t)by * TR, c0 = (int64_t)bx * TC;
@@ -654,11 +673,13 @@ static inline bool tile_ok(const void* x, int64_t cols, int64_t ldx) {
   return ((uintptr_t)x & 15) == 0 && (ldx & 7) == 0 && (cols & 7) == 0;
 }
 constexpr int kTileRows = 32 * MX_CAST_WAVES;
-static inline int64_t tile_grid_x(int64_t gx, int64_t gy) {
-  return ((gx + 7) / 8) * ((gy + 7) / 8) * 64;
+static inline int64_t tile_grid_x(int64_t gx, int64_t gy, bool col) {
+  const int64_t bx = col ? TileWalk<true>::BX : TileWalk<false>::BX;
+  const int64_t by = col ? TileWalk<true>::BY : TileWalk<false>::BY;
+  return ((gx + bx - 1) / bx) * ((gy + by - 1) / by) * (bx * by);
 }
-static inline dim3 tile_grid(int64_t gx, int64_t gy, int64_t batch) {
-  return dim3((unsigned)tile_grid_x(gx, gy), 1, (unsigned)batch);
+static inline dim3 tile_grid(int64_t gx, int64_t gy, int64_t batch, bool col) {
+  return dim3((unsigned)tile_grid_x(gx, gy, col), 1, (unsigned)batch);
 }
 
 static inline bool bad_enums(int scale_mode, int scale_order) {
@@ -700,9 +721,9 @@ extern "C" int mx_cast_dim0(const void* x, int64_t rows, int64_t cols, int64_t l
   hipStream_t st = (hipStream_t)stream;
   if (scale_order == MX_SCALES_MFMA && ((uintptr_t)scales & 3)) return MX_ERR_ALIGNMENT;
   const int64_t tgx = (cols + kT - 1) / kT, tgy = (rows + kTileRows - 1) / kTileRows;
-  if (scale_order == MX_SCALES_MFMA && tile_grid_x(tgx, tgy) <= 0x7FFFFFFF) {
+  if (scale_order == MX_SCALES_MFMA && tile_grid_x(tgx, tgy, false) <= 0x7FFFFFFF) {
     // scattered scale bytes cost more than the tiled read: stage them through LDS
-    dim3 grid = tile_grid(tgx, tgy, 1), block(64 * MX_CAST_WAVES);
+    dim3 grid = tile_grid(tgx, tgy, 1, false), block(64 * MX_CAST_WAVES);
     MX_DISPATCH_TILE(true, false, (const uint16_t*)x, rows, cols, ldx, codes, scales, nblk, ks_n,
                      (uint8_t*)nullptr, (uint8_t*)nullptr, (int64_t)0, (int64_t)0, (int64_t)0,
                      (int64_t)0, (int64_t)0, (uint32_t)tgx, (uint32_t)tgy);
@@ -735,8 +756,8 @@ extern "C" int mx_cast_dim1_batched(const void* x, int64_t batch, int64_t rows, 
   if (gy > 65535 || batch > 65535 || gx > 0x7FFFFFFF) return MX_ERR_UNSUPPORTED;
   hipStream_t st = (hipStream_t)stream;
   const int64_t tgy = (rows + kTileRows - 1) / kTileRows;
-  if (tile_ok(x, cols, ldx) && tile_grid_x(gx, tgy) <= 0x7FFFFFFF) {
-    dim3 grid = tile_grid(gx, tgy, batch), block(64 * MX_CAST_WAVES);
+  if (tile_ok(x, cols, ldx) && tile_grid_x(gx, tgy, true) <= 0x7FFFFFFF) {
+    dim3 grid = tile_grid(gx, tgy, batch, true), block(64 * MX_CAST_WAVES);
     MX_DISPATCH_TILE(false, true, (const uint16_t*)x, rows, cols, ldx, (uint8_t*)nullptr,
                      (uint8_t*)nullptr, (int64_t)0, (int64_t)0, codes_t, scales_t, nblk_t, ks_n_t,
                      rows * ldx, (int64_t)0, st_b, (uint32_t)gx, (uint32_t)tgy);
@@ -776,8 +797,8 @@ extern "C" int mx_cast_dim0_dim1_batched(const void* x, int64_t batch, int64_t r
   if (scale_order == MX_SCALES_MFMA && ((uintptr_t)scales & 3)) return MX_ERR_ALIGNMENT;
   const int64_t tgy = (rows + kTileRows - 1) / kTileRows;
   if (tile_ok(x, cols, ldx) && ((uintptr_t)codes & 7) == 0 && ((uintptr_t)scales & 3) == 0 &&
-      tile_grid_x(gx, tgy) <= 0x7FFFFFFF) {
-    dim3 grid = tile_grid(gx, tgy, batch), block(64 * MX_CAST_WAVES);
+      tile_grid_x(gx, tgy, true) <= 0x7FFFFFFF) {
+    dim3 grid = tile_grid(gx, tgy, batch, true), block(64 * MX_CAST_WAVES);
     MX_DISPATCH_TILE(true, true, (const uint16_t*)x, rows, cols, ldx, codes, scales, nblk, ks_n,
                      codes_t, scales_t, nblk_t, ks_n_t, rows * ldx, s_b, st_b, (uint32_t)gx,
                      (uint32_t)tgy);
