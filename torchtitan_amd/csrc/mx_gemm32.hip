@@ -1,23 +1,30 @@
-// Dense MXFP8 GEMM for large shapes: persistent 256x256 tiles on v_mfma_scale_f32_32x32x64_f8f6f4.
+// MXFP8 GEMM for large shapes, dense and grouped: persistent 256x256 tiles on
+// v_mfma_scale_f32_32x32x64_f8f6f4.
 //
 //   D[M,N] (bf16) = deq(A)[M,K] * deq(B)[N,K]^T, fp32 accumulate.
 //
 // One workgroup (4 waves, 2x2, 128x128 each = 256 accumulator registers per lane) per CU walks
-// a list of output tiles; the K loop of all its tiles is one flat stream, so the loads of the
-// next tile's first steps are already in flight while a tile is written out.
+// a list of output tiles; the K loops of all its tiles form one flat stream of 128-deep
+// blocks, so the loads of the next tile's first blocks are already in flight while a tile is
+// written out.
 //
 // Global -> LDS moves whole 128-byte rows (buffer_load_dwordx4 ... lds, 8 rows per instruction:
 // full cache lines, which the texture path delivers about twice as fast as 64-byte pieces), so
-// the ring holds two 128-deep "blocks" of 64 KB codes + 2 KB scales.  Compute runs in 64-deep
+// the ring holds two 128-deep blocks of 64 KB codes + 2 KB scales.  Compute runs in 64-deep
 // steps (two per block): 16 MFMAs per wave per step (1024 MFMA cycles), fragments LDS -> VGPR
 // double-buffered in registers and read one step ahead, conflict-free under the b128 pass
-// grouping.  The block that was just consumed is refilled two steps before it is needed
-// again; one barrier per block.
+// grouping.  Two barriers per block: one in the middle of the first step releases the ring
+// block whose last fragments have just been read (its refill starts there, spread over 22
+// MFMA slots because the copy path is the scarce resource), one before the second step makes
+// sure the next block has landed.
 //
 // Operand layout of the 32x32x64 f8 MFMA (measured): lane (i = l & 31, j = l >> 5) holds row i,
 // K bytes [16j, 16j+16) in registers 0-3 and [32+16j, 32+16j+16) in registers 4-7; the scale
 // of 32-element block b is taken from lane group b.  With the first operand = B rows and the
 // second = A rows, a lane ends up with D[row = l & 31][col = 8q + 4j + 0..3], q = 0..3.
+//
+// MX_ABL_NO_DMA / MX_ABL_NO_READ (never defined in the product build) drop the copies or the
+// fragment reads from the steady state, to time what is left; results are then meaningless.
 #include "mx_gemm_tile.h"
 
 namespace mx {
@@ -551,11 +558,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       // write path's pace
       static_for<0, 4>([&](auto q_) {
         constexpr int q = decltype(q_)::value;
-#ifndef MX_ABL_NO_STAGE
         if constexpr (pc < 7) stage_part(std::integral_constant<int, pc + 1>{}, q_);
-#else
-        if constexpr (pc < 7) lds_write_b128_hidden<q * 32>(patch_w, v4i{1, 2, 3, 4});
-#endif
         if constexpr (q == 0) {
           // the four reads are done once at most the one younger write is outstanding
           if constexpr (pc < 7) asm volatile("s_waitcnt lgkmcnt(1)" ::: "memory");
@@ -563,20 +566,13 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
         }
         const v4i rq = pin(r[pc & 1][q]);
         const u32x4 w = {(uint32_t)rq.x, (uint32_t)rq.y, (uint32_t)rq.z, (uint32_t)rq.w};
-#ifndef MX_ABL_NO_STORE
         __builtin_amdgcn_raw_buffer_store_b128(w, rd, v, (m * 32 + q * 8) * ldd_b, MX_STORE_AUX);
-#else
-        asm volatile("" ::"v"(w));
-#endif
         __builtin_amdgcn_sched_barrier(0);
       });
       if constexpr (PROF) prof_e_stage += __builtin_readcyclecounter() - e0;
     });
   };
 
-#ifdef MX_XCD_STAGGER
-  for (uint32_t i = 0, n = xcd * MX_XCD_STAGGER; i < n; ++i) __builtin_amdgcn_s_sleep(1);
-#endif
   // ---- prologue: fill the ring, fetch the first fragments
   loader_open_tile();
   issue_block();
