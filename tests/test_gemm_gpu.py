@@ -138,3 +138,27 @@ def test_full_size_linearity(device):
     ref = mo.mx_matmul_q(u8(a.codes[:64]), u8(a.scales[:64]), u8(b.codes[:96]), u8(b.scales[:96]))
     err = rel_l2(_f32(bits_of(d[:64, :96])), _f32(ref))
     assert err <= TOL
+
+
+def test_config1_full_size_against_the_oracle(device):
+    """The CPU-runnable baseline config at its full size: X[8192,4096], W[4096,4096] with 0.1 %
+    x100 outliers, FLOOR and RCEIL: codes and scales of all four casts bit-exact against the C
+    oracle, Y against the oracle's dequantize + fp32 matmul + bf16 round (rel-L2 <= 1e-3)."""
+    from oracle import c_oracle as co
+
+    x_bits, w_bits = mo.make_cfg1_inputs(0)
+    x, w = bf16_from_bits(x_bits, device), bf16_from_bits(w_bits, device)
+    R = ops.MX_SCALES_ROWMAJOR
+    for mode_name, mode in (("floor", mo.FLOOR), ("rceil", mo.RCEIL)):
+        for t_bits, t in ((x_bits, x), (w_bits, w)):
+            q0, q1 = ops.to_mx_dim0_dim1(t, mode_name, R)
+            c0, s0 = co.cast_dim0(t_bits, mode)
+            c1, s1 = co.cast_dim1(t_bits, mode)
+            assert np.array_equal(u8(q0.codes), c0) and np.array_equal(u8(q0.scales), s0)
+            assert np.array_equal(u8(q1.codes), c1) and np.array_equal(u8(q1.scales), s1)
+        L = ops.MX_SCALES_MFMA
+        y = ops.mx_gemm_nt(ops.to_mx_dim0(x, mode_name, L), ops.to_mx_dim0(w, mode_name, L))
+        xc, xs = co.cast_dim0(x_bits, mode)
+        wc, ws = co.cast_dim0(w_bits, mode)
+        ref = mo.f32_to_bf16_bits(co.dequant(xc, xs) @ co.dequant(wc, ws).T)
+        assert rel_l2(_f32(bits_of(y)), _f32(ref)) <= TOL
