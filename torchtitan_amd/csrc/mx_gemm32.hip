@@ -55,6 +55,7 @@ struct Gemm32Args {
   int64_t M, N, K, ldd;
   const int32_t* offs;  // grouped modes: inclusive cumulative group sizes, on the device
   int64_t G;
+  int32_t tn0, tn_cnt;  // grouped modes: this launch covers tile columns [tn0, tn0 + tn_cnt)
   uint64_t* prof;  // timing build only: per wave {vmcnt wait, barrier wait, step body} cycles
 };
 
@@ -118,6 +119,29 @@ __device__ __forceinline__ void mfma_asm(v16f& c, const v8i& b, const v8i& a, ui
         : "v"(b), "v"(a), "v"(sb), "v"(sa), "n"(N & 1), "n"(M & 1), "n"(N >> 1), "n"(M >> 1));
 }
 
+// A tile without K blocks: zeros (an empty group, the rows behind the last group), or NaN when
+// the group ends break the contract, so that the mistake cannot pass unnoticed.  Written
+// straight from registers: wave (wm, wn) owns rows 128 wm.., columns 128 wn...
+// (Inlined on purpose: a call would make the compiler save every live register around it.)
+__device__ __forceinline__ void fill_tile32(uint16_t* d, int64_t rows_a, int64_t rows_b,
+                                                      int64_t ldd, bool poison) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const uint32_t fill = poison ? 0x7FC07FC0u : 0u;
+  const u32x4 w = {fill, fill, fill, fill};
+  const uint32_t ldd_b = (uint32_t)ldd * 2;
+  const __amdgpu_buffer_rsrc_t rd = make_rsrc(d, rows_a * ldd_b);
+  const uint32_t cols_valid = (uint32_t)(rows_b < 256 ? rows_b : 256);
+  const uint32_t colp = wn * 128 + (lane & 7) * 8;
+  const uint32_t vrow = (wm * 128 + (lane >> 3)) * ldd_b + colp * 2;
+  for (uint32_t r8 = 0; r8 < 16; ++r8) {
+    const uint32_t v0 = colp < cols_valid ? vrow : 0x80000000u;
+    const uint32_t v1 = colp + 64 < cols_valid ? vrow + 128 : 0x80000000u;
+    __builtin_amdgcn_raw_buffer_store_b128(w, rd, v0, r8 * 8 * ldd_b, 0);
+    __builtin_amdgcn_raw_buffer_store_b128(w, rd, v1, r8 * 8 * ldd_b, 0);
+  }
+}
+
 struct Frags32 {
   v8i a[4];
   v8i b[4];
@@ -135,13 +159,13 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void_t*)smem;  // LDS byte address of the ring
   const uint32_t K = (uint32_t)p.K;  // bytes per operand row; a multiple of 128 for this kernel
   const uint32_t ks_n = K / kK32;    // 64-deep steps per 128-row scale group
-  const uint32_t tiles_n = (uint32_t)((p.N + kT32 - 1) / kT32);
+  const uint32_t tiles_n = MODE == kDense ? (uint32_t)((p.N + kT32 - 1) / kT32) : (uint32_t)p.tn_cnt;
+  const uint32_t tn0 = MODE == kDense ? 0u : (uint32_t)p.tn0;
   const uint32_t G = (uint32_t)p.G;
 
   // ---- tile count.  kGrouped2d3d: group g has ceil(rows_g / 256) x tiles_n tiles; the first
   //      tile number of every group (G + 2 entries, the last group being the zero rows behind
   //      offs[G-1]) is kept in the 2.5 KB that wave 0's output patch leaves unused.
-  const uint32_t lds_first = lds_base + kRing32 + 4608;
   bool poison = false;
   uint32_t nb;
   // "any thread saw a bad group end", through a word of wave 1's spare patch bytes (the
@@ -174,13 +198,20 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       first[g + 1] = (uint32_t)((rows + kT32 - 1) / kT32) * tiles_n;
     }
     poison = any_bad(bad);
-    if (tid == 0) {
-      uint32_t acc_t = 0;
-      first[0] = 0;
-      for (uint32_t g = 1; g <= G + 1; ++g) {
-        acc_t += first[g];
-        first[g] = acc_t;
+    if (tid < 64) {  // inclusive prefix sum of first[1 .. G+1] by wave 0, 10 entries per lane
+      uint32_t sum = 0;
+      for (uint32_t g = 1 + tid * 10; g < 11 + tid * 10 && g <= G + 1; ++g) sum += first[g];
+      uint32_t incl = sum;
+      for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t o = __shfl_up(incl, d);
+        if (tid >= d) incl += o;
       }
+      uint32_t run = incl - sum;
+      for (uint32_t g = 1 + tid * 10; g < 11 + tid * 10 && g <= G + 1; ++g) {
+        run += first[g];
+        first[g] = run;
+      }
+      if (tid == 0) first[0] = 0;
     }
     __syncthreads();
     nb = first[G + 1];
@@ -196,24 +227,17 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   const uint32_t t_hi = (xcd + 1) * per_xcd < nb ? (xcd + 1) * per_xcd : nb;
   const uint32_t n_my = t_lo < t_hi ? (t_hi - t_lo + wgs_per_xcd - 1) / wgs_per_xcd : 0;
   if (n_my == 0) return;
+  if (MODE != kDense && n_my > 120) return;  // more tiles than records: the host never launches this
 
-  // first tile number of group g (kGrouped2d3d), read so that the compiler's wait-count
-  // model does not see an LDS read (see read_piece)
-  auto group_first = [&](uint32_t g) -> uint32_t {
-    uint32_t v;
-    const uint32_t addr = lds_first + g * 4;
-    asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(addr) : "memory");
-    return __builtin_amdgcn_readfirstlane(v);
-  };
-  // Tile number -> operands.  `g` is the caller's cursor into the groups: a stream visits
-  // tiles in increasing order, so the group is found by walking forward from the last one.
-  auto describe = [&](uint32_t t, uint32_t& g) -> Tile32 {
+  // Tile number -> operands.
+  auto describe = [&](uint32_t t) -> Tile32 {
     Tile32 r;
     r.poison = poison;
     r.koff = 0;
     uint32_t tm, tn;
     if (MODE == kDense || (MODE == kGrouped2d3d && poison)) {
       tile_coords(t, (uint32_t)((p.M + kT32 - 1) / kT32), tiles_n, tm, tn);
+      tn += tn0;
       r.a = p.a_codes + (int64_t)tm * kT32 * K;
       r.b = p.b_codes + (int64_t)tn * kT32 * K;
       r.sa = p.a_scales + (int64_t)(tm * 2) * ks_n * 256;
@@ -223,10 +247,16 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       r.rows_b = p.N - (int64_t)tn * kT32;
       r.nblocks = poison ? 0 : K / kKB;
     } else if (MODE == kGrouped2d3d) {
-      while (t >= group_first(g + 1)) ++g;
+      const uint32_t* first = reinterpret_cast<const uint32_t*>(smem + kRing32 + 4608);
+      uint32_t g = 0, hi_g = G + 1;  // first[g] <= t < first[g + 1]
+      while (hi_g - g > 1) {
+        const uint32_t mid = (g + hi_g) >> 1;
+        if (first[mid] <= t) g = mid; else hi_g = mid;
+      }
       const int64_t lo = g ? p.offs[g - 1] : 0, hi = g < G ? (int64_t)p.offs[g] : p.M;
       const uint32_t tiles_mg = (uint32_t)((hi - lo + kT32 - 1) / kT32);
-      tile_coords(t - group_first(g), tiles_mg, tiles_n, tm, tn);
+      tile_coords(t - first[g], tiles_mg, tiles_n, tm, tn);
+      tn += tn0;
       const int64_t row0 = lo + (int64_t)tm * kT32;
       const uint32_t gb = g < G ? g : 0;  // the zero rows have no expert: any valid address
       r.a = p.a_codes + row0 * K;
@@ -239,8 +269,9 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       r.nblocks = g < G ? K / kKB : 0;
     } else {
       const uint32_t tiles_m = (uint32_t)((p.M + kT32 - 1) / kT32), per_g = tiles_m * tiles_n;
-      g = t / per_g;
+      const uint32_t g = t / per_g;
       tile_coords(t - g * per_g, tiles_m, tiles_n, tm, tn);
+      tn += tn0;
       const int64_t lo = poison ? 0 : (g ? p.offs[g - 1] : 0), hi = poison ? 0 : p.offs[g];
       r.a = p.a_codes + (int64_t)tm * kT32 * K + lo;
       r.b = p.b_codes + (int64_t)tn * kT32 * K + lo;
@@ -253,6 +284,64 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       r.nblocks = (uint32_t)((hi - lo) >> 7);
     }
     return r;
+  };
+
+  // Grouped modes: the map needs loads of the group ends and a search, far too slow for the
+  // in-order instruction stream of the MFMA waves.  Every thread works out one of this
+  // workgroup's tiles up front and leaves a 64-byte record in the spare 2.5 KB behind the
+  // output patches of waves 1-3 (40 records each; the host splits launches so that a
+  // workgroup never has more than kMaxRecords tiles).
+  auto record_offset = [&](uint32_t i) -> uint32_t {
+    return kRing32 + (1 + i / 40) * 7168 + 4608 + (i % 40) * 64;
+  };
+  if constexpr (MODE != kDense) {
+    for (uint32_t i = tid; i < n_my; i += 256) {
+      const Tile32 t = describe(t_lo + i * wgs_per_xcd);
+      uint64_t* q = reinterpret_cast<uint64_t*>(smem + record_offset(i));
+      q[0] = (uint64_t)(uintptr_t)t.a;
+      q[1] = (uint64_t)(uintptr_t)t.b;
+      q[2] = (uint64_t)(uintptr_t)t.sa;
+      q[3] = (uint64_t)(uintptr_t)t.sb;
+      q[4] = (uint64_t)(uintptr_t)t.d;
+      int32_t* w = reinterpret_cast<int32_t*>(q + 5);
+      w[0] = (int32_t)(t.rows_a > 0x7FFFFFFF ? 0x7FFFFFFF : t.rows_a);
+      w[1] = (int32_t)(t.rows_b > 0x7FFFFFFF ? 0x7FFFFFFF : t.rows_b);
+      w[2] = (int32_t)t.nblocks;
+      w[3] = (int32_t)t.koff;
+    }
+    __syncthreads();
+  }
+  // this workgroup's i-th tile (records are read so that the compiler's wait-count model
+  // does not see an LDS read, see read_piece; every lane reads the same 64 bytes)
+  auto get_tile = [&](uint32_t i) -> Tile32 {
+    if constexpr (MODE == kDense) {
+      return describe(t_lo + i * wgs_per_xcd);
+    } else {
+      const uint32_t addr = lds_base + record_offset(i);
+      v4i r0, r1, r2, r3;
+      asm volatile(
+          "ds_read_b128 %0, %4\n\tds_read_b128 %1, %4 offset:16\n\tds_read_b128 %2, %4 offset:32\n\t"
+          "ds_read_b128 %3, %4 offset:48\n\ts_waitcnt lgkmcnt(0)"
+          : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3)
+          : "v"(addr)
+          : "memory");
+      auto u64 = [](int lo, int hi) -> uint64_t {
+        return (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane(lo) |
+               ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane(hi) << 32);
+      };
+      Tile32 t;
+      t.a = (const uint8_t*)(uintptr_t)u64(r0.x, r0.y);
+      t.b = (const uint8_t*)(uintptr_t)u64(r0.z, r0.w);
+      t.sa = (const uint8_t*)(uintptr_t)u64(r1.x, r1.y);
+      t.sb = (const uint8_t*)(uintptr_t)u64(r1.z, r1.w);
+      t.d = (uint16_t*)(uintptr_t)u64(r2.x, r2.y);
+      t.rows_a = __builtin_amdgcn_readfirstlane(r2.z);
+      t.rows_b = __builtin_amdgcn_readfirstlane(r2.w);
+      t.nblocks = (uint32_t)__builtin_amdgcn_readfirstlane(r3.x);
+      t.koff = (uint32_t)__builtin_amdgcn_readfirstlane(r3.y);
+      t.poison = poison;
+      return t;
+    }
   };
 
   // ---- per-lane constants
@@ -273,14 +362,14 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   const uint32_t fsa_s = kCodes32 + wm * 512, fsb_s = kCodes32 + 1024 + wn * 512;
 
   // ---- loader stream: fills ring block `ld_slot` with K block `ld_kb` of tile `ld_tile`
-  uint32_t ld_tile = 0, ld_kb = 0, ld_nb = 1, ld_g = 0;
+  uint32_t ld_tile = 0, ld_kb = 0, ld_nb = 1;
   int ld_slot = 0;
   __amdgpu_buffer_rsrc_t ra, rb, rs;  // codes of A, codes of B, scales this wave copies
   auto loader_open_tile = [&]() {
     Tile32 t;
     t.nblocks = 0;
     while (ld_tile < n_my) {  // tiles without K blocks add nothing to the stream
-      t = describe(t_lo + ld_tile * wgs_per_xcd, ld_g);
+      t = get_tile(ld_tile);
       if (MODE == kDense || t.nblocks) break;
       ++ld_tile;
     }
@@ -519,7 +608,6 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   const uint32_t patch = lds_base + kRing32 + wave * 7168;
   const uint32_t patch_w = patch + li * kPatchPitch + lj * 16;                 // + (n&1)*64 + h*32
   const uint32_t patch_r = patch + (lane >> 3) * kPatchPitch + (lane & 7) * 16;  // + pass*8 rows
-  uint32_t ep_g = 0;
   auto epilogue = [&](const Tile32& t) {
     const int64_t rows_valid = t.rows_a;
     const uint32_t cols_valid = (uint32_t)(t.rows_b < kT32 ? t.rows_b : kT32);
@@ -589,7 +677,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   // last step of a tile has already read them from the next tile's first block, which the
   // loader fetched like any other block).
   for (uint32_t tile = 0; tile < n_my; ++tile) {
-    const Tile32 t = describe(t_lo + tile * wgs_per_xcd, ep_g);
+    const Tile32 t = get_tile(tile);
     if (MODE == kDense || t.nblocks) {
       block_steps(f0, f1, std::true_type{});
       for (uint32_t i = 1; i < t.nblocks; ++i) block_steps(f0, f1, std::false_type{});
@@ -608,22 +696,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
         epilogue(t);
       }
     } else {
-      // no K blocks: zeros (an empty group, the rows behind the last group), or NaN when the
-      // group ends break the contract, so that the mistake cannot pass unnoticed.  Written
-      // straight from registers: wave (wm, wn) owns rows 128 wm.., columns 128 wn..
-      const uint32_t fill = t.poison ? 0x7FC07FC0u : 0u;
-      const u32x4 w = {fill, fill, fill, fill};
-      const uint32_t ldd_b = (uint32_t)p.ldd * 2;
-      const __amdgpu_buffer_rsrc_t rd = make_rsrc(t.d, t.rows_a * ldd_b);
-      const uint32_t cols_valid = (uint32_t)(t.rows_b < kT32 ? t.rows_b : kT32);
-      const uint32_t colp = wn * 128 + (lane & 7) * 8;
-      const uint32_t vrow = (wm * 128 + (lane >> 3)) * ldd_b + colp * 2;
-      for (uint32_t r8 = 0; r8 < 16; ++r8) {
-        const uint32_t v0 = colp < cols_valid ? vrow : 0x80000000u;
-        const uint32_t v1 = colp + 64 < cols_valid ? vrow + 128 : 0x80000000u;
-        __builtin_amdgcn_raw_buffer_store_b128(w, rd, v0, r8 * 8 * ldd_b, 0);
-        __builtin_amdgcn_raw_buffer_store_b128(w, rd, v1, r8 * 8 * ldd_b, 0);
-      }
+      fill_tile32(t.d, t.rows_a, t.rows_b, p.ldd, t.poison);
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the over-issued prefetches before retiring
@@ -674,29 +747,53 @@ void set_debug_prof(uint64_t* buf) { debug_prof = buf; }
 int launch_gemm_nt32(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                      const uint8_t* b_scales, void* d, int64_t M, int64_t N, int64_t K,
                      int64_t ldd, hipStream_t st) {
-  Gemm32Args p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, M, N, K, ldd, nullptr, 0, debug_prof};
+  Gemm32Args p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, M, N, K, ldd, nullptr, 0, 0, 0, debug_prof};
   const int64_t nb = ((M + kT32 - 1) / kT32) * ((N + kT32 - 1) / kT32);
   if (debug_prof) return launch32<kDense, true>(p, nb, st);
   return launch32<kDense, false>(p, nb, st);
 }
 
 // Grouped forms with every group end a multiple of 128 and all scales in MFMA order
-// (a_scales over the whole [T, K/32] matrix, b_scales one block per expert).
+// (a_scales over the whole [T, K/32] matrix, b_scales one block per expert).  A workgroup keeps
+// a record per tile in LDS, at most kMaxRecords of them: larger problems are cut into several
+// launches over ranges of tile columns.
+constexpr int64_t kMaxRecords = 120;
+
+template <int MODE>
+static int launch_grouped32(Gemm32Args p, int64_t tiles_per_column, int64_t tiles_n, hipStream_t st) {
+  int cus = 0, dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+    return MX_ERR_LAUNCH;
+  const int64_t grid = cus / 8 * 8 < 8 ? 8 : cus / 8 * 8;
+  // tiles of one launch <= grid * kMaxRecords - slack for the rounding of the per-XCD runs
+  int64_t cols = (grid * kMaxRecords - 8 * (grid / 8)) / tiles_per_column;
+  if (cols < 1) return MX_ERR_UNSUPPORTED;
+  if (cols > tiles_n) cols = tiles_n;
+  for (int64_t tn0 = 0; tn0 < tiles_n; tn0 += cols) {
+    p.tn0 = (int32_t)tn0;
+    p.tn_cnt = (int32_t)(tiles_n - tn0 < cols ? tiles_n - tn0 : cols);
+    const int64_t nb = tiles_per_column * p.tn_cnt;
+    const int rc = p.prof ? launch32<MODE, true>(p, nb, st) : launch32<MODE, false>(p, nb, st);
+    if (rc != MX_OK) return rc;
+  }
+  return MX_OK;
+}
+
 int launch_grouped32_2d3d(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                           const uint8_t* b_scales, const int32_t* offs, void* d, int64_t T,
                           int64_t N, int64_t K, int64_t G, int64_t ldd, hipStream_t st) {
-  Gemm32Args p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, T, N, K, ldd, offs, G, nullptr};
-  const int64_t nb = ((T + kT32 - 1) / kT32 + G + 1) * ((N + kT32 - 1) / kT32);
-  return launch32<kGrouped2d3d, false>(p, nb, st);
+  Gemm32Args p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, T, N, K, ldd, offs, G, 0, 0, debug_prof};
+  // an upper bound of the tile rows: every group may add one partly filled tile
+  return launch_grouped32<kGrouped2d3d>(p, (T + kT32 - 1) / kT32 + G + 1, (N + kT32 - 1) / kT32, st);
 }
 
 // D[g][N, K] = A^T[N, lo:hi] B^T[K, lo:hi]^T; operand rows are T long.
 int launch_grouped32_2d2d(const uint8_t* at_codes, const uint8_t* at_scales,
                           const uint8_t* bt_codes, const uint8_t* bt_scales, const int32_t* offs,
                           void* d, int64_t T, int64_t N, int64_t K, int64_t G, hipStream_t st) {
-  Gemm32Args p{at_codes, at_scales, bt_codes, bt_scales, (uint16_t*)d, N, K, T, K, offs, G, nullptr};
-  const int64_t nb = G * ((N + kT32 - 1) / kT32) * ((K + kT32 - 1) / kT32);
-  return launch32<kGrouped2d2d, false>(p, nb, st);
+  Gemm32Args p{at_codes, at_scales, bt_codes, bt_scales, (uint16_t*)d, N, K, T, K, offs, G, 0, 0, debug_prof};
+  return launch_grouped32<kGrouped2d2d>(p, G * ((N + kT32 - 1) / kT32), (K + kT32 - 1) / kT32, st);
 }
 
 }  // namespace mx
