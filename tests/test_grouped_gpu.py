@@ -134,6 +134,44 @@ def test_grouped_wgrad_aligned_groups(device, sizes, N, K):
                 assert rel_l2(_f32(got[g]), _f32(ref[g])) <= TOL, g
 
 
+def test_aligned_group_forms_split_into_several_launches(device):
+    """More tiles than a workgroup can keep records for: the launch is cut by tile columns.
+
+    Forced here by running with 8 workgroups (a debug setting of the library), which lowers the
+    capacity of one launch to 952 tiles."""
+    from torchtitan_amd import _lib
+
+    lib = _lib.load()
+    rng = np.random.default_rng(23)
+    try:
+        lib.mx_debug_set_grid(8)
+        sizes, N, K = [512, 0, 1280], 25600, 128      # 12 tile rows x 100 tile columns
+        T = sum(sizes) + 256
+        x_bits = randn_bits(rng, (T, K), outliers=1e-3)
+        w_bits = randn_bits(rng, (len(sizes), N, K), std=0.02)
+        offs = _sizes_to_offs(sizes, device)
+        x, w = bf16_from_bits(x_bits, device), bf16_from_bits(w_bits, device)
+        y = ops.mx_grouped_gemm_2d3d(ops.to_mx_dim0(x, "rceil", L), ops.to_mx_dim0_batched(w, "rceil", L), offs)
+        ref = mo.grouped_fwd(x_bits, w_bits, np.cumsum(sizes), mo.RCEIL)
+        assert rel_l2(_f32(bits_of(y)), _f32(ref)) <= TOL
+        assert np.all(bits_of(y)[sum(sizes):] == 0)
+
+        sizes, N, K = [128, 0, 256], 2560, 10240      # 30 tiles per column x 40 tile columns
+        T = sum(sizes)
+        x_bits = randn_bits(rng, (T, K), outliers=1e-3)
+        dy_bits = randn_bits(rng, (T, N), std=1e-3)
+        offs = _sizes_to_offs(sizes, device)
+        x, dy = bf16_from_bits(x_bits, device), bf16_from_bits(dy_bits, device)
+        dw = ops.mx_grouped_gemm_2d2d(ops.to_mx_dim1(dy, "rceil", L), ops.to_mx_dim1(x, "rceil", L), offs)
+        ref = mo.grouped_wgrad(dy_bits, x_bits, np.cumsum(sizes), mo.RCEIL)
+        got = bits_of(dw)
+        assert np.all(got[1] == 0)
+        for g in (0, 2):
+            assert rel_l2(_f32(got[g]), _f32(ref[g])) <= TOL, g
+    finally:
+        lib.mx_debug_set_grid(0)
+
+
 def test_aligned_group_forms_poison_the_output_when_a_group_end_is_not_a_multiple_of_128(device):
     rng = np.random.default_rng(5)
     sizes, N, K = [128, 160, 96], 128, 128

@@ -717,26 +717,37 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
 static int debug_grid = 0;
 static uint64_t* debug_prof = nullptr;  // > 0: number of persistent workgroups (experiments only)
 
+// One persistent workgroup per CU, a multiple of the 8 XCDs (0: the device cannot be queried).
+static int64_t persistent_grid() {
+  static int num_cus = 0;
+  if (num_cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      return 0;
+    num_cus = n;
+  }
+  int64_t grid = (num_cus / 8) * 8;
+  if (grid < 8) grid = 8;
+  if (debug_grid > 0) grid = (debug_grid + 7) / 8 * 8;
+  return grid;
+}
+
 template <int MODE, bool PROF>
 static int launch32(const Gemm32Args& p, int64_t nb, hipStream_t st) {
   auto kern = gemm_nt32_kernel<MODE, PROF>;
   constexpr int lds = kRing32 + 4 * 7168;  // ring + one output patch per wave = all 160 KB
-  static int num_cus = 0;
-  if (num_cus == 0) {
+  static bool configured = false;
+  if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                             hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
       return MX_ERR_LAUNCH;
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-      return MX_ERR_LAUNCH;
-    num_cus = n;
+    configured = true;
   }
-  int64_t grid = (num_cus / 8) * 8;  // one persistent workgroup per CU, a multiple of the 8 XCDs
-  if (grid < 8) grid = 8;
+  int64_t grid = persistent_grid();
+  if (grid == 0) return MX_ERR_LAUNCH;
   const int64_t need = (nb + 7) / 8 * 8;  // nb: the tile count, or an upper bound of it
-  if (need < grid) grid = need;
-  if (debug_grid > 0) grid = (debug_grid + 7) / 8 * 8;
+  if (need < grid && debug_grid <= 0) grid = need;
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, st, p);
   return hipGetLastError() == hipSuccess ? MX_OK : MX_ERR_LAUNCH;
 }
@@ -761,11 +772,8 @@ constexpr int64_t kMaxRecords = 120;
 
 template <int MODE>
 static int launch_grouped32(Gemm32Args p, int64_t tiles_per_column, int64_t tiles_n, hipStream_t st) {
-  int cus = 0, dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess ||
-      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-    return MX_ERR_LAUNCH;
-  const int64_t grid = cus / 8 * 8 < 8 ? 8 : cus / 8 * 8;
+  const int64_t grid = persistent_grid();
+  if (grid == 0) return MX_ERR_LAUNCH;
   // tiles of one launch <= grid * kMaxRecords - slack for the rounding of the per-XCD runs
   int64_t cols = (grid * kMaxRecords - 8 * (grid / 8)) / tiles_per_column;
   if (cols < 1) return MX_ERR_UNSUPPORTED;
