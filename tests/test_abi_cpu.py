@@ -39,3 +39,18 @@ def test_host_side_entry_points_answer_without_a_gpu():
     assert lib.mx_cast_dim0(None, 0, 64, 64, None, None, 0, 0, None) == 0  # empty is a no-op
     assert lib.mx_gemm_nt(None, None, None, None, None, 16, 16, 33, 16, None) != 0
     assert lib.mx_group_offsets_pad(None, 0, 1, 0, 32, None, None, None, None) == 1
+
+
+def test_ctypes_prototypes_have_the_declared_number_of_arguments():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    for name, args in re.findall(r"\b(mx_[a-z0-9_]+)\s*\(([^)]*)\)\s*;", text):
+        args = args.strip()
+        n = 0 if args in ("", "void") else len(args.split(","))
+        assert len(_lib.SIGNATURES[name][1]) == n, name
+    # the grouped forms take the scale order just before the stream
+    assert lib_arg_kinds("mx_grouped_gemm_2d3d")[-2:] == [ctypes.c_int, ctypes.c_void_p]
+    assert lib_arg_kinds("mx_grouped_gemm_2d2d")[-2:] == [ctypes.c_int, ctypes.c_void_p]
+
+
+def lib_arg_kinds(name):
+    return list(_lib.SIGNATURES[name][1])

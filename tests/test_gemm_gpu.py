@@ -25,7 +25,9 @@ def _f32(bits):
 @pytest.mark.parametrize("M,N,K", [(16, 16, 32), (16, 16, 128), (64, 64, 128), (128, 128, 256),
                                    (256, 256, 128), (256, 256, 512), (512, 768, 1024),
                                    (300, 200, 160), (257, 129, 96), (1000, 1000, 2048),
-                                   (2048, 1024, 4096)])
+                                   (2048, 1024, 4096),
+                                   # more tiles than workgroups, one or two K blocks per tile
+                                   (4096, 4352, 128), (6144, 6400, 256)])
 def test_gemm_matches_oracle(device, M, N, K):
     rng = np.random.default_rng(M * 7 + N * 3 + K)
     a_bits = randn_bits(rng, (M, K), outliers=1e-3)

@@ -1,7 +1,7 @@
 // Library identification and status strings.
 #include "mx_common.h"
 
-extern "C" int mx_version(void) { return 100; }
+extern "C" int mx_version(void) { return 101; }
 
 extern "C" const char* mx_status_string(int status) {
   switch (status) {
