@@ -125,6 +125,53 @@ def time_casts(dev, recipe_mode):
     return out
 
 
+def time_moe_grouped(dev, recipe_mode):
+    """BASELINE configs[3] GEMMs (not the headline): 128 experts, hidden 2048, expert FFN 768,
+    top-8 routing of 16384 tokens from softmax over seeded Gumbel-perturbed logits (uneven
+    groups), groups padded to multiples of 128 rows for the persistent kernel.  TFLOP/s counts
+    the unpadded routed rows only."""
+    import torch
+
+    from torchtitan_amd import ops
+
+    E, dim, hid, tokens, topk = 128, 2048, 768, 16384, 8
+    g = torch.Generator(device=dev).manual_seed(3)
+    logits = torch.randn((tokens, E), generator=g, device=dev) + 0.5 * torch.randn((1, E), generator=g, device=dev)
+    gumbel = -torch.log(-torch.log(torch.rand((tokens, E), generator=g, device=dev).clamp_min(1e-9)))
+    top = torch.topk(torch.softmax(logits + gumbel, dim=-1), topk, dim=-1).indices
+    counts = torch.bincount(top.flatten(), minlength=E).to(torch.int32)
+    routed = tokens * topk
+    max_len = -(-(routed + 128 * E) // 128) * 128
+    _, m_sizes, offs = ops.group_offsets_pad(counts, E, 1, max_len, 128)
+    L = ops.MX_SCALES_MFMA
+    x = torch.randn((max_len, dim), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    w = (torch.randn((E, hid, dim), generator=g, device=dev, dtype=torch.float32) * 0.02).to(torch.bfloat16)
+    dy = (torch.randn((max_len, hid), generator=g, device=dev, dtype=torch.float32) * 1e-3).to(torch.bfloat16)
+    xq0, xq1 = ops.to_mx_dim0_dim1(x, recipe_mode, L)
+    dyq0, dyq1 = ops.to_mx_dim0_dim1(dy, recipe_mode, L)
+    wq0, wq1 = ops.to_mx_dim0_dim1_batched(w, recipe_mode, L)
+    y = torch.empty((max_len, hid), device=dev, dtype=torch.bfloat16)
+    dx = torch.empty((max_len, dim), device=dev, dtype=torch.bfloat16)
+    dw = torch.empty((E, hid, dim), device=dev, dtype=torch.bfloat16)
+    flops = 2.0 * routed * dim * hid
+    out = {"group_rows_min_max": [int(counts.min()), int(counts.max())], "padded_rows": int(offs[-1])}
+    for name, fn in (("fwd_2d3d", lambda: ops.mx_grouped_gemm_2d3d(xq0, wq0, offs, y)),
+                     ("dgrad_2d3d", lambda: ops.mx_grouped_gemm_2d3d(dyq0, wq1, offs, dx)),
+                     ("wgrad_2d2d", lambda: ops.mx_grouped_gemm_2d2d(dyq1, xq1, offs, dw))):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(8):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        sec = s.elapsed_time(e) * 1e-3 / 8
+        out[name] = {"us": round(sec * 1e6, 1), "TFLOP/s": round(flops / sec / 1e12, 1)}
+    return out
+
+
 def cpu_baseline(recipe_mode_int, target_s=15.0):
     """CPU oracle on a bounded sample of BASELINE config 1: the emulated MX linear forward
     (to_mx of X and W along K, dequantize, fp32 matmul, bf16 round) plus the column-wise casts
@@ -265,6 +312,7 @@ def main():
     }
     if not args.no_casts:
         line["casts"] = time_casts(dev, recipe_mode)
+        line["moe_grouped_gemms"] = time_moe_grouped(dev, recipe_mode)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(0 if recipe_mode == "floor" else 1, target_s=12.0)
     print(json.dumps(line))
