@@ -1,0 +1,29 @@
+/*
+ * Measurement hooks of libmxfp8_gfx950.so.  NOT part of the ABI in mxfp8.h: nothing in the
+ * product path calls them, their meaning may change with the kernels, and they are process-wide
+ * (not thread-safe).  They exist so that timing experiments can be run against the shipped
+ * library instead of a special build.
+ */
+#ifndef MXFP8_DEBUG_H_
+#define MXFP8_DEBUG_H_
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* 0: pick the dense GEMM kernel by shape (default); 1: the 16x16x128 tile kernel for every shape. */
+void mx_debug_force_kernel(int which);
+
+/* > 0: number of persistent workgroups of the 32x32x64 kernel, rounded up to a multiple of 8
+ * (also lowers how many tiles one grouped launch covers); 0: one per CU (default). */
+void mx_debug_set_grid(int workgroups);
+
+/* Device buffer of 256 * 4 * 8 uint64 that the timing build of the 32x32x64 kernel fills with
+ * per-wave cycle counts {copy wait, barriers, step body, epilogue, ...}; NULL switches the timing
+ * build off (default). */
+void mx_debug_set_prof(void* device_buffer);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MXFP8_DEBUG_H_ */

@@ -100,11 +100,15 @@ def test_feed_forward_close_to_bf16_and_trains(device):
 
 
 @pytest.mark.parametrize("pad,align", [(True, 8), (False, 32)])
-def test_grouped_experts_module(device, pad, align):
-    """torch._grouped_mm on converted 3-D weights, forward and backward, vs per-expert oracle."""
-    rng = np.random.default_rng(17 + align)
-    E, dim, hidden = 4, 128, 64
-    counts = np.array([40, 0, 72, 16]) if pad else np.array([64, 0, 96, 32])
+@pytest.mark.parametrize("dim,hidden", [(128, 64), (256, 128)])
+def test_grouped_experts_module(device, pad, align, dim, hidden):
+    """torch._grouped_mm on converted 3-D weights, forward and backward, vs per-expert oracle.
+
+    With padding on and both dims multiples of 128 the wrapper pads groups to 128 rows and the
+    persistent kernels run; otherwise the general ones.  The results must not depend on it."""
+    rng = np.random.default_rng(17 + align + dim)
+    E = 4
+    counts = np.array([40, 0, 200, 16]) if pad else np.array([64, 0, 96, 32])
     T = int(counts.sum())
     x_bits = randn_bits(rng, (T, dim))
     w_bits = randn_bits(rng, (E, hidden, dim), std=0.05)
