@@ -55,7 +55,8 @@ int launch_gemm_nt32(const uint8_t* a_codes, const uint8_t* a_scales, const uint
                      const uint8_t* b_scales, void* d, int64_t M, int64_t N, int64_t K,
                      int64_t ldd, hipStream_t st);
 }
-// 0: pick by shape; 1: the 16x16x128 tile kernel for every shape (kept for comparison runs)
+// 0: pick by shape; 1 / 2: the 16x16x128 tile kernel with 256x256 / 128x128 tiles for every
+// shape (kept for comparison runs)
 static int force_kernel = 0;
 extern "C" void mx_debug_force_kernel(int which) { force_kernel = which; }
 namespace mx { void set_debug_grid(int g); }
@@ -77,7 +78,19 @@ extern "C" int mx_gemm_nt(const uint8_t* a_codes, const uint8_t* a_scales,
   if (256 * K > 0x7FFFFFFFll) return MX_ERR_UNSUPPORTED;
   DenseArgs p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, M, N, K, ldd};
   hipStream_t st = (hipStream_t)stream;
-  if (M <= 128 || N <= 128) return launch_dense<128, 128>(p, st);
+  if (M <= 128 || N <= 128 || force_kernel == 2) return launch_dense<128, 128>(p, st);
+  // Few 256x256 tiles leave most CUs of the persistent kernel idle (it has no split along K):
+  // up to 3/8 of the CUs' worth of tiles, four times as many 128x128 tiles finish sooner
+  // (measured: 64 tiles 58 vs 71 us at K = 8192; 128 tiles 46 vs 43 us).
+  static int num_cus = 0;
+  if (num_cus == 0) {
+    int dev = 0, n = 0;
+    num_cus = (hipGetDevice(&dev) == hipSuccess &&
+               hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+                  ? n : 256;
+  }
+  const int64_t tiles256 = ((M + 255) / 256) * ((N + 255) / 256);
+  if (force_kernel == 0 && tiles256 * 8 <= (int64_t)num_cus * 3) return launch_dense<128, 128>(p, st);
   if (force_kernel == 1 || K % 128 || (uint64_t)K * 256 > 0x7FFFFFFFull || N % 8 || ldd % 8 ||
       ((uintptr_t)d & 15) || (uint64_t)ldd * 512 > 0x7FFFFFFFull) return launch_dense<256, 256>(p, st);
   return launch_gemm_nt32(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd, st);
