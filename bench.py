@@ -33,7 +33,7 @@ PEAK_MXFP8_TFLOPS = 5000.0  # MI355X dense fp8 / MXFP8 MFMA peak
 PEAK_HBM_GBPS = 8000.0
 # Bytes the GEMM kernel moves between L2 and the memory fabric per launch, mean over the step's
 # nine GEMMs: rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the same counter reads for a
-# known-size elementwise kernel (profiles/bench_ffn_M16384__hbm_traffic_pmc.txt).  Counters cannot
+# known-size elementwise kernel (profiles/gemm_nt32_kernel_and_cast_tile_kernel__ffn_fwd_bwd_M16384__hbm_traffic_pmc.txt).  Counters cannot
 # be read from inside this process, so the figure is carried here and re-measured when the kernel
 # changes.
 GEMM_TRAFFIC_BYTES_PER_LAUNCH = 1819200742
