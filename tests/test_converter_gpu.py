@@ -166,3 +166,58 @@ def test_grouped_experts_swiglu_block(device):
         assert rel_l2(ya.detach().float().cpu().numpy(), yb.detach().float().cpu().numpy()) < 0.1
     finally:
         moe_mod.set_token_group_alignment_size_m(8)
+
+
+class _MiniDecoderBlock(nn.Module):
+    """Llama-style block in small: RMSNorm, GQA attention with RoPE-free SDPA in bf16, SwiGLU FFN.
+    The seven linears are the `Linear` modules the converter selects by FQN."""
+
+    def __init__(self, dim, heads, kv_heads, ffn):
+        super().__init__()
+        self.heads, self.kv_heads, self.hd = heads, kv_heads, dim // heads
+        self.attention = nn.Module()
+        mk = lambda i, o: Linear.Config().build(in_features=i, out_features=o)
+        self.attention.wq = mk(dim, dim)
+        self.attention.wk = mk(dim, kv_heads * self.hd)
+        self.attention.wv = mk(dim, kv_heads * self.hd)
+        self.attention.wo = mk(dim, dim)
+        self.feed_forward = FeedForward.Config(hidden_dim=ffn).build(dim=dim)
+        self.n1 = nn.RMSNorm(dim, eps=1e-5)
+        self.n2 = nn.RMSNorm(dim, eps=1e-5)
+
+    def forward(self, x):
+        B, S, D = x.shape
+        h = self.n1(x)
+        q = self.attention.wq(h).view(B, S, self.heads, self.hd).transpose(1, 2)
+        k = self.attention.wk(h).view(B, S, self.kv_heads, self.hd).transpose(1, 2)
+        v = self.attention.wv(h).view(B, S, self.kv_heads, self.hd).transpose(1, 2)
+        rep = self.heads // self.kv_heads
+        k, v = k.repeat_interleave(rep, dim=1), v.repeat_interleave(rep, dim=1)
+        a = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True)
+        x = x + self.attention.wo(a.transpose(1, 2).reshape(B, S, D))
+        return x + self.feed_forward(self.n2(x))
+
+
+def test_decoder_block_with_all_seven_linears_converted(device):
+    """The converter drops into a whole block: same module tree, every linear selected by FQN,
+    output and gradients close to the unconverted bf16 block, parameters still trainable."""
+    torch.manual_seed(7)
+    blk = _MiniDecoderBlock(256, 4, 2, 512).to(device).to(torch.bfloat16)
+    for m in blk.modules():
+        if isinstance(m, nn.Linear):
+            nn.init.normal_(m.weight, std=0.02)
+    ref = _MiniDecoderBlock(256, 4, 2, 512).to(device).to(torch.bfloat16)
+    ref.load_state_dict(blk.state_dict())
+    _convert(blk, ["attention", "feed_forward"])
+    wrapped = [n for n, p in blk.named_parameters() if isinstance(p, MXFP8TrainingWeight)]
+    assert len(wrapped) == 7
+    x = torch.randn(1, 256, 256, device=device, dtype=torch.bfloat16)
+    xa, xb = x.clone().requires_grad_(True), x.clone().requires_grad_(True)
+    ya, yb = blk(xa), ref(xb)
+    ya.float().pow(2).mean().backward()
+    yb.float().pow(2).mean().backward()
+    assert rel_l2(ya.detach().float().cpu().numpy(), yb.detach().float().cpu().numpy()) < 0.05
+    assert rel_l2(xa.grad.float().cpu().numpy(), xb.grad.float().cpu().numpy()) < 0.1
+    for (n, pa), (_, pb) in zip(blk.named_parameters(), ref.named_parameters()):
+        if pa.ndim == 2:
+            assert rel_l2(pa.grad.float().cpu().numpy(), pb.grad.float().cpu().numpy()) < 0.15, n
