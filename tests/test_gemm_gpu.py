@@ -164,3 +164,20 @@ def test_config1_full_size_against_the_oracle(device):
         wc, ws = co.cast_dim0(w_bits, mode)
         ref = mo.f32_to_bf16_bits(co.dequant(xc, xs) @ co.dequant(wc, ws).T)
         assert rel_l2(_f32(bits_of(y)), _f32(ref)) <= TOL
+
+
+@pytest.mark.parametrize("M,N,K", [(512, 384, 256), (96, 80, 64), (1024, 1000, 128)])
+def test_output_row_stride(device, M, N, K):
+    """D may be a column slice of a wider buffer (ldd > N): nothing outside the slice is touched."""
+    rng = np.random.default_rng(M + N + K)
+    a_bits = randn_bits(rng, (M, K), outliers=1e-3)
+    b_bits = randn_bits(rng, (N, K), std=0.02)
+    ac, asc = mo.cast_dim0(a_bits, mo.RCEIL)
+    bc, bsc = mo.cast_dim0(b_bits, mo.RCEIL)
+    ref = mo.mx_matmul_q(ac, asc, bc, bsc)
+    a = ops.to_mx_dim0(bf16_from_bits(a_bits, device), "rceil")
+    b = ops.to_mx_dim0(bf16_from_bits(b_bits, device), "rceil")
+    wide = torch.full((M, N + 56), 7.0, dtype=torch.bfloat16, device=device)
+    ops.mx_gemm_nt(a, b, out=wide[:, 24:24 + N])
+    assert rel_l2(_f32(bits_of(wide[:, 24:24 + N].contiguous())), _f32(ref)) <= TOL
+    assert torch.all(wide[:, :24] == 7.0) and torch.all(wide[:, 24 + N:] == 7.0)
