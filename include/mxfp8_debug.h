@@ -11,7 +11,9 @@
 extern "C" {
 #endif
 
-/* 0: pick the dense GEMM kernel by shape (default); 1: the 16x16x128 tile kernel for every shape. */
+/* 0: pick the dense GEMM kernel by shape (default); 1 / 2: the 16x16x128 tile kernel with
+ * 256x256 / 128x128 tiles for every shape; 3: the persistent 32x32x64 kernel for every shape it
+ * can take, however few tiles there are. */
 void mx_debug_force_kernel(int which);
 
 /* > 0: number of persistent workgroups of the 32x32x64 kernel, rounded up to a multiple of 8

@@ -28,7 +28,20 @@ def _f32(bits):
                                    (2048, 1024, 4096),
                                    # more tiles than workgroups, one or two K blocks per tile
                                    (4096, 4352, 128), (6144, 6400, 256)])
-def test_gemm_matches_oracle(device, M, N, K):
+@pytest.mark.parametrize("force", [0, 3])
+def test_gemm_matches_oracle(device, M, N, K, force):
+    """force 0: the kernel the library picks for the shape; 3: the persistent 32x32x64 kernel
+    wherever it can run (small shapes would otherwise go to the tile kernel)."""
+    from torchtitan_amd import _lib
+
+    _lib.load().mx_debug_force_kernel(force)
+    try:
+        _check_gemm(device, M, N, K)
+    finally:
+        _lib.load().mx_debug_force_kernel(0)
+
+
+def _check_gemm(device, M, N, K):
     rng = np.random.default_rng(M * 7 + N * 3 + K)
     a_bits = randn_bits(rng, (M, K), outliers=1e-3)
     b_bits = randn_bits(rng, (N, K), std=0.02)

@@ -56,7 +56,7 @@ int launch_gemm_nt32(const uint8_t* a_codes, const uint8_t* a_scales, const uint
                      int64_t ldd, hipStream_t st);
 }
 // 0: pick by shape; 1 / 2: the 16x16x128 tile kernel with 256x256 / 128x128 tiles for every
-// shape (kept for comparison runs)
+// shape; 3: the persistent kernel wherever it is legal (comparison runs and tests)
 static int force_kernel = 0;
 extern "C" void mx_debug_force_kernel(int which) { force_kernel = which; }
 namespace mx { void set_debug_grid(int g); }
