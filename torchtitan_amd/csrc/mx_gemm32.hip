@@ -359,6 +359,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   const uint32_t fa0 = (wm * 128 + li) * kKB + ((lj ^ sw) << 4);
   const uint32_t fb_delta = kOperand32 + (wn - wm) * 128 * kKB;
   const uint32_t lane4 = lane * 4;
+  const uint32_t v_scale = (uint32_t)(lane >> 5) * ks_n * 256 + (lane & 31) * 16;  // scale copy
   const uint32_t fsa_s = kCodes32 + wm * 512, fsb_s = kCodes32 + 1024 + wn * 512;
 
   // ---- loader stream: fills ring block `ld_slot` with K block `ld_kb` of tile `ld_tile`
@@ -379,11 +380,13 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       //  the K range is exact because nblocks is)
       ra = make_rsrc(t.a, t.rows_a * K - t.koff);
       rb = make_rsrc(t.b, t.rows_b * K - t.koff);
-      // wave 0,1 copy A's two 128-row scale groups, wave 2,3 copy B's
+      // wave 0 copies the scales of A's two 128-row groups, wave 2 those of B's (one copy per
+      // block each: lanes 0-31 fetch group 0, lanes 32-63 group 1); a group beyond the operand
+      // is cut off by the range and arrives as zeros
       const int64_t rows = wave < 2 ? t.rows_a : t.rows_b;
-      const uint8_t* sbase = (wave < 2 ? t.sa : t.sb) + (int64_t)(wave & 1) * ks_n * 256;
-      const int64_t groups_left = ((rows + 127) >> 7) - (wave & 1);
-      rs = make_rsrc(sbase, groups_left > 0 ? (int64_t)ld_nb * 512 : 0);
+      const uint8_t* sbase = wave < 2 ? t.sa : t.sb;
+      rs = make_rsrc(sbase, rows > 128 ? (int64_t)ks_n * 256 + (int64_t)ld_nb * 512
+                                       : (rows > 0 ? (int64_t)ld_nb * 512 : 0));
     } else {  // past the last tile: every lane reads out of range (zeros, no traffic)
       ld_nb = 1;
       ra = make_rsrc(p.a_codes, 0);
@@ -391,8 +394,8 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       rs = ra;
     }
   };
-  // The 18 copies of a block are issued one at a time, between MFMAs (see block_steps):
-  // piece 0..15 = unit pairs (A unit, B unit alternating), 16,17 = scales, then advance.
+  // The 17 copies of a block are issued one at a time, between MFMAs (see block_steps):
+  // piece 0..15 = unit pairs (A unit, B unit alternating), 16 = scales, then advance.
   auto issue_piece = [&](auto i_) {
     constexpr int i = decltype(i_)::value;
     const uint32_t sbase = lds_base + ld_slot * kBlock32;
@@ -407,11 +410,12 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
         __builtin_amdgcn_raw_ptr_buffer_load_lds(
             rb, (lds_void_t*)(uintptr_t)(sbase + kOperand32 + unit * 1024), 16, v, so, 0, 0);
     } else {
-      // this wave's scale group: the block's two 64-deep steps are 512 contiguous bytes
-      constexpr int h = i - 16;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          rs, (lds_void_t*)(uintptr_t)(sbase + kCodes32 + wave * 512 + h * 256), 4,
-          lane4, ld_kb * 512 + h * 256, 0, 0);
+      // scales (waves 0 and 2 only): a group's two 64-deep steps are 512 contiguous bytes, the
+      // two groups land behind one another, which is the order the fragment reads expect
+      if ((wave & 1) == 0)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            rs, (lds_void_t*)(uintptr_t)(sbase + kCodes32 + wave * 512), 16, v_scale,
+            ld_kb * 512, 0, 0);
     }
   };
   auto issue_advance = [&]() {
@@ -423,7 +427,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     ld_slot ^= 1;
   };
   auto issue_block = [&]() {
-    static_for<0, 18>([&](auto i_) { issue_piece(i_); });
+    static_for<0, 17>([&](auto i_) { issue_piece(i_); });
     issue_advance();
   };
 
@@ -496,7 +500,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   //           slots; the first half of block b+1 is read into f0 in slots 0-8.
   // The copy unit serves all four waves at about 20 cycles per copy, so four waves issuing
   // one copy per 64-cycle slot keep it saturated and the MFMAs start to wait behind them:
-  // spreading the block's 18 copies over 22 slots instead of 16 is what the second barrier
+  // spreading the block's 17 copies over 22 slots instead of 16 is what the second barrier
   // buys.  A wave issues in order and an MFMA occupies the matrix pipe for 64 cycles, so every
   // other instruction is placed in the shadow of an MFMA; the sequence is pinned with
   // scheduling fences.  (Waits are written as assembly: the compiler rewrites the immediates
@@ -576,7 +580,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
         // copies kCopiesA .. 17, one per slot, every kSkipB-th slot left free
         constexpr int j = kSkipB ? i - i / kSkipB : i;
         constexpr bool skip = kSkipB && (i % kSkipB) == kSkipB - 1;
-        if constexpr (!skip && kCopiesA + j < 18) issue_piece(std::integral_constant<int, kCopiesA + j>{});
+        if constexpr (!skip && kCopiesA + j < 17) issue_piece(std::integral_constant<int, kCopiesA + j>{});
 #endif
 #ifndef MX_ABL_NO_READ
         if constexpr (i < kReadSlots) {
