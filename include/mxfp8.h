@@ -87,6 +87,19 @@ int mx_cast_dim0_dim1_batched(const void* x, int64_t batch, int64_t rows, int64_
                               int64_t ldx, uint8_t* codes, uint8_t* scales, uint8_t* codes_t,
                               uint8_t* scales_t, int scale_mode, int scale_order, void* stream);
 
+/* SwiGLU gate fused into the cast: g = silu(a) * b elementwise over bf16 [rows, cols] (row strides
+ * lda, ldb), each step rounded to bf16 as the unfused tensor ops round it, then both casts of g
+ * as mx_cast_dim0_dim1 produces them -- g itself never travels through HBM unless `g` is given
+ * (bf16 [rows, cols] dense, may be NULL).  The sigmoid uses the hardware exp2 / reciprocal: a
+ * bf16 value of g can be one ulp off a correctly rounded one; codes and scales are exact for
+ * the g that was formed.  Requires rows % 32 == 0, cols % 32 == 0, 16-byte aligned inputs.
+ * Stands in for the activation between the two halves of the feed-forward and the casts that
+ * feed w2 (torchtitan/models/common/feed_forward.py:61-62; models/common/moe/moe.py:68-73). */
+int mx_swiglu_cast_dim0_dim1(const void* a, const void* b, int64_t rows, int64_t cols,
+                             int64_t lda, int64_t ldb, uint8_t* codes, uint8_t* scales,
+                             uint8_t* codes_t, uint8_t* scales_t, void* g, int scale_mode,
+                             int scale_order, void* stream);
+
 /* Re-order a row-major [rows, nblk] scale matrix into MX_SCALES_MFMA order
  * (the "blocked layout" step the reference leaves to torch._scaled_mm, docs/mxfp8.md:36). */
 int mx_scale_layout(const uint8_t* scales, int64_t rows, int64_t nblk, uint8_t* out, void* stream);

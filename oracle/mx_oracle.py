@@ -36,6 +36,8 @@ Pinning status (what fixes each function independently of its own formula):
   grouped variants           pinned  -- loop of mx_matmul over groups, the shape of the
                                         reference's own per-expert loop
                                         (torchtitan/models/common/moe/moe.py:24-56)
+  swiglu_bf16                pinned  -- closed form in float64; the last bf16 ulp of a
+                                        float32 evaluation is PARITY UNPINNED (see its docstring)
   generate_permute_indices   pinned  -- the worked example and invariants of
                                         torchtitan/models/common/moe/kernels.py:145-218
                                         and tests/unit_tests/test_permute_indices_kernel.py
@@ -354,6 +356,33 @@ def padded_max_len(num_tokens: int, num_experts: int, alignment: int) -> int:
 
 
 # --------------------------------------------------------------------------- inputs
+def silu_bf16(a_bits: np.ndarray) -> np.ndarray:
+    """bf16 silu as one tensor op: x / (1 + exp(-x)) evaluated in float64 with float32's range
+    (exp(-x) beyond float32 is infinite, so x below about -88.7 gives -0), rounded to bf16."""
+    with np.errstate(over="ignore", invalid="ignore"):
+        a = bf16_bits_to_f32(a_bits).astype(np.float64)
+        e = np.exp(-a).astype(np.float32).astype(np.float64)
+        s = a / (1.0 + e)
+    return f32_to_bf16_bits(s.astype(np.float32))
+
+
+def mul_bf16(x_bits: np.ndarray, y_bits: np.ndarray) -> np.ndarray:
+    """bf16 product as one tensor op: exact in float32 (8 x 8 significand bits), rounded to bf16."""
+    with np.errstate(over="ignore", invalid="ignore"):
+        return f32_to_bf16_bits(bf16_bits_to_f32(x_bits) * bf16_bits_to_f32(y_bits))
+
+
+def swiglu_bf16(a_bits: np.ndarray, b_bits: np.ndarray) -> np.ndarray:
+    """g = silu(a) * b as two bf16 tensor ops (torchtitan/models/common/feed_forward.py:61-62:
+    ``F.silu(self.w1(x)) * self.w3(x)`` on bf16 activations).
+
+    Pinning: the sigmoid is the textbook closed form in float64 and the product is exact before
+    its rounding.  A float32 evaluation of silu with a library or hardware exp can land on the
+    other side of a bf16 rounding boundary (the neighbouring bf16 value) for a few elements in
+    ten thousand: PARITY UNPINNED to that extent, and the tests bound it to exactly that."""
+    return mul_bf16(silu_bf16(a_bits), b_bits)
+
+
 def make_cfg1_inputs(seed: int, M: int = 8192, K: int = 4096, N: int = 4096):
     """Seeded N(0,1) bf16 X[M,K], W[N,K] with 0.1 % of entries scaled by 100."""
     rng = np.random.default_rng(seed)

@@ -20,9 +20,10 @@ def _f32(bits):
     return mo.bf16_bits_to_f32(bits)
 
 
-def _convert(model, fqns, recipe="mxfp8_rceil", pad=True):
+def _convert(model, fqns, recipe="mxfp8_rceil", pad=True, fuse=True):
     box = ModelConvertersContainer.Config(
-        converters=[MXFP8Converter.Config(fqns=fqns, recipe_name=recipe, pad_token_groups_for_grouped_mm=pad)]
+        converters=[MXFP8Converter.Config(fqns=fqns, recipe_name=recipe, pad_token_groups_for_grouped_mm=pad,
+                                          fuse_swiglu_cast=fuse)]
     ).build(parallel_dims=None, model_compile_enabled=False)
     box.convert(model)
     return box
@@ -97,6 +98,39 @@ def test_feed_forward_close_to_bf16_and_trains(device):
     before = ff.w1.weight.detach().clone()
     opt.step()
     assert isinstance(ff.w1.weight, MXFP8TrainingWeight) and not torch.equal(before, ff.w1.weight)
+
+
+@pytest.mark.parametrize("recipe", ["mxfp8_rceil", "mxfp8_floor"])
+@pytest.mark.parametrize("tokens,dim,hidden", [(256, 256, 512), (96, 128, 352)])
+def test_feed_forward_fused_gate_matches_separate_ops(device, recipe, tokens, dim, hidden):
+    """The SwiGLU block with the gate inside the cast kernel against the same block with silu and
+    the product as separate bf16 ops: the output and every gradient are bit-identical."""
+    torch.manual_seed(7)
+    blocks = []
+    for fuse in (True, False):
+        ff = FeedForward.Config(hidden_dim=hidden).build(dim=dim).to(device).to(torch.bfloat16)
+        if blocks:
+            ff.load_state_dict(blocks[0].feed_forward.state_dict())
+        else:
+            ff.init_weights(init_std=0.05)
+        holder = nn.Module()
+        holder.feed_forward = ff
+        _convert(holder, ["feed_forward"], recipe=recipe, fuse=fuse)
+        blocks.append(holder)
+    x = torch.randn(tokens, dim, device=device, dtype=torch.bfloat16) * 2
+    dy = torch.randn(tokens, dim, device=device, dtype=torch.bfloat16)
+    outs = []
+    for holder in blocks:
+        xi = x.clone().requires_grad_(True)
+        y = holder.feed_forward(xi)
+        y.backward(dy)
+        ff = holder.feed_forward
+        outs.append([y.detach(), xi.grad, ff.w1.weight.grad, ff.w2.weight.grad, ff.w3.weight.grad])
+    for got, want in zip(*outs):
+        assert torch.equal(got, want)
+    # the fused forward keeps no bf16 gate tensor: the graph node of y is the fused function
+    y = blocks[0].feed_forward(x.clone().requires_grad_(True))
+    assert type(y.grad_fn).__name__ == "_MXSwiGLULinearBackward"
 
 
 @pytest.mark.parametrize("pad,align", [(True, 8), (False, 32)])

@@ -56,6 +56,21 @@ def test_bf16_conversions_vs_torch():
     assert np.array_equal(mo.f32_to_bf16_bits(x), ref)
 
 
+def test_swiglu_vs_torch_bf16_ops_every_gate_input():
+    """silu over every bf16 bit pattern, and the gate product on a random pairing, against
+    torch's CPU bf16 tensor ops (the ops feed_forward.py:61-62 runs)."""
+    t = lambda bits: torch.from_numpy(bits.view(np.int16)).view(torch.bfloat16)
+    b = lambda x: x.view(torch.int16).numpy().view(np.uint16)
+    nan = lambda x: (x & 0x7FFF) > 0x7F80
+    s_ref = b(torch.nn.functional.silu(t(ALL_BF16)))
+    s = mo.silu_bf16(ALL_BF16)
+    assert np.array_equal(np.where(nan(s), 0x7FC0, s), np.where(nan(s_ref), 0x7FC0, s_ref))
+    other = np.random.default_rng(5).permutation(ALL_BF16)
+    g_ref = b(torch.nn.functional.silu(t(ALL_BF16)) * t(other))
+    g = mo.swiglu_bf16(ALL_BF16, other)
+    assert np.array_equal(np.where(nan(g), 0x7FC0, g), np.where(nan(g_ref), 0x7FC0, g_ref))
+
+
 # ------------------------------------------------------------------ scales
 def _normal_finite():
     a = ALL_BF16[(ALL_BF16 >= 0x0080) & (ALL_BF16 < 0x7F80)]

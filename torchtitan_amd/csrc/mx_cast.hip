@@ -323,6 +323,8 @@ __device__ __forceinline__ uint32_t cvt2_finite(float lo, float hi, uint32_t old
   return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(lo, hi, (int)old, HIGH);
 }
 
+typedef float v2f_t __attribute__((ext_vector_type(2)));
+typedef __bf16 v2bf_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xFFFF0000u); }
 
@@ -440,13 +442,35 @@ struct TileWalk {
   static constexpr uint32_t BY = COL ? MX_CAST_COL_BY : MX_CAST_ROW_BY;
 };
 
-template <int MODE, int ORDER, bool ROW, bool COL, int WAVES>
+// SwiGLU gate in front of the cast: g = bf16(bf16(silu(a)) * b) per element, each step rounded
+// to bf16 like the unfused bf16 tensor ops.  silu follows the float32 formula a / (1 + exp(-a))
+// with a correctly rounded quotient (hardware reciprocal plus one Newton step on the
+// remainder): the bf16 result equals torch's GPU silu for every one of the 65536 bf16 inputs.
+__device__ __forceinline__ float silu_f32(float a) {
+  // the hardware reciprocal flushes a denormal result: a denominator beyond 2^100 (a below -69)
+  // is scaled into range first; an infinite one gives a * 0 as the float32 division would
+  const float d = 1.0f + __expf(-a);
+  const float sc = d > 0x1p100f ? 0x1p-32f : 1.0f;
+  const float ds = d * sc, r = __builtin_amdgcn_rcpf(ds);
+  const float q = a * r;
+  const float e = __builtin_fmaf(-q, ds, a);  // NaN for a = +inf, +0 for a = -0: keep q then
+  const float q2 = __builtin_islessgreater(e, 0.0f) ? __builtin_fmaf(e, r, q) : q;
+  return d == __builtin_inff() ? a * 0.0f : q2 * sc;
+}
+__device__ __forceinline__ uint32_t swiglu2(uint32_t a2, uint32_t b2) {
+  const float s_lo = silu_f32(bf16_lo(a2)), s_hi = silu_f32(bf16_hi(a2));
+  const uint32_t s2 = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f_t{s_lo, s_hi}, v2bf_t));
+  const float g_lo = bf16_lo(s2) * bf16_lo(b2), g_hi = bf16_hi(s2) * bf16_hi(b2);
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f_t{g_lo, g_hi}, v2bf_t));
+}
+
+template <int MODE, int ORDER, bool ROW, bool COL, int WAVES, bool SWIGLU>
 __global__ __launch_bounds__(64 * WAVES) void cast_tile_kernel(
     const uint16_t* __restrict__ x, int64_t rows, int64_t cols, int64_t ldx,
     uint8_t* __restrict__ codes, uint8_t* __restrict__ scales, int64_t nblk, int64_t ks_n,
     uint8_t* __restrict__ codes_t, uint8_t* __restrict__ scales_t, int64_t nblk_t,
     int64_t ks_n_t, int64_t x_bstride, int64_t s_bstride, int64_t st_bstride, uint32_t gx,
-    uint32_t gy) {
+    uint32_t gy, const uint16_t* __restrict__ x3, int64_t ldx3, uint16_t* __restrict__ g_out) {
   constexpr int TR = 32 * WAVES, TC = 128, PITCH = TR + 16;
   __shared__ __attribute__((aligned(16))) uint8_t lds_codes[COL ? TC * PITCH : 16];
   __shared__ __attribute__((aligned(16))) uint8_t lds_st[COL ? TC * WAVES : 16];
@@ -484,6 +508,23 @@ __global__ __launch_bounds__(64 * WAVES) void cast_tile_kernel(
       v[k] = u32x4{0, 0, 0, 0};
       if (col_ok && k < rows_left)
         v[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + k * ldx));
+    }
+  }
+  if constexpr (SWIGLU) {  // x = gate input a, x3 = b: quantize g = silu(a) * b
+    const uint16_t* src3 = x3 + (r0 + rl0) * ldx3 + c;
+    u32x4 b[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      b[k] = u32x4{0, 0, 0, 0};
+      if (col_ok && k < rows_left)
+        b[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src3 + k * ldx3));
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      v[k] = u32x4{swiglu2(v[k].x, b[k].x), swiglu2(v[k].y, b[k].y), swiglu2(v[k].z, b[k].z),
+                   swiglu2(v[k].w, b[k].w)};
+      if (g_out && col_ok && k < rows_left)
+        *reinterpret_cast<u32x4*>(g_out + (r0 + rl0 + k) * cols + c) = v[k];
     }
   }
 
@@ -648,23 +689,23 @@ using namespace mx;
 #ifndef MX_CAST_WAVES
 #define MX_CAST_WAVES 4
 #endif
-#define MX_DISPATCH_TILE(ROW, COL, ...)                                                          \
+#define MX_DISPATCH_TILE(ROW, COL, SWIGLU, ...)                                                         \
   do {                                                                                           \
     if (scale_mode == MX_SCALE_FLOOR && scale_order == MX_SCALES_ROWMAJOR)                       \
       hipLaunchKernelGGL(                                                                        \
-          (cast_tile_kernel<MX_SCALE_FLOOR, MX_SCALES_ROWMAJOR, ROW, COL, MX_CAST_WAVES>), grid, \
+          (cast_tile_kernel<MX_SCALE_FLOOR, MX_SCALES_ROWMAJOR, ROW, COL, MX_CAST_WAVES, SWIGLU>), grid, \
           block, 0, st, __VA_ARGS__);                                                            \
     else if (scale_mode == MX_SCALE_FLOOR)                                                       \
       hipLaunchKernelGGL(                                                                        \
-          (cast_tile_kernel<MX_SCALE_FLOOR, MX_SCALES_MFMA, ROW, COL, MX_CAST_WAVES>), grid,     \
+          (cast_tile_kernel<MX_SCALE_FLOOR, MX_SCALES_MFMA, ROW, COL, MX_CAST_WAVES, SWIGLU>), grid,     \
           block, 0, st, __VA_ARGS__);                                                            \
     else if (scale_order == MX_SCALES_ROWMAJOR)                                                  \
       hipLaunchKernelGGL(                                                                        \
-          (cast_tile_kernel<MX_SCALE_RCEIL, MX_SCALES_ROWMAJOR, ROW, COL, MX_CAST_WAVES>), grid, \
+          (cast_tile_kernel<MX_SCALE_RCEIL, MX_SCALES_ROWMAJOR, ROW, COL, MX_CAST_WAVES, SWIGLU>), grid, \
           block, 0, st, __VA_ARGS__);                                                            \
     else                                                                                         \
       hipLaunchKernelGGL(                                                                        \
-          (cast_tile_kernel<MX_SCALE_RCEIL, MX_SCALES_MFMA, ROW, COL, MX_CAST_WAVES>), grid,     \
+          (cast_tile_kernel<MX_SCALE_RCEIL, MX_SCALES_MFMA, ROW, COL, MX_CAST_WAVES, SWIGLU>), grid,     \
           block, 0, st, __VA_ARGS__);                                                            \
   } while (0)
 
@@ -724,9 +765,10 @@ extern "C" int mx_cast_dim0(const void* x, int64_t rows, int64_t cols, int64_t l
   if (scale_order == MX_SCALES_MFMA && tile_grid_x(tgx, tgy, false) <= 0x7FFFFFFF) {
     // scattered scale bytes cost more than the tiled read: stage them through LDS
     dim3 grid = tile_grid(tgx, tgy, 1, false), block(64 * MX_CAST_WAVES);
-    MX_DISPATCH_TILE(true, false, (const uint16_t*)x, rows, cols, ldx, codes, scales, nblk, ks_n,
-                     (uint8_t*)nullptr, (uint8_t*)nullptr, (int64_t)0, (int64_t)0, (int64_t)0,
-                     (int64_t)0, (int64_t)0, (uint32_t)tgx, (uint32_t)tgy);
+    MX_DISPATCH_TILE(true, false, false, (const uint16_t*)x, rows, cols, ldx, codes, scales, nblk,
+                     ks_n, (uint8_t*)nullptr, (uint8_t*)nullptr, (int64_t)0, (int64_t)0, (int64_t)0,
+                     (int64_t)0, (int64_t)0, (uint32_t)tgx, (uint32_t)tgy, (const uint16_t*)nullptr,
+                     (int64_t)0, (uint16_t*)nullptr);
     return launch_status();
   }
   clear_mfma_padding(scales, rows, nblk, scale_order, st);
@@ -758,9 +800,10 @@ extern "C" int mx_cast_dim1_batched(const void* x, int64_t batch, int64_t rows, 
   const int64_t tgy = (rows + kTileRows - 1) / kTileRows;
   if (tile_ok(x, cols, ldx) && tile_grid_x(gx, tgy, true) <= 0x7FFFFFFF) {
     dim3 grid = tile_grid(gx, tgy, batch, true), block(64 * MX_CAST_WAVES);
-    MX_DISPATCH_TILE(false, true, (const uint16_t*)x, rows, cols, ldx, (uint8_t*)nullptr,
+    MX_DISPATCH_TILE(false, true, false, (const uint16_t*)x, rows, cols, ldx, (uint8_t*)nullptr,
                      (uint8_t*)nullptr, (int64_t)0, (int64_t)0, codes_t, scales_t, nblk_t, ks_n_t,
-                     rows * ldx, (int64_t)0, st_b, (uint32_t)gx, (uint32_t)tgy);
+                     rows * ldx, (int64_t)0, st_b, (uint32_t)gx, (uint32_t)tgy,
+                     (const uint16_t*)nullptr, (int64_t)0, (uint16_t*)nullptr);
     return launch_status();
   }
   dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch), block(256);
@@ -799,9 +842,9 @@ extern "C" int mx_cast_dim0_dim1_batched(const void* x, int64_t batch, int64_t r
   if (tile_ok(x, cols, ldx) && ((uintptr_t)codes & 7) == 0 && ((uintptr_t)scales & 3) == 0 &&
       tile_grid_x(gx, tgy, true) <= 0x7FFFFFFF) {
     dim3 grid = tile_grid(gx, tgy, batch, true), block(64 * MX_CAST_WAVES);
-    MX_DISPATCH_TILE(true, true, (const uint16_t*)x, rows, cols, ldx, codes, scales, nblk, ks_n,
-                     codes_t, scales_t, nblk_t, ks_n_t, rows * ldx, s_b, st_b, (uint32_t)gx,
-                     (uint32_t)tgy);
+    MX_DISPATCH_TILE(true, true, false, (const uint16_t*)x, rows, cols, ldx, codes, scales, nblk,
+                     ks_n, codes_t, scales_t, nblk_t, ks_n_t, rows * ldx, s_b, st_b, (uint32_t)gx,
+                     (uint32_t)tgy, (const uint16_t*)nullptr, (int64_t)0, (uint16_t*)nullptr);
     return launch_status();
   }
   dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch), block(256);
@@ -852,5 +895,29 @@ extern "C" int mx_scale_unlayout(const uint8_t* laid, int64_t rows, int64_t nblk
   const int64_t n = rows * nblk;
   hipLaunchKernelGGL(scale_unlayout_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
                      (hipStream_t)stream, laid, rows, nblk, ks_n, out);
+  return launch_status();
+}
+
+extern "C" int mx_swiglu_cast_dim0_dim1(const void* a, const void* b, int64_t rows, int64_t cols,
+                                        int64_t lda, int64_t ldb, uint8_t* codes, uint8_t* scales,
+                                        uint8_t* codes_t, uint8_t* scales_t, void* g,
+                                        int scale_mode, int scale_order, void* stream) {
+  if (rows < 0 || cols < 0 || lda < cols || ldb < cols || bad_enums(scale_mode, scale_order))
+    return MX_ERR_INVALID_ARG;
+  if (rows == 0 || cols == 0) return MX_OK;
+  if (!a || !b || !codes || !scales || !codes_t || !scales_t) return MX_ERR_INVALID_ARG;
+  if (rows % 32 || cols % 32 || lda % 8 || ldb % 8 || ((uintptr_t)a & 15) || ((uintptr_t)b & 15) ||
+      ((uintptr_t)codes & 7) || ((uintptr_t)codes_t & 15) || ((uintptr_t)scales & 3) ||
+      ((uintptr_t)scales_t & 3) || ((uintptr_t)g & 15))
+    return MX_ERR_ALIGNMENT;
+  const int64_t nblk = cols / 32, ks_n = (nblk + 1) / 2;
+  const int64_t nblk_t = rows / 32, ks_n_t = (nblk_t + 1) / 2;
+  const int64_t gx = (cols + kT - 1) / kT, tgy = (rows + kTileRows - 1) / kTileRows;
+  if (tile_grid_x(gx, tgy, true) > 0x7FFFFFFF) return MX_ERR_UNSUPPORTED;
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid = tile_grid(gx, tgy, 1, true), block(64 * MX_CAST_WAVES);
+  MX_DISPATCH_TILE(true, true, true, (const uint16_t*)a, rows, cols, lda, codes, scales, nblk, ks_n,
+                   codes_t, scales_t, nblk_t, ks_n_t, (int64_t)0, (int64_t)0, (int64_t)0,
+                   (uint32_t)gx, (uint32_t)tgy, (const uint16_t*)b, ldb, (uint16_t*)g);
   return launch_status();
 }

@@ -4,6 +4,7 @@ from dataclasses import dataclass, field
 import torch
 import torch.nn.functional as F
 
+from ..mx_tensor import mx_swiglu_linear, swiglu_fusable
 from ..protocols import Module
 from .linear import Linear
 
@@ -32,7 +33,10 @@ class FeedForward(Module):
         self.w3 = lin.build(in_features=config.dim, out_features=config.hidden_dim)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return self.w2(F.silu(self.w1(x)) * self.w3(x))
+        h1, h3 = self.w1(x), self.w3(x)
+        if swiglu_fusable(h1, h3, self.w2.weight):  # converted w2: gate inside the MXFP8 cast
+            return mx_swiglu_linear(h1, h3, self.w2.weight, self.w2.bias)
+        return self.w2(F.silu(h1) * h3)
 
     def init_weights(self, init_std: float = 0.02, **kwargs):
         self.w1.init_weights()

@@ -28,13 +28,15 @@ from .ops import MX_SCALES_MFMA, MX_SCALES_ROWMAJOR, MXData
 class MXFP8Config:
     """Per-weight recipe: scale mode and whether grouped GEMMs pad token groups to 32."""
 
-    __slots__ = ("scale_mode", "pad_token_groups_for_grouped_mm")
+    __slots__ = ("scale_mode", "pad_token_groups_for_grouped_mm", "fuse_swiglu_cast")
 
-    def __init__(self, scale_mode: str = "rceil", pad_token_groups_for_grouped_mm: bool = True):
+    def __init__(self, scale_mode: str = "rceil", pad_token_groups_for_grouped_mm: bool = True,
+                 fuse_swiglu_cast: bool = True):
         if scale_mode not in ops.SCALE_MODES:
             raise ValueError(f"unknown scale mode {scale_mode!r}")
         self.scale_mode = scale_mode
         self.pad_token_groups_for_grouped_mm = pad_token_groups_for_grouped_mm
+        self.fuse_swiglu_cast = fuse_swiglu_cast
 
     def __repr__(self):
         return (f"MXFP8Config(scale_mode={self.scale_mode!r}, "
@@ -191,6 +193,95 @@ def mx_linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, 
         y = y.to(out_dtype)
     if bias is not None:
         y = y + bias.to(y.dtype)
+    return y
+
+
+# ----------------------------------------------------------------------------- SwiGLU + linear
+class _MXSwiGLULinear(torch.autograd.Function):
+    """y = (silu(h1) * h3) W^T with the gate formed inside the cast kernel: g is never written
+    to memory in forward and only its column-wise MXFP8 form is kept for wgrad.  Backward
+    returns the gradients the unfused bf16 ops would (silu and the products rounded to bf16
+    tensor by tensor, torchtitan/models/common/feed_forward.py:61-62 under autograd)."""
+
+    @staticmethod
+    def forward(ctx, h1, h3, weight, cfg: MXFP8Config):
+        mode = cfg.scale_mode
+        H, N = h1.shape[-1], weight.shape[0]
+        a, b = h1.reshape(-1, H), h3.reshape(-1, H)
+        w = weight if weight.dtype == torch.bfloat16 else weight.to(torch.bfloat16)
+        gq0, gq1, _ = ops.swiglu_to_mx_dim0_dim1(a, b, mode, MX_SCALES_MFMA)
+        need_dh = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
+        if need_dh and N % ops.BLOCK == 0:
+            wq0, wq1 = ops.to_mx_dim0_dim1(w, mode, MX_SCALES_MFMA)
+        else:
+            wq0, wq1 = ops.to_mx_dim0(w, mode, MX_SCALES_MFMA), None
+        y = ops.mx_gemm_nt(gq0, wq0)
+        ctx.cfg, ctx.w_dtype, ctx.have_wq1 = cfg, weight.dtype, wq1 is not None
+        saved = [h1, h3]
+        if ctx.needs_input_grad[2]:
+            saved += [gq1.codes, gq1.scales]
+        if need_dh:
+            saved += [wq1.codes, wq1.scales] if wq1 is not None else [w]
+        ctx.save_for_backward(*saved)
+        return y.view(*h1.shape[:-1], N)
+
+    @staticmethod
+    def backward(ctx, dy):
+        mode = ctx.cfg.scale_mode
+        need_dh = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
+        need_dw = ctx.needs_input_grad[2]
+        saved = list(ctx.saved_tensors)
+        h1, h3 = saved.pop(0), saved.pop(0)
+        N = dy.shape[-1]
+        dy2 = dy.reshape(-1, N)
+        if dy2.dtype != torch.bfloat16:
+            dy2 = dy2.to(torch.bfloat16)
+        dy2 = dy2.contiguous()
+        gq1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA) if need_dw else None
+        wq1 = None
+        if need_dh:
+            if ctx.have_wq1:
+                wq1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
+            else:
+                wq1 = _cast_cols_padded(saved.pop(0), mode)
+        if need_dh and need_dw and N % ops.BLOCK == 0:
+            dyq0, dyq1 = ops.to_mx_dim0_dim1(dy2, mode, MX_SCALES_MFMA)
+        else:
+            dyq0 = _cast_rows_padded(dy2, mode) if need_dh else None
+            dyq1 = ops.to_mx_dim1(dy2, mode, MX_SCALES_MFMA) if need_dw else None
+        dh1 = dh3 = dw = None
+        if need_dh:
+            dg = ops.mx_gemm_nt(dyq0, wq1).view(h1.shape)
+            if ctx.needs_input_grad[1]:
+                dh3 = dg * F.silu(h1)
+            if ctx.needs_input_grad[0]:
+                dh1 = torch.ops.aten.silu_backward(dg * h3, h1)
+        if need_dw:
+            dw = ops.mx_gemm_nt(dyq1, gq1)
+            if dw.dtype != ctx.w_dtype:
+                dw = dw.to(ctx.w_dtype)
+        return dh1, dh3, dw, None
+
+
+def swiglu_fusable(h1: torch.Tensor, h3: torch.Tensor, weight: torch.Tensor) -> bool:
+    """The fused gate + cast needs bf16 row-contiguous inputs of one shape with 32-aligned token
+    and hidden counts (what a converted SwiGLU block produces) and a converted weight."""
+    if not isinstance(weight, MXFP8TrainingWeight) or not weight.mx_config.fuse_swiglu_cast:
+        return False
+    if h1.dtype != torch.bfloat16 or h3.dtype != torch.bfloat16 or h1.shape != h3.shape:
+        return False
+    H = h1.shape[-1]
+    return (h1.is_contiguous() and h3.is_contiguous() and h1.is_cuda and H % ops.BLOCK == 0
+            and h1.numel() // max(H, 1) % ops.BLOCK == 0 and h1.numel() > 0)
+
+
+def mx_swiglu_linear(h1: torch.Tensor, h3: torch.Tensor, weight: torch.Tensor,
+                     bias: torch.Tensor | None = None):
+    """``F.linear(F.silu(h1) * h3, weight, bias)`` for a converted weight, with the gate computed
+    inside the MXFP8 cast.  Callers check `swiglu_fusable` first."""
+    y = _MXSwiGLULinear.apply(h1, h3, _unwrap(weight), weight.mx_config)
+    if bias is not None:
+        y = y + _unwrap(bias).to(y.dtype)
     return y
 
 

@@ -149,6 +149,27 @@ def to_mx_dim0_dim1(x: torch.Tensor, mode="floor", order: int = MX_SCALES_ROWMAJ
     return MXData(codes, scales, order), MXData(codes_t, scales_t, order)
 
 
+def swiglu_to_mx_dim0_dim1(a: torch.Tensor, b: torch.Tensor, mode="floor",
+                           order: int = MX_SCALES_ROWMAJOR, want_g: bool = False):
+    """Both casts of g = silu(a) * b (bf16, every step rounded to bf16) without g passing through
+    memory; returns (row-wise MXData, column-wise MXData, g or None)."""
+    a, b = _check_hp(a), _check_hp(b)
+    if a.shape != b.shape:
+        raise ValueError(f"shape mismatch: {tuple(a.shape)} vs {tuple(b.shape)}")
+    R, C = a.shape
+    if R % BLOCK or C % BLOCK:
+        raise ValueError(f"both dims of {tuple(a.shape)} must be multiples of {BLOCK}")
+    codes = torch.empty((R, C), dtype=torch.uint8, device=a.device)
+    scales = _alloc_scales(R, C // BLOCK, order, a.device)
+    codes_t = torch.empty((C, R), dtype=torch.uint8, device=a.device)
+    scales_t = _alloc_scales(C, R // BLOCK, order, a.device)
+    g = torch.empty((R, C), dtype=torch.bfloat16, device=a.device) if want_g else None
+    _call("mx_swiglu_cast_dim0_dim1", "swiglu_cast_dim0_dim1", a.device, _ptr(a), _ptr(b), R, C,
+          a.stride(0), b.stride(0), _ptr(codes), _ptr(scales), _ptr(codes_t), _ptr(scales_t),
+          _ptr(g) if g is not None else None, _mode(mode), order, _stream(a))
+    return MXData(codes, scales, order), MXData(codes_t, scales_t, order), g
+
+
 def scale_layout(scales: torch.Tensor) -> torch.Tensor:
     """Row-major [rows, nblk] scales -> flat buffer in MFMA order."""
     rows, nblk = scales.shape

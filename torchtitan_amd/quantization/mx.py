@@ -62,6 +62,13 @@ class MXFP8Converter(QuantizationConverter):
         """Pad token groups to multiples of 32 inside the grouped GEMM.  Set to false when the
         dispatcher already delivers 32-aligned groups."""
 
+        fuse_swiglu_cast: bool = True
+        """Not in the reference's Config.  A SwiGLU block whose w2 is converted forms
+        silu(w1 x) * w3 x inside the cast kernel that feeds w2 (one pass over the two
+        projections instead of three elementwise passes and a cast).  The bf16 gate value can
+        differ from the unfused ops' by one rounding step at a few elements in ten thousand;
+        false keeps the three separate ops."""
+
     def __init__(self, config: Config, *, parallel_dims: Any, model_compile_enabled: bool):
         self.enabled = False
         if not _lib.LIB_PATH.exists():
@@ -89,7 +96,8 @@ class MXFP8Converter(QuantizationConverter):
         verify_module_protocol(model, nn.Linear, Linear)
         saved = capture_module_attrs(model, ["_init_mean", "_init_std"], nn_module_cls=nn.Linear)
         cfg = MXFP8Config(_RECIPES[self.config.recipe_name],
-                          self.config.pad_token_groups_for_grouped_mm)
+                          self.config.pad_token_groups_for_grouped_mm,
+                          self.config.fuse_swiglu_cast)
         n_linear = n_grouped = 0
         for fqn, mod in model.named_modules():
             if not self._matches(fqn):
