@@ -90,15 +90,31 @@ int mx_cast_dim0_dim1_batched(const void* x, int64_t batch, int64_t rows, int64_
 /* SwiGLU gate fused into the cast: g = silu(a) * b elementwise over bf16 [rows, cols] (row strides
  * lda, ldb), each step rounded to bf16 as the unfused tensor ops round it, then both casts of g
  * as mx_cast_dim0_dim1 produces them -- g itself never travels through HBM unless `g` is given
- * (bf16 [rows, cols] dense, may be NULL).  The sigmoid uses the hardware exp2 / reciprocal: a
- * bf16 value of g can be one ulp off a correctly rounded one; codes and scales are exact for
- * the g that was formed.  Requires rows % 32 == 0, cols % 32 == 0, 16-byte aligned inputs.
+ * (bf16 [rows, cols] dense, may be NULL).  silu is a / (1 + exp(-a)) in float32 with a
+ * correctly rounded quotient: its bf16 value equals the GPU tensor op's for every bf16 input.
+ * Requires rows % 32 == 0, cols % 32 == 0, lda % 8 == 0, ldb % 8 == 0, 16-byte aligned inputs.
  * Stands in for the activation between the two halves of the feed-forward and the casts that
  * feed w2 (torchtitan/models/common/feed_forward.py:61-62; models/common/moe/moe.py:68-73). */
 int mx_swiglu_cast_dim0_dim1(const void* a, const void* b, int64_t rows, int64_t cols,
                              int64_t lda, int64_t ldb, uint8_t* codes, uint8_t* scales,
                              uint8_t* codes_t, uint8_t* scales_t, void* g, int scale_mode,
                              int scale_order, void* stream);
+
+/* Backward of that gate fused into the casts that feed the dgrad and wgrad GEMMs of w1 and w3:
+ * from dg, a, b (bf16 [rows, cols], row strides lddg, lda, ldb) forms, as bf16 autograd does
+ * tensor op by tensor op,
+ *     da = silu_backward(bf16(dg * b), a),   db = bf16(dg * bf16(silu(a)))
+ * and writes both casts of each.  Every output holds da's part followed by db's part:
+ * codes [2, rows, cols], codes_t [2, cols, rows], scales and scales_t two buffers of the size a
+ * single cast would use, back to back.  `dab` (bf16 [2, rows, cols], may be NULL) receives da and
+ * db themselves.  Same shape and alignment rules as mx_swiglu_cast_dim0_dim1.
+ * Stands in for the autograd nodes of feed_forward.py:61-62 (mul, silu) and the casts of their
+ * results under the converted w1 / w3. */
+int mx_swiglu_bwd_cast_dim0_dim1(const void* dg, const void* a, const void* b, int64_t rows,
+                                 int64_t cols, int64_t lddg, int64_t lda, int64_t ldb,
+                                 uint8_t* codes, uint8_t* scales, uint8_t* codes_t,
+                                 uint8_t* scales_t, void* dab, int scale_mode, int scale_order,
+                                 void* stream);
 
 /* Re-order a row-major [rows, nblk] scale matrix into MX_SCALES_MFMA order
  * (the "blocked layout" step the reference leaves to torch._scaled_mm, docs/mxfp8.md:36). */

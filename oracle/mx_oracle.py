@@ -38,6 +38,8 @@ Pinning status (what fixes each function independently of its own formula):
                                         (torchtitan/models/common/moe/moe.py:24-56)
   swiglu_bf16                pinned  -- closed form in float64; the last bf16 ulp of a
                                         float32 evaluation is PARITY UNPINNED (see its docstring)
+  swiglu_backward_bf16       pinned  -- closed form vs a central difference and torch's CPU op;
+                                        last bf16 ulp of da PARITY UNPINNED (see its docstring)
   generate_permute_indices   pinned  -- the worked example and invariants of
                                         torchtitan/models/common/moe/kernels.py:145-218
                                         and tests/unit_tests/test_permute_indices_kernel.py
@@ -381,6 +383,25 @@ def swiglu_bf16(a_bits: np.ndarray, b_bits: np.ndarray) -> np.ndarray:
     other side of a bf16 rounding boundary (the neighbouring bf16 value) for a few elements in
     ten thousand: PARITY UNPINNED to that extent, and the tests bound it to exactly that."""
     return mul_bf16(silu_bf16(a_bits), b_bits)
+
+
+def swiglu_backward_bf16(dg_bits: np.ndarray, a_bits: np.ndarray, b_bits: np.ndarray):
+    """(da, db) of g = silu(a) * b as bf16 autograd forms them (feed_forward.py:61-62 under
+    autograd): the product node gives db = bf16(dg * silu_bf16(a)) and t = bf16(dg * b); the silu
+    node gives da = bf16(t * s * (1 + a * (1 - s))), s = 1 / (1 + exp(-a)), evaluated here in
+    float64 with float32's exp range.
+
+    Pinning: db is exact given silu_bf16; da is the closed form of d silu / da (checked against
+    a central difference and torch's CPU op in the tests); its last bf16 ulp under a float32
+    evaluation is PARITY UNPINNED, as for silu_bf16."""
+    db = mul_bf16(dg_bits, silu_bf16(a_bits))
+    t = bf16_bits_to_f32(mul_bf16(dg_bits, b_bits)).astype(np.float64)
+    with np.errstate(over="ignore", invalid="ignore"):
+        a = bf16_bits_to_f32(a_bits).astype(np.float64)
+        e = np.exp(-a).astype(np.float32).astype(np.float64)
+        s = 1.0 / (1.0 + e)
+        da = t * s * (1.0 + a * (1.0 - s))
+        return f32_to_bf16_bits(da.astype(np.float32)), db
 
 
 def make_cfg1_inputs(seed: int, M: int = 8192, K: int = 4096, N: int = 4096):

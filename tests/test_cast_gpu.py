@@ -217,3 +217,56 @@ def test_swiglu_gate_every_bf16_input(device):
     want = torch.nn.functional.silu(a) * b
     both_nan = torch.isnan(g) & torch.isnan(want)
     assert torch.equal(g.view(torch.int16)[~both_nan], want.view(torch.int16)[~both_nan])
+
+
+def _equal_or_nan(got, want):
+    both_nan = torch.isnan(got) & torch.isnan(want)
+    return torch.equal(got.view(torch.int16)[~both_nan], want.view(torch.int16)[~both_nan])
+
+
+@pytest.mark.parametrize("mode_name,mode", MODES)
+@pytest.mark.parametrize("shape", [(32, 32), (160, 224), (256, 384), (1024, 768)])
+def test_swiglu_backward_fused_cast(device, mode_name, mode, shape):
+    """Gate backward fused in front of four casts: gradients within the oracle's bound (db exact,
+    da equal or the neighbouring bf16 value at a few elements in ten thousand) and bit-identical
+    to torch's GPU autograd of the two bf16 ops; codes and scales exact for those gradients."""
+    rng = np.random.default_rng(shape[0] * 7 + shape[1])
+    a_bits = randn_bits(rng, shape, std=2.0, outliers=1e-3)
+    b_bits = randn_bits(rng, shape, std=1.0)
+    dg_bits = randn_bits(rng, shape, std=0.5, outliers=1e-3)
+    a, b, dg = (bf16_from_bits(x, device) for x in (a_bits, b_bits, dg_bits))
+    ta, tb = a.clone().requires_grad_(True), b.clone().requires_grad_(True)
+    (torch.nn.functional.silu(ta) * tb).backward(dg)
+    da_o, db_o = mo.swiglu_backward_bf16(dg_bits, a_bits, b_bits)
+    for order in (ops.MX_SCALES_ROWMAJOR, ops.MX_SCALES_MFMA):
+        qa, qb, grads = ops.swiglu_bwd_to_mx_dim0_dim1(dg, a, b, mode_name, order, want_grads=True)
+        assert _equal_or_nan(grads[0], ta.grad) and _equal_or_nan(grads[1], tb.grad)
+        da_bits, db_bits = bits_of(grads[0]), bits_of(grads[1])
+        nan = lambda x: (x & 0x7FFF) > 0x7F80
+        assert ((db_bits == db_o) | (nan(db_bits) & nan(db_o))).all()
+        off = (da_bits != da_o) & ~(nan(da_bits) & nan(da_o))
+        assert off.mean() <= 2e-3
+        assert (np.abs(da_bits[off].astype(np.int32) - da_o[off].astype(np.int32)) <= 1).all()
+        for (q0, q1), bits in ((qa, da_bits), (qb, db_bits)):
+            c0, s0 = mo.cast_dim0(bits, mode)
+            c1, s1 = mo.cast_dim1(bits, mode)
+            if order == ops.MX_SCALES_MFMA:
+                s0, s1 = mo.scale_layout(s0), mo.scale_layout(s1)
+            assert np.array_equal(u8(q0.codes), c0) and np.array_equal(u8(q0.scales).reshape(-1), s0.reshape(-1))
+            assert np.array_equal(u8(q1.codes), c1) and np.array_equal(u8(q1.scales).reshape(-1), s1.reshape(-1))
+        pa, pb, none = ops.swiglu_bwd_to_mx_dim0_dim1(dg, a, b, mode_name, order)
+        assert none is None and torch.equal(pa[0].codes, qa[0].codes) and torch.equal(pb[1].codes, qb[1].codes)
+        assert torch.equal(pa[1].scales, qa[1].scales) and torch.equal(pb[0].scales, qb[0].scales)
+
+
+def test_swiglu_backward_every_bf16_gate_input(device):
+    """Every bf16 bit pattern as the gate input, against torch's GPU autograd."""
+    rng = np.random.default_rng(78)
+    a = bf16_from_bits(np.arange(65536, dtype=np.uint16).reshape(256, 256), device)
+    for std in (1.0, 30.0):
+        b = bf16_from_bits(randn_bits(rng, (256, 256), std=std), device)
+        dg = bf16_from_bits(randn_bits(rng, (256, 256), std=std), device)
+        ta, tb = a.clone().requires_grad_(True), b.clone().requires_grad_(True)
+        (torch.nn.functional.silu(ta) * tb).backward(dg)
+        _, _, grads = ops.swiglu_bwd_to_mx_dim0_dim1(dg, a, b, "rceil", ops.MX_SCALES_MFMA, want_grads=True)
+        assert _equal_or_nan(grads[0], ta.grad) and _equal_or_nan(grads[1], tb.grad)

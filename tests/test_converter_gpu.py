@@ -130,7 +130,64 @@ def test_feed_forward_fused_gate_matches_separate_ops(device, recipe, tokens, di
         assert torch.equal(got, want)
     # the fused forward keeps no bf16 gate tensor: the graph node of y is the fused function
     y = blocks[0].feed_forward(x.clone().requires_grad_(True))
+    assert type(y.grad_fn).__name__ == "_MXFeedForwardBackward"
+
+
+def test_feed_forward_with_only_w2_converted_fuses_the_gate(device):
+    """w1 / w3 left in bf16, w2 converted: the gate still runs inside the cast that feeds w2 and
+    the block matches the same block built from separate ops bit for bit."""
+    torch.manual_seed(11)
+    blocks = []
+    for fuse in (True, False):
+        ff = FeedForward.Config(hidden_dim=384).build(dim=128).to(device).to(torch.bfloat16)
+        if blocks:
+            ff.load_state_dict(blocks[0].feed_forward.state_dict())
+        else:
+            ff.init_weights(init_std=0.05)
+        holder = nn.Module()
+        holder.feed_forward = ff
+        _convert(holder, ["feed_forward.w2"], fuse=fuse)
+        blocks.append(holder)
+    x = torch.randn(4, 40, 128, device=device, dtype=torch.bfloat16)
+    dy = torch.randn(4, 40, 128, device=device, dtype=torch.bfloat16)
+    outs = []
+    for holder in blocks:
+        xi = x.clone().requires_grad_(True)
+        y = holder.feed_forward(xi)
+        y.backward(dy)
+        ff = holder.feed_forward
+        outs.append([y.detach(), xi.grad, ff.w1.weight.grad, ff.w2.weight.grad, ff.w3.weight.grad])
+    for got, want in zip(*outs):
+        assert torch.equal(got, want)
+    y = blocks[0].feed_forward(x.clone().requires_grad_(True))
     assert type(y.grad_fn).__name__ == "_MXSwiGLULinearBackward"
+
+
+def test_feed_forward_fused_with_frozen_parts(device):
+    """Only some inputs of the fused block require gradients."""
+    torch.manual_seed(12)
+    ff = FeedForward.Config(hidden_dim=256).build(dim=128).to(device).to(torch.bfloat16)
+    ff.init_weights(init_std=0.05)
+    ref = FeedForward.Config(hidden_dim=256).build(dim=128).to(device).to(torch.bfloat16)
+    ref.load_state_dict(ff.state_dict())
+    for m, fuse in ((ff, True), (ref, False)):
+        holder = nn.Module()
+        holder.feed_forward = m
+        _convert(holder, ["feed_forward"], fuse=fuse)
+        m.w1.weight.requires_grad_(False)
+    x = torch.randn(64, 128, device=device, dtype=torch.bfloat16)
+    dy = torch.randn(64, 128, device=device, dtype=torch.bfloat16)
+    ff(x).backward(dy)   # x needs no gradient
+    ref(x).backward(dy)
+    assert ff.w1.weight.grad is None
+    assert torch.equal(ff.w2.weight.grad, ref.w2.weight.grad) and torch.equal(ff.w3.weight.grad, ref.w3.weight.grad)
+    for m in (ff, ref):
+        for p in m.parameters():
+            p.requires_grad_(False)
+    xa, xb = x.clone().requires_grad_(True), x.clone().requires_grad_(True)
+    ff(xa).backward(dy)
+    ref(xb).backward(dy)
+    assert torch.equal(xa.grad, xb.grad)
 
 
 @pytest.mark.parametrize("pad,align", [(True, 8), (False, 32)])

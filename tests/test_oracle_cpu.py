@@ -71,6 +71,31 @@ def test_swiglu_vs_torch_bf16_ops_every_gate_input():
     assert np.array_equal(np.where(nan(g), 0x7FC0, g), np.where(nan(g_ref), 0x7FC0, g_ref))
 
 
+def test_swiglu_backward_vs_torch_autograd_and_central_difference():
+    """Gate gradients against torch's CPU bf16 autograd over every bf16 gate input (db exact; da
+    equal except where a float32 evaluation rounds to the neighbouring bf16 value), and the
+    float64 derivative inside against a central difference."""
+    t = lambda bits: torch.from_numpy(bits.view(np.int16)).view(torch.bfloat16)
+    b = lambda x: x.view(torch.int16).numpy().view(np.uint16)
+    nan = lambda x: (x & 0x7FFF) > 0x7F80
+    rng = np.random.default_rng(3)
+    dg = mo.f32_to_bf16_bits(rng.standard_normal(65536).astype(np.float32))
+    h3 = mo.f32_to_bf16_bits(rng.standard_normal(65536).astype(np.float32))
+    da, db = mo.swiglu_backward_bf16(dg, ALL_BF16, h3)
+    ta, tb = t(ALL_BF16).clone().requires_grad_(True), t(h3).clone().requires_grad_(True)
+    (torch.nn.functional.silu(ta) * tb).backward(t(dg))
+    ra, rb = b(ta.grad), b(tb.grad)
+    assert not ((db != rb) & ~(nan(db) & nan(rb))).any()
+    off = (da != ra) & ~(nan(da) & nan(ra))
+    assert off.sum() <= 4
+    assert (np.abs(da[off].astype(np.int32) - ra[off].astype(np.int32)) <= 1).all()
+    # d/da [a * sigmoid(a)] = s * (1 + a * (1 - s))
+    x = np.linspace(-20, 20, 4001)
+    silu = lambda v: v / (1 + np.exp(-v))
+    s = 1 / (1 + np.exp(-x))
+    assert np.allclose(s * (1 + x * (1 - s)), (silu(x + 1e-6) - silu(x - 1e-6)) / 2e-6, atol=1e-8)
+
+
 # ------------------------------------------------------------------ scales
 def _normal_finite():
     a = ALL_BF16[(ALL_BF16 >= 0x0080) & (ALL_BF16 < 0x7F80)]

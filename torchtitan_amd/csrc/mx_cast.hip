@@ -464,70 +464,51 @@ __device__ __forceinline__ uint32_t swiglu2(uint32_t a2, uint32_t b2) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f_t{g_lo, g_hi}, v2bf_t));
 }
 
-template <int MODE, int ORDER, bool ROW, bool COL, int WAVES, bool SWIGLU>
-__global__ __launch_bounds__(64 * WAVES) void cast_tile_kernel(
-    const uint16_t* __restrict__ x, int64_t rows, int64_t cols, int64_t ldx,
-    uint8_t* __restrict__ codes, uint8_t* __restrict__ scales, int64_t nblk, int64_t ks_n,
-    uint8_t* __restrict__ codes_t, uint8_t* __restrict__ scales_t, int64_t nblk_t,
-    int64_t ks_n_t, int64_t x_bstride, int64_t s_bstride, int64_t st_bstride, uint32_t gx,
-    uint32_t gy, const uint16_t* __restrict__ x3, int64_t ldx3, uint16_t* __restrict__ g_out) {
+// Backward of g = silu(a) * b under bf16 autograd, tensor op by tensor op:
+//   d/db = bf16(dg * bf16(silu(a)))
+//   d/da = silu_backward(bf16(dg * b), a) = bf16(t * s * (1 + a * (1 - s))),  s = 1 / (1 + exp(-a))
+// with the float32 formula of the unfused silu backward op.
+__device__ __forceinline__ float silu_grad_f32(float t, float a) {
+  const float s = 1.0f / (1.0f + expf(-a));
+  return t * s * (1.0f + a * (1.0f - s));
+}
+__device__ __forceinline__ uint32_t swiglu_da2(uint32_t dg2, uint32_t a2, uint32_t b2) {
+  const uint32_t t2 = __builtin_bit_cast(
+      uint32_t, __builtin_convertvector(v2f_t{bf16_lo(dg2) * bf16_lo(b2), bf16_hi(dg2) * bf16_hi(b2)}, v2bf_t));
+  return __builtin_bit_cast(
+      uint32_t, __builtin_convertvector(v2f_t{silu_grad_f32(bf16_lo(t2), bf16_lo(a2)),
+                                              silu_grad_f32(bf16_hi(t2), bf16_hi(a2))}, v2bf_t));
+}
+__device__ __forceinline__ uint32_t swiglu_db2(uint32_t dg2, uint32_t a2) {
+  const uint32_t s2 = __builtin_bit_cast(
+      uint32_t, __builtin_convertvector(v2f_t{silu_f32(bf16_lo(a2)), silu_f32(bf16_hi(a2))}, v2bf_t));
+  return __builtin_bit_cast(
+      uint32_t, __builtin_convertvector(v2f_t{bf16_lo(dg2) * bf16_lo(s2), bf16_hi(dg2) * bf16_hi(s2)}, v2bf_t));
+}
+
+// 8 rows x 16 bytes of a bf16 matrix per lane; rows past `rows_left` and lanes past the last
+// column read as zero.
+__device__ __forceinline__ void load_patch(u32x4 (&v)[8], const uint16_t* src, int64_t ld,
+                                           bool col_ok, int rows_left) {
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    v[k] = u32x4{0, 0, 0, 0};
+    if (col_ok && k < rows_left)
+      v[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + k * ld));
+  }
+}
+
+// Second half of the tile kernel: block maxima, quantization and the stores of one 8 x 8 patch
+// per lane.  Ends with every wave past its reads of the shared staging buffers only after the
+// caller's next barrier.
+template <int MODE, int ORDER, bool ROW, bool COL, int WAVES>
+__device__ __forceinline__ void emit_tile(
+    u32x4 (&v)[8], uint8_t* __restrict__ codes, uint8_t* __restrict__ scales,
+    uint8_t* __restrict__ codes_t, uint8_t* __restrict__ scales_t, uint8_t* lds_codes,
+    uint8_t* lds_st, uint8_t* lds_sr, int64_t rows, int64_t cols, int64_t nblk, int64_t ks_n,
+    int64_t nblk_t, int64_t ks_n_t, int64_t r0, int64_t c0, int64_t c, int rl0, int rows_left,
+    bool col_ok, int tid, int wave, int lane) {
   constexpr int TR = 32 * WAVES, TC = 128, PITCH = TR + 16;
-  __shared__ __attribute__((aligned(16))) uint8_t lds_codes[COL ? TC * PITCH : 16];
-  __shared__ __attribute__((aligned(16))) uint8_t lds_st[COL ? TC * WAVES : 16];
-  __shared__ __attribute__((aligned(16))) uint8_t lds_sr[ROW ? TR * 4 : 16];
-  x += blockIdx.z * x_bstride;  // batch of independent [rows, cols] matrices
-  if (ROW) {
-    codes += blockIdx.z * rows * cols;
-    scales += blockIdx.z * s_bstride;
-  }
-  if (COL) {
-    codes_t += blockIdx.z * rows * cols;
-    scales_t += blockIdx.z * st_bstride;
-  }
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 4, q = lane & 15;
-  const int rl0 = wave * 32 + 8 * g;  // first tile-local row of this lane
-
-  constexpr uint32_t BX = TileWalk<COL>::BX, BY = TileWalk<COL>::BY;
-  const uint32_t spr = (gx + BX - 1) / BX;
-  const uint32_t sup = blockIdx.x / (BX * BY), in = blockIdx.x % (BX * BY);
-  const uint32_t bx = (sup % spr) * BX + in / BY;
-  const uint32_t by = (sup / spr) * BY + in % BY;
-  if (bx >= gx || by >= gy) return;
-
-  const int64_t r0 = (int64_t)by * TR, c0 = (int64_t)bx * TC;
-  const int64_t c = c0 + 8 * q;
-  const bool col_ok = c < cols;
-  const int64_t left64 = rows - (r0 + rl0);
-  const int rows_left = left64 > 8 ? 8 : (left64 < 0 ? 0 : (int)left64);
-
-  u32x4 v[8];
-  {
-    const uint16_t* src = x + (r0 + rl0) * ldx + c;
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      v[k] = u32x4{0, 0, 0, 0};
-      if (col_ok && k < rows_left)
-        v[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + k * ldx));
-    }
-  }
-  if constexpr (SWIGLU) {  // x = gate input a, x3 = b: quantize g = silu(a) * b
-    const uint16_t* src3 = x3 + (r0 + rl0) * ldx3 + c;
-    u32x4 b[8];
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      b[k] = u32x4{0, 0, 0, 0};
-      if (col_ok && k < rows_left)
-        b[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src3 + k * ldx3));
-    }
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      v[k] = u32x4{swiglu2(v[k].x, b[k].x), swiglu2(v[k].y, b[k].y), swiglu2(v[k].z, b[k].z),
-                   swiglu2(v[k].w, b[k].w)};
-      if (g_out && col_ok && k < rows_left)
-        *reinterpret_cast<u32x4*>(g_out + (r0 + rl0 + k) * cols + c) = v[k];
-    }
-  }
-
   // block maxima first: they also tell whether the wave holds any Inf / NaN
   uint32_t mr[8] = {0, 0, 0, 0, 0, 0, 0, 0}, mc[4] = {0, 0, 0, 0};
   uint32_t top = 0;
@@ -625,6 +606,93 @@ __global__ __launch_bounds__(64 * WAVES) void cast_tile_kernel(
   }
 }
 
+template <int MODE, int ORDER, bool ROW, bool COL, int WAVES, int GATE>
+__global__ __launch_bounds__(64 * WAVES) void cast_tile_kernel(
+    const uint16_t* __restrict__ x, int64_t rows, int64_t cols, int64_t ldx,
+    uint8_t* __restrict__ codes, uint8_t* __restrict__ scales, int64_t nblk, int64_t ks_n,
+    uint8_t* __restrict__ codes_t, uint8_t* __restrict__ scales_t, int64_t nblk_t,
+    int64_t ks_n_t, int64_t x_bstride, int64_t s_bstride, int64_t st_bstride, uint32_t gx,
+    uint32_t gy, const uint16_t* __restrict__ x3, int64_t ldx3, uint16_t* __restrict__ g_out,
+    const uint16_t* __restrict__ x4, int64_t ldx4) {
+  constexpr int TR = 32 * WAVES, TC = 128, PITCH = TR + 16;
+  __shared__ __attribute__((aligned(16))) uint8_t lds_codes[COL ? TC * PITCH : 16];
+  __shared__ __attribute__((aligned(16))) uint8_t lds_st[COL ? TC * WAVES : 16];
+  __shared__ __attribute__((aligned(16))) uint8_t lds_sr[ROW ? TR * 4 : 16];
+  x += blockIdx.z * x_bstride;  // batch of independent [rows, cols] matrices
+  if (ROW) {
+    codes += blockIdx.z * rows * cols;
+    scales += blockIdx.z * s_bstride;
+  }
+  if (COL) {
+    codes_t += blockIdx.z * rows * cols;
+    scales_t += blockIdx.z * st_bstride;
+  }
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 4, q = lane & 15;
+  const int rl0 = wave * 32 + 8 * g;  // first tile-local row of this lane
+
+  constexpr uint32_t BX = TileWalk<COL>::BX, BY = TileWalk<COL>::BY;
+  const uint32_t spr = (gx + BX - 1) / BX;
+  const uint32_t sup = blockIdx.x / (BX * BY), in = blockIdx.x % (BX * BY);
+  const uint32_t bx = (sup % spr) * BX + in / BY;
+  const uint32_t by = (sup / spr) * BY + in % BY;
+  if (bx >= gx || by >= gy) return;
+
+  const int64_t r0 = (int64_t)by * TR, c0 = (int64_t)bx * TC;
+  const int64_t c = c0 + 8 * q;
+  const bool col_ok = c < cols;
+  const int64_t left64 = rows - (r0 + rl0);
+  const int rows_left = left64 > 8 ? 8 : (left64 < 0 ? 0 : (int)left64);
+
+  u32x4 v[8];
+  load_patch(v, x + (r0 + rl0) * ldx + c, ldx, col_ok, rows_left);
+  if constexpr (GATE == 1) {  // x = gate input a, x3 = b: quantize g = silu(a) * b
+    u32x4 b[8];
+    load_patch(b, x3 + (r0 + rl0) * ldx3 + c, ldx3, col_ok, rows_left);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      v[k] = u32x4{swiglu2(v[k].x, b[k].x), swiglu2(v[k].y, b[k].y), swiglu2(v[k].z, b[k].z),
+                   swiglu2(v[k].w, b[k].w)};
+      if (g_out && col_ok && k < rows_left)
+        *reinterpret_cast<u32x4*>(g_out + (r0 + rl0 + k) * cols + c) = v[k];
+    }
+  }
+  if constexpr (GATE == 2) {
+    // backward of the gate: x = a, x3 = b, x4 = dg; two stacked outputs, d/da then d/db
+    u32x4 b[8], dg[8], w[8];
+    load_patch(b, x3 + (r0 + rl0) * ldx3 + c, ldx3, col_ok, rows_left);
+    load_patch(dg, x4 + (r0 + rl0) * ldx4 + c, ldx4, col_ok, rows_left);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      w[k] = u32x4{swiglu_da2(dg[k].x, v[k].x, b[k].x), swiglu_da2(dg[k].y, v[k].y, b[k].y),
+                   swiglu_da2(dg[k].z, v[k].z, b[k].z), swiglu_da2(dg[k].w, v[k].w, b[k].w)};
+      if (g_out && col_ok && k < rows_left)
+        *reinterpret_cast<u32x4*>(g_out + (r0 + rl0 + k) * cols + c) = w[k];
+    }
+    emit_tile<MODE, ORDER, ROW, COL, WAVES>(w, codes, scales, codes_t, scales_t, lds_codes, lds_st,
+                                            lds_sr, rows, cols, nblk, ks_n, nblk_t, ks_n_t, r0, c0,
+                                            c, rl0, rows_left, col_ok, tid, wave, lane);
+    __syncthreads();  // the staging buffers are reused by the second output
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      v[k] = u32x4{swiglu_db2(dg[k].x, v[k].x), swiglu_db2(dg[k].y, v[k].y),
+                   swiglu_db2(dg[k].z, v[k].z), swiglu_db2(dg[k].w, v[k].w)};
+      if (g_out && col_ok && k < rows_left)
+        *reinterpret_cast<u32x4*>(g_out + (rows + r0 + rl0 + k) * cols + c) = v[k];
+    }
+    if (ROW) {
+      codes += rows * cols;
+      scales += s_bstride;
+    }
+    if (COL) {
+      codes_t += rows * cols;
+      scales_t += st_bstride;
+    }
+  }
+  emit_tile<MODE, ORDER, ROW, COL, WAVES>(v, codes, scales, codes_t, scales_t, lds_codes, lds_st,
+                                          lds_sr, rows, cols, nblk, ks_n, nblk_t, ks_n_t, r0, c0, c,
+                                          rl0, rows_left, col_ok, tid, wave, lane);
+}
+
 // ------------------------------------------------------------------------------------
 // Scale re-layout (pure byte permutation) and its inverse.
 // ------------------------------------------------------------------------------------
@@ -689,23 +757,23 @@ using namespace mx;
 #ifndef MX_CAST_WAVES
 #define MX_CAST_WAVES 4
 #endif
-#define MX_DISPATCH_TILE(ROW, COL, SWIGLU, ...)                                                         \
+#define MX_DISPATCH_TILE(ROW, COL, GATE, ...)                                                           \
   do {                                                                                           \
     if (scale_mode == MX_SCALE_FLOOR && scale_order == MX_SCALES_ROWMAJOR)                       \
       hipLaunchKernelGGL(                                                                        \
-          (cast_tile_kernel<MX_SCALE_FLOOR, MX_SCALES_ROWMAJOR, ROW, COL, MX_CAST_WAVES, SWIGLU>), grid, \
+          (cast_tile_kernel<MX_SCALE_FLOOR, MX_SCALES_ROWMAJOR, ROW, COL, MX_CAST_WAVES, GATE>), grid, \
           block, 0, st, __VA_ARGS__);                                                            \
     else if (scale_mode == MX_SCALE_FLOOR)                                                       \
       hipLaunchKernelGGL(                                                                        \
-          (cast_tile_kernel<MX_SCALE_FLOOR, MX_SCALES_MFMA, ROW, COL, MX_CAST_WAVES, SWIGLU>), grid,     \
+          (cast_tile_kernel<MX_SCALE_FLOOR, MX_SCALES_MFMA, ROW, COL, MX_CAST_WAVES, GATE>), grid,     \
           block, 0, st, __VA_ARGS__);                                                            \
     else if (scale_order == MX_SCALES_ROWMAJOR)                                                  \
       hipLaunchKernelGGL(                                                                        \
-          (cast_tile_kernel<MX_SCALE_RCEIL, MX_SCALES_ROWMAJOR, ROW, COL, MX_CAST_WAVES, SWIGLU>), grid, \
+          (cast_tile_kernel<MX_SCALE_RCEIL, MX_SCALES_ROWMAJOR, ROW, COL, MX_CAST_WAVES, GATE>), grid, \
           block, 0, st, __VA_ARGS__);                                                            \
     else                                                                                         \
       hipLaunchKernelGGL(                                                                        \
-          (cast_tile_kernel<MX_SCALE_RCEIL, MX_SCALES_MFMA, ROW, COL, MX_CAST_WAVES, SWIGLU>), grid,     \
+          (cast_tile_kernel<MX_SCALE_RCEIL, MX_SCALES_MFMA, ROW, COL, MX_CAST_WAVES, GATE>), grid,     \
           block, 0, st, __VA_ARGS__);                                                            \
   } while (0)
 
@@ -765,10 +833,10 @@ extern "C" int mx_cast_dim0(const void* x, int64_t rows, int64_t cols, int64_t l
   if (scale_order == MX_SCALES_MFMA && tile_grid_x(tgx, tgy, false) <= 0x7FFFFFFF) {
     // scattered scale bytes cost more than the tiled read: stage them through LDS
     dim3 grid = tile_grid(tgx, tgy, 1, false), block(64 * MX_CAST_WAVES);
-    MX_DISPATCH_TILE(true, false, false, (const uint16_t*)x, rows, cols, ldx, codes, scales, nblk,
+    MX_DISPATCH_TILE(true, false, 0, (const uint16_t*)x, rows, cols, ldx, codes, scales, nblk,
                      ks_n, (uint8_t*)nullptr, (uint8_t*)nullptr, (int64_t)0, (int64_t)0, (int64_t)0,
                      (int64_t)0, (int64_t)0, (uint32_t)tgx, (uint32_t)tgy, (const uint16_t*)nullptr,
-                     (int64_t)0, (uint16_t*)nullptr);
+                     (int64_t)0, (uint16_t*)nullptr, (const uint16_t*)nullptr, (int64_t)0);
     return launch_status();
   }
   clear_mfma_padding(scales, rows, nblk, scale_order, st);
@@ -800,10 +868,11 @@ extern "C" int mx_cast_dim1_batched(const void* x, int64_t batch, int64_t rows, 
   const int64_t tgy = (rows + kTileRows - 1) / kTileRows;
   if (tile_ok(x, cols, ldx) && tile_grid_x(gx, tgy, true) <= 0x7FFFFFFF) {
     dim3 grid = tile_grid(gx, tgy, batch, true), block(64 * MX_CAST_WAVES);
-    MX_DISPATCH_TILE(false, true, false, (const uint16_t*)x, rows, cols, ldx, (uint8_t*)nullptr,
+    MX_DISPATCH_TILE(false, true, 0, (const uint16_t*)x, rows, cols, ldx, (uint8_t*)nullptr,
                      (uint8_t*)nullptr, (int64_t)0, (int64_t)0, codes_t, scales_t, nblk_t, ks_n_t,
                      rows * ldx, (int64_t)0, st_b, (uint32_t)gx, (uint32_t)tgy,
-                     (const uint16_t*)nullptr, (int64_t)0, (uint16_t*)nullptr);
+                     (const uint16_t*)nullptr, (int64_t)0, (uint16_t*)nullptr,
+                     (const uint16_t*)nullptr, (int64_t)0);
     return launch_status();
   }
   dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch), block(256);
@@ -842,9 +911,10 @@ extern "C" int mx_cast_dim0_dim1_batched(const void* x, int64_t batch, int64_t r
   if (tile_ok(x, cols, ldx) && ((uintptr_t)codes & 7) == 0 && ((uintptr_t)scales & 3) == 0 &&
       tile_grid_x(gx, tgy, true) <= 0x7FFFFFFF) {
     dim3 grid = tile_grid(gx, tgy, batch, true), block(64 * MX_CAST_WAVES);
-    MX_DISPATCH_TILE(true, true, false, (const uint16_t*)x, rows, cols, ldx, codes, scales, nblk,
+    MX_DISPATCH_TILE(true, true, 0, (const uint16_t*)x, rows, cols, ldx, codes, scales, nblk,
                      ks_n, codes_t, scales_t, nblk_t, ks_n_t, rows * ldx, s_b, st_b, (uint32_t)gx,
-                     (uint32_t)tgy, (const uint16_t*)nullptr, (int64_t)0, (uint16_t*)nullptr);
+                     (uint32_t)tgy, (const uint16_t*)nullptr, (int64_t)0, (uint16_t*)nullptr,
+                     (const uint16_t*)nullptr, (int64_t)0);
     return launch_status();
   }
   dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch), block(256);
@@ -916,8 +986,39 @@ extern "C" int mx_swiglu_cast_dim0_dim1(const void* a, const void* b, int64_t ro
   if (tile_grid_x(gx, tgy, true) > 0x7FFFFFFF) return MX_ERR_UNSUPPORTED;
   hipStream_t st = (hipStream_t)stream;
   dim3 grid = tile_grid(gx, tgy, 1, true), block(64 * MX_CAST_WAVES);
-  MX_DISPATCH_TILE(true, true, true, (const uint16_t*)a, rows, cols, lda, codes, scales, nblk, ks_n,
+  MX_DISPATCH_TILE(true, true, 1, (const uint16_t*)a, rows, cols, lda, codes, scales, nblk, ks_n,
                    codes_t, scales_t, nblk_t, ks_n_t, (int64_t)0, (int64_t)0, (int64_t)0,
-                   (uint32_t)gx, (uint32_t)tgy, (const uint16_t*)b, ldb, (uint16_t*)g);
+                   (uint32_t)gx, (uint32_t)tgy, (const uint16_t*)b, ldb, (uint16_t*)g,
+                   (const uint16_t*)nullptr, (int64_t)0);
+  return launch_status();
+}
+
+extern "C" int mx_swiglu_bwd_cast_dim0_dim1(const void* dg, const void* a, const void* b,
+                                            int64_t rows, int64_t cols, int64_t lddg, int64_t lda,
+                                            int64_t ldb, uint8_t* codes, uint8_t* scales,
+                                            uint8_t* codes_t, uint8_t* scales_t, void* dab,
+                                            int scale_mode, int scale_order, void* stream) {
+  if (rows < 0 || cols < 0 || lddg < cols || lda < cols || ldb < cols ||
+      bad_enums(scale_mode, scale_order))
+    return MX_ERR_INVALID_ARG;
+  if (rows == 0 || cols == 0) return MX_OK;
+  if (!dg || !a || !b || !codes || !scales || !codes_t || !scales_t) return MX_ERR_INVALID_ARG;
+  if (rows % 32 || cols % 32 || lddg % 8 || lda % 8 || ldb % 8 || ((uintptr_t)dg & 15) ||
+      ((uintptr_t)a & 15) || ((uintptr_t)b & 15) || ((uintptr_t)codes & 7) ||
+      ((uintptr_t)codes_t & 15) || ((uintptr_t)scales & 3) || ((uintptr_t)scales_t & 3) ||
+      ((uintptr_t)dab & 15))
+    return MX_ERR_ALIGNMENT;
+  const int64_t nblk = cols / 32, ks_n = (nblk + 1) / 2;
+  const int64_t nblk_t = rows / 32, ks_n_t = (nblk_t + 1) / 2;
+  // the second output follows the first: one matrix of codes and one scale buffer further on
+  const int64_t s_b = scale_bytes(rows, nblk, scale_order);
+  const int64_t st_b = scale_bytes(cols, nblk_t, scale_order);
+  const int64_t gx = (cols + kT - 1) / kT, tgy = (rows + kTileRows - 1) / kTileRows;
+  if (tile_grid_x(gx, tgy, true) > 0x7FFFFFFF) return MX_ERR_UNSUPPORTED;
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid = tile_grid(gx, tgy, 1, true), block(64 * MX_CAST_WAVES);
+  MX_DISPATCH_TILE(true, true, 2, (const uint16_t*)a, rows, cols, lda, codes, scales, nblk, ks_n,
+                   codes_t, scales_t, nblk_t, ks_n_t, (int64_t)0, s_b, st_b, (uint32_t)gx,
+                   (uint32_t)tgy, (const uint16_t*)b, ldb, (uint16_t*)dab, (const uint16_t*)dg, lddg);
   return launch_status();
 }

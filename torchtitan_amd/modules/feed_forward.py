@@ -4,7 +4,7 @@ from dataclasses import dataclass, field
 import torch
 import torch.nn.functional as F
 
-from ..mx_tensor import mx_swiglu_linear, swiglu_fusable
+from ..mx_tensor import feed_forward_fusable, mx_feed_forward, mx_swiglu_linear, swiglu_fusable
 from ..protocols import Module
 from .linear import Linear
 
@@ -33,6 +33,10 @@ class FeedForward(Module):
         self.w3 = lin.build(in_features=config.dim, out_features=config.hidden_dim)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if (self.w1.bias is None and self.w3.bias is None
+                and feed_forward_fusable(x, self.w1.weight, self.w2.weight, self.w3.weight)):
+            # all three converted: gate and its backward inside the MXFP8 cast kernels
+            return mx_feed_forward(x, self.w1.weight, self.w2.weight, self.w3.weight, self.w2.bias)
         h1, h3 = self.w1(x), self.w3(x)
         if swiglu_fusable(h1, h3, self.w2.weight):  # converted w2: gate inside the MXFP8 cast
             return mx_swiglu_linear(h1, h3, self.w2.weight, self.w2.bias)

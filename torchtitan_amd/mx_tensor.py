@@ -285,6 +285,104 @@ def mx_swiglu_linear(h1: torch.Tensor, h3: torch.Tensor, weight: torch.Tensor,
     return y
 
 
+# ----------------------------------------------------------------------------- whole SwiGLU block
+def _bf16(t: torch.Tensor) -> torch.Tensor:
+    return t if t.dtype == torch.bfloat16 else t.to(torch.bfloat16)
+
+
+class _MXFeedForward(torch.autograd.Function):
+    """y = (silu(x W1^T) * (x W3^T)) W2^T with every elementwise step folded into a cast kernel.
+
+    Forward: one cast of x, the gate inside the cast that feeds W2.  Backward: the gate's
+    gradients inside the cast that feeds the dgrad / wgrad GEMMs of W1 and W3.  Neither g nor
+    dh1 / dh3 is written to memory; kept for backward are h1, h3 and the column-wise MXFP8 forms
+    of x, g and the weights.  Results are bit-identical to the three converted linears around
+    bf16 ``F.silu`` and ``*`` (torchtitan/models/common/feed_forward.py:61-62)."""
+
+    @staticmethod
+    def forward(ctx, x, w1, w2, w3, cfg: MXFP8Config):
+        mode = cfg.scale_mode
+        D, H = x.shape[-1], w1.shape[0]
+        x2 = x.reshape(-1, D)
+        need_dx = ctx.needs_input_grad[0]
+        need_dw = any(ctx.needs_input_grad[1:4])
+        xq0, xq1 = _cast_activation(x2, x, mode, need_cols=need_dw)
+        both = lambda w: ops.to_mx_dim0_dim1(_bf16(w), mode, MX_SCALES_MFMA)
+        rows = lambda w: (ops.to_mx_dim0(_bf16(w), mode, MX_SCALES_MFMA), None)
+        w1q0, w1q1 = both(w1) if need_dx else rows(w1)
+        w3q0, w3q1 = both(w3) if need_dx else rows(w3)
+        w2q0, w2q1 = both(w2) if (need_dx or need_dw) else rows(w2)
+        h1 = ops.mx_gemm_nt(xq0, w1q0)
+        h3 = ops.mx_gemm_nt(xq0, w3q0)
+        gq0, gq1, _ = ops.swiglu_to_mx_dim0_dim1(h1, h3, mode, MX_SCALES_MFMA)
+        y = ops.mx_gemm_nt(gq0, w2q0)
+        ctx.cfg, ctx.x_shape = cfg, x.shape
+        ctx.w_dtypes = (w1.dtype, w2.dtype, w3.dtype)
+        ctx.need_dx, ctx.need_dw = need_dx, need_dw
+        saved = []
+        if need_dx or need_dw:
+            saved += [h1, h3, w2q1.codes, w2q1.scales]
+        if need_dw:
+            saved += [xq1.codes, xq1.scales, gq1.codes, gq1.scales]
+        if need_dx:
+            saved += [w1q1.codes, w1q1.scales, w3q1.codes, w3q1.scales]
+        ctx.save_for_backward(*saved)
+        return y.view(*x.shape[:-1], w2.shape[0])
+
+    @staticmethod
+    def backward(ctx, dy):
+        mode = ctx.cfg.scale_mode
+        saved = list(ctx.saved_tensors)
+        take = lambda: MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
+        h1, h3 = saved.pop(0), saved.pop(0)
+        w2q1 = take()
+        dy2 = _bf16(dy.reshape(-1, dy.shape[-1])).contiguous()
+        if ctx.needs_input_grad[2]:
+            dyq0, dyq1 = ops.to_mx_dim0_dim1(dy2, mode, MX_SCALES_MFMA)
+        else:
+            dyq0, dyq1 = ops.to_mx_dim0(dy2, mode, MX_SCALES_MFMA), None
+        dg = ops.mx_gemm_nt(dyq0, w2q1)
+        (da0, da1), (db0, db1), _ = ops.swiglu_bwd_to_mx_dim0_dim1(dg, h1, h3, mode, MX_SCALES_MFMA)
+        dx = dw1 = dw2 = dw3 = None
+        if ctx.need_dw:
+            xq1, gq1 = take(), take()
+            cast_back = lambda g, dt: g if g.dtype == dt else g.to(dt)
+            if ctx.needs_input_grad[1]:
+                dw1 = cast_back(ops.mx_gemm_nt(da1, xq1), ctx.w_dtypes[0])
+            if ctx.needs_input_grad[2]:
+                dw2 = cast_back(ops.mx_gemm_nt(dyq1, gq1), ctx.w_dtypes[1])
+            if ctx.needs_input_grad[3]:
+                dw3 = cast_back(ops.mx_gemm_nt(db1, xq1), ctx.w_dtypes[2])
+        if ctx.need_dx:
+            w1q1, w3q1 = take(), take()
+            dx = (ops.mx_gemm_nt(da0, w1q1) + ops.mx_gemm_nt(db0, w3q1)).view(ctx.x_shape)
+        return dx, dw1, dw2, dw3, None
+
+
+def feed_forward_fusable(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, w3: torch.Tensor) -> bool:
+    """The whole-block function needs all three weights converted with gate fusion on, a bf16
+    GPU activation and 32-aligned token, model and hidden sizes."""
+    ws = (w1, w2, w3)
+    if not all(isinstance(w, MXFP8TrainingWeight) and w.mx_config.fuse_swiglu_cast for w in ws):
+        return False
+    if w1.mx_config.scale_mode != w2.mx_config.scale_mode or w1.mx_config.scale_mode != w3.mx_config.scale_mode:
+        return False
+    if x.dtype != torch.bfloat16 or not x.is_cuda or x.numel() == 0 or w1.shape != w3.shape:
+        return False
+    D, H = x.shape[-1], w1.shape[0]
+    return D % ops.BLOCK == 0 and H % ops.BLOCK == 0 and (x.numel() // D) % ops.BLOCK == 0
+
+
+def mx_feed_forward(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, w3: torch.Tensor,
+                    bias2: torch.Tensor | None = None):
+    """``F.linear(F.silu(F.linear(x, w1)) * F.linear(x, w3), w2, bias2)`` for converted weights.
+    Callers check `feed_forward_fusable` first."""
+    y = _MXFeedForward.apply(x, _unwrap(w1), _unwrap(w2), _unwrap(w3), w2.mx_config)
+    if bias2 is not None:
+        y = y + _unwrap(bias2).to(y.dtype)
+    return y
+
+
 # ----------------------------------------------------------------------------- grouped GEMM
 def _pad_plan(offs: torch.Tensor, T: int, align: int = 32):
     """Device-side plan that moves rows of variable-size groups into `align`-aligned groups.

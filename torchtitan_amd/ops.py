@@ -170,6 +170,42 @@ def swiglu_to_mx_dim0_dim1(a: torch.Tensor, b: torch.Tensor, mode="floor",
     return MXData(codes, scales, order), MXData(codes_t, scales_t, order), g
 
 
+def _scale_count(rows: int, nblk: int, order: int) -> int:
+    return mfma_scale_bytes(rows, nblk) if order == MX_SCALES_MFMA else rows * nblk
+
+
+def swiglu_bwd_to_mx_dim0_dim1(dg: torch.Tensor, a: torch.Tensor, b: torch.Tensor, mode="floor",
+                               order: int = MX_SCALES_ROWMAJOR, want_grads: bool = False):
+    """Backward of g = silu(a) * b with both casts of each gradient from one pass over dg, a, b.
+
+    Returns ((da row-wise, da column-wise), (db row-wise, db column-wise), stacked bf16 [2, R, C]
+    gradients or None).  The two row-wise (column-wise) results are the halves of one buffer."""
+    dg, a, b = _check_hp(dg), _check_hp(a), _check_hp(b)
+    if a.shape != b.shape or a.shape != dg.shape:
+        raise ValueError(f"shape mismatch: {tuple(dg.shape)}, {tuple(a.shape)}, {tuple(b.shape)}")
+    R, C = a.shape
+    if R % BLOCK or C % BLOCK:
+        raise ValueError(f"both dims of {tuple(a.shape)} must be multiples of {BLOCK}")
+    dev = a.device
+    n_s, n_st = _scale_count(R, C // BLOCK, order), _scale_count(C, R // BLOCK, order)
+    codes = torch.empty((2, R, C), dtype=torch.uint8, device=dev)
+    codes_t = torch.empty((2, C, R), dtype=torch.uint8, device=dev)
+    scales = torch.empty(2 * n_s, dtype=torch.uint8, device=dev)
+    scales_t = torch.empty(2 * n_st, dtype=torch.uint8, device=dev)
+    dab = torch.empty((2, R, C), dtype=torch.bfloat16, device=dev) if want_grads else None
+    _call("mx_swiglu_bwd_cast_dim0_dim1", "swiglu_bwd_cast_dim0_dim1", dev, _ptr(dg), _ptr(a), _ptr(b),
+          R, C, dg.stride(0), a.stride(0), b.stride(0), _ptr(codes), _ptr(scales), _ptr(codes_t),
+          _ptr(scales_t), _ptr(dab) if dab is not None else None, _mode(mode), order, _stream(a))
+
+    def half(i):
+        s, st = scales[i * n_s:(i + 1) * n_s], scales_t[i * n_st:(i + 1) * n_st]
+        if order == MX_SCALES_ROWMAJOR:
+            s, st = s.view(R, C // BLOCK), st.view(C, R // BLOCK)
+        return MXData(codes[i], s, order), MXData(codes_t[i], st, order)
+
+    return half(0), half(1), dab
+
+
 def scale_layout(scales: torch.Tensor) -> torch.Tensor:
     """Row-major [rows, nblk] scales -> flat buffer in MFMA order."""
     rows, nblk = scales.shape
