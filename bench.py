@@ -125,6 +125,74 @@ def time_casts(dev, recipe_mode):
     return out
 
 
+def time_ffn_block(dev, recipe):
+    """Beyond the headline: the whole SwiGLU block w2(silu(w1 x) * w3 x), forward + backward, at
+    the same shapes, with the gate (and its backward) inside the cast kernels and with silu and
+    the products as separate bf16 ops.  Same nine GEMMs either way; results are bit-identical."""
+    import torch
+    import torch.nn as nn
+
+    from torchtitan_amd import mx_tensor, ops
+    from torchtitan_amd.modules import FeedForward
+    from torchtitan_amd.protocols import ModelConvertersContainer
+    from torchtitan_amd.quantization.mx import MXFP8Converter
+
+    x = torch.randn((M, DIM), device=dev, dtype=torch.bfloat16).requires_grad_(True)
+    dy = torch.randn((M, DIM), device=dev, dtype=torch.bfloat16) * 1e-3
+    out = {}
+    for name, fuse in (("fused_gate", True), ("separate_ops", False)):
+        ff = FeedForward.Config(hidden_dim=HIDDEN).build(dim=DIM)
+        holder = nn.Module()
+        holder.feed_forward = ff
+        ModelConvertersContainer.Config(
+            converters=[MXFP8Converter.Config(fqns=["feed_forward"], recipe_name=recipe, fuse_swiglu_cast=fuse)]
+        ).build(parallel_dims=None, model_compile_enabled=False).convert(holder)
+        holder.to(dev).to(torch.bfloat16)
+        ff.init_weights(init_std=0.02)
+
+        def step():
+            mx_tensor._cast_cache.clear()
+            x.grad = None
+            for p in ff.parameters():
+                p.grad = None
+            ff(x).backward(dy)
+
+        for _ in range(2):
+            step()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        reps = 5
+        s.record()
+        for _ in range(reps):
+            step()
+        e.record()
+        torch.cuda.synchronize()
+        ms = s.elapsed_time(e) / reps
+        out[name] = {"ms": round(ms, 3), "TFLOP/s": round(18.0 * M * DIM * HIDDEN / ms / 1e9, 1)}
+        del ff, holder
+    el = M * HIDDEN
+    a = torch.randn((M, HIDDEN), device=dev, dtype=torch.bfloat16)
+    b = torch.randn((M, HIDDEN), device=dev, dtype=torch.bfloat16)
+    dg = torch.randn((M, HIDDEN), device=dev, dtype=torch.bfloat16)
+    L = ops.MX_SCALES_MFMA
+    mode = {"mxfp8_rceil": "rceil", "mxfp8_floor": "floor"}[recipe]
+    for name, fn, bpe in (("swiglu_cast_dim0_dim1", lambda: ops.swiglu_to_mx_dim0_dim1(a, b, mode, L), 6.0625),
+                          ("swiglu_bwd_cast_dim0_dim1", lambda: ops.swiglu_bwd_to_mx_dim0_dim1(dg, a, b, mode, L), 10.125)):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(10):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        sec = s.elapsed_time(e) * 1e-4
+        out[name] = {"us": round(sec * 1e6, 1), "GB/s": round(el * bpe / sec / 1e9, 1),
+                     "frac_hbm": round(el * bpe / sec / 1e9 / PEAK_HBM_GBPS, 3)}
+    return out
+
+
 def time_moe_grouped(dev, recipe_mode):
     """BASELINE configs[3] GEMMs (not the headline): 128 experts, hidden 2048, expert FFN 768,
     top-8 routing of 16384 tokens from softmax over seeded Gumbel-perturbed logits (uneven
@@ -313,6 +381,9 @@ def main():
     if not args.no_casts:
         line["casts"] = time_casts(dev, recipe_mode)
         line["moe_grouped_gemms"] = time_moe_grouped(dev, recipe_mode)
+        del ffn, x, h, dy_h, dy_o
+        torch.cuda.empty_cache()
+        line["swiglu_block"] = time_ffn_block(dev, args.recipe)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(0 if recipe_mode == "floor" else 1, target_s=12.0)
     print(json.dumps(line))

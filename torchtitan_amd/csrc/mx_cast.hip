@@ -467,23 +467,32 @@ __device__ __forceinline__ uint32_t swiglu2(uint32_t a2, uint32_t b2) {
 // Backward of g = silu(a) * b under bf16 autograd, tensor op by tensor op:
 //   d/db = bf16(dg * bf16(silu(a)))
 //   d/da = silu_backward(bf16(dg * b), a) = bf16(t * s * (1 + a * (1 - s))),  s = 1 / (1 + exp(-a))
-// with the float32 formula of the unfused silu backward op.
-__device__ __forceinline__ float silu_grad_f32(float t, float a) {
-  const float s = 1.0f / (1.0f + expf(-a));
-  return t * s * (1.0f + a * (1.0f - s));
+// with the float32 formula of the unfused silu backward op.  silu(a) = a / (1 + exp(-a)) shares
+// the denominator: a * s corrected by one Newton step on the remainder is the correctly rounded
+// quotient (the remainder is NaN or zero for infinite a, an infinite denominator and a = -0:
+// the uncorrected product is the answer there).
+__device__ __forceinline__ void swiglu_bwd_f32(float dg, float a, float b, float& da, float& db) {
+  // exp as the library computes it (the fast hardware path moves a few results in a million by
+  // one bf16 step); 1 / d = hardware reciprocal, scaled into its range, plus one Newton step
+  const float d = 1.0f + expf(-a);
+  const float sc = d > 0x1p100f ? 0x1p-32f : 1.0f;
+  const float ds = d * sc, r0 = __builtin_amdgcn_rcpf(ds);
+  const float s = d == __builtin_inff() ? 0.0f : __builtin_fmaf(__builtin_fmaf(-r0, ds, 1.0f), r0, r0) * sc;
+  const float q = a * s;
+  const float rem = __builtin_fmaf(-q, d, a);
+  const float silu = __builtin_islessgreater(rem, 0.0f) ? __builtin_fmaf(rem, s, q) : q;
+  const uint32_t sb = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f_t{silu, dg * b}, v2bf_t));
+  db = dg * bf16_lo(sb);
+  const float t = bf16_hi(sb);
+  da = t * s * (1.0f + a * (1.0f - s));
 }
-__device__ __forceinline__ uint32_t swiglu_da2(uint32_t dg2, uint32_t a2, uint32_t b2) {
-  const uint32_t t2 = __builtin_bit_cast(
-      uint32_t, __builtin_convertvector(v2f_t{bf16_lo(dg2) * bf16_lo(b2), bf16_hi(dg2) * bf16_hi(b2)}, v2bf_t));
-  return __builtin_bit_cast(
-      uint32_t, __builtin_convertvector(v2f_t{silu_grad_f32(bf16_lo(t2), bf16_lo(a2)),
-                                              silu_grad_f32(bf16_hi(t2), bf16_hi(a2))}, v2bf_t));
-}
-__device__ __forceinline__ uint32_t swiglu_db2(uint32_t dg2, uint32_t a2) {
-  const uint32_t s2 = __builtin_bit_cast(
-      uint32_t, __builtin_convertvector(v2f_t{silu_f32(bf16_lo(a2)), silu_f32(bf16_hi(a2))}, v2bf_t));
-  return __builtin_bit_cast(
-      uint32_t, __builtin_convertvector(v2f_t{bf16_lo(dg2) * bf16_lo(s2), bf16_hi(dg2) * bf16_hi(s2)}, v2bf_t));
+__device__ __forceinline__ void swiglu_bwd2(uint32_t dg2, uint32_t a2, uint32_t b2, uint32_t& da2,
+                                            uint32_t& db2) {
+  float da_lo, da_hi, db_lo, db_hi;
+  swiglu_bwd_f32(bf16_lo(dg2), bf16_lo(a2), bf16_lo(b2), da_lo, db_lo);
+  swiglu_bwd_f32(bf16_hi(dg2), bf16_hi(a2), bf16_hi(b2), da_hi, db_hi);
+  da2 = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f_t{da_lo, da_hi}, v2bf_t));
+  db2 = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f_t{db_lo, db_hi}, v2bf_t));
 }
 
 // 8 rows x 16 bytes of a bf16 matrix per lane; rows past `rows_left` and lanes past the last
@@ -606,8 +615,9 @@ __device__ __forceinline__ void emit_tile(
   }
 }
 
+// The gate-backward variant is bound by vector ALU work: four workgroups per CU (128 VGPRs).
 template <int MODE, int ORDER, bool ROW, bool COL, int WAVES, int GATE>
-__global__ __launch_bounds__(64 * WAVES) void cast_tile_kernel(
+__global__ __launch_bounds__(64 * WAVES, GATE == 2 ? 4 : 1) void cast_tile_kernel(
     const uint16_t* __restrict__ x, int64_t rows, int64_t cols, int64_t ldx,
     uint8_t* __restrict__ codes, uint8_t* __restrict__ scales, int64_t nblk, int64_t ks_n,
     uint8_t* __restrict__ codes_t, uint8_t* __restrict__ scales_t, int64_t nblk_t,
@@ -658,27 +668,30 @@ __global__ __launch_bounds__(64 * WAVES) void cast_tile_kernel(
   }
   if constexpr (GATE == 2) {
     // backward of the gate: x = a, x3 = b, x4 = dg; two stacked outputs, d/da then d/db
-    u32x4 b[8], dg[8], w[8];
-    load_patch(b, x3 + (r0 + rl0) * ldx3 + c, ldx3, col_ok, rows_left);
-    load_patch(dg, x4 + (r0 + rl0) * ldx4 + c, ldx4, col_ok, rows_left);
+    u32x4 w[8];
+    {
+      u32x4 b[8], dg[8];
+      load_patch(b, x3 + (r0 + rl0) * ldx3 + c, ldx3, col_ok, rows_left);
+      load_patch(dg, x4 + (r0 + rl0) * ldx4 + c, ldx4, col_ok, rows_left);
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      w[k] = u32x4{swiglu_da2(dg[k].x, v[k].x, b[k].x), swiglu_da2(dg[k].y, v[k].y, b[k].y),
-                   swiglu_da2(dg[k].z, v[k].z, b[k].z), swiglu_da2(dg[k].w, v[k].w, b[k].w)};
-      if (g_out && col_ok && k < rows_left)
-        *reinterpret_cast<u32x4*>(g_out + (r0 + rl0 + k) * cols + c) = w[k];
+      for (int k = 0; k < 8; ++k) {
+        uint32_t da[4], db[4];
+        swiglu_bwd2(dg[k].x, v[k].x, b[k].x, da[0], db[0]);
+        swiglu_bwd2(dg[k].y, v[k].y, b[k].y, da[1], db[1]);
+        swiglu_bwd2(dg[k].z, v[k].z, b[k].z, da[2], db[2]);
+        swiglu_bwd2(dg[k].w, v[k].w, b[k].w, da[3], db[3]);
+        w[k] = u32x4{da[0], da[1], da[2], da[3]};
+        v[k] = u32x4{db[0], db[1], db[2], db[3]};
+        if (g_out && col_ok && k < rows_left) {
+          *reinterpret_cast<u32x4*>(g_out + (r0 + rl0 + k) * cols + c) = w[k];
+          *reinterpret_cast<u32x4*>(g_out + (rows + r0 + rl0 + k) * cols + c) = v[k];
+        }
+      }
     }
     emit_tile<MODE, ORDER, ROW, COL, WAVES>(w, codes, scales, codes_t, scales_t, lds_codes, lds_st,
                                             lds_sr, rows, cols, nblk, ks_n, nblk_t, ks_n_t, r0, c0,
                                             c, rl0, rows_left, col_ok, tid, wave, lane);
     __syncthreads();  // the staging buffers are reused by the second output
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      v[k] = u32x4{swiglu_db2(dg[k].x, v[k].x), swiglu_db2(dg[k].y, v[k].y),
-                   swiglu_db2(dg[k].z, v[k].z), swiglu_db2(dg[k].w, v[k].w)};
-      if (g_out && col_ok && k < rows_left)
-        *reinterpret_cast<u32x4*>(g_out + (rows + r0 + rl0 + k) * cols + c) = v[k];
-    }
     if (ROW) {
       codes += rows * cols;
       scales += s_bstride;
