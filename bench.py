@@ -237,6 +237,56 @@ def time_moe_grouped(dev, recipe_mode):
         torch.cuda.synchronize()
         sec = s.elapsed_time(e) * 1e-3 / 8
         out[name] = {"us": round(sec * 1e6, 1), "TFLOP/s": round(flops / sec / 1e12, 1)}
+    del x, w, dy, xq0, xq1, dyq0, dyq1, wq0, wq1, y, dx, dw
+    out["expert_block"] = time_expert_block(dev, recipe_mode, counts)
+    return out
+
+
+def time_expert_block(dev, recipe_mode, counts):
+    """The whole expert SwiGLU block (three grouped GEMMs forward, six backward, padding, casts,
+    gate) through the converted module on the routed rows in expert order: as one fused function
+    and as separate grouped GEMMs around bf16 silu / product ops.  Bit-identical results."""
+    import torch
+    import torch.nn as nn
+
+    from torchtitan_amd.modules import GroupedExperts
+    from torchtitan_amd.protocols import ModelConvertersContainer
+    from torchtitan_amd.quantization.mx import MXFP8Converter
+
+    E, dim, hid = counts.numel(), 2048, 768
+    routed = int(counts.sum())
+    recipe = {"rceil": "mxfp8_rceil", "floor": "mxfp8_floor"}[recipe_mode]
+    x = torch.randn((routed, dim), device=dev, dtype=torch.bfloat16).requires_grad_(True)
+    dy = torch.randn((routed, dim), device=dev, dtype=torch.bfloat16) * 1e-3
+    out = {}
+    for name, fuse in (("fused", True), ("separate_ops", False)):
+        ex = GroupedExperts(dim=dim, hidden_dim=hid, num_experts=E, use_grouped_mm=True)
+        holder = nn.Module()
+        holder.experts = ex
+        ModelConvertersContainer.Config(
+            converters=[MXFP8Converter.Config(fqns=["experts"], recipe_name=recipe, fuse_swiglu_cast=fuse)]
+        ).build(parallel_dims=None, model_compile_enabled=False).convert(holder)
+        holder.to(dev).to(torch.bfloat16)
+        ex.init_weights(init_std=0.02)
+
+        def step():
+            x.grad = None
+            for p in ex.parameters():
+                p.grad = None
+            ex(x, counts).backward(dy)
+
+        for _ in range(2):
+            step()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(5):
+            step()
+        e.record()
+        torch.cuda.synchronize()
+        ms = s.elapsed_time(e) / 5
+        out[name] = {"ms": round(ms, 3), "TFLOP/s": round(18.0 * routed * dim * hid / ms / 1e9, 1)}
+        del ex, holder
     return out
 
 

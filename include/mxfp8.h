@@ -87,6 +87,18 @@ int mx_cast_dim0_dim1_batched(const void* x, int64_t batch, int64_t rows, int64_
                               int64_t ldx, uint8_t* codes, uint8_t* scales, uint8_t* codes_t,
                               uint8_t* scales_t, int scale_mode, int scale_order, void* stream);
 
+/* Cast of gathered rows: output row r is row row_index[r] of x (bf16 [src_rows, cols], row
+ * stride ldx); an index outside [0, src_rows) gives a row of zeros (the padding slots of an
+ * aligned token-group layout hold -1).  Row-wise cast always; the column-wise cast too unless
+ * codes_t and scales_t are both NULL (then `rows` need not be a multiple of 32).  Outputs as
+ * mx_cast_dim0_dim1 for a [rows, cols] matrix.  Requires cols % 32 == 0, ldx % 8 == 0, x 16-byte
+ * aligned.  Stands in for the token permutation `x[permuted_indices, :]` in front of the grouped
+ * GEMMs (torchtitan/models/common/moe/utils.py:65-89) followed by the cast of its result. */
+int mx_cast_rows_gathered(const void* x, const int64_t* row_index, int64_t src_rows, int64_t rows,
+                          int64_t cols, int64_t ldx, uint8_t* codes, uint8_t* scales,
+                          uint8_t* codes_t, uint8_t* scales_t, int scale_mode, int scale_order,
+                          void* stream);
+
 /* SwiGLU gate fused into the cast: g = silu(a) * b elementwise over bf16 [rows, cols] (row strides
  * lda, ldb), each step rounded to bf16 as the unfused tensor ops round it, then both casts of g
  * as mx_cast_dim0_dim1 produces them -- g itself never travels through HBM unless `g` is given

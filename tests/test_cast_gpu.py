@@ -270,3 +270,30 @@ def test_swiglu_backward_every_bf16_gate_input(device):
         (torch.nn.functional.silu(ta) * tb).backward(dg)
         _, _, grads = ops.swiglu_bwd_to_mx_dim0_dim1(dg, a, b, "rceil", ops.MX_SCALES_MFMA, want_grads=True)
         assert _equal_or_nan(grads[0], ta.grad) and _equal_or_nan(grads[1], tb.grad)
+
+
+@pytest.mark.parametrize("mode_name,mode", MODES)
+@pytest.mark.parametrize("src_rows,rows,cols", [(50, 64, 96), (300, 512, 256), (1000, 1184, 160)])
+def test_cast_of_gathered_rows(device, mode_name, mode, src_rows, rows, cols):
+    """Cast of x[row_index] with -1 (and out-of-range) slots as zero rows == cast of the tensor
+    the gather would have formed; with and without the column-wise output."""
+    rng = np.random.default_rng(rows + cols)
+    bits = randn_bits(rng, (src_rows, cols), outliers=1e-3)
+    idx = np.full(rows, -1, dtype=np.int64)
+    slots = rng.permutation(rows)[:src_rows] if src_rows <= rows else rng.permutation(rows)
+    idx[slots] = rng.permutation(src_rows)[:len(slots)]
+    idx[rng.integers(0, rows)] = src_rows + 5  # outside the source: zeros as well
+    valid = (idx >= 0) & (idx < src_rows)
+    gathered = np.where(valid[:, None], bits[np.clip(idx, 0, src_rows - 1)], 0).astype(np.uint16)
+    x = bf16_from_bits(bits, device)
+    ti = torch.from_numpy(idx).to(device)
+    for order in (ops.MX_SCALES_ROWMAJOR, ops.MX_SCALES_MFMA):
+        q0, q1 = ops.to_mx_rows_gathered(x, ti, mode_name, order)
+        c0, s0 = mo.cast_dim0(gathered, mode)
+        c1, s1 = mo.cast_dim1(gathered, mode)
+        if order == ops.MX_SCALES_MFMA:
+            s0, s1 = mo.scale_layout(s0), mo.scale_layout(s1)
+        assert np.array_equal(u8(q0.codes), c0) and np.array_equal(u8(q0.scales).reshape(-1), s0.reshape(-1))
+        assert np.array_equal(u8(q1.codes), c1) and np.array_equal(u8(q1.scales).reshape(-1), s1.reshape(-1))
+        r0, none = ops.to_mx_rows_gathered(x, ti, mode_name, order, want_cols=False)
+        assert none is None and torch.equal(r0.codes, q0.codes) and torch.equal(r0.scales, q0.scales)

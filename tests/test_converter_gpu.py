@@ -259,6 +259,45 @@ def test_grouped_experts_swiglu_block(device):
         moe_mod.set_token_group_alignment_size_m(8)
 
 
+@pytest.mark.parametrize("pad,align", [(True, 8), (False, 32)])
+@pytest.mark.parametrize("dim,hidden", [(128, 64), (256, 128)])
+def test_grouped_experts_fused_block_matches_separate_ops(device, pad, align, dim, hidden):
+    """The expert block as one fused function (one padding pass, gate inside the casts) against
+    three converted grouped GEMMs around separate bf16 silu / product ops: bit-identical output
+    and gradients, on the persistent kernels (pad on, dims % 128) and on the general ones."""
+    torch.manual_seed(21)
+    moe_mod.set_token_group_alignment_size_m(align)
+    try:
+        counts = torch.tensor([40, 0, 200, 16, 7, 130] if pad else [64, 0, 96, 32, 32, 160], device=device)
+        blocks = []
+        for fuse in (True, False):
+            ex = GroupedExperts(dim=dim, hidden_dim=hidden, num_experts=6, use_grouped_mm=True).to(device).to(torch.bfloat16)
+            if blocks:
+                ex.load_state_dict(blocks[0].state_dict())
+            else:
+                ex.init_weights(init_std=0.05)
+            holder = nn.Module()
+            holder.experts = ex
+            _convert(holder, ["experts"], pad=pad, fuse=fuse)
+            blocks.append(ex)
+        x = torch.randn(int(counts.sum()), dim, device=device, dtype=torch.bfloat16)
+        dy = torch.randn(int(counts.sum()), dim, device=device, dtype=torch.bfloat16)
+        outs = []
+        for ex in blocks:
+            xi = x.clone().requires_grad_(True)
+            y = ex(xi, counts)
+            y.backward(dy)
+            outs.append([y.detach(), xi.grad, ex.w1.grad, ex.w2.grad, ex.w3.grad])
+        for got, want in zip(*outs):
+            assert torch.equal(got, want)
+        assert not torch.isnan(outs[0][0]).any() and outs[0][2].abs().sum() > 0
+        from torchtitan_amd.mx_tensor import grouped_feed_forward_fusable as fusable
+        assert fusable(x, blocks[0].w1, blocks[0].w2, blocks[0].w3)
+        assert not fusable(x, blocks[1].w1, blocks[1].w2, blocks[1].w3)
+    finally:
+        moe_mod.set_token_group_alignment_size_m(8)
+
+
 class _MiniDecoderBlock(nn.Module):
     """Llama-style block in small: RMSNorm, GQA attention with RoPE-free SDPA in bf16, SwiGLU FFN.
     The seven linears are the `Linear` modules the converter selects by FQN."""

@@ -615,15 +615,45 @@ __device__ __forceinline__ void emit_tile(
   }
 }
 
+// As load_patch, with the source row of output row r taken from row_idx[r]; an index outside
+// [0, src_rows) (the padding slots of a token-group layout hold -1) reads as a row of zeros.
+__device__ __forceinline__ void load_patch_rows(u32x4 (&v)[8], const uint16_t* x, int64_t ld,
+                                                int64_t c, const int64_t* row_idx, int64_t src_rows,
+                                                bool col_ok, int rows_left) {
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    v[k] = u32x4{0, 0, 0, 0};
+    if (col_ok && k < rows_left) {
+      const int64_t r = row_idx[k];
+      if (r >= 0 && r < src_rows)
+        v[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(x + r * ld + c));
+    }
+  }
+}
+
+// Operands of the tile kernel's variants beyond the plain cast.
+struct TileExtras {
+  const uint16_t* x3 = nullptr;  // GATE 1, 2: second gate input b
+  int64_t ldx3 = 0;
+  uint16_t* g_out = nullptr;     // GATE 1: g; GATE 2: stacked da, db (optional)
+  const uint16_t* x4 = nullptr;  // GATE 2: dg
+  int64_t ldx4 = 0;
+  const int64_t* row_idx = nullptr;  // GATHER: source row of every output row
+  int64_t src_rows = 0;
+};
+
 // The gate-backward variant is bound by vector ALU work: four workgroups per CU (128 VGPRs).
-template <int MODE, int ORDER, bool ROW, bool COL, int WAVES, int GATE>
+template <int MODE, int ORDER, bool ROW, bool COL, int WAVES, int GATE, bool GATHER>
 __global__ __launch_bounds__(64 * WAVES, GATE == 2 ? 4 : 1) void cast_tile_kernel(
     const uint16_t* __restrict__ x, int64_t rows, int64_t cols, int64_t ldx,
     uint8_t* __restrict__ codes, uint8_t* __restrict__ scales, int64_t nblk, int64_t ks_n,
     uint8_t* __restrict__ codes_t, uint8_t* __restrict__ scales_t, int64_t nblk_t,
     int64_t ks_n_t, int64_t x_bstride, int64_t s_bstride, int64_t st_bstride, uint32_t gx,
-    uint32_t gy, const uint16_t* __restrict__ x3, int64_t ldx3, uint16_t* __restrict__ g_out,
-    const uint16_t* __restrict__ x4, int64_t ldx4) {
+    uint32_t gy, TileExtras ex) {
+  const uint16_t* __restrict__ x3 = ex.x3;
+  const uint16_t* __restrict__ x4 = ex.x4;
+  uint16_t* __restrict__ g_out = ex.g_out;
+  const int64_t ldx3 = ex.ldx3, ldx4 = ex.ldx4;
   constexpr int TR = 32 * WAVES, TC = 128, PITCH = TR + 16;
   __shared__ __attribute__((aligned(16))) uint8_t lds_codes[COL ? TC * PITCH : 16];
   __shared__ __attribute__((aligned(16))) uint8_t lds_st[COL ? TC * WAVES : 16];
@@ -654,7 +684,10 @@ __global__ __launch_bounds__(64 * WAVES, GATE == 2 ? 4 : 1) void cast_tile_kerne
   const int rows_left = left64 > 8 ? 8 : (left64 < 0 ? 0 : (int)left64);
 
   u32x4 v[8];
-  load_patch(v, x + (r0 + rl0) * ldx + c, ldx, col_ok, rows_left);
+  if constexpr (GATHER)
+    load_patch_rows(v, x, ldx, c, ex.row_idx + r0 + rl0, ex.src_rows, col_ok, rows_left);
+  else
+    load_patch(v, x + (r0 + rl0) * ldx + c, ldx, col_ok, rows_left);
   if constexpr (GATE == 1) {  // x = gate input a, x3 = b: quantize g = silu(a) * b
     u32x4 b[8];
     load_patch(b, x3 + (r0 + rl0) * ldx3 + c, ldx3, col_ok, rows_left);
@@ -770,23 +803,23 @@ using namespace mx;
 #ifndef MX_CAST_WAVES
 #define MX_CAST_WAVES 4
 #endif
-#define MX_DISPATCH_TILE(ROW, COL, GATE, ...)                                                           \
+#define MX_DISPATCH_TILE(ROW, COL, GATE, GATHER, ...)                                                         \
   do {                                                                                           \
     if (scale_mode == MX_SCALE_FLOOR && scale_order == MX_SCALES_ROWMAJOR)                       \
       hipLaunchKernelGGL(                                                                        \
-          (cast_tile_kernel<MX_SCALE_FLOOR, MX_SCALES_ROWMAJOR, ROW, COL, MX_CAST_WAVES, GATE>), grid, \
+          (cast_tile_kernel<MX_SCALE_FLOOR, MX_SCALES_ROWMAJOR, ROW, COL, MX_CAST_WAVES, GATE, GATHER>), grid, \
           block, 0, st, __VA_ARGS__);                                                            \
     else if (scale_mode == MX_SCALE_FLOOR)                                                       \
       hipLaunchKernelGGL(                                                                        \
-          (cast_tile_kernel<MX_SCALE_FLOOR, MX_SCALES_MFMA, ROW, COL, MX_CAST_WAVES, GATE>), grid,     \
+          (cast_tile_kernel<MX_SCALE_FLOOR, MX_SCALES_MFMA, ROW, COL, MX_CAST_WAVES, GATE, GATHER>), grid,     \
           block, 0, st, __VA_ARGS__);                                                            \
     else if (scale_order == MX_SCALES_ROWMAJOR)                                                  \
       hipLaunchKernelGGL(                                                                        \
-          (cast_tile_kernel<MX_SCALE_RCEIL, MX_SCALES_ROWMAJOR, ROW, COL, MX_CAST_WAVES, GATE>), grid, \
+          (cast_tile_kernel<MX_SCALE_RCEIL, MX_SCALES_ROWMAJOR, ROW, COL, MX_CAST_WAVES, GATE, GATHER>), grid, \
           block, 0, st, __VA_ARGS__);                                                            \
     else                                                                                         \
       hipLaunchKernelGGL(                                                                        \
-          (cast_tile_kernel<MX_SCALE_RCEIL, MX_SCALES_MFMA, ROW, COL, MX_CAST_WAVES, GATE>), grid,     \
+          (cast_tile_kernel<MX_SCALE_RCEIL, MX_SCALES_MFMA, ROW, COL, MX_CAST_WAVES, GATE, GATHER>), grid,     \
           block, 0, st, __VA_ARGS__);                                                            \
   } while (0)
 
@@ -846,10 +879,9 @@ extern "C" int mx_cast_dim0(const void* x, int64_t rows, int64_t cols, int64_t l
   if (scale_order == MX_SCALES_MFMA && tile_grid_x(tgx, tgy, false) <= 0x7FFFFFFF) {
     // scattered scale bytes cost more than the tiled read: stage them through LDS
     dim3 grid = tile_grid(tgx, tgy, 1, false), block(64 * MX_CAST_WAVES);
-    MX_DISPATCH_TILE(true, false, 0, (const uint16_t*)x, rows, cols, ldx, codes, scales, nblk,
+    MX_DISPATCH_TILE(true, false, 0, false, (const uint16_t*)x, rows, cols, ldx, codes, scales, nblk,
                      ks_n, (uint8_t*)nullptr, (uint8_t*)nullptr, (int64_t)0, (int64_t)0, (int64_t)0,
-                     (int64_t)0, (int64_t)0, (uint32_t)tgx, (uint32_t)tgy, (const uint16_t*)nullptr,
-                     (int64_t)0, (uint16_t*)nullptr, (const uint16_t*)nullptr, (int64_t)0);
+                     (int64_t)0, (int64_t)0, (uint32_t)tgx, (uint32_t)tgy, TileExtras{});
     return launch_status();
   }
   clear_mfma_padding(scales, rows, nblk, scale_order, st);
@@ -881,11 +913,10 @@ extern "C" int mx_cast_dim1_batched(const void* x, int64_t batch, int64_t rows, 
   const int64_t tgy = (rows + kTileRows - 1) / kTileRows;
   if (tile_ok(x, cols, ldx) && tile_grid_x(gx, tgy, true) <= 0x7FFFFFFF) {
     dim3 grid = tile_grid(gx, tgy, batch, true), block(64 * MX_CAST_WAVES);
-    MX_DISPATCH_TILE(false, true, 0, (const uint16_t*)x, rows, cols, ldx, (uint8_t*)nullptr,
+    MX_DISPATCH_TILE(false, true, 0, false, (const uint16_t*)x, rows, cols, ldx, (uint8_t*)nullptr,
                      (uint8_t*)nullptr, (int64_t)0, (int64_t)0, codes_t, scales_t, nblk_t, ks_n_t,
                      rows * ldx, (int64_t)0, st_b, (uint32_t)gx, (uint32_t)tgy,
-                     (const uint16_t*)nullptr, (int64_t)0, (uint16_t*)nullptr,
-                     (const uint16_t*)nullptr, (int64_t)0);
+                     TileExtras{});
     return launch_status();
   }
   dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch), block(256);
@@ -924,10 +955,9 @@ extern "C" int mx_cast_dim0_dim1_batched(const void* x, int64_t batch, int64_t r
   if (tile_ok(x, cols, ldx) && ((uintptr_t)codes & 7) == 0 && ((uintptr_t)scales & 3) == 0 &&
       tile_grid_x(gx, tgy, true) <= 0x7FFFFFFF) {
     dim3 grid = tile_grid(gx, tgy, batch, true), block(64 * MX_CAST_WAVES);
-    MX_DISPATCH_TILE(true, true, 0, (const uint16_t*)x, rows, cols, ldx, codes, scales, nblk,
+    MX_DISPATCH_TILE(true, true, 0, false, (const uint16_t*)x, rows, cols, ldx, codes, scales, nblk,
                      ks_n, codes_t, scales_t, nblk_t, ks_n_t, rows * ldx, s_b, st_b, (uint32_t)gx,
-                     (uint32_t)tgy, (const uint16_t*)nullptr, (int64_t)0, (uint16_t*)nullptr,
-                     (const uint16_t*)nullptr, (int64_t)0);
+                     (uint32_t)tgy, TileExtras{});
     return launch_status();
   }
   dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch), block(256);
@@ -981,6 +1011,37 @@ extern "C" int mx_scale_unlayout(const uint8_t* laid, int64_t rows, int64_t nblk
   return launch_status();
 }
 
+extern "C" int mx_cast_rows_gathered(const void* x, const int64_t* row_index, int64_t src_rows,
+                                     int64_t rows, int64_t cols, int64_t ldx, uint8_t* codes,
+                                     uint8_t* scales, uint8_t* codes_t, uint8_t* scales_t,
+                                     int scale_mode, int scale_order, void* stream) {
+  if (rows < 0 || cols < 0 || src_rows < 0 || ldx < cols || bad_enums(scale_mode, scale_order))
+    return MX_ERR_INVALID_ARG;
+  if (rows == 0 || cols == 0) return MX_OK;
+  if (!x || !row_index || !codes || !scales || (!codes_t) != (!scales_t)) return MX_ERR_INVALID_ARG;
+  if (cols % 32 || ldx % 8 || ((uintptr_t)x & 15) || ((uintptr_t)codes & 7) ||
+      ((uintptr_t)scales & 3) || ((uintptr_t)row_index & 7))
+    return MX_ERR_ALIGNMENT;
+  if (codes_t && (rows % 32 || ((uintptr_t)codes_t & 15) || ((uintptr_t)scales_t & 3)))
+    return MX_ERR_ALIGNMENT;
+  const int64_t nblk = cols / 32, ks_n = (nblk + 1) / 2;
+  const int64_t nblk_t = rows / 32, ks_n_t = (nblk_t + 1) / 2;
+  const int64_t gx = (cols + kT - 1) / kT, tgy = (rows + kTileRows - 1) / kTileRows;
+  if (tile_grid_x(gx, tgy, codes_t != nullptr) > 0x7FFFFFFF) return MX_ERR_UNSUPPORTED;
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid = tile_grid(gx, tgy, 1, codes_t != nullptr), block(64 * MX_CAST_WAVES);
+  const TileExtras ex{nullptr, 0, nullptr, nullptr, 0, row_index, src_rows};
+  if (codes_t)
+    MX_DISPATCH_TILE(true, true, 0, true, (const uint16_t*)x, rows, cols, ldx, codes, scales, nblk,
+                     ks_n, codes_t, scales_t, nblk_t, ks_n_t, (int64_t)0, (int64_t)0, (int64_t)0,
+                     (uint32_t)gx, (uint32_t)tgy, ex);
+  else
+    MX_DISPATCH_TILE(true, false, 0, true, (const uint16_t*)x, rows, cols, ldx, codes, scales, nblk,
+                     ks_n, (uint8_t*)nullptr, (uint8_t*)nullptr, (int64_t)0, (int64_t)0, (int64_t)0,
+                     (int64_t)0, (int64_t)0, (uint32_t)gx, (uint32_t)tgy, ex);
+  return launch_status();
+}
+
 extern "C" int mx_swiglu_cast_dim0_dim1(const void* a, const void* b, int64_t rows, int64_t cols,
                                         int64_t lda, int64_t ldb, uint8_t* codes, uint8_t* scales,
                                         uint8_t* codes_t, uint8_t* scales_t, void* g,
@@ -999,10 +1060,10 @@ extern "C" int mx_swiglu_cast_dim0_dim1(const void* a, const void* b, int64_t ro
   if (tile_grid_x(gx, tgy, true) > 0x7FFFFFFF) return MX_ERR_UNSUPPORTED;
   hipStream_t st = (hipStream_t)stream;
   dim3 grid = tile_grid(gx, tgy, 1, true), block(64 * MX_CAST_WAVES);
-  MX_DISPATCH_TILE(true, true, 1, (const uint16_t*)a, rows, cols, lda, codes, scales, nblk, ks_n,
+  MX_DISPATCH_TILE(true, true, 1, false, (const uint16_t*)a, rows, cols, lda, codes, scales, nblk, ks_n,
                    codes_t, scales_t, nblk_t, ks_n_t, (int64_t)0, (int64_t)0, (int64_t)0,
-                   (uint32_t)gx, (uint32_t)tgy, (const uint16_t*)b, ldb, (uint16_t*)g,
-                   (const uint16_t*)nullptr, (int64_t)0);
+                   (uint32_t)gx, (uint32_t)tgy,
+                   TileExtras{(const uint16_t*)b, ldb, (uint16_t*)g, nullptr, 0, nullptr, 0});
   return launch_status();
 }
 
@@ -1030,8 +1091,9 @@ extern "C" int mx_swiglu_bwd_cast_dim0_dim1(const void* dg, const void* a, const
   if (tile_grid_x(gx, tgy, true) > 0x7FFFFFFF) return MX_ERR_UNSUPPORTED;
   hipStream_t st = (hipStream_t)stream;
   dim3 grid = tile_grid(gx, tgy, 1, true), block(64 * MX_CAST_WAVES);
-  MX_DISPATCH_TILE(true, true, 2, (const uint16_t*)a, rows, cols, lda, codes, scales, nblk, ks_n,
+  MX_DISPATCH_TILE(true, true, 2, false, (const uint16_t*)a, rows, cols, lda, codes, scales, nblk, ks_n,
                    codes_t, scales_t, nblk_t, ks_n_t, (int64_t)0, s_b, st_b, (uint32_t)gx,
-                   (uint32_t)tgy, (const uint16_t*)b, ldb, (uint16_t*)dab, (const uint16_t*)dg, lddg);
+                   (uint32_t)tgy,
+                   TileExtras{(const uint16_t*)b, ldb, (uint16_t*)dab, (const uint16_t*)dg, lddg, nullptr, 0});
   return launch_status();
 }

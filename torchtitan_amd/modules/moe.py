@@ -15,6 +15,7 @@ import torch
 import torch.nn.functional as F
 from torch import nn
 
+from ..mx_tensor import grouped_feed_forward_fusable, mx_grouped_feed_forward
 from ..protocols import Module
 from ..quantization import MXFP8_GROUP_ALIGNMENT_SIZE
 
@@ -114,6 +115,8 @@ def _run_experts_for_loop(w1, w2, w3, x, num_tokens_per_expert):
 
 def _run_experts_grouped_mm(w1, w2, w3, x, num_tokens_per_expert):
     offsets = torch.cumsum(num_tokens_per_expert, dim=0, dtype=torch.int32)
+    if grouped_feed_forward_fusable(x, w1, w2, w3):  # converted experts: one fused function
+        return mx_grouped_feed_forward(x, w1, w2, w3, offsets).type_as(x)
     xb = x.bfloat16()
     h = F.silu(torch._grouped_mm(xb, w1.bfloat16().transpose(-2, -1), offs=offsets))
     h = h * torch._grouped_mm(xb, w3.bfloat16().transpose(-2, -1), offs=offsets)
@@ -134,6 +137,11 @@ class GroupedExperts(Module):
     def forward(self, x: torch.Tensor, num_tokens_per_expert: torch.Tensor) -> torch.Tensor:
         if self.use_grouped_mm:
             run = indices_padding_wrapper(_run_experts_grouped_mm)
+            if (num_tokens_per_expert.shape[0] == self.w1.shape[0]
+                    and grouped_feed_forward_fusable(x, self.w1, self.w2, self.w3)
+                    and self.w2.mx_config.pad_token_groups_for_grouped_mm):
+                # tokens already in expert order and the converted block aligns the groups itself
+                run = _run_experts_grouped_mm
         else:
             run = _run_experts_for_loop
         return run(self.w1, self.w2, self.w3, x, num_tokens_per_expert)

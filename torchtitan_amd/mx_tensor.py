@@ -400,6 +400,28 @@ def _pad_plan(offs: torch.Tensor, T: int, align: int = 32):
     return perm, m_offsets, back[:T]
 
 
+def _cast_into_groups(t: torch.Tensor, perm, mode: str, order: int, want_cols: bool):
+    """(row-wise, column-wise or None) casts of `t` moved into its padded group layout: the
+    gather by `perm` happens inside the cast kernel (padding slots read as zero rows)."""
+    if perm is not None:
+        return ops.to_mx_rows_gathered(t, perm, mode, order, want_cols)
+    if want_cols:
+        return ops.to_mx_dim0_dim1(t, mode, order)
+    return ops.to_mx_dim0(t, mode, order), None
+
+
+def _grouped_2d3d_padded(a: MXData, b: MXData, offs_p: torch.Tensor, back):
+    """Grouped GEMM in the padded layout, result moved back to the original row order.  One
+    spare zero row behind the GEMM's output serves rows that belong to no group."""
+    Tp, N = a.codes.shape[0], b.codes.shape[1]
+    if back is None:
+        return ops.mx_grouped_gemm_2d3d(a, b, offs_p)
+    buf = torch.empty((Tp + 1, N), dtype=torch.bfloat16, device=a.codes.device)
+    buf[Tp].zero_()
+    ops.mx_grouped_gemm_2d3d(a, b, offs_p, buf[:Tp])
+    return buf[back]
+
+
 class _MXGroupedMM(torch.autograd.Function):
     """out[rows of g] = x[rows of g] @ w[g]^T with w [G, N, K]; offs = inclusive cumsum, int32."""
 
@@ -416,28 +438,23 @@ class _MXGroupedMM(torch.autograd.Function):
         # run on the persistent kernel, which wants whole 128-row scale groups per expert.
         fast = (cfg.pad_token_groups_for_grouped_mm and K % 128 == 0 and N % 128 == 0 and G <= 638)
         order = MX_SCALES_MFMA if fast else MX_SCALES_ROWMAJOR
+        perm = back = None
         if cfg.pad_token_groups_for_grouped_mm:
             plan = _pad_plan(offs, T, 128 if fast else ops.BLOCK)
             perm, offs_p, back = plan
-            xb = torch.cat((xb, xb.new_zeros((1, K))), dim=0)[perm]
         else:
             offs_p = offs
             if T % ops.BLOCK:
                 raise ValueError("without padding the token dimension must be a multiple of 32")
         xb = xb.contiguous()
         need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
-        if need_dw:
-            xq0, xq1 = ops.to_mx_dim0_dim1(xb, mode, order)
-        else:
-            xq0, xq1 = ops.to_mx_dim0(xb, mode, order), None
+        xq0, xq1 = _cast_into_groups(xb, perm, mode, order, need_dw)
         if need_dx and N % ops.BLOCK == 0:
             wq0, wq1 = ops.to_mx_dim0_dim1_batched(w, mode, MX_SCALES_MFMA)
         else:
             wq0 = _cast_w_rows(w, mode)
             wq1 = None
-        y = ops.mx_grouped_gemm_2d3d(xq0, wq0, offs_p)
-        if plan is not None:
-            y = torch.cat((y, y.new_zeros((1, N))), dim=0)[back]
+        y = _grouped_2d3d_padded(xq0, wq0, offs_p, back)
         ctx.cfg = cfg
         ctx.dims = (T, K, N, G)
         ctx.dtypes = (x.dtype, weight.dtype)
@@ -461,16 +478,15 @@ class _MXGroupedMM(torch.autograd.Function):
         need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         saved = list(ctx.saved_tensors)
         offs_p = saved.pop(0)
-        dyb = dy if dy.dtype == torch.bfloat16 else dy.to(torch.bfloat16)
+        dyb = (dy if dy.dtype == torch.bfloat16 else dy.to(torch.bfloat16)).contiguous()
+        perm = back = None
         if ctx.padded:
             perm, back = saved.pop(0), saved.pop(0)
-            dyb = torch.cat((dyb, dyb.new_zeros((1, N))), dim=0)[perm]
-        dyb = dyb.contiguous()
         dx = dw = None
         if need_dw:
             xq1 = MXData(saved.pop(0), saved.pop(0), ctx.order)
-        if need_dx and need_dw and N % ops.BLOCK == 0:
-            dyq0, dyq1 = ops.to_mx_dim0_dim1(dyb, mode, ctx.order)
+        if ctx.padded or (need_dx and need_dw and N % ops.BLOCK == 0):
+            dyq0, dyq1 = _cast_into_groups(dyb, perm, mode, ctx.order, need_dw)
         else:
             dyq0 = ops.to_mx_dim0(dyb, mode, ctx.order) if need_dx else None
             dyq1 = ops.to_mx_dim1(dyb, mode, ctx.order) if need_dw else None
@@ -479,9 +495,7 @@ class _MXGroupedMM(torch.autograd.Function):
                 wq1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
             else:
                 wq1 = ops.to_mx_dim1_batched(saved.pop(0), mode, MX_SCALES_MFMA)
-            dx = ops.mx_grouped_gemm_2d3d(dyq0, wq1, offs_p)
-            if ctx.padded:
-                dx = torch.cat((dx, dx.new_zeros((1, K))), dim=0)[back]
+            dx = _grouped_2d3d_padded(dyq0, wq1, offs_p, back)
             if dx.dtype != ctx.dtypes[0]:
                 dx = dx.to(ctx.dtypes[0])
         if need_dw:
@@ -489,6 +503,114 @@ class _MXGroupedMM(torch.autograd.Function):
             if dw.dtype != ctx.dtypes[1]:
                 dw = dw.to(ctx.dtypes[1])
         return dx, dw, None, None
+
+
+class _MXGroupedFeedForward(torch.autograd.Function):
+    """The expert block ``grouped_mm(silu(grouped_mm(x, w1)) * grouped_mm(x, w3), w2)`` as one
+    function (torchtitan/models/common/moe/moe.py:59-76): tokens are moved into aligned groups
+    once instead of once per GEMM, x is cast once for w1 and w3, and the gate and its backward
+    run inside the cast kernels as in `_MXFeedForward`.  Bit-identical to the three converted
+    grouped GEMMs around bf16 ``F.silu`` and ``*``."""
+
+    @staticmethod
+    def forward(ctx, x, w1, w2, w3, offs, cfg: MXFP8Config):
+        mode = cfg.scale_mode
+        T, D = x.shape
+        G, H, _ = w1.shape
+        xb = _bf16(x)
+        pad = cfg.pad_token_groups_for_grouped_mm
+        fast = pad and D % 128 == 0 and H % 128 == 0 and G <= 638
+        order = MX_SCALES_MFMA if fast else MX_SCALES_ROWMAJOR
+        plan = perm = back = None
+        if pad:
+            plan = _pad_plan(offs, T, 128 if fast else ops.BLOCK)
+            perm, offs_p, back = plan
+        else:
+            offs_p = offs
+            if T % ops.BLOCK:
+                raise ValueError("without padding the token dimension must be a multiple of 32")
+        xb = xb.contiguous()
+        need_dx = ctx.needs_input_grad[0]
+        need_dw = any(ctx.needs_input_grad[1:4])
+        xq0, xq1 = _cast_into_groups(xb, perm, mode, order, need_dw)
+        both = lambda w: ops.to_mx_dim0_dim1_batched(_bf16(w).contiguous(), mode, MX_SCALES_MFMA)
+        rows = lambda w: (_cast_w_rows(_bf16(w).contiguous(), mode), None)
+        w1q0, w1q1 = both(w1) if need_dx else rows(w1)
+        w3q0, w3q1 = both(w3) if need_dx else rows(w3)
+        w2q0, w2q1 = both(w2) if (need_dx or need_dw) else rows(w2)
+        h1 = ops.mx_grouped_gemm_2d3d(xq0, w1q0, offs_p)
+        h3 = ops.mx_grouped_gemm_2d3d(xq0, w3q0, offs_p)
+        gq0, gq1, _ = ops.swiglu_to_mx_dim0_dim1(h1, h3, mode, order)
+        y = _grouped_2d3d_padded(gq0, w2q0, offs_p, back)
+        ctx.cfg, ctx.order, ctx.padded, ctx.D = cfg, order, plan is not None, D
+        ctx.dtypes = (x.dtype, w1.dtype, w2.dtype, w3.dtype)
+        ctx.need_dx, ctx.need_dw = need_dx, need_dw
+        saved = [offs_p]
+        if plan is not None:
+            saved += [plan[0], plan[2]]
+        if need_dx or need_dw:
+            saved += [h1, h3, w2q1.codes, w2q1.scales]
+        if need_dw:
+            saved += [xq1.codes, xq1.scales, gq1.codes, gq1.scales]
+        if need_dx:
+            saved += [w1q1.codes, w1q1.scales, w3q1.codes, w3q1.scales]
+        ctx.save_for_backward(*saved)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        mode, order = ctx.cfg.scale_mode, ctx.order
+        saved = list(ctx.saved_tensors)
+        offs_p = saved.pop(0)
+        dyb = _bf16(dy).contiguous()
+        perm = back = None
+        if ctx.padded:
+            perm, back = saved.pop(0), saved.pop(0)
+        h1, h3 = saved.pop(0), saved.pop(0)
+        w2q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
+        dyq0, dyq1 = _cast_into_groups(dyb, perm, mode, order, ctx.needs_input_grad[2])
+        dg = ops.mx_grouped_gemm_2d3d(dyq0, w2q1, offs_p)
+        (da0, da1), (db0, db1), _ = ops.swiglu_bwd_to_mx_dim0_dim1(dg, h1, h3, mode, order)
+        dx = dw1 = dw2 = dw3 = None
+        cast_back = lambda g, dt: g if g.dtype == dt else g.to(dt)
+        if ctx.need_dw:
+            xq1 = MXData(saved.pop(0), saved.pop(0), order)
+            gq1 = MXData(saved.pop(0), saved.pop(0), order)
+            if ctx.needs_input_grad[1]:
+                dw1 = cast_back(ops.mx_grouped_gemm_2d2d(da1, xq1, offs_p), ctx.dtypes[1])
+            if ctx.needs_input_grad[2]:
+                dw2 = cast_back(ops.mx_grouped_gemm_2d2d(dyq1, gq1, offs_p), ctx.dtypes[2])
+            if ctx.needs_input_grad[3]:
+                dw3 = cast_back(ops.mx_grouped_gemm_2d2d(db1, xq1, offs_p), ctx.dtypes[3])
+        if ctx.need_dx:
+            w1q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
+            w3q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
+            dx = _grouped_2d3d_padded(da0, w1q1, offs_p, back) + _grouped_2d3d_padded(db0, w3q1, offs_p, back)
+            dx = cast_back(dx, ctx.dtypes[0])
+        return dx, dw1, dw2, dw3, None, None
+
+
+def grouped_feed_forward_fusable(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
+                                 w3: torch.Tensor) -> bool:
+    """All three expert parameters converted with gate fusion on, a 2-D GPU activation, model
+    and hidden sizes multiples of 32."""
+    ws = (w1, w2, w3)
+    if not all(isinstance(w, MXFP8TrainingWeight) and w.mx_config.fuse_swiglu_cast and w.dim() == 3 for w in ws):
+        return False
+    if x.dim() != 2 or not x.is_cuda or x.numel() == 0 or w1.shape != w3.shape:
+        return False
+    if w1.mx_config.scale_mode != w2.mx_config.scale_mode or w1.mx_config.scale_mode != w3.mx_config.scale_mode:
+        return False
+    return x.shape[-1] % ops.BLOCK == 0 and w1.shape[1] % ops.BLOCK == 0
+
+
+def mx_grouped_feed_forward(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, w3: torch.Tensor,
+                            offs: torch.Tensor):
+    """The SwiGLU expert block for converted 3-D parameters w1, w3 [G, hidden, dim] and
+    w2 [G, dim, hidden]; offs = inclusive cumulative group sizes.  Returns bf16.
+    Callers check `grouped_feed_forward_fusable` first."""
+    return _MXGroupedFeedForward.apply(x, _unwrap(w1), _unwrap(w2), _unwrap(w3), offs.to(torch.int32),
+                                       w2.mx_config)
 
 
 def _cast_w_rows(w: torch.Tensor, mode: str) -> MXData:

@@ -149,6 +149,29 @@ def to_mx_dim0_dim1(x: torch.Tensor, mode="floor", order: int = MX_SCALES_ROWMAJ
     return MXData(codes, scales, order), MXData(codes_t, scales_t, order)
 
 
+def to_mx_rows_gathered(x: torch.Tensor, row_index: torch.Tensor, mode="floor",
+                        order: int = MX_SCALES_ROWMAJOR, want_cols: bool = True):
+    """Casts of x[row_index] (index -1, or any index outside x, = a row of zeros) without forming
+    the gathered tensor; returns (row-wise MXData, column-wise MXData or None)."""
+    x = _check_hp(x)
+    if row_index.dtype != torch.int64 or row_index.dim() != 1 or row_index.device != x.device:
+        raise TypeError("row_index must be a 1-D int64 tensor on x's device")
+    row_index = row_index.contiguous()
+    R, C = row_index.numel(), x.shape[1]
+    if C % BLOCK or (want_cols and R % BLOCK):
+        raise ValueError(f"dims {R}, {C} must be multiples of {BLOCK}")
+    codes = torch.empty((R, C), dtype=torch.uint8, device=x.device)
+    scales = _alloc_scales(R, C // BLOCK, order, x.device)
+    codes_t = scales_t = None
+    if want_cols:
+        codes_t = torch.empty((C, R), dtype=torch.uint8, device=x.device)
+        scales_t = _alloc_scales(C, R // BLOCK, order, x.device)
+    _call("mx_cast_rows_gathered", "cast_rows_gathered", x.device, _ptr(x), _ptr(row_index), x.shape[0],
+          R, C, x.stride(0), _ptr(codes), _ptr(scales), _ptr(codes_t) if want_cols else None,
+          _ptr(scales_t) if want_cols else None, _mode(mode), order, _stream(x))
+    return MXData(codes, scales, order), (MXData(codes_t, scales_t, order) if want_cols else None)
+
+
 def swiglu_to_mx_dim0_dim1(a: torch.Tensor, b: torch.Tensor, mode="floor",
                            order: int = MX_SCALES_ROWMAJOR, want_g: bool = False):
     """Both casts of g = silu(a) * b (bf16, every step rounded to bf16) without g passing through
