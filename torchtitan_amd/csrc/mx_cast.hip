@@ -640,6 +640,7 @@ struct TileExtras {
   int64_t ldx4 = 0;
   const int64_t* row_idx = nullptr;  // GATHER: source row of every output row
   int64_t src_rows = 0;
+  uint32_t batch = 1;  // stacked independent matrices
 };
 
 // The gate-backward variant is bound by vector ALU work: four workgroups per CU (128 VGPRs).
@@ -658,24 +659,27 @@ __global__ __launch_bounds__(64 * WAVES, GATE == 2 ? 4 : 1) void cast_tile_kerne
   __shared__ __attribute__((aligned(16))) uint8_t lds_codes[COL ? TC * PITCH : 16];
   __shared__ __attribute__((aligned(16))) uint8_t lds_st[COL ? TC * WAVES : 16];
   __shared__ __attribute__((aligned(16))) uint8_t lds_sr[ROW ? TR * 4 : 16];
-  x += blockIdx.z * x_bstride;  // batch of independent [rows, cols] matrices
-  if (ROW) {
-    codes += blockIdx.z * rows * cols;
-    scales += blockIdx.z * s_bstride;
-  }
-  if (COL) {
-    codes_t += blockIdx.z * rows * cols;
-    scales_t += blockIdx.z * st_bstride;
-  }
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 4, q = lane & 15;
   const int rl0 = wave * 32 + 8 * g;  // first tile-local row of this lane
 
+  // a batch of independent [rows, cols] matrices is walked as one stack of gy * batch tile rows
   constexpr uint32_t BX = TileWalk<COL>::BX, BY = TileWalk<COL>::BY;
+  const uint32_t gy_all = gy * ex.batch;
   const uint32_t spr = (gx + BX - 1) / BX;
   const uint32_t sup = blockIdx.x / (BX * BY), in = blockIdx.x % (BX * BY);
   const uint32_t bx = (sup % spr) * BX + in / BY;
-  const uint32_t by = (sup / spr) * BY + in % BY;
-  if (bx >= gx || by >= gy) return;
+  const uint32_t by_all = (sup / spr) * BY + in % BY;
+  if (bx >= gx || by_all >= gy_all) return;
+  const uint32_t bz = by_all / gy, by = by_all - bz * gy;
+  x += bz * x_bstride;
+  if (ROW) {
+    codes += bz * rows * cols;
+    scales += bz * s_bstride;
+  }
+  if (COL) {
+    codes_t += bz * rows * cols;
+    scales_t += bz * st_bstride;
+  }
 
   const int64_t r0 = (int64_t)by * TR, c0 = (int64_t)bx * TC;
   const int64_t c = c0 + 8 * q;
@@ -834,7 +838,12 @@ static inline int64_t tile_grid_x(int64_t gx, int64_t gy, bool col) {
   return ((gx + bx - 1) / bx) * ((gy + by - 1) / by) * (bx * by);
 }
 static inline dim3 tile_grid(int64_t gx, int64_t gy, int64_t batch, bool col) {
-  return dim3((unsigned)tile_grid_x(gx, gy, col), 1, (unsigned)batch);
+  return dim3((unsigned)tile_grid_x(gx, gy * batch, col));
+}
+static inline TileExtras tile_batch(int64_t batch) {
+  TileExtras ex;
+  ex.batch = (uint32_t)batch;
+  return ex;
 }
 
 static inline bool bad_enums(int scale_mode, int scale_order) {
@@ -911,12 +920,12 @@ extern "C" int mx_cast_dim1_batched(const void* x, int64_t batch, int64_t rows, 
   if (gy > 65535 || batch > 65535 || gx > 0x7FFFFFFF) return MX_ERR_UNSUPPORTED;
   hipStream_t st = (hipStream_t)stream;
   const int64_t tgy = (rows + kTileRows - 1) / kTileRows;
-  if (tile_ok(x, cols, ldx) && tile_grid_x(gx, tgy, true) <= 0x7FFFFFFF) {
+  if (tile_ok(x, cols, ldx) && tile_grid_x(gx, tgy * batch, true) <= 0x7FFFFFFF) {
     dim3 grid = tile_grid(gx, tgy, batch, true), block(64 * MX_CAST_WAVES);
     MX_DISPATCH_TILE(false, true, 0, false, (const uint16_t*)x, rows, cols, ldx, (uint8_t*)nullptr,
                      (uint8_t*)nullptr, (int64_t)0, (int64_t)0, codes_t, scales_t, nblk_t, ks_n_t,
                      rows * ldx, (int64_t)0, st_b, (uint32_t)gx, (uint32_t)tgy,
-                     TileExtras{});
+                     tile_batch(batch));
     return launch_status();
   }
   dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch), block(256);
@@ -953,11 +962,11 @@ extern "C" int mx_cast_dim0_dim1_batched(const void* x, int64_t batch, int64_t r
   if (scale_order == MX_SCALES_MFMA && ((uintptr_t)scales & 3)) return MX_ERR_ALIGNMENT;
   const int64_t tgy = (rows + kTileRows - 1) / kTileRows;
   if (tile_ok(x, cols, ldx) && ((uintptr_t)codes & 7) == 0 && ((uintptr_t)scales & 3) == 0 &&
-      tile_grid_x(gx, tgy, true) <= 0x7FFFFFFF) {
+      tile_grid_x(gx, tgy * batch, true) <= 0x7FFFFFFF) {
     dim3 grid = tile_grid(gx, tgy, batch, true), block(64 * MX_CAST_WAVES);
     MX_DISPATCH_TILE(true, true, 0, false, (const uint16_t*)x, rows, cols, ldx, codes, scales, nblk,
                      ks_n, codes_t, scales_t, nblk_t, ks_n_t, rows * ldx, s_b, st_b, (uint32_t)gx,
-                     (uint32_t)tgy, TileExtras{});
+                     (uint32_t)tgy, tile_batch(batch));
     return launch_status();
   }
   dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch), block(256);
