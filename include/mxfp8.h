@@ -89,15 +89,36 @@ int mx_cast_dim0_dim1_batched(const void* x, int64_t batch, int64_t rows, int64_
 
 /* Cast of gathered rows: output row r is row row_index[r] of x (bf16 [src_rows, cols], row
  * stride ldx); an index outside [0, src_rows) gives a row of zeros (the padding slots of an
- * aligned token-group layout hold -1).  Row-wise cast always; the column-wise cast too unless
+ * aligned token-group layout hold -1).  With row_scale (float32 [rows], may be NULL) row r is
+ * first multiplied by row_scale[r] in float32 and rounded to bf16: the routing-score multiply
+ * `(routed_input.float() * top_scores).to(dtype)` of torchtitan/models/common/moe/moe.py:519-527.  Row-wise cast always; the column-wise cast too unless
  * codes_t and scales_t are both NULL (then `rows` need not be a multiple of 32).  Outputs as
  * mx_cast_dim0_dim1 for a [rows, cols] matrix.  Requires cols % 32 == 0, ldx % 8 == 0, x 16-byte
  * aligned.  Stands in for the token permutation `x[permuted_indices, :]` in front of the grouped
  * GEMMs (torchtitan/models/common/moe/utils.py:65-89) followed by the cast of its result. */
-int mx_cast_rows_gathered(const void* x, const int64_t* row_index, int64_t src_rows, int64_t rows,
-                          int64_t cols, int64_t ldx, uint8_t* codes, uint8_t* scales,
-                          uint8_t* codes_t, uint8_t* scales_t, int scale_mode, int scale_order,
-                          void* stream);
+int mx_cast_rows_gathered(const void* x, const int64_t* row_index, const float* row_scale,
+                          int64_t src_rows, int64_t rows, int64_t cols, int64_t ldx,
+                          uint8_t* codes, uint8_t* scales, uint8_t* codes_t, uint8_t* scales_t,
+                          int scale_mode, int scale_order, void* stream);
+
+/* Combine of the routed expert outputs: out[t, :] = sum_j weights[t, j] * y[pos[t, j], :] for
+ * j = 0 .. top_k-1 in that order, in float32 (product and sum rounded separately), result
+ * rounded to bf16; weights == NULL gives the plain sum.  y: bf16 [y_rows, cols] (row stride
+ * ldy), pos: int64 [tokens, top_k] rows of y (outside [0, y_rows): contributes nothing), out:
+ * bf16 [tokens, cols] (row stride ldo).  cols % 8 == 0, 16-byte aligned rows.
+ * Stands in for the un-sort scatter and the score-weighted sum over top_k of
+ * torchtitan/models/common/moe/moe.py:535-555, and (with y = the gradient of the routed input)
+ * for the backward of the token gather `x[token_indices // top_k]` (moe.py:519). */
+int mx_moe_combine(const void* y, int64_t y_rows, int64_t ldy, const int64_t* pos,
+                   const float* weights, int64_t tokens, int64_t top_k, int64_t cols, void* out,
+                   int64_t ldo, void* stream);
+
+/* Row dot products out[i] = sum_d a[ia[i], d] * b[ib[i], d] in float32 over bf16 matrices
+ * a [a_rows, cols], b [b_rows, cols]; an index outside its matrix gives 0.  The gradient of the
+ * routing scores on either side of the experts (backward of moe.py:521-527 and :541-551). */
+int mx_moe_row_dot(const void* a, int64_t a_rows, int64_t lda, const int64_t* ia, const void* b,
+                   int64_t b_rows, int64_t ldb, const int64_t* ib, int64_t n, int64_t cols,
+                   float* out, void* stream);
 
 /* SwiGLU gate fused into the cast: g = silu(a) * b elementwise over bf16 [rows, cols] (row strides
  * lda, ldb), each step rounded to bf16 as the unfused tensor ops round it, then both casts of g

@@ -40,6 +40,11 @@ Pinning status (what fixes each function independently of its own formula):
                                         float32 evaluation is PARITY UNPINNED (see its docstring)
   swiglu_backward_bf16       pinned  -- closed form vs a central difference and torch's CPU op;
                                         last bf16 ulp of da PARITY UNPINNED (see its docstring)
+  gather_rows                pinned  -- index semantics vs torch indexing; score product exact
+                                        before its bf16 rounding (torch CPU ops)
+  moe_combine                pinned  -- vs an exact float64 sum (within one bf16 step) and torch's
+                                        scatter + bmm on the CPU; accumulation order PARITY UNPINNED
+  moe_row_dot                pinned  -- float64 dot products (textbook)
   generate_permute_indices   pinned  -- the worked example and invariants of
                                         torchtitan/models/common/moe/kernels.py:145-218
                                         and tests/unit_tests/test_permute_indices_kernel.py
@@ -402,6 +407,49 @@ def swiglu_backward_bf16(dg_bits: np.ndarray, a_bits: np.ndarray, b_bits: np.nda
         s = 1.0 / (1.0 + e)
         da = t * s * (1.0 + a * (1.0 - s))
         return f32_to_bf16_bits(da.astype(np.float32)), db
+
+
+def gather_rows(x_bits: np.ndarray, row_index: np.ndarray, row_scale: np.ndarray | None = None) -> np.ndarray:
+    """Rows x[row_index] with rows of zeros where the index is outside x (the -1 padding slots
+    of torchtitan/models/common/moe/utils.py:78-80), optionally multiplied by a float32 score
+    per row with the product rounded to bf16 (moe.py:521-527)."""
+    n = x_bits.shape[0]
+    ok = (row_index >= 0) & (row_index < n)
+    rows = np.where(ok[:, None], x_bits[np.clip(row_index, 0, max(n - 1, 0))], 0).astype(np.uint16)
+    if row_scale is None:
+        return rows
+    with np.errstate(over="ignore", invalid="ignore"):
+        scaled = f32_to_bf16_bits(bf16_bits_to_f32(rows) * row_scale.astype(np.float32)[:, None])
+    return np.where(ok[:, None], scaled, 0).astype(np.uint16)
+
+
+def moe_combine(y_bits: np.ndarray, pos: np.ndarray, weights: np.ndarray | None = None) -> np.ndarray:
+    """out[t] = sum_j weights[t, j] * y[pos[t, j]] accumulated in float32 for j = 0 .. k-1 in
+    that order (product and sum rounded separately), rounded to bf16: the score-weighted
+    combine of the top-k expert outputs (moe.py:535-555, where a scatter, a float upcast and a
+    bmm / sum do it).  The reference's own summation order inside bmm / sum is not specified:
+    PARITY UNPINNED in the last float32 bit of the accumulation; against an exact sum the result
+    is within one bf16 step (tested)."""
+    T, k = pos.shape
+    y = bf16_bits_to_f32(y_bits)
+    acc = np.zeros((T, y.shape[1]), dtype=np.float32)
+    for j in range(k):
+        r = pos[:, j]
+        ok = (r >= 0) & (r < y.shape[0])
+        rows = y[np.clip(r, 0, y.shape[0] - 1)]
+        with np.errstate(over="ignore", invalid="ignore"):
+            term = rows if weights is None else (weights[:, j].astype(np.float32)[:, None] * rows).astype(np.float32)
+            acc = np.where(ok[:, None], (acc + term).astype(np.float32), acc)
+    return f32_to_bf16_bits(acc)
+
+
+def moe_row_dot(a_bits: np.ndarray, ia: np.ndarray, b_bits: np.ndarray, ib: np.ndarray) -> np.ndarray:
+    """out[i] = <a[ia[i]], b[ib[i]]> in float64 (the gradient of a routing score is the dot
+    product of the two rows its product joined); 0 where an index is outside its matrix."""
+    a, b = bf16_bits_to_f32(a_bits).astype(np.float64), bf16_bits_to_f32(b_bits).astype(np.float64)
+    ok = (ia >= 0) & (ia < a.shape[0]) & (ib >= 0) & (ib < b.shape[0])
+    d = np.einsum("ij,ij->i", a[np.clip(ia, 0, a.shape[0] - 1)], b[np.clip(ib, 0, b.shape[0] - 1)])
+    return np.where(ok, d, 0.0)
 
 
 def make_cfg1_inputs(seed: int, M: int = 8192, K: int = 4096, N: int = 4096):

@@ -297,3 +297,44 @@ def test_cast_of_gathered_rows(device, mode_name, mode, src_rows, rows, cols):
         assert np.array_equal(u8(q1.codes), c1) and np.array_equal(u8(q1.scales).reshape(-1), s1.reshape(-1))
         r0, none = ops.to_mx_rows_gathered(x, ti, mode_name, order, want_cols=False)
         assert none is None and torch.equal(r0.codes, q0.codes) and torch.equal(r0.scales, q0.scales)
+
+
+@pytest.mark.parametrize("mode_name,mode", MODES)
+def test_cast_of_gathered_rows_with_scores(device, mode_name, mode):
+    """The routing-score multiply in front of the experts folded into the gathered cast."""
+    rng = np.random.default_rng(31)
+    src_rows, rows, cols = 200, 672, 192
+    bits = randn_bits(rng, (src_rows, cols), outliers=1e-3)
+    idx = rng.integers(-1, src_rows, rows).astype(np.int64)
+    scale = rng.random(rows).astype(np.float32) * 2
+    gathered = mo.gather_rows(bits, idx, scale)
+    q0, q1 = ops.to_mx_rows_gathered(bf16_from_bits(bits, device), torch.from_numpy(idx).to(device), mode_name,
+                                     ops.MX_SCALES_MFMA, row_scale=torch.from_numpy(scale).to(device))
+    c0, s0 = mo.cast_dim0(gathered, mode)
+    c1, s1 = mo.cast_dim1(gathered, mode)
+    assert np.array_equal(u8(q0.codes), c0) and np.array_equal(u8(q0.scales).reshape(-1), mo.scale_layout(s0).reshape(-1))
+    assert np.array_equal(u8(q1.codes), c1) and np.array_equal(u8(q1.scales).reshape(-1), mo.scale_layout(s1).reshape(-1))
+
+
+@pytest.mark.parametrize("tokens,k,cols", [(64, 1, 64), (300, 4, 256), (1000, 8, 2048)])
+def test_moe_combine_and_row_dot(device, tokens, k, cols):
+    """Weighted top-k combine bit-exact against the oracle's float32 sequential sum; score
+    gradients (row dot products) to 1e-5 of the float64 oracle (float32 reduction)."""
+    rng = np.random.default_rng(tokens + k)
+    rows = tokens * k + 40
+    y_bits = randn_bits(rng, (rows, cols))
+    pos = rng.permutation(rows)[: tokens * k].astype(np.int64).reshape(tokens, k)
+    pos[rng.integers(0, tokens), rng.integers(0, k)] = -1
+    pos[rng.integers(0, tokens), rng.integers(0, k)] = rows + 3
+    w = rng.random((tokens, k)).astype(np.float32)
+    y = bf16_from_bits(y_bits, device)
+    tp = torch.from_numpy(pos).to(device)
+    got = ops.moe_combine(y, tp, torch.from_numpy(w).to(device))
+    assert np.array_equal(bits_of(got), mo.moe_combine(y_bits, pos, w))
+    got = ops.moe_combine(y, tp)
+    assert np.array_equal(bits_of(got), mo.moe_combine(y_bits, pos, None))
+    x_bits = randn_bits(rng, (tokens, cols))
+    ib = (np.arange(tokens * k) // k).astype(np.int64)
+    d = ops.moe_row_dot(y, tp.view(-1), bf16_from_bits(x_bits, device), torch.from_numpy(ib).to(device))
+    ref = mo.moe_row_dot(y_bits, pos.reshape(-1), x_bits, ib)
+    assert np.allclose(d.cpu().numpy().astype(np.float64), ref, rtol=1e-5, atol=1e-5 * np.sqrt(cols))

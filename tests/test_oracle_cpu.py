@@ -96,6 +96,46 @@ def test_swiglu_backward_vs_torch_autograd_and_central_difference():
     assert np.allclose(s * (1 + x * (1 - s)), (silu(x + 1e-6) - silu(x - 1e-6)) / 2e-6, atol=1e-8)
 
 
+def test_moe_gather_and_combine_vs_torch_cpu_ops():
+    """gather_rows against torch indexing + the float32 score multiply; moe_combine against the
+    reference's un-sort scatter + float bmm / sum (moe.py:519-555) run with torch on the CPU and
+    against an exact float64 sum."""
+    rng = np.random.default_rng(9)
+    T, k, D = 96, 4, 64
+    t = lambda bits: torch.from_numpy(bits.view(np.int16)).view(torch.bfloat16)
+    b = lambda x: x.contiguous().view(torch.int16).numpy().view(np.uint16)
+    x = mo.f32_to_bf16_bits(rng.standard_normal((T, D)).astype(np.float32))
+    scores = rng.random((T, k)).astype(np.float32)
+    order = rng.permutation(T * k)  # token_indices_experts_sorted
+    # dispatch: routed_input = (x[order // k].float() * scores_sorted).to(bf16)
+    want = (t(x)[torch.from_numpy(order // k)].float() * torch.from_numpy(scores.reshape(-1)[order])[:, None]).to(torch.bfloat16)
+    got = mo.gather_rows(x, order // k, scores.reshape(-1)[order])
+    assert np.array_equal(got, b(want))
+    idx = np.array([3, -1, T + 2, 0])
+    assert np.array_equal(mo.gather_rows(x, idx)[[1, 2]], np.zeros((2, D), np.uint16))
+    assert np.array_equal(mo.gather_rows(x, idx)[[0, 3]], x[[3, 0]])
+    # combine: y rows in sorted order; unsorted[order] = y; out = bmm(scores, unsorted.float())
+    y = mo.f32_to_bf16_bits(rng.standard_normal((T * k, D)).astype(np.float32))
+    pos = np.empty(T * k, dtype=np.int64)
+    pos[order] = np.arange(T * k)
+    pos = pos.reshape(T, k)
+    unsorted = torch.zeros((T * k, D), dtype=torch.bfloat16)
+    unsorted[torch.from_numpy(order)] = t(y)
+    unsorted = unsorted.reshape(T, k, D)
+    exact = lambda w: np.einsum("tk,tkd->td", w.astype(np.float64), mo.bf16_bits_to_f32(b(unsorted)).astype(np.float64))
+    near = lambda got, ex: np.abs(mo.bf16_bits_to_f32(got).astype(np.float64) - ex) <= np.abs(ex) * 2.0 ** -8 + 1e-30
+    for w in (scores, None):
+        got = mo.moe_combine(y, pos, w)
+        ref = (torch.bmm(torch.from_numpy(scores).reshape(T, 1, k), unsorted.float()).to(torch.bfloat16).squeeze(1)
+               if w is not None else unsorted.sum(dim=1))
+        differ = got != b(ref)
+        assert differ.mean() < 0.02          # only accumulation-order effects
+        assert near(got, exact(w if w is not None else np.ones((T, k), np.float32))).all()
+    d = mo.moe_row_dot(y, pos.reshape(-1), x, np.arange(T * k) // k)
+    ref = (unsorted.float() * t(x).float()[:, None, :]).sum(-1).numpy().reshape(-1)
+    assert np.allclose(d, ref, rtol=1e-4, atol=1e-5)
+
+
 # ------------------------------------------------------------------ scales
 def _normal_finite():
     a = ALL_BF16[(ALL_BF16 >= 0x0080) & (ALL_BF16 < 0x7F80)]

@@ -617,16 +617,26 @@ __device__ __forceinline__ void emit_tile(
 
 // As load_patch, with the source row of output row r taken from row_idx[r]; an index outside
 // [0, src_rows) (the padding slots of a token-group layout hold -1) reads as a row of zeros.
+// With row_scale, every element of output row r is multiplied by row_scale[r] in float32 and
+// rounded back to bf16 first (the routing-score multiply in front of the experts).
+__device__ __forceinline__ uint32_t scale2(uint32_t w, float s) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f_t{bf16_lo(w) * s, bf16_hi(w) * s}, v2bf_t));
+}
 __device__ __forceinline__ void load_patch_rows(u32x4 (&v)[8], const uint16_t* x, int64_t ld,
                                                 int64_t c, const int64_t* row_idx, int64_t src_rows,
-                                                bool col_ok, int rows_left) {
+                                                const float* row_scale, bool col_ok, int rows_left) {
 #pragma unroll
   for (int k = 0; k < 8; ++k) {
     v[k] = u32x4{0, 0, 0, 0};
     if (col_ok && k < rows_left) {
       const int64_t r = row_idx[k];
-      if (r >= 0 && r < src_rows)
+      if (r >= 0 && r < src_rows) {
         v[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(x + r * ld + c));
+        if (row_scale) {
+          const float s = row_scale[k];
+          v[k] = u32x4{scale2(v[k].x, s), scale2(v[k].y, s), scale2(v[k].z, s), scale2(v[k].w, s)};
+        }
+      }
     }
   }
 }
@@ -641,6 +651,7 @@ struct TileExtras {
   const int64_t* row_idx = nullptr;  // GATHER: source row of every output row
   int64_t src_rows = 0;
   uint32_t batch = 1;  // stacked independent matrices
+  const float* row_scale = nullptr;  // GATHER: optional multiplier of every output row
 };
 
 // The gate-backward variant is bound by vector ALU work: four workgroups per CU (128 VGPRs).
@@ -689,7 +700,8 @@ __global__ __launch_bounds__(64 * WAVES, GATE == 2 ? 4 : 1) void cast_tile_kerne
 
   u32x4 v[8];
   if constexpr (GATHER)
-    load_patch_rows(v, x, ldx, c, ex.row_idx + r0 + rl0, ex.src_rows, col_ok, rows_left);
+    load_patch_rows(v, x, ldx, c, ex.row_idx + r0 + rl0, ex.src_rows,
+                    ex.row_scale ? ex.row_scale + r0 + rl0 : nullptr, col_ok, rows_left);
   else
     load_patch(v, x + (r0 + rl0) * ldx + c, ldx, col_ok, rows_left);
   if constexpr (GATE == 1) {  // x = gate input a, x3 = b: quantize g = silu(a) * b
@@ -1020,7 +1032,8 @@ extern "C" int mx_scale_unlayout(const uint8_t* laid, int64_t rows, int64_t nblk
   return launch_status();
 }
 
-extern "C" int mx_cast_rows_gathered(const void* x, const int64_t* row_index, int64_t src_rows,
+extern "C" int mx_cast_rows_gathered(const void* x, const int64_t* row_index,
+                                     const float* row_scale, int64_t src_rows,
                                      int64_t rows, int64_t cols, int64_t ldx, uint8_t* codes,
                                      uint8_t* scales, uint8_t* codes_t, uint8_t* scales_t,
                                      int scale_mode, int scale_order, void* stream) {
@@ -1029,7 +1042,7 @@ extern "C" int mx_cast_rows_gathered(const void* x, const int64_t* row_index, in
   if (rows == 0 || cols == 0) return MX_OK;
   if (!x || !row_index || !codes || !scales || (!codes_t) != (!scales_t)) return MX_ERR_INVALID_ARG;
   if (cols % 32 || ldx % 8 || ((uintptr_t)x & 15) || ((uintptr_t)codes & 7) ||
-      ((uintptr_t)scales & 3) || ((uintptr_t)row_index & 7))
+      ((uintptr_t)scales & 3) || ((uintptr_t)row_index & 7) || ((uintptr_t)row_scale & 3))
     return MX_ERR_ALIGNMENT;
   if (codes_t && (rows % 32 || ((uintptr_t)codes_t & 15) || ((uintptr_t)scales_t & 3)))
     return MX_ERR_ALIGNMENT;
@@ -1039,7 +1052,10 @@ extern "C" int mx_cast_rows_gathered(const void* x, const int64_t* row_index, in
   if (tile_grid_x(gx, tgy, codes_t != nullptr) > 0x7FFFFFFF) return MX_ERR_UNSUPPORTED;
   hipStream_t st = (hipStream_t)stream;
   dim3 grid = tile_grid(gx, tgy, 1, codes_t != nullptr), block(64 * MX_CAST_WAVES);
-  const TileExtras ex{nullptr, 0, nullptr, nullptr, 0, row_index, src_rows};
+  TileExtras ex;
+  ex.row_idx = row_index;
+  ex.src_rows = src_rows;
+  ex.row_scale = row_scale;
   if (codes_t)
     MX_DISPATCH_TILE(true, true, 0, true, (const uint16_t*)x, rows, cols, ldx, codes, scales, nblk,
                      ks_n, codes_t, scales_t, nblk_t, ks_n_t, (int64_t)0, (int64_t)0, (int64_t)0,

@@ -150,10 +150,16 @@ def to_mx_dim0_dim1(x: torch.Tensor, mode="floor", order: int = MX_SCALES_ROWMAJ
 
 
 def to_mx_rows_gathered(x: torch.Tensor, row_index: torch.Tensor, mode="floor",
-                        order: int = MX_SCALES_ROWMAJOR, want_cols: bool = True):
+                        order: int = MX_SCALES_ROWMAJOR, want_cols: bool = True,
+                        row_scale: torch.Tensor | None = None):
     """Casts of x[row_index] (index -1, or any index outside x, = a row of zeros) without forming
-    the gathered tensor; returns (row-wise MXData, column-wise MXData or None)."""
+    the gathered tensor; returns (row-wise MXData, column-wise MXData or None).  `row_scale`
+    (float32, one per output row) multiplies the rows in float32, rounded to bf16, first."""
     x = _check_hp(x)
+    if row_scale is not None:
+        if row_scale.dtype != torch.float32 or row_scale.shape != row_index.shape or row_scale.device != x.device:
+            raise TypeError("row_scale must be float32 with one entry per output row on x's device")
+        row_scale = row_scale.contiguous()
     if row_index.dtype != torch.int64 or row_index.dim() != 1 or row_index.device != x.device:
         raise TypeError("row_index must be a 1-D int64 tensor on x's device")
     row_index = row_index.contiguous()
@@ -166,10 +172,49 @@ def to_mx_rows_gathered(x: torch.Tensor, row_index: torch.Tensor, mode="floor",
     if want_cols:
         codes_t = torch.empty((C, R), dtype=torch.uint8, device=x.device)
         scales_t = _alloc_scales(C, R // BLOCK, order, x.device)
-    _call("mx_cast_rows_gathered", "cast_rows_gathered", x.device, _ptr(x), _ptr(row_index), x.shape[0],
+    _call("mx_cast_rows_gathered", "cast_rows_gathered", x.device, _ptr(x), _ptr(row_index),
+          _ptr(row_scale) if row_scale is not None else None, x.shape[0],
           R, C, x.stride(0), _ptr(codes), _ptr(scales), _ptr(codes_t) if want_cols else None,
           _ptr(scales_t) if want_cols else None, _mode(mode), order, _stream(x))
     return MXData(codes, scales, order), (MXData(codes_t, scales_t, order) if want_cols else None)
+
+
+def moe_combine(y: torch.Tensor, pos: torch.Tensor, weights: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t] = sum_j weights[t, j] * y[pos[t, j]] (float32, j in order; plain sum without
+    weights), bf16 [tokens, cols].  y: bf16 [rows, cols]; pos: int64 [tokens, top_k]; a position
+    outside y contributes nothing."""
+    y = _check_hp(y)
+    if pos.dtype != torch.int64 or pos.dim() != 2 or pos.device != y.device:
+        raise TypeError("pos must be a 2-D int64 tensor on y's device")
+    pos = pos.contiguous()
+    T, k = pos.shape
+    if weights is not None:
+        if weights.dtype != torch.float32 or weights.shape != pos.shape or weights.device != y.device:
+            raise TypeError("weights must be float32 of pos's shape on y's device")
+        weights = weights.contiguous()
+    out = torch.empty((T, y.shape[1]), dtype=torch.bfloat16, device=y.device)
+    _call("mx_moe_combine", "moe_combine", y.device, _ptr(y), y.shape[0], y.stride(0), _ptr(pos),
+          _ptr(weights) if weights is not None else None, T, k, y.shape[1], _ptr(out), out.stride(0),
+          _stream(y))
+    return out
+
+
+def moe_row_dot(a: torch.Tensor, ia: torch.Tensor, b: torch.Tensor, ib: torch.Tensor) -> torch.Tensor:
+    """out[i] = <a[ia[i]], b[ib[i]]> in float32 for bf16 matrices a, b with equal column counts;
+    an index outside its matrix gives 0."""
+    a, b = _check_hp(a), _check_hp(b)
+    if a.shape[1] != b.shape[1]:
+        raise ValueError(f"column mismatch: {a.shape[1]} vs {b.shape[1]}")
+    for idx in (ia, ib):
+        if idx.dtype != torch.int64 or idx.device != a.device:
+            raise TypeError("indices must be int64 on the matrices' device")
+    if ia.shape != ib.shape:
+        raise ValueError("index shapes differ")
+    ia_c, ib_c = ia.contiguous().view(-1), ib.contiguous().view(-1)
+    out = torch.empty(ia.shape, dtype=torch.float32, device=a.device)
+    _call("mx_moe_row_dot", "moe_row_dot", a.device, _ptr(a), a.shape[0], a.stride(0), _ptr(ia_c), _ptr(b),
+          b.shape[0], b.stride(0), _ptr(ib_c), ia_c.numel(), a.shape[1], _ptr(out), _stream(a))
+    return out
 
 
 def swiglu_to_mx_dim0_dim1(a: torch.Tensor, b: torch.Tensor, mode="floor",
