@@ -6,7 +6,7 @@ import torch.nn as nn
 
 from oracle import mx_oracle as mo
 from tests.helpers import bf16_from_bits, bits_of, randn_bits, rel_l2
-from torchtitan_amd.modules import FeedForward, GroupedExperts, Linear
+from torchtitan_amd.modules import FeedForward, GroupedExperts, Linear, MoE
 from torchtitan_amd.modules import moe as moe_mod
 from torchtitan_amd.mx_tensor import MXFP8TrainingWeight
 from torchtitan_amd.protocols import ModelConvertersContainer
@@ -296,6 +296,45 @@ def test_grouped_experts_fused_block_matches_separate_ops(device, pad, align, di
         assert not fusable(x, blocks[1].w1, blocks[1].w2, blocks[1].w3)
     finally:
         moe_mod.set_token_group_alignment_size_m(8)
+
+
+@pytest.mark.parametrize("score_before", [True, False])
+@pytest.mark.parametrize("dim,hidden,experts,top_k", [(128, 64, 8, 2), (256, 128, 16, 4)])
+def test_moe_layer_fused_routing_matches_torch_ops(device, score_before, dim, hidden, experts, top_k):
+    """MoE layer with gather + score + experts + combine as one fused function against the same
+    layer built from torch's gather / scatter / bmm around the converted experts.  Expert weight
+    gradients are bit-identical (the experts see bit-identical inputs and output gradients); the
+    output, dx and the router's gradient differ only by float32 summation order over top_k and
+    over the row dot products: rel-L2 <= 2e-3 (bf16 rounding of a differently ordered sum)."""
+    torch.manual_seed(5)
+    layers = []
+    for fuse in (True, False):
+        cfg = MoE.Config(num_experts=experts, num_shared_experts=1, top_k=top_k, hidden_dim=hidden,
+                         score_before_experts=score_before, score_func="softmax", route_norm=True)
+        moe = MoE(cfg, dim=dim).to(device).to(torch.bfloat16)
+        if layers:
+            moe.load_state_dict(layers[0].state_dict())
+        else:
+            moe.init_weights(init_std=0.05, buffer_device=device)
+        holder = nn.Module()
+        holder.moe = moe
+        _convert(holder, ["experts"], fuse=fuse)   # shared experts and the router stay in bf16
+        layers.append(moe)
+    x = torch.randn(2, 96, dim, device=device, dtype=torch.bfloat16)
+    dy = torch.randn(2, 96, dim, device=device, dtype=torch.bfloat16)
+    outs = []
+    for moe in layers:
+        xi = x.clone().requires_grad_(True)
+        y = moe(xi)
+        y.backward(dy)
+        outs.append(dict(y=y.detach(), dx=xi.grad, gate=moe.router.gate.weight.grad, w1=moe.experts.w1.grad,
+                         w2=moe.experts.w2.grad, w3=moe.experts.w3.grad, counts=moe.tokens_per_expert.clone()))
+    a, b = outs
+    assert torch.equal(a["counts"], b["counts"]) and a["counts"].sum() == 2 * 96 * top_k
+    for name in ("w1", "w2", "w3"):
+        assert torch.equal(a[name], b[name]), name
+    for name in ("y", "dx", "gate"):
+        assert rel_l2(a[name].float().cpu().numpy(), b[name].float().cpu().numpy()) <= 2e-3, name
 
 
 class _MiniDecoderBlock(nn.Module):

@@ -15,8 +15,12 @@ import torch
 import torch.nn.functional as F
 from torch import nn
 
-from ..mx_tensor import grouped_feed_forward_fusable, mx_grouped_feed_forward
+from dataclasses import dataclass
+
+from ..mx_tensor import grouped_feed_forward_fusable, mx_grouped_feed_forward, mx_routed_experts
 from ..protocols import Module
+from .feed_forward import FeedForward
+from .linear import Linear
 from ..quantization import MXFP8_GROUP_ALIGNMENT_SIZE
 
 TOKEN_GROUP_ALIGN_SIZE_M = 8
@@ -152,3 +156,181 @@ class GroupedExperts(Module):
         nn.init.trunc_normal_(self.w1, mean=0.0, std=0.02)
         nn.init.trunc_normal_(self.w2, mean=0.0, std=init_std)
         nn.init.trunc_normal_(self.w3, mean=0.0, std=init_std)
+
+
+class TokenChoiceTopKRouter(Module):
+    """Token-choice routing: every token goes to its top_k experts by router score, optionally
+    restricted to the best `num_limited_groups` of `num_expert_groups` expert groups
+    (torchtitan/models/common/moe/moe.py:137-315).  Gate and scores run in float32."""
+
+    def __init__(self, *, dim: int, num_experts: int, num_expert_groups: int | None,
+                 num_limited_groups: int | None, top_k: int, score_func: Literal["softmax", "sigmoid"],
+                 route_norm: bool, route_scale: float, gate_bias: bool,
+                 _debug_force_load_balance: bool = False):
+        super().__init__()
+        self.gate = Linear.Config(bias=gate_bias).build(in_features=dim, out_features=num_experts)
+        self.num_experts = num_experts
+        self.num_expert_groups = num_expert_groups
+        self.num_limited_groups = num_limited_groups
+        self.top_k = top_k
+        self.score_func = score_func
+        self.route_norm = route_norm
+        self.route_scale = route_scale
+        self._debug_force_load_balance = _debug_force_load_balance
+
+    def _limit_to_groups(self, scores: torch.Tensor) -> torch.Tensor:
+        """-inf for the experts of every group outside the `num_limited_groups` best ones, a
+        group's score being the sum of its two best experts."""
+        if self.num_limited_groups is None:
+            raise ValueError("num_limited_groups must be set when num_expert_groups is set")
+        if self.num_experts % self.num_expert_groups != 0:
+            raise ValueError(f"num_experts ({self.num_experts}) must be divisible by "
+                             f"num_expert_groups ({self.num_expert_groups})")
+        per_group = self.num_experts // self.num_expert_groups
+        if per_group < 2:
+            raise ValueError(f"experts_per_group ({per_group}) must be >= 2")
+        grouped = scores.view(-1, self.num_expert_groups, per_group)
+        group_score = grouped.topk(2, dim=-1).values.sum(dim=-1)
+        keep = torch.topk(group_score, k=self.num_limited_groups, dim=-1, sorted=False).indices
+        drop = torch.ones_like(group_score, dtype=torch.bool).scatter_(1, keep, False)
+        return grouped.masked_fill(drop.unsqueeze(-1), float("-inf")).view(-1, self.num_experts)
+
+    def forward(self, x: torch.Tensor, expert_bias: torch.Tensor | None = None):
+        """x [tokens, dim] -> (top_scores [tokens, top_k] float32, expert indices [tokens, top_k],
+        tokens per expert [num_experts])."""
+        with torch.autocast(device_type=x.device.type, dtype=torch.float32):
+            scores = self.gate(x)
+        if self.score_func == "sigmoid":
+            scores = torch.sigmoid(scores)
+        elif self.score_func == "softmax":
+            scores = F.softmax(scores, dim=1)
+        else:
+            raise NotImplementedError(f"Unknown score function {self.score_func}")
+        choice = scores if expert_bias is None else scores + expert_bias  # the bias only steers routing
+        if self.num_expert_groups is not None:
+            choice = self._limit_to_groups(choice)
+        selected = torch.topk(choice, k=self.top_k, dim=-1, sorted=False).indices
+        top_scores = scores.gather(dim=1, index=selected)
+        if self._debug_force_load_balance:  # round-robin assignment, exactly balanced
+            n = scores.size(0)
+            selected = (torch.arange(n * self.top_k, device=scores.device, dtype=torch.int64)
+                        .reshape(n, self.top_k) % self.num_experts)
+            top_scores = scores.gather(dim=1, index=selected)
+        if self.route_norm:
+            top_scores = top_scores / (top_scores.sum(dim=-1, keepdim=True) + 1e-20)
+        top_scores = top_scores * self.route_scale
+        counts = torch.histc(selected.view(-1), bins=self.num_experts, min=0, max=self.num_experts)
+        return top_scores, selected, counts
+
+    def init_weights(self, **kwargs) -> None:
+        init_std = kwargs.get("init_std")
+        assert init_std is not None
+        self.gate.init_weights(init_std=init_std)
+
+
+class TokenReorderer(Module):
+    """Order of the (token, choice) pairs that groups them by expert
+    (torchtitan/models/common/moe/moe.py:320-370)."""
+
+    def __init__(self, *, num_experts: int, top_k: int):
+        super().__init__()
+        self.num_experts = num_experts
+        self.top_k = top_k
+
+    def forward(self, top_scores: torch.Tensor, selected_experts_indices: torch.Tensor):
+        flat = selected_experts_indices.view(-1)
+        counts = torch.histc(flat, bins=self.num_experts, min=0, max=self.num_experts)
+        order = torch.argsort(flat, stable=True)
+        return top_scores.view(-1)[order], order, counts
+
+
+class MoE(Module):
+    """Router + routed experts (+ shared experts) with auxiliary-loss-free load balancing buffers
+    (torchtitan/models/common/moe/moe.py:373-575, single-device part)."""
+
+    @dataclass(kw_only=True, slots=True)
+    class Config(Module.Config):
+        num_experts: int = 8
+        num_shared_experts: int = 1
+        score_func: Literal["softmax", "sigmoid"] = "sigmoid"
+        route_norm: bool = False
+        route_scale: float = 1.0
+        gate_bias: bool = False
+        score_before_experts: bool = True
+        top_k: int = 1
+        num_expert_groups: int | None = None
+        num_limited_groups: int | None = None
+        use_grouped_mm: bool = True
+        load_balance_coeff: float | None = 1e-3
+        _debug_force_load_balance: bool = False
+        hidden_dim: int = 0
+
+    def __init__(self, config: Config, *, dim: int):
+        super().__init__()
+        self.experts = GroupedExperts(dim=dim, hidden_dim=config.hidden_dim, num_experts=config.num_experts,
+                                      use_grouped_mm=config.use_grouped_mm)
+        self.router = TokenChoiceTopKRouter(
+            dim=dim, num_experts=config.num_experts, num_expert_groups=config.num_expert_groups,
+            num_limited_groups=config.num_limited_groups, top_k=config.top_k, score_func=config.score_func,
+            route_norm=config.route_norm, route_scale=config.route_scale, gate_bias=config.gate_bias,
+            _debug_force_load_balance=config._debug_force_load_balance)
+        self.reorderer = TokenReorderer(num_experts=config.num_experts, top_k=config.top_k)
+        self.shared_experts = (
+            FeedForward.Config(hidden_dim=config.hidden_dim * config.num_shared_experts).build(dim=dim)
+            if config.num_shared_experts > 0 else None)
+        self.score_before_experts = config.score_before_experts
+        self.load_balance_coeff = config.load_balance_coeff
+        if self.load_balance_coeff is not None:
+            assert self.load_balance_coeff > 0.0
+            self.register_buffer("expert_bias", torch.zeros(config.num_experts, dtype=torch.float32), persistent=True)
+        else:
+            self.expert_bias = None
+        self.register_buffer("tokens_per_expert", torch.zeros(config.num_experts, dtype=torch.float32),
+                             persistent=False)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        bs, slen, dim = x.shape
+        x = x.view(-1, dim)
+        top_scores, selected, counts = self.router(x, self.expert_bias)
+        with torch.no_grad():
+            self.tokens_per_expert.add_(counts)
+        scores_sorted, order, counts = self.reorderer(top_scores, selected)
+        top_k = self.router.top_k
+        ex = self.experts
+        if (ex.use_grouped_mm and x.dtype == torch.bfloat16
+                and grouped_feed_forward_fusable(x, ex.w1, ex.w2, ex.w3)
+                and ex.w2.mx_config.pad_token_groups_for_grouped_mm):
+            # converted experts: gather, score, experts and combine as one fused function
+            out_experts = mx_routed_experts(x, top_scores, ex.w1, ex.w2, ex.w3, order, counts,
+                                            self.score_before_experts)
+            shared = self.shared_experts(x) if self.shared_experts is not None else None
+        else:
+            routed_in = x[order // top_k]
+            if self.score_before_experts:
+                routed_in = (routed_in.to(torch.float32) * scores_sorted.reshape(-1, 1)).to(x.dtype)
+            routed_out = ex(routed_in, counts)
+            shared = self.shared_experts(x) if self.shared_experts is not None else None
+            unsorted = torch.zeros((bs * slen * top_k, dim), dtype=routed_out.dtype, device=routed_out.device)
+            unsorted[order] = routed_out
+            unsorted = unsorted.reshape(-1, top_k, dim)
+            if not self.score_before_experts:
+                out_experts = torch.bmm(top_scores.reshape(-1, 1, top_k), unsorted.float()).to(x.dtype).squeeze(1)
+            else:
+                out_experts = unsorted.sum(dim=1)
+        if shared is None:
+            return out_experts.reshape(bs, slen, dim)
+        return (shared + out_experts).reshape(bs, slen, dim)
+
+    def init_weights(self, **kwargs) -> None:
+        init_std = kwargs.get("init_std")
+        buffer_device = kwargs.get("buffer_device")
+        assert init_std is not None
+        assert isinstance(buffer_device, torch.device)
+        self.experts.init_weights(init_std=init_std)
+        self.router.init_weights(init_std=init_std)
+        if self.shared_experts is not None:
+            self.shared_experts.init_weights(init_std=init_std)
+        with torch.device(buffer_device):
+            self.tokens_per_expert = torch.zeros(self.experts.num_experts, dtype=torch.float32)
+            if self.load_balance_coeff is not None:
+                self.expert_bias = torch.zeros(self.experts.num_experts, dtype=torch.float32)

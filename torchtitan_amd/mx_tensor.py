@@ -613,6 +613,123 @@ def mx_grouped_feed_forward(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
                                        w2.mx_config)
 
 
+class _MXRoutedExperts(torch.autograd.Function):
+    """The routed half of an MoE layer as one function (torchtitan/models/common/moe/moe.py:519-555):
+
+        out[t] = sum_j  c[t, j] * experts(x[t] * r[t, j])        j over the token's top_k experts
+
+    with r = scores, c = 1 when the scores multiply the expert inputs (`score_before_experts`)
+    and r = 1, c = scores otherwise.  The token gather, the score multiply and the move into
+    aligned expert groups happen inside the cast kernel (no routed copy of x exists); the
+    un-sort and the weighted sum over top_k are one kernel over the padded expert outputs; in
+    backward the same two kernels swap roles and the score gradients are row dot products."""
+
+    @staticmethod
+    def forward(ctx, x, top_scores, w1, w2, w3, tok_sorted, counts, score_before: bool, cfg: MXFP8Config):
+        mode = cfg.scale_mode
+        T, D = x.shape
+        k = top_scores.shape[1]
+        R = T * k
+        G, H, _ = w1.shape
+        xb = _bf16(x).contiguous()
+        scores = top_scores.float().contiguous()
+        fast = D % 128 == 0 and H % 128 == 0 and G <= 638
+        order = MX_SCALES_MFMA if fast else MX_SCALES_ROWMAJOR
+        offs = torch.cumsum(counts, dim=0, dtype=torch.int32)
+        perm, offs_p, back = _pad_plan(offs, R, 128 if fast else ops.BLOCK)
+        slot = tok_sorted[perm.clamp_min(0)]              # (token, j) pair of every padded row
+        src_row = torch.where(perm >= 0, slot // k, -1)   # its token, -1 for padding
+        row_score = scores.view(-1)[slot]
+        pos = torch.empty(R, dtype=torch.int64, device=x.device)
+        pos[tok_sorted] = back                            # padded row of pair (t, j)
+        pos = pos.view(T, k)
+        need_dx = ctx.needs_input_grad[0]
+        need_ds = ctx.needs_input_grad[1]
+        need_dw = any(ctx.needs_input_grad[2:5])
+        xq0, xq1 = ops.to_mx_rows_gathered(xb, src_row, mode, order, need_dw,
+                                           row_score if score_before else None)
+        need_dg = need_dx or need_ds or need_dw
+        both = lambda w: ops.to_mx_dim0_dim1_batched(_bf16(w).contiguous(), mode, MX_SCALES_MFMA)
+        rows = lambda w: (_cast_w_rows(_bf16(w).contiguous(), mode), None)
+        w1q0, w1q1 = both(w1) if (need_dx or need_ds) else rows(w1)
+        w3q0, w3q1 = both(w3) if (need_dx or need_ds) else rows(w3)
+        w2q0, w2q1 = both(w2) if need_dg else rows(w2)
+        h1 = ops.mx_grouped_gemm_2d3d(xq0, w1q0, offs_p)
+        h3 = ops.mx_grouped_gemm_2d3d(xq0, w3q0, offs_p)
+        gq0, gq1, _ = ops.swiglu_to_mx_dim0_dim1(h1, h3, mode, order)
+        yp = ops.mx_grouped_gemm_2d3d(gq0, w2q0, offs_p)
+        out = ops.moe_combine(yp, pos, None if score_before else scores)
+        ctx.cfg, ctx.order, ctx.score_before = cfg, order, score_before
+        ctx.dtypes = (x.dtype, top_scores.dtype, w1.dtype, w2.dtype, w3.dtype)
+        ctx.flags = (need_dx, need_ds, need_dw)
+        saved = [offs_p, src_row, row_score, pos, scores]
+        if need_dg:
+            saved += [h1, h3, w2q1.codes, w2q1.scales]
+        if need_dw:
+            saved += [xq1.codes, xq1.scales, gq1.codes, gq1.scales]
+        if need_dx or need_ds:
+            saved += [w1q1.codes, w1q1.scales, w3q1.codes, w3q1.scales]
+        if need_ds:
+            saved += [xb if score_before else yp]
+        ctx.save_for_backward(*saved)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        mode, order, score_before = ctx.cfg.scale_mode, ctx.order, ctx.score_before
+        need_dx, need_ds, need_dw = ctx.flags
+        saved = list(ctx.saved_tensors)
+        offs_p, src_row, row_score, pos, scores = (saved.pop(0) for _ in range(5))
+        T, k = pos.shape
+        dob = _bf16(dout).contiguous()
+        h1, h3 = saved.pop(0), saved.pop(0)
+        w2q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
+        # gradient of the padded expert outputs: dout of the row's token (times its score)
+        dyq0, dyq1 = ops.to_mx_rows_gathered(dob, src_row, mode, order, ctx.needs_input_grad[3],
+                                             None if score_before else row_score)
+        dg = ops.mx_grouped_gemm_2d3d(dyq0, w2q1, offs_p)
+        (da0, da1), (db0, db1), _ = ops.swiglu_bwd_to_mx_dim0_dim1(dg, h1, h3, mode, order)
+        dx = ds = dw1 = dw2 = dw3 = None
+        cast_back = lambda g, dt: g if g.dtype == dt else g.to(dt)
+        if need_dw:
+            xq1 = MXData(saved.pop(0), saved.pop(0), order)
+            gq1 = MXData(saved.pop(0), saved.pop(0), order)
+            if ctx.needs_input_grad[2]:
+                dw1 = cast_back(ops.mx_grouped_gemm_2d2d(da1, xq1, offs_p), ctx.dtypes[2])
+            if ctx.needs_input_grad[3]:
+                dw2 = cast_back(ops.mx_grouped_gemm_2d2d(dyq1, gq1, offs_p), ctx.dtypes[3])
+            if ctx.needs_input_grad[4]:
+                dw3 = cast_back(ops.mx_grouped_gemm_2d2d(db1, xq1, offs_p), ctx.dtypes[4])
+        if need_dx or need_ds:
+            w1q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
+            w3q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
+            need_dxp = need_dx or (need_ds and score_before)
+            if need_dxp:  # gradient of the (scaled) routed inputs, padded layout
+                dxp = ops.mx_grouped_gemm_2d3d(da0, w1q1, offs_p) + ops.mx_grouped_gemm_2d3d(db0, w3q1, offs_p)
+            if need_dx:
+                dx = cast_back(ops.moe_combine(dxp, pos, scores if score_before else None), ctx.dtypes[0])
+            if need_ds:
+                other = saved.pop(0)  # x (scores in front of the experts) or the expert outputs
+                token = torch.arange(T * k, device=pos.device, dtype=torch.int64).div_(k, rounding_mode="floor")
+                if score_before:
+                    ds = ops.moe_row_dot(dxp, pos.view(-1), other, token)
+                else:
+                    ds = ops.moe_row_dot(other, pos.view(-1), dob, token)
+                ds = cast_back(ds.view(T, k), ctx.dtypes[1])
+        return dx, ds, dw1, dw2, dw3, None, None, None, None
+
+
+def mx_routed_experts(x: torch.Tensor, top_scores: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
+                      w3: torch.Tensor, token_indices_experts_sorted: torch.Tensor,
+                      num_tokens_per_expert: torch.Tensor, score_before_experts: bool) -> torch.Tensor:
+    """Gather, score, run the SwiGLU experts and combine, for converted expert parameters.
+    x [T, dim] bf16, top_scores [T, top_k]; the index tensor is the stable argsort of the
+    flattened expert choices.  Callers check `grouped_feed_forward_fusable` first."""
+    return _MXRoutedExperts.apply(x, top_scores, _unwrap(w1), _unwrap(w2), _unwrap(w3),
+                                  token_indices_experts_sorted, num_tokens_per_expert,
+                                  bool(score_before_experts), w2.mx_config)
+
+
 def _cast_w_rows(w: torch.Tensor, mode: str) -> MXData:
     """Row-wise cast of stacked matrices w [G, N, K] with one MFMA-order scale block each."""
     return ops.to_mx_dim0_batched(w, mode, MX_SCALES_MFMA)
