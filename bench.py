@@ -239,6 +239,57 @@ def time_moe_grouped(dev, recipe_mode):
         out[name] = {"us": round(sec * 1e6, 1), "TFLOP/s": round(flops / sec / 1e12, 1)}
     del x, w, dy, xq0, xq1, dyq0, dyq1, wq0, wq1, y, dx, dw
     out["expert_block"] = time_expert_block(dev, recipe_mode, counts)
+    out["moe_layer"] = time_moe_layer(dev, recipe_mode)
+    return out
+
+
+def time_moe_layer(dev, recipe_mode):
+    """The whole MoE layer of the same config (router, top-8 of 128 experts, softmax scores
+    normalised over the chosen experts and applied in front of the experts, no shared expert),
+    forward + backward on 16384 tokens: routed half as one fused function (gather + score inside
+    the cast, fused experts, weighted combine) and as torch gather / scatter / sum around three
+    converted grouped GEMMs with separate gate ops."""
+    import torch
+    import torch.nn as nn
+
+    from torchtitan_amd.modules import MoE
+    from torchtitan_amd.protocols import ModelConvertersContainer
+    from torchtitan_amd.quantization.mx import MXFP8Converter
+
+    recipe = {"rceil": "mxfp8_rceil", "floor": "mxfp8_floor"}[recipe_mode]
+    x = torch.randn((2, 8192, 2048), device=dev, dtype=torch.bfloat16).requires_grad_(True)
+    dy = torch.randn((2, 8192, 2048), device=dev, dtype=torch.bfloat16) * 1e-3
+    out = {}
+    for name, fuse in (("fused", True), ("torch_ops_around_grouped_gemms", False)):
+        torch.manual_seed(0)
+        moe = MoE(MoE.Config(num_experts=128, num_shared_experts=0, top_k=8, hidden_dim=768,
+                             score_before_experts=True, score_func="softmax", route_norm=True), dim=2048)
+        holder = nn.Module()
+        holder.moe = moe
+        ModelConvertersContainer.Config(
+            converters=[MXFP8Converter.Config(fqns=["experts"], recipe_name=recipe, fuse_swiglu_cast=fuse)]
+        ).build(parallel_dims=None, model_compile_enabled=False).convert(holder)
+        holder.to(dev).to(torch.bfloat16)
+        moe.init_weights(init_std=0.02, buffer_device=dev)
+
+        def step():
+            x.grad = None
+            for p in moe.parameters():
+                p.grad = None
+            moe(x).backward(dy)
+
+        for _ in range(2):
+            step()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(5):
+            step()
+        e.record()
+        torch.cuda.synchronize()
+        ms = s.elapsed_time(e) / 5
+        out[name] = {"ms": round(ms, 3), "TFLOP/s": round(18.0 * 16384 * 8 * 2048 * 768 / ms / 1e9, 1)}
+        del moe, holder
     return out
 
 
