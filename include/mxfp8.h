@@ -149,6 +149,19 @@ int mx_swiglu_bwd_cast_dim0_dim1(const void* dg, const void* a, const void* b, i
                                  uint8_t* scales_t, void* dab, int scale_mode, int scale_order,
                                  void* stream);
 
+/* Log-probabilities of chosen tokens: logprob[r] = x[r, target[r]] - lse[r],
+ * lse[r] = log sum_v exp(x[r, v]) in float32 over bf16 logits x [rows, vocab] (row stride ld,
+ * ld % 8 == 0, 16-byte aligned); target int64 [rows] (outside [0, vocab): NaN).  One read of
+ * the logits.  Stands in for `.to(float32)`, `F.log_softmax` and `gather` on the policy's
+ * logits (torchtitan/experiments/rl/unified/actors/utils.py:37-50). */
+int mx_token_logprob_fwd(const void* logits, int64_t rows, int64_t vocab, int64_t ld,
+                         const int64_t* target, float* logprob, float* lse, void* stream);
+/* Its backward: dlogits[r, v] = grad_logprob[r] * ((v == target[r]) - exp(x[r, v] - lse[r]))
+ * rounded to bf16 (dlogits bf16 [rows, vocab], row stride ldd); rows <= 65535 per call. */
+int mx_token_logprob_bwd(const void* logits, int64_t rows, int64_t vocab, int64_t ld,
+                         const int64_t* target, const float* lse, const float* grad_logprob,
+                         void* dlogits, int64_t ldd, void* stream);
+
 /* Re-order a row-major [rows, nblk] scale matrix into MX_SCALES_MFMA order
  * (the "blocked layout" step the reference leaves to torch._scaled_mm, docs/mxfp8.md:36). */
 int mx_scale_layout(const uint8_t* scales, int64_t rows, int64_t nblk, uint8_t* out, void* stream);

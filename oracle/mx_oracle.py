@@ -45,6 +45,9 @@ Pinning status (what fixes each function independently of its own formula):
   moe_combine                pinned  -- vs an exact float64 sum (within one bf16 step) and torch's
                                         scatter + bmm on the CPU; accumulation order PARITY UNPINNED
   moe_row_dot                pinned  -- float64 dot products (textbook)
+  token_log_probs(_grad)     pinned  -- torch CPU float32 log_softmax + gather and its autograd
+  policy_gradient_loss       pinned  -- closed forms (policy == reference; hand example) and the
+                                        formulas run with torch ops on the CPU
   generate_permute_indices   pinned  -- the worked example and invariants of
                                         torchtitan/models/common/moe/kernels.py:145-218
                                         and tests/unit_tests/test_permute_indices_kernel.py
@@ -450,6 +453,44 @@ def moe_row_dot(a_bits: np.ndarray, ia: np.ndarray, b_bits: np.ndarray, ib: np.n
     ok = (ia >= 0) & (ia < a.shape[0]) & (ib >= 0) & (ib < b.shape[0])
     d = np.einsum("ij,ij->i", a[np.clip(ia, 0, a.shape[0] - 1)], b[np.clip(ib, 0, b.shape[0] - 1)])
     return np.where(ok, d, 0.0)
+
+
+def token_log_probs(logits_bits: np.ndarray, target: np.ndarray):
+    """(log-probability of target[r] under softmax(logits[r]), log-sum-exp per row) in float64
+    from bf16 logits: what `.to(float32)`, `F.log_softmax` and `gather` compute in
+    torchtitan/experiments/rl/unified/actors/utils.py:37-50."""
+    x = bf16_bits_to_f32(logits_bits).astype(np.float64)
+    m = x.max(axis=1, keepdims=True)
+    lse = (m + np.log(np.exp(x - m).sum(axis=1, keepdims=True)))[:, 0]
+    return x[np.arange(x.shape[0]), target] - lse, lse
+
+
+def token_log_probs_grad(logits_bits: np.ndarray, target: np.ndarray, grad: np.ndarray) -> np.ndarray:
+    """d/dlogits of sum_r grad[r] * logprob[r]: grad[r] * (onehot(target[r]) - softmax(x[r])), float64."""
+    x = bf16_bits_to_f32(logits_bits).astype(np.float64)
+    _, lse = token_log_probs(logits_bits, target)
+    d = -np.exp(x - lse[:, None])
+    d[np.arange(x.shape[0]), target] += 1.0
+    return d * grad[:, None]
+
+
+def policy_gradient_loss(policy_lps, ref_lps, advantages, kl_coef=0.1, ppo_clip_eps=0.2, entropy_coef=0.01):
+    """GRPO / PPO loss of actors/utils.py:97-134 in float64 from per-sample token log-probs.
+    Returns (total, dict of pg_loss, entropy, kl_div, ratio_mean, ratio_clipped_frac)."""
+    mlr, mkl = [], []
+    for p, r in zip(policy_lps, ref_lps):
+        d = np.asarray(p, np.float64) - np.asarray(r, np.float64)
+        mlr.append(d.mean())
+        mkl.append((np.exp(d) - 1.0 - d).mean())
+    ratio = np.exp(np.array(mlr))
+    adv = np.asarray(advantages, np.float64)
+    clipped = np.clip(ratio, 1 - ppo_clip_eps, 1 + ppo_clip_eps)
+    pg = -np.minimum(ratio * adv, clipped * adv).mean()
+    entropy = -np.concatenate([np.asarray(p, np.float64) for p in policy_lps]).mean()
+    kl = float(np.mean(mkl))
+    total = pg - entropy_coef * entropy + kl_coef * kl
+    return total, {"pg_loss": pg, "entropy": entropy, "kl_div": kl, "ratio_mean": ratio.mean(),
+                   "ratio_clipped_frac": float((np.abs(ratio - clipped) > 1e-6).mean())}
 
 
 def make_cfg1_inputs(seed: int, M: int = 8192, K: int = 4096, N: int = 4096):

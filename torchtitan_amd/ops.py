@@ -217,6 +217,51 @@ def moe_row_dot(a: torch.Tensor, ia: torch.Tensor, b: torch.Tensor, ib: torch.Te
     return out
 
 
+def token_logprob_fwd(logits: torch.Tensor, target: torch.Tensor):
+    """(log-probability of target[r] under softmax(logits[r]), log-sum-exp of row r), float32
+    [rows], from bf16 logits [rows, vocab] read once."""
+    logits = _check_hp(logits)
+    if target.dtype != torch.int64 or target.shape != (logits.shape[0],) or target.device != logits.device:
+        raise TypeError("target must be int64 [rows] on the logits' device")
+    if logits.stride(0) % 8 or logits.data_ptr() % 16:
+        logits = logits.contiguous().clone() if logits.shape[1] % 8 == 0 else _pad_row_stride(logits)
+    target = target.contiguous()
+    rows, vocab = logits.shape
+    lp = torch.empty(rows, dtype=torch.float32, device=logits.device)
+    lse = torch.empty(rows, dtype=torch.float32, device=logits.device)
+    _call("mx_token_logprob_fwd", "token_logprob_fwd", logits.device, _ptr(logits), rows, vocab,
+          logits.stride(0), _ptr(target), _ptr(lp), _ptr(lse), _stream(logits))
+    return lp, lse
+
+
+def _pad_row_stride(x: torch.Tensor) -> torch.Tensor:
+    """Copy of x [rows, cols] whose row stride is a multiple of 8 elements (16-byte aligned rows)."""
+    rows, cols = x.shape
+    buf = torch.empty((rows, -(-cols // 8) * 8), dtype=x.dtype, device=x.device)
+    view = buf[:, :cols]
+    view.copy_(x)
+    return view
+
+
+def token_logprob_bwd(logits: torch.Tensor, target: torch.Tensor, lse: torch.Tensor,
+                      grad_logprob: torch.Tensor) -> torch.Tensor:
+    """Gradient of `token_logprob_fwd`'s first output with respect to the logits, bf16."""
+    logits = _check_hp(logits)
+    if logits.stride(0) % 8 or logits.data_ptr() % 16:
+        logits = logits.contiguous().clone() if logits.shape[1] % 8 == 0 else _pad_row_stride(logits)
+    rows, vocab = logits.shape
+    g = grad_logprob.to(torch.float32).contiguous()
+    lse, target = lse.contiguous(), target.contiguous()
+    out = torch.empty((rows, -(-vocab // 8) * 8), dtype=torch.bfloat16, device=logits.device)[:, :vocab]
+    step = 65535
+    for lo in range(0, rows, step):
+        n = min(step, rows - lo)
+        _call("mx_token_logprob_bwd", "token_logprob_bwd", logits.device, _ptr(logits[lo:]), n, vocab,
+              logits.stride(0), _ptr(target[lo:]), _ptr(lse[lo:]), _ptr(g[lo:]), _ptr(out[lo:]),
+              out.stride(0), _stream(logits))
+    return out
+
+
 def swiglu_to_mx_dim0_dim1(a: torch.Tensor, b: torch.Tensor, mode="floor",
                            order: int = MX_SCALES_ROWMAJOR, want_g: bool = False):
     """Both casts of g = silu(a) * b (bf16, every step rounded to bf16) without g passing through
