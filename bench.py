@@ -193,6 +193,48 @@ def time_ffn_block(dev, recipe):
     return out
 
 
+def time_policy_loss(dev):
+    """Beyond the headline: the log-probabilities of one 2048-token completion over the RL
+    config's vocabulary (151 936) from bf16 logits, forward + backward: fused kernels against
+    the float32 log_softmax + gather of the reference's loss.  Same inputs; results agree to
+    1e-5 (tests)."""
+    import torch
+    import torch.nn.functional as F
+
+    from torchtitan_amd.rl import token_log_probs
+
+    rows, vocab = 2048, 151936
+    logits = (torch.randn((rows, vocab), device=dev) * 3).to(torch.bfloat16).requires_grad_(True)
+    target = torch.randint(0, vocab, (rows,), device=dev)
+    w = torch.randn(rows, device=dev)
+    out = {}
+
+    def torch_ops():
+        lp = F.log_softmax(logits.to(torch.float32), dim=-1).gather(1, target[:, None]).squeeze(-1)
+        (lp * w).sum().backward()
+
+    def fused():
+        (token_log_probs(logits, target) * w).sum().backward()
+
+    for name, fn in (("fused", fused), ("torch_ops", torch_ops)):
+        for _ in range(2):
+            logits.grad = None
+            fn()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(5):
+            logits.grad = None
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        sec = s.elapsed_time(e) * 1e-3 / 5
+        # algorithmic bytes: logits read once forward; read once and gradient written backward
+        out[name] = {"us": round(sec * 1e6, 1), "GB/s": round(rows * vocab * 6 / sec / 1e9, 1)}
+    out["fused"]["frac_hbm"] = round(out["fused"]["GB/s"] / PEAK_HBM_GBPS, 3)
+    return out
+
+
 def time_moe_grouped(dev, recipe_mode):
     """BASELINE configs[3] GEMMs (not the headline): 128 experts, hidden 2048, expert FFN 768,
     top-8 routing of 16384 tokens from softmax over seeded Gumbel-perturbed logits (uneven
@@ -485,6 +527,8 @@ def main():
         del ffn, x, h, dy_h, dy_o
         torch.cuda.empty_cache()
         line["swiglu_block"] = time_ffn_block(dev, args.recipe)
+        torch.cuda.empty_cache()
+        line["policy_loss_logprobs"] = time_policy_loss(dev)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(0 if recipe_mode == "floor" else 1, target_s=12.0)
     print(json.dumps(line))
