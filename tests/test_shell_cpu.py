@@ -269,3 +269,17 @@ def test_alignment_switch():
         assert moe_mod.get_mxfp8_pad_multiple() == 32
     finally:
         moe_mod.set_token_group_alignment_size_m(8)
+
+
+def test_module_filter_fn_rules():
+    """Linear only, both dims % 16, no filtered substring in the FQN (quantization/utils.py:10-27)."""
+    import torch.nn as nn
+
+    from torchtitan_amd.quantization.utils import module_filter_fn
+
+    assert module_filter_fn(nn.Linear(32, 48), "layers.0.attention.wq", [])
+    assert not module_filter_fn(nn.Linear(32, 48), "layers.0.attention.wq", ["attention.wq"])
+    assert not module_filter_fn(nn.Linear(30, 48), "w", [])
+    assert not module_filter_fn(nn.Linear(32, 40), "w", [])
+    assert not module_filter_fn(nn.Embedding(32, 48), "tok_embeddings", [])
+    assert module_filter_fn(nn.Linear(16, 16), "output", ["router"])
