@@ -149,6 +149,15 @@ int mx_swiglu_bwd_cast_dim0_dim1(const void* dg, const void* a, const void* b, i
                                  uint8_t* scales_t, void* dab, int scale_mode, int scale_order,
                                  void* stream);
 
+/* MXFP8 -> bf16: out[r, c] = e4m3(codes[r, c]) * 2^(scale of row r, block c / 32 - 127) rounded
+ * to bf16 (exact above bf16's subnormal range); a scale byte 255 gives NaN.  codes uint8
+ * [rows, cols] dense (16-byte aligned, cols % 32 == 0), scales in either order, out bf16
+ * [rows, cols] with row stride ldo (% 8).  The receiving side of a weight hand-over in MXFP8
+ * form (in place of the bf16 state dict of
+ * torchtitan/experiments/rl/unified/actors/trainer.py:226-239 -> generator.py:307-335). */
+int mx_dequant(const uint8_t* codes, const uint8_t* scales, int64_t rows, int64_t cols,
+               int scale_order, void* out, int64_t ldo, void* stream);
+
 /* Log-probabilities of chosen tokens: logprob[r] = x[r, target[r]] - lse[r],
  * lse[r] = log sum_v exp(x[r, v]) in float32 over bf16 logits x [rows, vocab] (row stride ld,
  * ld % 8 == 0, 16-byte aligned); target int64 [rows] (outside [0, vocab): NaN).  One read of

@@ -338,3 +338,22 @@ def test_moe_combine_and_row_dot(device, tokens, k, cols):
     d = ops.moe_row_dot(y, tp.view(-1), bf16_from_bits(x_bits, device), torch.from_numpy(ib).to(device))
     ref = mo.moe_row_dot(y_bits, pos.reshape(-1), x_bits, ib)
     assert np.allclose(d.cpu().numpy().astype(np.float64), ref, rtol=1e-5, atol=1e-5 * np.sqrt(cols))
+
+
+@pytest.mark.parametrize("mode_name,mode", MODES)
+def test_dequant_is_exact(device, mode_name, mode):
+    """codes x 2^(scale - 127) back to bf16: equal to the oracle's dequantization bit for bit, in
+    both scale orders, including all-zero blocks, a NaN block and the smallest scales."""
+    rng = np.random.default_rng(8)
+    bits = randn_bits(rng, (192, 160), outliers=1e-2)
+    bits[3, 32:64] = 0
+    bits[5, 70] = 0x7FC0
+    bits[7, :32] = mo.f32_to_bf16_bits((rng.standard_normal(32) * 1e-38).astype(np.float32))
+    x = bf16_from_bits(bits, device)
+    for order in (ops.MX_SCALES_ROWMAJOR, ops.MX_SCALES_MFMA):
+        q = ops.to_mx_dim0(x, mode_name, order)
+        got = bits_of(ops.mx_dequant(q))
+        codes, scales = mo.cast_dim0(bits, mode)
+        want = mo.f32_to_bf16_bits(mo.dequant(codes, scales))
+        nan = lambda v: (v & 0x7FFF) > 0x7F80
+        assert (nan(got) == nan(want)).all() and np.array_equal(got[~nan(want)], want[~nan(want)])

@@ -20,10 +20,10 @@ def _f32(bits):
     return mo.bf16_bits_to_f32(bits)
 
 
-def _convert(model, fqns, recipe="mxfp8_rceil", pad=True, fuse=True):
+def _convert(model, fqns, recipe="mxfp8_rceil", pad=True, fuse=True, cache=False):
     box = ModelConvertersContainer.Config(
         converters=[MXFP8Converter.Config(fqns=fqns, recipe_name=recipe, pad_token_groups_for_grouped_mm=pad,
-                                          fuse_swiglu_cast=fuse)]
+                                          fuse_swiglu_cast=fuse, cache_weight_casts=cache)]
     ).build(parallel_dims=None, model_compile_enabled=False)
     box.convert(model)
     return box
@@ -335,6 +335,74 @@ def test_moe_layer_fused_routing_matches_torch_ops(device, score_before, dim, hi
         assert torch.equal(a[name], b[name]), name
     for name in ("y", "dx", "gate"):
         assert rel_l2(a[name].float().cpu().numpy(), b[name].float().cpu().numpy()) <= 2e-3, name
+
+
+def test_weight_cast_cache_and_mxfp8_hand_over(device):
+    """cache_weight_casts: same results as without; the casts are reused until the weight is
+    updated in place; the post-optimizer hook refreshes them; the exported MXFP8 state dict
+    dequantizes to exactly what the GEMMs multiply by and takes 33/64 of the bf16 bytes."""
+    from torchtitan_amd import mx_tensor, ops
+    from torchtitan_amd.quantization.mx import export_mxfp8_state_dict, load_mxfp8_state_dict
+
+    torch.manual_seed(9)
+    mx_tensor._weight_cache.clear()
+    blocks, boxes = [], []
+    for cache in (True, False):
+        ff = FeedForward.Config(hidden_dim=256).build(dim=128).to(device).to(torch.bfloat16)
+        if blocks:
+            ff.load_state_dict(blocks[0].state_dict())
+        else:
+            ff.init_weights(init_std=0.05)
+        holder = nn.Module()
+        holder.feed_forward = ff
+        boxes.append(_convert(holder, ["feed_forward"], cache=cache))
+        blocks.append(ff)
+    cached, plain = blocks
+    x = torch.randn(64, 128, device=device, dtype=torch.bfloat16).requires_grad_(True)
+    calls = []
+    real = ops.to_mx_dim0_dim1
+    ops.to_mx_dim0_dim1 = lambda t, *a, **k: (calls.append(tuple(t.shape)), real(t, *a, **k))[1]
+    try:
+        for step in range(2):
+            for micro in range(2):          # two micro-batches per optimizer step
+                ya, yb = cached(x), plain(x)
+                assert torch.equal(ya, yb)
+                ya.sum().backward()
+                yb.sum().backward()
+            for a, b in zip(cached.parameters(), plain.parameters()):
+                assert torch.equal(a.grad, b.grad)
+            w_casts = [c for c in calls if c in ((256, 128), (128, 256))]
+            # plain: 3 weights x 2 micro-batches; cached: 3 weights once in the first step, none
+            # after the hook has cast them
+            assert len(w_casts) == (9 if step == 0 else 6), (step, w_casts)
+            calls.clear()
+            with torch.no_grad():
+                for m in (cached, plain):
+                    for p in m.parameters():
+                        p.add_(p.grad, alpha=-0.1)   # the optimizer's in-place update
+                        p.grad = None
+            holder = nn.Module()
+            holder.feed_forward = cached
+            boxes[0].post_optimizer_hook(holder)
+            assert len([c for c in calls if c in ((256, 128), (128, 256))]) == 3  # cast once, in the hook
+            calls.clear()
+        ya, yb = cached(x), plain(x)
+        assert torch.equal(ya, yb)
+        assert len([c for c in calls if c in ((256, 128), (128, 256))]) == 3  # only the uncached block casts
+    finally:
+        ops.to_mx_dim0_dim1 = real
+    payload = export_mxfp8_state_dict(cached)
+    sd = cached.state_dict()
+    assert set(payload) == set(sd)
+    entry = payload["w1.weight"]
+    assert entry["codes"].shape == (256, 128) and entry["scales"].shape == (256, 4)
+    sent = sum(v["codes"].numel() + v["scales"].numel() for v in payload.values())
+    assert sent * 64 == sum(t.numel() * 2 for t in sd.values()) * 33
+    back = load_mxfp8_state_dict(payload)
+    q = ops.to_mx_dim0(sd["w1.weight"].as_subclass(torch.Tensor), "rceil", ops.MX_SCALES_ROWMAJOR)
+    assert torch.equal(back["w1.weight"], ops.mx_dequant(q))
+    assert rel_l2(back["w2.weight"].float().cpu().numpy(), sd["w2.weight"].float().cpu().numpy()) < 0.04
+    mx_tensor._weight_cache.clear()
 
 
 class _MiniDecoderBlock(nn.Module):

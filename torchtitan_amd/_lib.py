@@ -30,6 +30,7 @@ SIGNATURES = {
     "mx_cast_dim1_batched": (c_int, [_P, _I, _I, _I, _I, _P, _P, c_int, c_int, _P]),
     "mx_cast_dim0_dim1_batched": (c_int, [_P, _I, _I, _I, _I, _P, _P, _P, _P, c_int, c_int, _P]),
     "mx_cast_rows_gathered": (c_int, [_P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P, c_int, c_int, _P]),
+    "mx_dequant": (c_int, [_P, _P, _I, _I, c_int, _P, _I, _P]),
     "mx_token_logprob_fwd": (c_int, [_P, _I, _I, _I, _P, _P, _P, _P]),
     "mx_token_logprob_bwd": (c_int, [_P, _I, _I, _I, _P, _P, _P, _P, _I, _P]),
     "mx_moe_combine": (c_int, [_P, _I, _I, _P, _P, _I, _I, _I, _P, _I, _P]),

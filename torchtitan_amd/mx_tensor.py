@@ -28,15 +28,16 @@ from .ops import MX_SCALES_MFMA, MX_SCALES_ROWMAJOR, MXData
 class MXFP8Config:
     """Per-weight recipe: scale mode and whether grouped GEMMs pad token groups to 32."""
 
-    __slots__ = ("scale_mode", "pad_token_groups_for_grouped_mm", "fuse_swiglu_cast")
+    __slots__ = ("scale_mode", "pad_token_groups_for_grouped_mm", "fuse_swiglu_cast", "cache_weight_casts")
 
     def __init__(self, scale_mode: str = "rceil", pad_token_groups_for_grouped_mm: bool = True,
-                 fuse_swiglu_cast: bool = True):
+                 fuse_swiglu_cast: bool = True, cache_weight_casts: bool = False):
         if scale_mode not in ops.SCALE_MODES:
             raise ValueError(f"unknown scale mode {scale_mode!r}")
         self.scale_mode = scale_mode
         self.pad_token_groups_for_grouped_mm = pad_token_groups_for_grouped_mm
         self.fuse_swiglu_cast = fuse_swiglu_cast
+        self.cache_weight_casts = cache_weight_casts
 
     def __repr__(self):
         return (f"MXFP8Config(scale_mode={self.scale_mode!r}, "
@@ -87,6 +88,71 @@ def _cast_activation(x2: torch.Tensor, src: torch.Tensor, mode: str, need_cols: 
     return rows, cols
 
 
+# ----------------------------------------------------------------------------- weight casts
+class _WeightCastCache:
+    """MXFP8 forms of weights that have not changed since they were cast.
+
+    A weight changes once per optimizer step but is cast in every forward; with gradient
+    accumulation, several forwards per step, or a hand-over of the weights in MXFP8 form, the
+    casts after the first are repeats.  An entry is keyed on the weight's memory (address, shape,
+    strides) and valid while that storage is alive and its version counter is unchanged: every
+    in-place update (optimizer step, ``copy_``, init) invalidates it.  Off unless the converter
+    is built with ``cache_weight_casts=True``; holds 2 bytes per weight element."""
+
+    def __init__(self):
+        self._entries = {}
+
+    @staticmethod
+    def _key(w: torch.Tensor, mode: str):
+        return (w.data_ptr(), tuple(w.shape), tuple(w.stride()), w.dtype, mode)
+
+    def get(self, w: torch.Tensor, mode: str):
+        e = self._entries.get(self._key(w, mode))
+        if e is None:
+            return None
+        ref, version, rows, cols = e
+        if ref.expired() or version != w._version:
+            return None
+        return rows, cols
+
+    def put(self, w: torch.Tensor, mode: str, rows: MXData, cols):
+        from torch.multiprocessing.reductions import StorageWeakRef
+
+        dead = [k for k, e in self._entries.items() if e[0].expired()]
+        for k in dead:
+            del self._entries[k]
+        self._entries[self._key(w, mode)] = (StorageWeakRef(w.untyped_storage()), w._version, rows, cols)
+
+    def clear(self):
+        self._entries.clear()
+
+    def __len__(self):
+        return len(self._entries)
+
+
+_weight_cache = _WeightCastCache()
+
+
+def _cast_weight(w: torch.Tensor, mode: str, need_cols: bool, cfg: MXFP8Config):
+    """(row-wise, column-wise or None) MXFP8 forms of a weight [N, K] or stacked [G, N, K], MFMA
+    scale order.  The column-wise form exists when asked for and N is a multiple of 32."""
+    cached = cfg.cache_weight_casts
+    if cached:
+        hit = _weight_cache.get(w, mode)
+        if hit is not None and (hit[1] is not None or not need_cols or w.shape[-2] % ops.BLOCK):
+            return hit
+        need_cols = True  # cast once in full, whoever asks first
+    wb = (w if w.dtype == torch.bfloat16 else w.to(torch.bfloat16)).contiguous()
+    both = need_cols and wb.shape[-2] % ops.BLOCK == 0
+    if wb.dim() == 3:
+        q = ops.to_mx_dim0_dim1_batched(wb, mode, MX_SCALES_MFMA) if both else (_cast_w_rows(wb, mode), None)
+    else:
+        q = ops.to_mx_dim0_dim1(wb, mode, MX_SCALES_MFMA) if both else (ops.to_mx_dim0(wb, mode, MX_SCALES_MFMA), None)
+    if cached:
+        _weight_cache.put(w, mode, q[0], q[1])
+    return q
+
+
 # ----------------------------------------------------------------------------- dense linear
 class _MXLinear(torch.autograd.Function):
     @staticmethod
@@ -101,10 +167,7 @@ class _MXLinear(torch.autograd.Function):
         needs_bwd = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
         M = x2.shape[0]
         xq0, xq1 = _cast_activation(x2, x, mode, need_cols=ctx.needs_input_grad[1])
-        if needs_bwd and ctx.needs_input_grad[0] and N % ops.BLOCK == 0:
-            wq0, wq1 = ops.to_mx_dim0_dim1(w, mode, MX_SCALES_MFMA)
-        else:
-            wq0, wq1 = ops.to_mx_dim0(w, mode, MX_SCALES_MFMA), None
+        wq0, wq1 = _cast_weight(weight, mode, needs_bwd and ctx.needs_input_grad[0], cfg)
         y = ops.mx_gemm_nt(xq0, wq0)
         ctx.cfg = cfg
         ctx.x_shape = x.shape
@@ -211,10 +274,7 @@ class _MXSwiGLULinear(torch.autograd.Function):
         w = weight if weight.dtype == torch.bfloat16 else weight.to(torch.bfloat16)
         gq0, gq1, _ = ops.swiglu_to_mx_dim0_dim1(a, b, mode, MX_SCALES_MFMA)
         need_dh = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
-        if need_dh and N % ops.BLOCK == 0:
-            wq0, wq1 = ops.to_mx_dim0_dim1(w, mode, MX_SCALES_MFMA)
-        else:
-            wq0, wq1 = ops.to_mx_dim0(w, mode, MX_SCALES_MFMA), None
+        wq0, wq1 = _cast_weight(weight, mode, need_dh, cfg)
         y = ops.mx_gemm_nt(gq0, wq0)
         ctx.cfg, ctx.w_dtype, ctx.have_wq1 = cfg, weight.dtype, wq1 is not None
         saved = [h1, h3]
@@ -307,11 +367,9 @@ class _MXFeedForward(torch.autograd.Function):
         need_dx = ctx.needs_input_grad[0]
         need_dw = any(ctx.needs_input_grad[1:4])
         xq0, xq1 = _cast_activation(x2, x, mode, need_cols=need_dw)
-        both = lambda w: ops.to_mx_dim0_dim1(_bf16(w), mode, MX_SCALES_MFMA)
-        rows = lambda w: (ops.to_mx_dim0(_bf16(w), mode, MX_SCALES_MFMA), None)
-        w1q0, w1q1 = both(w1) if need_dx else rows(w1)
-        w3q0, w3q1 = both(w3) if need_dx else rows(w3)
-        w2q0, w2q1 = both(w2) if (need_dx or need_dw) else rows(w2)
+        w1q0, w1q1 = _cast_weight(w1, mode, need_dx, cfg)
+        w3q0, w3q1 = _cast_weight(w3, mode, need_dx, cfg)
+        w2q0, w2q1 = _cast_weight(w2, mode, need_dx or need_dw, cfg)
         h1 = ops.mx_gemm_nt(xq0, w1q0)
         h3 = ops.mx_gemm_nt(xq0, w3q0)
         gq0, gq1, _ = ops.swiglu_to_mx_dim0_dim1(h1, h3, mode, MX_SCALES_MFMA)
@@ -449,11 +507,7 @@ class _MXGroupedMM(torch.autograd.Function):
         xb = xb.contiguous()
         need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         xq0, xq1 = _cast_into_groups(xb, perm, mode, order, need_dw)
-        if need_dx and N % ops.BLOCK == 0:
-            wq0, wq1 = ops.to_mx_dim0_dim1_batched(w, mode, MX_SCALES_MFMA)
-        else:
-            wq0 = _cast_w_rows(w, mode)
-            wq1 = None
+        wq0, wq1 = _cast_weight(weight, mode, need_dx, cfg)
         y = _grouped_2d3d_padded(xq0, wq0, offs_p, back)
         ctx.cfg = cfg
         ctx.dims = (T, K, N, G)
@@ -533,11 +587,9 @@ class _MXGroupedFeedForward(torch.autograd.Function):
         need_dx = ctx.needs_input_grad[0]
         need_dw = any(ctx.needs_input_grad[1:4])
         xq0, xq1 = _cast_into_groups(xb, perm, mode, order, need_dw)
-        both = lambda w: ops.to_mx_dim0_dim1_batched(_bf16(w).contiguous(), mode, MX_SCALES_MFMA)
-        rows = lambda w: (_cast_w_rows(_bf16(w).contiguous(), mode), None)
-        w1q0, w1q1 = both(w1) if need_dx else rows(w1)
-        w3q0, w3q1 = both(w3) if need_dx else rows(w3)
-        w2q0, w2q1 = both(w2) if (need_dx or need_dw) else rows(w2)
+        w1q0, w1q1 = _cast_weight(w1, mode, need_dx, cfg)
+        w3q0, w3q1 = _cast_weight(w3, mode, need_dx, cfg)
+        w2q0, w2q1 = _cast_weight(w2, mode, need_dx or need_dw, cfg)
         h1 = ops.mx_grouped_gemm_2d3d(xq0, w1q0, offs_p)
         h3 = ops.mx_grouped_gemm_2d3d(xq0, w3q0, offs_p)
         gq0, gq1, _ = ops.swiglu_to_mx_dim0_dim1(h1, h3, mode, order)
@@ -649,11 +701,9 @@ class _MXRoutedExperts(torch.autograd.Function):
         xq0, xq1 = ops.to_mx_rows_gathered(xb, src_row, mode, order, need_dw,
                                            row_score if score_before else None)
         need_dg = need_dx or need_ds or need_dw
-        both = lambda w: ops.to_mx_dim0_dim1_batched(_bf16(w).contiguous(), mode, MX_SCALES_MFMA)
-        rows = lambda w: (_cast_w_rows(_bf16(w).contiguous(), mode), None)
-        w1q0, w1q1 = both(w1) if (need_dx or need_ds) else rows(w1)
-        w3q0, w3q1 = both(w3) if (need_dx or need_ds) else rows(w3)
-        w2q0, w2q1 = both(w2) if need_dg else rows(w2)
+        w1q0, w1q1 = _cast_weight(w1, mode, need_dx or need_ds, cfg)
+        w3q0, w3q1 = _cast_weight(w3, mode, need_dx or need_ds, cfg)
+        w2q0, w2q1 = _cast_weight(w2, mode, need_dg, cfg)
         h1 = ops.mx_grouped_gemm_2d3d(xq0, w1q0, offs_p)
         h3 = ops.mx_grouped_gemm_2d3d(xq0, w3q0, offs_p)
         gq0, gq1, _ = ops.swiglu_to_mx_dim0_dim1(h1, h3, mode, order)

@@ -217,6 +217,23 @@ def moe_row_dot(a: torch.Tensor, ia: torch.Tensor, b: torch.Tensor, ib: torch.Te
     return out
 
 
+def mx_dequant(d: MXData, out: torch.Tensor | None = None) -> torch.Tensor:
+    """bf16 [rows, cols] values of row-wise MXFP8 data (codes [rows, cols], blocks along cols)."""
+    codes = d.codes
+    if codes.dtype != torch.uint8 or codes.dim() != 2 or not codes.is_cuda:
+        raise TypeError("expected 2-D uint8 codes on the GPU")
+    codes = codes.contiguous()
+    rows, cols = codes.shape
+    if cols % BLOCK:
+        raise ValueError(f"cols {cols} is not a multiple of {BLOCK}")
+    if out is None:
+        out = torch.empty((rows, cols), dtype=torch.bfloat16, device=codes.device)
+    scales = d.scales.contiguous()
+    _call("mx_dequant", "dequant", codes.device, _ptr(codes), _ptr(scales), rows, cols, d.scale_order,
+          _ptr(out), out.stride(0), _stream(codes))
+    return out
+
+
 def token_logprob_fwd(logits: torch.Tensor, target: torch.Tensor):
     """(log-probability of target[r] under softmax(logits[r]), log-sum-exp of row r), float32
     [rows], from bf16 logits [rows, vocab] read once."""

@@ -19,7 +19,7 @@ import torch.nn as nn
 
 from .. import _lib
 from ..modules.linear import Linear
-from ..mx_tensor import MXFP8Config, MXFP8TrainingWeight, wrap_parameter
+from ..mx_tensor import MXFP8Config, MXFP8TrainingWeight, _cast_weight, wrap_parameter
 from . import QuantizationConverter
 from .module_utils import capture_module_attrs, inject_module_protocol, verify_module_protocol
 
@@ -69,6 +69,13 @@ class MXFP8Converter(QuantizationConverter):
         differ from the unfused ops' by one rounding step at a few elements in ten thousand;
         false keeps the three separate ops."""
 
+        cache_weight_casts: bool = False
+        """Not in the reference's Config.  Keep the MXFP8 forms of a converted weight until the
+        weight is next updated in place (2 extra bytes per weight element): `post_optimizer_hook`
+        then casts every converted weight once per optimizer step, and every forward until the
+        next step (gradient accumulation, evaluation, several micro-batches) and
+        `export_mxfp8_state_dict` reuse those codes."""
+
     def __init__(self, config: Config, *, parallel_dims: Any, model_compile_enabled: bool):
         self.enabled = False
         if not _lib.LIB_PATH.exists():
@@ -97,7 +104,7 @@ class MXFP8Converter(QuantizationConverter):
         saved = capture_module_attrs(model, ["_init_mean", "_init_std"], nn_module_cls=nn.Linear)
         cfg = MXFP8Config(_RECIPES[self.config.recipe_name],
                           self.config.pad_token_groups_for_grouped_mm,
-                          self.config.fuse_swiglu_cast)
+                          self.config.fuse_swiglu_cast, self.config.cache_weight_casts)
         n_linear = n_grouped = 0
         for fqn, mod in model.named_modules():
             if not self._matches(fqn):
@@ -122,5 +129,66 @@ class MXFP8Converter(QuantizationConverter):
         )
 
     def post_optimizer_hook(self, model: nn.Module | list[nn.Module]):
-        """MXFP8 training needs no post-optimizer work: weights are re-quantized every forward."""
-        return
+        """Nothing to do by default: weights are re-quantized in every forward, as in the
+        reference.  With `cache_weight_casts` the freshly updated weights are cast here, once per
+        optimizer step, for the forwards that follow and for a hand-over in MXFP8 form."""
+        if not self.enabled or not self.config.cache_weight_casts:
+            return
+        for m in model if isinstance(model, (list, tuple)) else [model]:
+            for p in m.parameters():
+                if isinstance(p, MXFP8TrainingWeight) and p.is_cuda:
+                    with torch.no_grad():
+                        _cast_weight(p.as_subclass(torch.Tensor), p.mx_config.scale_mode, True, p.mx_config)
+
+
+MXFP8_PAYLOAD_FORMAT = "mxfp8:e4m3fn+e8m0:block32:dim-1"
+
+
+def export_mxfp8_state_dict(model: nn.Module) -> dict:
+    """The model's state dict with every converted weight in MXFP8 form: for such a key the
+    value is ``{"format", "codes" (uint8, the weight's shape), "scales" (uint8, one E8M0 byte
+    per 32 elements of the last dim, row-major), "dtype" (of the original)}`` -- 1.03 bytes per
+    element instead of 2 -- and every other tensor is passed through.  What a trainer can hand
+    to a generator in place of the bf16 state dict
+    (torchtitan/experiments/rl/unified/actors/trainer.py:226-239)."""
+    from .. import ops
+
+    converted = {name: p for name, p in model.named_parameters() if isinstance(p, MXFP8TrainingWeight)}
+    out = {}
+    for name, t in model.state_dict().items():
+        p = converted.get(name)
+        if p is None or not p.is_cuda or p.shape[-1] % 32:
+            out[name] = t
+            continue
+        with torch.no_grad():
+            rows, _ = _cast_weight(p.as_subclass(torch.Tensor), p.mx_config.scale_mode, False, p.mx_config)
+        lead = p.shape[:-1]
+        n_rows, nblk = int(torch.Size(lead).numel()), p.shape[-1] // 32
+        if p.dim() == 3 and p.shape[1] % 128:  # per-matrix scale blocks: undo them one by one
+            per = ops.mfma_scale_bytes(p.shape[1], nblk)
+            scales = torch.stack([ops.scale_unlayout(rows.scales[g * per:(g + 1) * per], p.shape[1], nblk)
+                                  for g in range(p.shape[0])])
+        else:
+            scales = ops.scale_unlayout(rows.scales, n_rows, nblk)
+        out[name] = {"format": MXFP8_PAYLOAD_FORMAT, "codes": rows.codes.view(*p.shape),
+                     "scales": scales.view(*lead, nblk), "dtype": p.dtype}
+    return out
+
+
+def load_mxfp8_state_dict(payload: dict) -> dict:
+    """Plain state dict from `export_mxfp8_state_dict`'s output: MXFP8 entries are dequantized to
+    their original dtype (what `load_weights_from_state_dict` on the receiving side expects,
+    torchtitan/experiments/rl/unified/actors/generator.py:307-335)."""
+    from .. import ops
+    from ..ops import MX_SCALES_ROWMAJOR, MXData
+
+    out = {}
+    for name, v in payload.items():
+        if not (isinstance(v, dict) and v.get("format") == MXFP8_PAYLOAD_FORMAT):
+            out[name] = v
+            continue
+        codes, scales = v["codes"], v["scales"]
+        flat = ops.mx_dequant(MXData(codes.reshape(-1, codes.shape[-1]),
+                                     scales.reshape(-1, scales.shape[-1]).contiguous(), MX_SCALES_ROWMAJOR))
+        out[name] = flat.view(codes.shape).to(v["dtype"])
+    return out
