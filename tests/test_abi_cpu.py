@@ -54,3 +54,42 @@ def test_ctypes_prototypes_have_the_declared_number_of_arguments():
 
 def lib_arg_kinds(name):
     return list(_lib.SIGNATURES[name][1])
+
+
+def test_new_entry_points_validate_arguments_before_any_launch():
+    """Status 1 (invalid argument) for null pointers / negative sizes, 2 (alignment) for shapes or
+    pointers the kernels cannot take, 0 for empty problems: decided on the host, no GPU needed."""
+    lib = _lib.load()
+    P = ctypes.c_void_p
+    a16, odd = P(0x1000), P(0x1004)
+    # gate-fused casts
+    assert lib.mx_swiglu_cast_dim0_dim1(None, None, 0, 64, 64, 64, None, None, None, None, None, 1, 1, None) == 0
+    assert lib.mx_swiglu_cast_dim0_dim1(None, a16, 32, 64, 64, 64, a16, a16, a16, a16, None, 1, 1, None) == 1
+    assert lib.mx_swiglu_cast_dim0_dim1(a16, a16, 33, 64, 64, 64, a16, a16, a16, a16, None, 1, 1, None) == 2
+    assert lib.mx_swiglu_cast_dim0_dim1(a16, odd, 32, 64, 64, 64, a16, a16, a16, a16, None, 1, 1, None) == 2
+    assert lib.mx_swiglu_cast_dim0_dim1(a16, a16, 32, 64, 64, 64, a16, a16, a16, a16, None, 7, 1, None) == 1
+    assert lib.mx_swiglu_bwd_cast_dim0_dim1(a16, a16, None, 32, 64, 64, 64, 64, a16, a16, a16, a16, None, 1, 1, None) == 1
+    assert lib.mx_swiglu_bwd_cast_dim0_dim1(a16, a16, a16, 32, 64, 60, 64, 64, a16, a16, a16, a16, None, 1, 1, None) == 1
+    assert lib.mx_swiglu_bwd_cast_dim0_dim1(a16, a16, a16, 32, 48, 64, 64, 64, a16, a16, a16, a16, None, 1, 1, None) == 2
+    # gathered cast: the column-wise outputs come as a pair or not at all
+    assert lib.mx_cast_rows_gathered(a16, a16, None, 10, 0, 64, 64, a16, a16, None, None, 1, 1, None) == 0
+    assert lib.mx_cast_rows_gathered(a16, None, None, 10, 32, 64, 64, a16, a16, None, None, 1, 1, None) == 1
+    assert lib.mx_cast_rows_gathered(a16, a16, None, 10, 32, 64, 64, a16, a16, a16, None, 1, 1, None) == 1
+    assert lib.mx_cast_rows_gathered(a16, a16, None, 10, 40, 64, 64, a16, a16, a16, a16, 1, 1, None) == 2
+    assert lib.mx_cast_rows_gathered(a16, a16, None, 10, 32, 72, 72, a16, a16, None, None, 1, 1, None) == 2
+    # combine / row dot
+    assert lib.mx_moe_combine(a16, 8, 64, a16, None, 0, 2, 64, a16, 64, None) == 0
+    assert lib.mx_moe_combine(a16, 8, 64, None, None, 4, 2, 64, a16, 64, None) == 1
+    assert lib.mx_moe_combine(a16, 8, 60, a16, None, 4, 2, 64, a16, 64, None) == 1
+    assert lib.mx_moe_combine(a16, 8, 68, a16, None, 4, 2, 68, a16, 68, None) == 2
+    assert lib.mx_moe_row_dot(a16, 8, 64, a16, a16, 8, 64, None, 4, 64, a16, None) == 1
+    assert lib.mx_moe_row_dot(a16, 8, 64, a16, odd, 8, 64, a16, 4, 64, a16, None) == 2
+    # dequantization and token log-probabilities
+    assert lib.mx_dequant(a16, a16, 4, 48, 0, a16, 48, None) == 2
+    assert lib.mx_dequant(a16, None, 4, 64, 0, a16, 64, None) == 1
+    assert lib.mx_dequant(a16, a16, 4, 64, 5, a16, 64, None) == 1
+    assert lib.mx_token_logprob_fwd(a16, 0, 100, 104, a16, a16, a16, None) == 0
+    assert lib.mx_token_logprob_fwd(a16, 4, 0, 104, a16, a16, a16, None) == 1
+    assert lib.mx_token_logprob_fwd(a16, 4, 100, 100, a16, a16, a16, None) == 2
+    assert lib.mx_token_logprob_bwd(a16, 70000, 104, 104, a16, a16, a16, a16, 104, None) == 4
+    assert lib.mx_token_logprob_bwd(a16, 4, 104, 104, a16, a16, None, a16, 104, None) == 1
