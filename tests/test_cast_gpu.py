@@ -357,3 +357,42 @@ def test_dequant_is_exact(device, mode_name, mode):
         want = mo.f32_to_bf16_bits(mo.dequant(codes, scales))
         nan = lambda v: (v & 0x7FFF) > 0x7F80
         assert (nan(got) == nan(want)).all() and np.array_equal(got[~nan(want)], want[~nan(want)])
+
+
+def test_fused_casts_at_benchmark_sizes_equal_separate_kernels(device):
+    """At the sizes the benchmark runs (16384 x 14336 activations; 139264 padded rows of 2048 for
+    the MoE config) the gate-fused and gathered casts equal the plain cast of the tensor the
+    separate ops would have formed, byte for byte."""
+    torch.manual_seed(3)
+    M, H = 16384, 14336
+    a = (torch.randn(M, H, device=device) * 2).to(torch.bfloat16)
+    b = torch.randn(M, H, device=device).to(torch.bfloat16)
+    L = ops.MX_SCALES_MFMA
+    q0, q1, _ = ops.swiglu_to_mx_dim0_dim1(a, b, "rceil", L)
+    g = torch.nn.functional.silu(a) * b
+    r0, r1 = ops.to_mx_dim0_dim1(g, "rceil", L)
+    for got, want in ((q0, r0), (q1, r1)):
+        assert torch.equal(got.codes, want.codes) and torch.equal(got.scales, want.scales)
+    del q0, q1, r0, r1, g
+    dg = (torch.randn(M, H, device=device) * 1e-3).to(torch.bfloat16)
+    ta, tb = a.clone().requires_grad_(True), b.clone().requires_grad_(True)
+    (torch.nn.functional.silu(ta) * tb).backward(dg)
+    (da0, da1), (db0, db1), _ = ops.swiglu_bwd_to_mx_dim0_dim1(dg, a, b, "rceil", L)
+    for (got0, got1), grad in (((da0, da1), ta.grad), ((db0, db1), tb.grad)):
+        w0, w1 = ops.to_mx_dim0_dim1(grad, "rceil", L)
+        assert torch.equal(got0.codes, w0.codes) and torch.equal(got0.scales, w0.scales)
+        assert torch.equal(got1.codes, w1.codes) and torch.equal(got1.scales, w1.scales)
+    del a, b, dg, ta, tb, da0, da1, db0, db1, w0, w1
+    torch.cuda.empty_cache()
+    T, k, D, rows = 16384, 8, 2048, 139264
+    x = torch.randn(T, D, device=device).to(torch.bfloat16)
+    idx = torch.full((rows,), -1, dtype=torch.int64, device=device)
+    slots = torch.randperm(rows, device=device)[: T * k]
+    idx[slots] = torch.randint(0, T, (T * k,), device=device)
+    score = torch.rand(rows, device=device)
+    q0, q1 = ops.to_mx_rows_gathered(x, idx, "rceil", L, row_scale=score)
+    gathered = torch.cat((x, x.new_zeros((1, D))))[idx]
+    gathered = (gathered.float() * score[:, None]).to(torch.bfloat16)
+    r0, r1 = ops.to_mx_dim0_dim1(gathered, "rceil", L)
+    for got, want in ((q0, r0), (q1, r1)):
+        assert torch.equal(got.codes, want.codes) and torch.equal(got.scales, want.scales)
