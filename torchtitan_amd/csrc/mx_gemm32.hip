@@ -66,7 +66,9 @@ struct Tile32 {
   uint16_t* d;
   int64_t rows_a, rows_b;  // valid rows from the tile's origin (may exceed 256; <= 0: none)
   uint32_t koff;           // first K byte of the range inside an operand row (kGrouped2d2d)
-  uint32_t nblocks;        // 128-deep K blocks (0: the tile is written as zeros)
+  uint32_t nblocks;        // 128-deep K blocks, at least 1
+  bool empty;              // no K range (an empty group, rows behind the last group, or poison):
+                           // one block of out-of-range reads, i.e. zeros, stands in for it
   bool poison;             // grouped modes: the group ends break the alignment contract
 };
 
@@ -117,29 +119,6 @@ __device__ __forceinline__ void mfma_asm(v16f& c, const v8i& b, const v8i& a, ui
         "v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[%5,%6,0] op_sel_hi:[%7,%8,0]"
         : "+a"(c)
         : "v"(b), "v"(a), "v"(sb), "v"(sa), "n"(N & 1), "n"(M & 1), "n"(N >> 1), "n"(M >> 1));
-}
-
-// A tile without K blocks: zeros (an empty group, the rows behind the last group), or NaN when
-// the group ends break the contract, so that the mistake cannot pass unnoticed.  Written
-// straight from registers: wave (wm, wn) owns rows 128 wm.., columns 128 wn...
-// (Inlined on purpose: a call would make the compiler save every live register around it.)
-__device__ __forceinline__ void fill_tile32(uint16_t* d, int64_t rows_a, int64_t rows_b,
-                                                      int64_t ldd, bool poison) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-  const uint32_t fill = poison ? 0x7FC07FC0u : 0u;
-  const u32x4 w = {fill, fill, fill, fill};
-  const uint32_t ldd_b = (uint32_t)ldd * 2;
-  const __amdgpu_buffer_rsrc_t rd = make_rsrc(d, rows_a * ldd_b);
-  const uint32_t cols_valid = (uint32_t)(rows_b < 256 ? rows_b : 256);
-  const uint32_t colp = wn * 128 + (lane & 7) * 8;
-  const uint32_t vrow = (wm * 128 + (lane >> 3)) * ldd_b + colp * 2;
-  for (uint32_t r8 = 0; r8 < 16; ++r8) {
-    const uint32_t v0 = colp < cols_valid ? vrow : 0x80000000u;
-    const uint32_t v1 = colp + 64 < cols_valid ? vrow + 128 : 0x80000000u;
-    __builtin_amdgcn_raw_buffer_store_b128(w, rd, v0, r8 * 8 * ldd_b, 0);
-    __builtin_amdgcn_raw_buffer_store_b128(w, rd, v1, r8 * 8 * ldd_b, 0);
-  }
 }
 
 struct Frags32 {
@@ -234,6 +213,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     Tile32 r;
     r.poison = poison;
     r.koff = 0;
+    r.empty = false;
     uint32_t tm, tn;
     if (MODE == kDense || (MODE == kGrouped2d3d && poison)) {
       tile_coords(t, (uint32_t)((p.M + kT32 - 1) / kT32), tiles_n, tm, tn);
@@ -245,7 +225,8 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       r.d = p.d + (int64_t)tm * kT32 * p.ldd + (int64_t)tn * kT32;
       r.rows_a = p.M - (int64_t)tm * kT32;
       r.rows_b = p.N - (int64_t)tn * kT32;
-      r.nblocks = poison ? 0 : K / kKB;
+      r.nblocks = poison ? 1 : K / kKB;
+      r.empty = poison;
     } else if (MODE == kGrouped2d3d) {
       const uint32_t* first = reinterpret_cast<const uint32_t*>(smem + kRing32 + 4608);
       uint32_t g = 0, hi_g = G + 1;  // first[g] <= t < first[g + 1]
@@ -266,7 +247,8 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       r.d = p.d + row0 * p.ldd + (int64_t)tn * kT32;
       r.rows_a = hi - row0;
       r.rows_b = p.N - (int64_t)tn * kT32;
-      r.nblocks = g < G ? K / kKB : 0;
+      r.nblocks = g < G ? K / kKB : 1;
+      r.empty = g >= G;
     } else {
       const uint32_t tiles_m = (uint32_t)((p.M + kT32 - 1) / kT32), per_g = tiles_m * tiles_n;
       const uint32_t g = t / per_g;
@@ -282,6 +264,10 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       r.rows_b = p.N - (int64_t)tn * kT32;
       r.koff = (uint32_t)lo;
       r.nblocks = (uint32_t)((hi - lo) >> 7);
+      if (r.nblocks == 0) {
+        r.nblocks = 1;
+        r.empty = true;
+      }
     }
     return r;
   };
@@ -308,6 +294,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       w[1] = (int32_t)(t.rows_b > 0x7FFFFFFF ? 0x7FFFFFFF : t.rows_b);
       w[2] = (int32_t)t.nblocks;
       w[3] = (int32_t)t.koff;
+      w[4] = t.empty ? 1 : 0;
     }
     __syncthreads();
   }
@@ -339,6 +326,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       t.rows_b = __builtin_amdgcn_readfirstlane(r2.w);
       t.nblocks = (uint32_t)__builtin_amdgcn_readfirstlane(r3.x);
       t.koff = (uint32_t)__builtin_amdgcn_readfirstlane(r3.y);
+      t.empty = __builtin_amdgcn_readfirstlane(r3.z) != 0;
       t.poison = poison;
       return t;
     }
@@ -367,26 +355,23 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   int ld_slot = 0;
   __amdgpu_buffer_rsrc_t ra, rb, rs;  // codes of A, codes of B, scales this wave copies
   auto loader_open_tile = [&]() {
-    Tile32 t;
-    t.nblocks = 0;
-    while (ld_tile < n_my) {  // tiles without K blocks add nothing to the stream
-      t = get_tile(ld_tile);
-      if (MODE == kDense || t.nblocks) break;
-      ++ld_tile;
-    }
     if (ld_tile < n_my) {
+      const Tile32 t = get_tile(ld_tile);
       ld_nb = t.nblocks;
       // (kGrouped2d2d: the range stops at the end of the operand rows, not of the K range;
-      //  the K range is exact because nblocks is)
-      ra = make_rsrc(t.a, t.rows_a * K - t.koff);
-      rb = make_rsrc(t.b, t.rows_b * K - t.koff);
+      //  the K range is exact because nblocks is.)  A tile without a K range reads nothing:
+      // its one block arrives as zeros, scales included.
+      const bool none = MODE != kDense && t.empty;
+      ra = make_rsrc(t.a, none ? 0 : t.rows_a * K - t.koff);
+      rb = make_rsrc(t.b, none ? 0 : t.rows_b * K - t.koff);
       // wave 0 copies the scales of A's two 128-row groups, wave 2 those of B's (one copy per
       // block each: lanes 0-31 fetch group 0, lanes 32-63 group 1); a group beyond the operand
       // is cut off by the range and arrives as zeros
       const int64_t rows = wave < 2 ? t.rows_a : t.rows_b;
       const uint8_t* sbase = wave < 2 ? t.sa : t.sb;
-      rs = make_rsrc(sbase, rows > 128 ? (int64_t)ks_n * 256 + (int64_t)ld_nb * 512
-                                       : (rows > 0 ? (int64_t)ld_nb * 512 : 0));
+      rs = make_rsrc(sbase, none ? 0
+                                 : rows > 128 ? (int64_t)ks_n * 256 + (int64_t)ld_nb * 512
+                                              : (rows > 0 ? (int64_t)ld_nb * 512 : 0));
     } else {  // past the last tile: every lane reads out of range (zeros, no traffic)
       ld_nb = 1;
       ra = make_rsrc(p.a_codes, 0);
@@ -612,6 +597,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   const uint32_t patch = lds_base + kRing32 + wave * 7168;
   const uint32_t patch_w = patch + li * kPatchPitch + lj * 16;                 // + (n&1)*64 + h*32
   const uint32_t patch_r = patch + (lane >> 3) * kPatchPitch + (lane & 7) * 16;  // + pass*8 rows
+  const uint32_t nan_mask = (MODE != kDense && poison) ? 0x7FC07FC0u : 0u;
   auto epilogue = [&](const Tile32& t) {
     const int64_t rows_valid = t.rows_a;
     const uint32_t cols_valid = (uint32_t)(t.rows_b < kT32 ? t.rows_b : kT32);
@@ -628,8 +614,14 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       constexpr int m = decltype(p_)::value >> 1, np = decltype(p_)::value & 1;
       constexpr int n = 2 * np + (decltype(k_)::value >> 1), h = decltype(k_)::value & 1;
       const v16f a = acc[m][n];
-      const uint32_t x0 = pack_bf16(a[8 * h + 0], a[8 * h + 1]), y0 = pack_bf16(a[8 * h + 2], a[8 * h + 3]);
-      const uint32_t x1 = pack_bf16(a[8 * h + 4], a[8 * h + 5]), y1 = pack_bf16(a[8 * h + 6], a[8 * h + 7]);
+      uint32_t x0 = pack_bf16(a[8 * h + 0], a[8 * h + 1]), y0 = pack_bf16(a[8 * h + 2], a[8 * h + 3]);
+      uint32_t x1 = pack_bf16(a[8 * h + 4], a[8 * h + 5]), y1 = pack_bf16(a[8 * h + 6], a[8 * h + 7]);
+      if constexpr (MODE != kDense) {  // a broken group contract must not pass unnoticed: NaN
+        x0 |= nan_mask;
+        y0 |= nan_mask;
+        x1 |= nan_mask;
+        y1 |= nan_mask;
+      }
       const u32x2 sx = __builtin_amdgcn_permlane32_swap(x0, x1, false, false);
       const u32x2 sy = __builtin_amdgcn_permlane32_swap(y0, y1, false, false);
       const v4i w = {(int)sx.x, (int)sy.x, (int)sx.y, (int)sy.y};
@@ -682,7 +674,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   // loader fetched like any other block).
   for (uint32_t tile = 0; tile < n_my; ++tile) {
     const Tile32 t = get_tile(tile);
-    if (MODE == kDense || t.nblocks) {
+    {
       block_steps(f0, f1, std::true_type{});
       for (uint32_t i = 1; i < t.nblocks; ++i) block_steps(f0, f1, std::false_type{});
       // the next tile's first fragments were read in the last step: make them ordinary
@@ -699,8 +691,6 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       } else {
         epilogue(t);
       }
-    } else {
-      fill_tile32(t.d, t.rows_a, t.rows_b, p.ldd, t.poison);
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the over-issued prefetches before retiring
