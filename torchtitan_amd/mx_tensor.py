@@ -494,10 +494,12 @@ class _MXGroupedMM(torch.autograd.Function):
         plan = None
         # Padding to 128-row groups (instead of the 32 the format needs) lets all three GEMMs
         # run on the persistent kernel, which wants whole 128-row scale groups per expert.
-        fast = (cfg.pad_token_groups_for_grouped_mm and K % 128 == 0 and N % 128 == 0 and G <= 638)
+        # (also when the caller's groups are already 32-aligned: the move costs nothing extra
+        # inside the gathered cast and the persistent kernel is about twice as fast)
+        fast = K % 128 == 0 and N % 128 == 0 and G <= 638
         order = MX_SCALES_MFMA if fast else MX_SCALES_ROWMAJOR
         perm = back = None
-        if cfg.pad_token_groups_for_grouped_mm:
+        if cfg.pad_token_groups_for_grouped_mm or fast:
             plan = _pad_plan(offs, T, 128 if fast else ops.BLOCK)
             perm, offs_p, back = plan
         else:
@@ -573,10 +575,10 @@ class _MXGroupedFeedForward(torch.autograd.Function):
         G, H, _ = w1.shape
         xb = _bf16(x)
         pad = cfg.pad_token_groups_for_grouped_mm
-        fast = pad and D % 128 == 0 and H % 128 == 0 and G <= 638
+        fast = D % 128 == 0 and H % 128 == 0 and G <= 638  # 128-row groups: persistent kernel
         order = MX_SCALES_MFMA if fast else MX_SCALES_ROWMAJOR
         plan = perm = back = None
-        if pad:
+        if pad or fast:
             plan = _pad_plan(offs, T, 128 if fast else ops.BLOCK)
             perm, offs_p, back = plan
         else:
