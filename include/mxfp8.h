@@ -105,18 +105,21 @@ int mx_cast_rows_gathered(const void* x, const int64_t* row_index, const float* 
  * j = 0 .. top_k-1 in that order, in float32 (product and sum rounded separately), result
  * rounded to bf16; weights == NULL gives the plain sum.  y: bf16 [y_rows, cols] (row stride
  * ldy), pos: int64 [tokens, top_k] rows of y (outside [0, y_rows): contributes nothing), out:
- * bf16 [tokens, cols] (row stride ldo).  cols % 8 == 0, 16-byte aligned rows.
+ * bf16 [tokens, cols] (row stride ldo).  cols % 8 == 0, 16-byte aligned rows.  With y2 (same
+ * shape and stride as y, may be NULL) the rows summed are bf16(y + y2): the bf16 addition of two
+ * partial gradients (dx from w1 and from w3) without a pass of its own.
  * Stands in for the un-sort scatter and the score-weighted sum over top_k of
  * torchtitan/models/common/moe/moe.py:535-555, and (with y = the gradient of the routed input)
  * for the backward of the token gather `x[token_indices // top_k]` (moe.py:519). */
-int mx_moe_combine(const void* y, int64_t y_rows, int64_t ldy, const int64_t* pos,
+int mx_moe_combine(const void* y, const void* y2, int64_t y_rows, int64_t ldy, const int64_t* pos,
                    const float* weights, int64_t tokens, int64_t top_k, int64_t cols, void* out,
                    int64_t ldo, void* stream);
 
 /* Row dot products out[i] = sum_d a[ia[i], d] * b[ib[i], d] in float32 over bf16 matrices
- * a [a_rows, cols], b [b_rows, cols]; an index outside its matrix gives 0.  The gradient of the
+ * a [a_rows, cols], b [b_rows, cols]; an index outside its matrix gives 0; with a2 (a's shape,
+ * may be NULL) a's rows are bf16(a + a2).  The gradient of the
  * routing scores on either side of the experts (backward of moe.py:521-527 and :541-551). */
-int mx_moe_row_dot(const void* a, int64_t a_rows, int64_t lda, const int64_t* ia, const void* b,
+int mx_moe_row_dot(const void* a, const void* a2, int64_t a_rows, int64_t lda, const int64_t* ia, const void* b,
                    int64_t b_rows, int64_t ldb, const int64_t* ib, int64_t n, int64_t cols,
                    float* out, void* stream);
 

@@ -426,6 +426,13 @@ def gather_rows(x_bits: np.ndarray, row_index: np.ndarray, row_scale: np.ndarray
     return np.where(ok[:, None], scaled, 0).astype(np.uint16)
 
 
+def add_bf16(x_bits: np.ndarray, y_bits: np.ndarray) -> np.ndarray:
+    """bf16 sum as one tensor op: float32 addition (exact for two bf16 operands up to its own
+    rounding) rounded to bf16."""
+    with np.errstate(over="ignore", invalid="ignore"):
+        return f32_to_bf16_bits(bf16_bits_to_f32(x_bits) + bf16_bits_to_f32(y_bits))
+
+
 def moe_combine(y_bits: np.ndarray, pos: np.ndarray, weights: np.ndarray | None = None) -> np.ndarray:
     """out[t] = sum_j weights[t, j] * y[pos[t, j]] accumulated in float32 for j = 0 .. k-1 in
     that order (product and sum rounded separately), rounded to bf16: the score-weighted

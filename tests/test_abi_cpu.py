@@ -78,12 +78,13 @@ def test_new_entry_points_validate_arguments_before_any_launch():
     assert lib.mx_cast_rows_gathered(a16, a16, None, 10, 40, 64, 64, a16, a16, a16, a16, 1, 1, None) == 2
     assert lib.mx_cast_rows_gathered(a16, a16, None, 10, 32, 72, 72, a16, a16, None, None, 1, 1, None) == 2
     # combine / row dot
-    assert lib.mx_moe_combine(a16, 8, 64, a16, None, 0, 2, 64, a16, 64, None) == 0
-    assert lib.mx_moe_combine(a16, 8, 64, None, None, 4, 2, 64, a16, 64, None) == 1
-    assert lib.mx_moe_combine(a16, 8, 60, a16, None, 4, 2, 64, a16, 64, None) == 1
-    assert lib.mx_moe_combine(a16, 8, 68, a16, None, 4, 2, 68, a16, 68, None) == 2
-    assert lib.mx_moe_row_dot(a16, 8, 64, a16, a16, 8, 64, None, 4, 64, a16, None) == 1
-    assert lib.mx_moe_row_dot(a16, 8, 64, a16, odd, 8, 64, a16, 4, 64, a16, None) == 2
+    assert lib.mx_moe_combine(a16, None, 8, 64, a16, None, 0, 2, 64, a16, 64, None) == 0
+    assert lib.mx_moe_combine(a16, None, 8, 64, None, None, 4, 2, 64, a16, 64, None) == 1
+    assert lib.mx_moe_combine(a16, None, 8, 60, a16, None, 4, 2, 64, a16, 64, None) == 1
+    assert lib.mx_moe_combine(a16, None, 8, 68, a16, None, 4, 2, 68, a16, 68, None) == 2
+    assert lib.mx_moe_combine(a16, odd, 8, 64, a16, None, 4, 2, 64, a16, 64, None) == 2
+    assert lib.mx_moe_row_dot(a16, None, 8, 64, a16, a16, 8, 64, None, 4, 64, a16, None) == 1
+    assert lib.mx_moe_row_dot(a16, None, 8, 64, a16, odd, 8, 64, a16, 4, 64, a16, None) == 2
     # dequantization and token log-probabilities
     assert lib.mx_dequant(a16, a16, 4, 48, 0, a16, 48, None) == 2
     assert lib.mx_dequant(a16, None, 4, 64, 0, a16, 64, None) == 1

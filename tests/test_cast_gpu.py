@@ -333,10 +333,19 @@ def test_moe_combine_and_row_dot(device, tokens, k, cols):
     assert np.array_equal(bits_of(got), mo.moe_combine(y_bits, pos, w))
     got = ops.moe_combine(y, tp)
     assert np.array_equal(bits_of(got), mo.moe_combine(y_bits, pos, None))
+    # two partial matrices merged by a bf16 addition on the way in
+    y2_bits = randn_bits(rng, (rows, cols))
+    y2 = bf16_from_bits(y2_bits, device)
+    merged = mo.add_bf16(y_bits, y2_bits)
+    got = ops.moe_combine(y, tp, torch.from_numpy(w).to(device), y2)
+    assert np.array_equal(bits_of(got), mo.moe_combine(merged, pos, w))
     x_bits = randn_bits(rng, (tokens, cols))
     ib = (np.arange(tokens * k) // k).astype(np.int64)
     d = ops.moe_row_dot(y, tp.view(-1), bf16_from_bits(x_bits, device), torch.from_numpy(ib).to(device))
     ref = mo.moe_row_dot(y_bits, pos.reshape(-1), x_bits, ib)
+    assert np.allclose(d.cpu().numpy().astype(np.float64), ref, rtol=1e-5, atol=1e-5 * np.sqrt(cols))
+    d = ops.moe_row_dot(y, tp.view(-1), bf16_from_bits(x_bits, device), torch.from_numpy(ib).to(device), y2)
+    ref = mo.moe_row_dot(merged, pos.reshape(-1), x_bits, ib)
     assert np.allclose(d.cpu().numpy().astype(np.float64), ref, rtol=1e-5, atol=1e-5 * np.sqrt(cols))
 
 

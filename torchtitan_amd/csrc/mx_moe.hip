@@ -24,11 +24,19 @@ __device__ __forceinline__ float rounded_product(float a, float b) {
   return p;
 }
 
+// bf16(a + b) of two bf16 values, as a bf16 tensor addition forms it.
+__device__ __forceinline__ float bf16_sum(uint32_t a16, uint32_t b16) {
+  return bf16_bits_f32(f32_bf16_bits(bf16_bits_f32(a16) + bf16_bits_f32(b16)));
+}
+
 // out[t, :] = sum_j w[t, j] * y[pos[t, j], :]   (j = 0 .. k-1 in that order, float32, the product
 // and the sum rounded separately; w == nullptr: plain sum).  A position outside [0, y_rows)
-// contributes nothing.  One lane per 8 columns, grid-stride over (token, column chunk).
+// contributes nothing.  With y2, the rows summed are bf16(y + y2) (two matrices of one shape
+// that a bf16 addition would have merged first).  One lane per 8 columns, grid-stride over
+// (token, column chunk).
 __global__ __launch_bounds__(kMoeThreads) void moe_combine_kernel(
-    const uint16_t* __restrict__ y, int64_t y_rows, int64_t ldy, const int64_t* __restrict__ pos,
+    const uint16_t* __restrict__ y, const uint16_t* __restrict__ y2, int64_t y_rows, int64_t ldy,
+    const int64_t* __restrict__ pos,
     const float* __restrict__ w, int64_t tokens, int k, int64_t cols, uint16_t* __restrict__ out,
     int64_t ldo) {
   const int64_t chunks = cols / 8;
@@ -42,19 +50,28 @@ __global__ __launch_bounds__(kMoeThreads) void moe_combine_kernel(
       if (r < 0 || r >= y_rows) continue;
       const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(y + r * ldy + c));
       const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+      float x[8];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        x[2 * e] = bf16_bits_f32(d[e] & 0xFFFFu);
+        x[2 * e + 1] = bf16_bits_f32(d[e] >> 16);
+      }
+      if (y2) {
+        const u32x4 v2 = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(y2 + r * ldy + c));
+        const uint32_t d2[4] = {v2.x, v2.y, v2.z, v2.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          x[2 * e] = bf16_sum(d[e] & 0xFFFFu, d2[e] & 0xFFFFu);
+          x[2 * e + 1] = bf16_sum(d[e] >> 16, d2[e] >> 16);
+        }
+      }
       if (w) {
         const float s = w[t * k + j];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          acc[2 * e] += rounded_product(s, bf16_bits_f32(d[e] & 0xFFFFu));
-          acc[2 * e + 1] += rounded_product(s, bf16_bits_f32(d[e] >> 16));
-        }
+        for (int e = 0; e < 8; ++e) acc[e] += rounded_product(s, x[e]);
       } else {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          acc[2 * e] = acc[2 * e] + bf16_bits_f32(d[e] & 0xFFFFu);
-          acc[2 * e + 1] = acc[2 * e + 1] + bf16_bits_f32(d[e] >> 16);
-        }
+        for (int e = 0; e < 8; ++e) acc[e] = acc[e] + x[e];
       }
     }
     u32x4 o;
@@ -67,9 +84,11 @@ __global__ __launch_bounds__(kMoeThreads) void moe_combine_kernel(
 }
 
 // out[i] = sum_d a[ia[i], d] * b[ib[i], d] in float32; a row index outside its matrix gives 0.
-// One wave per output: lanes stride over 8-column chunks, then a butterfly over the 64 lanes.
+// With a2, a's rows are bf16(a + a2).  One wave per output: lanes stride over 8-column chunks,
+// then a butterfly over the 64 lanes.
 __global__ __launch_bounds__(kMoeThreads) void moe_row_dot_kernel(
-    const uint16_t* __restrict__ a, int64_t a_rows, int64_t lda, const int64_t* __restrict__ ia,
+    const uint16_t* __restrict__ a, const uint16_t* __restrict__ a2, int64_t a_rows, int64_t lda,
+    const int64_t* __restrict__ ia,
     const uint16_t* __restrict__ b, int64_t b_rows, int64_t ldb, const int64_t* __restrict__ ib,
     int64_t n, int64_t cols, float* __restrict__ out) {
   const int lane = threadIdx.x & 63;
@@ -83,10 +102,25 @@ __global__ __launch_bounds__(kMoeThreads) void moe_row_dot_kernel(
         const u32x4 va = *reinterpret_cast<const u32x4*>(a + ra * lda + c);
         const u32x4 vb = *reinterpret_cast<const u32x4*>(b + rb * ldb + c);
         const uint32_t da[4] = {va.x, va.y, va.z, va.w}, db[4] = {vb.x, vb.y, vb.z, vb.w};
+        float xa[8];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          acc = __builtin_fmaf(bf16_bits_f32(da[e] & 0xFFFFu), bf16_bits_f32(db[e] & 0xFFFFu), acc);
-          acc = __builtin_fmaf(bf16_bits_f32(da[e] >> 16), bf16_bits_f32(db[e] >> 16), acc);
+          xa[2 * e] = bf16_bits_f32(da[e] & 0xFFFFu);
+          xa[2 * e + 1] = bf16_bits_f32(da[e] >> 16);
+        }
+        if (a2) {
+          const u32x4 v2 = *reinterpret_cast<const u32x4*>(a2 + ra * lda + c);
+          const uint32_t d2[4] = {v2.x, v2.y, v2.z, v2.w};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            xa[2 * e] = bf16_sum(da[e] & 0xFFFFu, d2[e] & 0xFFFFu);
+            xa[2 * e + 1] = bf16_sum(da[e] >> 16, d2[e] >> 16);
+          }
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          acc = __builtin_fmaf(xa[2 * e], bf16_bits_f32(db[e] & 0xFFFFu), acc);
+          acc = __builtin_fmaf(xa[2 * e + 1], bf16_bits_f32(db[e] >> 16), acc);
         }
       }
     }
@@ -106,34 +140,39 @@ static inline unsigned moe_grid(int64_t work_items) {
 
 using namespace mx;
 
-extern "C" int mx_moe_combine(const void* y, int64_t y_rows, int64_t ldy, const int64_t* pos,
+extern "C" int mx_moe_combine(const void* y, const void* y2, int64_t y_rows, int64_t ldy,
+                              const int64_t* pos,
                               const float* weights, int64_t tokens, int64_t top_k, int64_t cols,
                               void* out, int64_t ldo, void* stream) {
   if (y_rows < 0 || tokens < 0 || top_k < 0 || top_k > 1024 || cols < 0 || ldy < cols || ldo < cols)
     return MX_ERR_INVALID_ARG;
   if (tokens == 0 || cols == 0) return MX_OK;
   if (!out || (top_k > 0 && (!y || !pos))) return MX_ERR_INVALID_ARG;
-  if (cols % 8 || ldy % 8 || ldo % 8 || ((uintptr_t)y & 15) || ((uintptr_t)out & 15) ||
-      ((uintptr_t)pos & 7) || ((uintptr_t)weights & 3))
+  if (cols % 8 || ldy % 8 || ldo % 8 || ((uintptr_t)y & 15) || ((uintptr_t)y2 & 15) ||
+      ((uintptr_t)out & 15) || ((uintptr_t)pos & 7) || ((uintptr_t)weights & 3))
     return MX_ERR_ALIGNMENT;
   hipLaunchKernelGGL(moe_combine_kernel, dim3(moe_grid(tokens * (cols / 8))), dim3(kMoeThreads), 0,
-                     (hipStream_t)stream, (const uint16_t*)y, y_rows, ldy, pos, weights, tokens,
+                     (hipStream_t)stream, (const uint16_t*)y, (const uint16_t*)y2, y_rows, ldy, pos,
+                     weights, tokens,
                      (int)top_k, cols, (uint16_t*)out, ldo);
   return hipGetLastError() == hipSuccess ? MX_OK : MX_ERR_LAUNCH;
 }
 
-extern "C" int mx_moe_row_dot(const void* a, int64_t a_rows, int64_t lda, const int64_t* ia,
+extern "C" int mx_moe_row_dot(const void* a, const void* a2, int64_t a_rows, int64_t lda,
+                              const int64_t* ia,
                               const void* b, int64_t b_rows, int64_t ldb, const int64_t* ib,
                               int64_t n, int64_t cols, float* out, void* stream) {
   if (a_rows < 0 || b_rows < 0 || n < 0 || cols < 0 || lda < cols || ldb < cols)
     return MX_ERR_INVALID_ARG;
   if (n == 0) return MX_OK;
   if (!a || !b || !ia || !ib || !out) return MX_ERR_INVALID_ARG;
-  if (cols % 8 || lda % 8 || ldb % 8 || ((uintptr_t)a & 15) || ((uintptr_t)b & 15) ||
+  if (cols % 8 || lda % 8 || ldb % 8 || ((uintptr_t)a & 15) || ((uintptr_t)a2 & 15) ||
+      ((uintptr_t)b & 15) ||
       ((uintptr_t)ia & 7) || ((uintptr_t)ib & 7) || ((uintptr_t)out & 3))
     return MX_ERR_ALIGNMENT;
   hipLaunchKernelGGL(moe_row_dot_kernel, dim3(moe_grid(n * 64)), dim3(kMoeThreads), 0,
-                     (hipStream_t)stream, (const uint16_t*)a, a_rows, lda, ia, (const uint16_t*)b,
+                     (hipStream_t)stream, (const uint16_t*)a, (const uint16_t*)a2, a_rows, lda, ia,
+                     (const uint16_t*)b,
                      b_rows, ldb, ib, n, cols, out);
   return hipGetLastError() == hipSuccess ? MX_OK : MX_ERR_LAUNCH;
 }

@@ -756,15 +756,18 @@ class _MXRoutedExperts(torch.autograd.Function):
             w1q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
             w3q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
             need_dxp = need_dx or (need_ds and score_before)
-            if need_dxp:  # gradient of the (scaled) routed inputs, padded layout
-                dxp = ops.mx_grouped_gemm_2d3d(da0, w1q1, offs_p) + ops.mx_grouped_gemm_2d3d(db0, w3q1, offs_p)
+            if need_dxp:
+                # gradient of the (scaled) routed inputs, padded layout: the two halves from w1
+                # and w3; their bf16 sum is formed inside the kernels that consume it
+                dxp1 = ops.mx_grouped_gemm_2d3d(da0, w1q1, offs_p)
+                dxp3 = ops.mx_grouped_gemm_2d3d(db0, w3q1, offs_p)
             if need_dx:
-                dx = cast_back(ops.moe_combine(dxp, pos, scores if score_before else None), ctx.dtypes[0])
+                dx = cast_back(ops.moe_combine(dxp1, pos, scores if score_before else None, dxp3), ctx.dtypes[0])
             if need_ds:
                 other = saved.pop(0)  # x (scores in front of the experts) or the expert outputs
                 token = torch.arange(T * k, device=pos.device, dtype=torch.int64).div_(k, rounding_mode="floor")
                 if score_before:
-                    ds = ops.moe_row_dot(dxp, pos.view(-1), other, token)
+                    ds = ops.moe_row_dot(dxp1, pos.view(-1), other, token, dxp3)
                 else:
                     ds = ops.moe_row_dot(other, pos.view(-1), dob, token)
                 ds = cast_back(ds.view(T, k), ctx.dtypes[1])

@@ -179,11 +179,16 @@ def to_mx_rows_gathered(x: torch.Tensor, row_index: torch.Tensor, mode="floor",
     return MXData(codes, scales, order), (MXData(codes_t, scales_t, order) if want_cols else None)
 
 
-def moe_combine(y: torch.Tensor, pos: torch.Tensor, weights: torch.Tensor | None = None) -> torch.Tensor:
+def moe_combine(y: torch.Tensor, pos: torch.Tensor, weights: torch.Tensor | None = None,
+                y2: torch.Tensor | None = None) -> torch.Tensor:
     """out[t] = sum_j weights[t, j] * y[pos[t, j]] (float32, j in order; plain sum without
     weights), bf16 [tokens, cols].  y: bf16 [rows, cols]; pos: int64 [tokens, top_k]; a position
-    outside y contributes nothing."""
+    outside y contributes nothing.  With y2 (y's shape) the rows are bf16(y + y2)."""
     y = _check_hp(y)
+    if y2 is not None:
+        y2 = _check_hp(y2)
+        if y2.shape != y.shape or y2.stride(0) != y.stride(0):
+            raise ValueError("y2 must have y's shape and row stride")
     if pos.dtype != torch.int64 or pos.dim() != 2 or pos.device != y.device:
         raise TypeError("pos must be a 2-D int64 tensor on y's device")
     pos = pos.contiguous()
@@ -193,16 +198,22 @@ def moe_combine(y: torch.Tensor, pos: torch.Tensor, weights: torch.Tensor | None
             raise TypeError("weights must be float32 of pos's shape on y's device")
         weights = weights.contiguous()
     out = torch.empty((T, y.shape[1]), dtype=torch.bfloat16, device=y.device)
-    _call("mx_moe_combine", "moe_combine", y.device, _ptr(y), y.shape[0], y.stride(0), _ptr(pos),
+    _call("mx_moe_combine", "moe_combine", y.device, _ptr(y), _ptr(y2) if y2 is not None else None,
+          y.shape[0], y.stride(0), _ptr(pos),
           _ptr(weights) if weights is not None else None, T, k, y.shape[1], _ptr(out), out.stride(0),
           _stream(y))
     return out
 
 
-def moe_row_dot(a: torch.Tensor, ia: torch.Tensor, b: torch.Tensor, ib: torch.Tensor) -> torch.Tensor:
+def moe_row_dot(a: torch.Tensor, ia: torch.Tensor, b: torch.Tensor, ib: torch.Tensor,
+                a2: torch.Tensor | None = None) -> torch.Tensor:
     """out[i] = <a[ia[i]], b[ib[i]]> in float32 for bf16 matrices a, b with equal column counts;
-    an index outside its matrix gives 0."""
+    an index outside its matrix gives 0.  With a2 (a's shape) a's rows are bf16(a + a2)."""
     a, b = _check_hp(a), _check_hp(b)
+    if a2 is not None:
+        a2 = _check_hp(a2)
+        if a2.shape != a.shape or a2.stride(0) != a.stride(0):
+            raise ValueError("a2 must have a's shape and row stride")
     if a.shape[1] != b.shape[1]:
         raise ValueError(f"column mismatch: {a.shape[1]} vs {b.shape[1]}")
     for idx in (ia, ib):
@@ -212,7 +223,8 @@ def moe_row_dot(a: torch.Tensor, ia: torch.Tensor, b: torch.Tensor, ib: torch.Te
         raise ValueError("index shapes differ")
     ia_c, ib_c = ia.contiguous().view(-1), ib.contiguous().view(-1)
     out = torch.empty(ia.shape, dtype=torch.float32, device=a.device)
-    _call("mx_moe_row_dot", "moe_row_dot", a.device, _ptr(a), a.shape[0], a.stride(0), _ptr(ia_c), _ptr(b),
+    _call("mx_moe_row_dot", "moe_row_dot", a.device, _ptr(a), _ptr(a2) if a2 is not None else None,
+          a.shape[0], a.stride(0), _ptr(ia_c), _ptr(b),
           b.shape[0], b.stride(0), _ptr(ib_c), ia_c.numel(), a.shape[1], _ptr(out), _stream(a))
     return out
 
