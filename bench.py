@@ -125,6 +125,51 @@ def time_casts(dev, recipe_mode):
     return out
 
 
+def time_yardsticks(dev):
+    """What the same box does on the same shapes with stock kernels, for scale (not targets and not
+    part of `value`): the vendor library's GEMMs through torch at M 16384, N 14336, K 4096, and
+    torch's device-to-device copy as the practical HBM ceiling for the casts."""
+    import torch
+
+    def timed(fn, reps=6):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(reps):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        return s.elapsed_time(e) * 1e-3 / reps
+
+    out = {}
+    flops = 2.0 * M * HIDDEN * DIM
+    a = torch.randn((M, DIM), device=dev).to(torch.float8_e4m3fn)
+    b = (torch.randn((HIDDEN, DIM), device=dev) * 1.28).to(torch.float8_e4m3fn)
+    one = torch.ones((), device=dev)
+    unit = lambda rows: torch.full((rows, DIM // 32), 127, dtype=torch.uint8, device=dev).view(torch.float8_e8m0fnu)
+    sa, sb = unit(M), unit(HIDDEN)
+    xb, wb = a.to(torch.bfloat16), b.to(torch.bfloat16)
+    cases = (
+        ("vendor_fp8_tensorwise_gemm", lambda: torch._scaled_mm(a, b.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16)),
+        ("vendor_mx_block_scaled_gemm", lambda: torch._scaled_mm(a, b.t(), scale_a=sa, scale_b=sb, out_dtype=torch.bfloat16)),
+        ("vendor_bf16_gemm", lambda: xb @ wb.t()),
+    )
+    for name, fn in cases:
+        try:
+            out[name] = {"TFLOP/s": round(flops / timed(fn) / 1e12, 1)}
+        except Exception as ex:  # a build of torch without that kernel: say so, measure the rest
+            out[name] = {"error": f"{type(ex).__name__}: {str(ex)[:120]}"}
+    del a, b, sa, sb, xb, wb
+    src = torch.empty(256 * 1024 * 1024, device=dev, dtype=torch.bfloat16).normal_()
+    dst = torch.empty_like(src)
+    sec = timed(lambda: dst.copy_(src), reps=10)
+    out["device_copy_512MiB"] = {"GB/s": round(2 * src.numel() * 2 / sec / 1e9, 1),
+                                 "frac_hbm": round(2 * src.numel() * 2 / sec / 1e9 / PEAK_HBM_GBPS, 3)}
+    return out
+
+
 def time_ffn_block(dev, recipe):
     """Beyond the headline: the whole SwiGLU block w2(silu(w1 x) * w3 x), forward + backward, at
     the same shapes, with the gate (and its backward) inside the cast kernels and with silu and
@@ -529,6 +574,8 @@ def main():
         line["swiglu_block"] = time_ffn_block(dev, args.recipe)
         torch.cuda.empty_cache()
         line["policy_loss_logprobs"] = time_policy_loss(dev)
+        torch.cuda.empty_cache()
+        line["yardsticks"] = time_yardsticks(dev)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(0 if recipe_mode == "floor" else 1, target_s=12.0)
     print(json.dumps(line))
