@@ -170,6 +170,103 @@ def time_yardsticks(dev):
     return out
 
 
+def time_decoder_block(dev, recipe):
+    """BASELINE configs[2] for scale (not the headline): one Llama-3-8B-style decoder block (dim
+    4096, 32 heads / 8 KV heads, FFN 14336, RMSNorm eps 1e-5, RoPE theta 5e5, init N(0, 0.02)),
+    forward + backward at batch 1 x seq 8192, with all seven linears converted to MXFP8
+    (attention itself in bf16 through torch's SDPA) and unconverted in bf16."""
+    import torch
+    import torch.nn as nn
+    import torch.nn.functional as F
+
+    from torchtitan_amd import mx_tensor
+    from torchtitan_amd.modules import FeedForward, Linear
+    from torchtitan_amd.protocols import ModelConvertersContainer
+    from torchtitan_amd.quantization.mx import MXFP8Converter
+
+    dim, heads, kv_heads, ffn, seq = 4096, 32, 8, 14336, 8192
+    hd = dim // heads
+
+    class Attention(nn.Module):
+        def __init__(self):
+            super().__init__()
+            mk = lambda i, o: Linear.Config().build(in_features=i, out_features=o)
+            self.wq, self.wk, self.wv, self.wo = mk(dim, dim), mk(dim, kv_heads * hd), mk(dim, kv_heads * hd), mk(dim, dim)
+
+        def forward(self, x, rope):
+            B, S, _ = x.shape
+            q = self.wq(x).view(B, S, heads, hd)
+            k = self.wk(x).view(B, S, kv_heads, hd)
+            v = self.wv(x).view(B, S, kv_heads, hd)
+            cos, sin = rope
+
+            def rot(t):  # rotate pairs (even, odd) of the head dimension
+                t2 = t.float().reshape(*t.shape[:-1], hd // 2, 2)
+                a, b = t2[..., 0], t2[..., 1]
+                return torch.stack((a * cos - b * sin, a * sin + b * cos), dim=-1).reshape(t.shape).to(t.dtype)
+
+            q, k = rot(q), rot(k)
+            o = F.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2),
+                                               is_causal=True, enable_gqa=True)
+            return self.wo(o.transpose(1, 2).reshape(B, S, dim))
+
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.attention = Attention()
+            self.feed_forward = FeedForward.Config(hidden_dim=ffn).build(dim=dim)
+            self.attention_norm = nn.RMSNorm(dim, eps=1e-5)
+            self.ffn_norm = nn.RMSNorm(dim, eps=1e-5)
+
+        def forward(self, x, rope):
+            h = x + self.attention(self.attention_norm(x), rope)
+            return h + self.feed_forward(self.ffn_norm(h))
+
+    pos = torch.arange(seq, device=dev, dtype=torch.float32)
+    freqs = 1.0 / (500000.0 ** (torch.arange(0, hd, 2, device=dev, dtype=torch.float32) / hd))
+    ang = torch.outer(pos, freqs)[None, :, None, :]
+    rope = (ang.cos(), ang.sin())
+    x = torch.randn((1, seq, dim), device=dev, dtype=torch.bfloat16).requires_grad_(True)
+    dy = torch.randn((1, seq, dim), device=dev, dtype=torch.bfloat16) * 1e-3
+    flops = 3 * 2.0 * seq * (2 * dim * dim + 2 * dim * kv_heads * hd + 3 * dim * ffn)  # the seven linears
+    out = {}
+    for name, convert in (("mxfp8_linears", True), ("bf16", False)):
+        torch.manual_seed(0)
+        blk = Block()
+        if convert:
+            ModelConvertersContainer.Config(
+                converters=[MXFP8Converter.Config(fqns=["attention", "feed_forward"], recipe_name=recipe)]
+            ).build(parallel_dims=None, model_compile_enabled=False).convert(blk)
+        blk.to(dev).to(torch.bfloat16)
+        with torch.no_grad():
+            for m in blk.modules():
+                if isinstance(m, nn.Linear):
+                    m.weight.normal_(0.0, 0.02)
+
+        def step():
+            mx_tensor._cast_cache.clear()
+            x.grad = None
+            for p in blk.parameters():
+                p.grad = None
+            blk(x, rope).backward(dy)
+
+        for _ in range(2):
+            step()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(4):
+            step()
+        e.record()
+        torch.cuda.synchronize()
+        ms = s.elapsed_time(e) / 4
+        out[name] = {"ms": round(ms, 3), "linear_TFLOP/s_over_block_time": round(flops / ms / 1e9, 1)}
+        del blk
+        torch.cuda.empty_cache()
+    out["speedup_over_bf16"] = round(out["bf16"]["ms"] / out["mxfp8_linears"]["ms"], 3)
+    return out
+
+
 def time_ffn_block(dev, recipe):
     """Beyond the headline: the whole SwiGLU block w2(silu(w1 x) * w3 x), forward + backward, at
     the same shapes, with the gate (and its backward) inside the cast kernels and with silu and
@@ -576,6 +673,8 @@ def main():
         line["policy_loss_logprobs"] = time_policy_loss(dev)
         torch.cuda.empty_cache()
         line["yardsticks"] = time_yardsticks(dev)
+        torch.cuda.empty_cache()
+        line["llama3_8b_decoder_block"] = time_decoder_block(dev, args.recipe)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(0 if recipe_mode == "floor" else 1, target_s=12.0)
     print(json.dumps(line))
