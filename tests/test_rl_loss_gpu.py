@@ -93,3 +93,78 @@ def test_policy_gradient_loss_fused_vs_oracle(device):
         assert math.isclose(metrics[k], v, rel_tol=1e-4, abs_tol=1e-5), k
     total.backward()
     assert torch.isfinite(model.out.weight.grad).all() and model.out.weight.grad.abs().sum() > 0
+
+
+def test_policy_step_on_a_small_converted_model_then_weight_hand_over(device):
+    """BASELINE configs[4] in small: a dense decoder-only model with MXFP8 linears, packed
+    prompts / completions of different lengths, the policy-gradient loss on fused log-probs,
+    backward, an optimizer step, then the re-cast of all converted weights for the hand-over."""
+    from tests.test_converter_gpu import _MiniDecoderBlock
+    from torchtitan_amd import ops
+    from torchtitan_amd.modules import Linear
+    from torchtitan_amd.mx_tensor import MXFP8TrainingWeight
+    from torchtitan_amd.protocols import ModelConvertersContainer
+    from torchtitan_amd.quantization.mx import MXFP8Converter, export_mxfp8_state_dict, load_mxfp8_state_dict
+
+    vocab, dim = 512, 128
+
+    class TinyLM(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.tok_embeddings = nn.Embedding(vocab, dim)
+            self.layers = nn.ModuleList([_MiniDecoderBlock(dim, 4, 2, 256) for _ in range(2)])
+            self.norm = nn.RMSNorm(dim, eps=1e-5)
+            self.output = Linear.Config().build(in_features=dim, out_features=vocab)
+
+        def forward(self, tokens, attention_masks=None):
+            h = self.tok_embeddings(tokens)
+            # the MXFP8 linears want a multiple of 32 tokens: pad the sequence on the right
+            # (causal attention: the real positions do not see the padding)
+            S = h.shape[1]
+            pad = -S % 32
+            if pad:
+                h = torch.cat((h, h.new_zeros((1, pad, dim))), dim=1)
+            for layer in self.layers:
+                h = layer(h)
+            return self.output(self.norm(h[:, :S]))
+
+    torch.manual_seed(3)
+    model = TinyLM().to(device).to(torch.bfloat16)
+    box = ModelConvertersContainer.Config(
+        converters=[MXFP8Converter.Config(fqns=["attention", "feed_forward"], cache_weight_casts=True)]
+    ).build(parallel_dims=None, model_compile_enabled=False)
+    box.convert(model)
+    assert sum(isinstance(p, MXFP8TrainingWeight) for p in model.parameters()) == 14
+    rng = np.random.default_rng(6)
+    prompts = [rng.integers(0, vocab, n).tolist() for n in (7, 20, 12)]
+    gens = [rng.integers(0, vocab, n).tolist() for n in (25, 9, 40)]
+    adv = torch.tensor([1.0, -0.5, 0.25])
+    with torch.no_grad():
+        ref = [token_log_probs(model(torch.tensor([p + g], device=device))[0, len(p) - 1:len(p) - 1 + len(g)],
+                               torch.tensor(g, device=device)) + 0.05 for p, g in zip(prompts, gens)]
+    total, metrics, lps = compute_policy_gradient_loss(model, gens, prompts, adv, ref)
+    o_total, o_m = mo.policy_gradient_loss([l.detach().cpu().numpy() for l in lps], [r.cpu().numpy() for r in ref],
+                                           adv.numpy())
+    assert math.isclose(total.item(), o_total, rel_tol=1e-4, abs_tol=1e-5)
+    assert math.isclose(metrics["kl_div"], o_m["kl_div"], rel_tol=1e-3, abs_tol=1e-6)
+    total.backward()
+    before = {n: p.detach().clone() for n, p in model.named_parameters()}
+    with torch.no_grad():
+        for p in model.parameters():
+            assert p.grad is not None and torch.isfinite(p.grad).all()
+            p.add_(p.grad, alpha=-0.5)
+    box.post_optimizer_hook(model)
+    payload = export_mxfp8_state_dict(model)
+    restored = load_mxfp8_state_dict(payload)
+    n_mx = 0
+    for name, p in model.named_parameters():
+        plain = p.detach().as_subclass(torch.Tensor)
+        if isinstance(p, MXFP8TrainingWeight):
+            n_mx += 1
+            assert not torch.equal(plain, before[name])                 # the step moved it
+            q = ops.to_mx_dim0(plain, "rceil", ops.MX_SCALES_ROWMAJOR)   # cast of the NEW weight
+            assert torch.equal(payload[name]["codes"], q.codes) and torch.equal(payload[name]["scales"], q.scales)
+            assert torch.equal(restored[name], ops.mx_dequant(q))
+        else:
+            assert torch.equal(restored[name], plain)
+    assert n_mx == 14
