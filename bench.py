@@ -36,6 +36,10 @@ PEAK_HBM_GBPS = 8000.0
 # known-size elementwise kernel (profiles/gemm_nt32_kernel_and_cast_tile_kernel__ffn_fwd_bwd_M16384__hbm_traffic_pmc.txt).  Counters cannot
 # be read from inside this process, so the figure is carried here and re-measured when the kernel
 # changes.
+# Share of the GPU's active cycles in which the matrix pipes are busy under the GEMM kernel:
+# rocprofv3's MfmaUtil (SQ_VALU_MFMA_BUSY_CYCLES / (GRBM_GUI_ACTIVE x SIMDs)), measured offline
+# on the same command (profiles/gemm_nt32_kernel__ffn_fwd_bwd_M16384__mfma_utilisation_pmc.txt).
+GEMM_MFMA_UTIL_ROCPROF = 0.725
 GEMM_TRAFFIC_BYTES_PER_LAUNCH = 1813553618
 
 
@@ -653,6 +657,9 @@ def main():
             "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH,
             "traffic_note": "bytes per launch between L2 and fabric (rocprofv3 FETCH_SIZE + WRITE_SIZE, offline); "
                             "operands and output once would be 488.5e6",
+            "mfma_util_rocprof": GEMM_MFMA_UTIL_ROCPROF,
+            "mfma_util_note": "matrix-pipe busy cycles / active cycles (rocprofv3 MfmaUtil, offline); frac = this x "
+                              "shader clock under the kernel (about 1.75 GHz) / 2.4 GHz",
             "launches_timed": n_gemm,
             "avg_launch_ms": round(gemm_ms, 4),
         },
