@@ -291,7 +291,7 @@ def test_grouped_experts_fused_block_matches_separate_ops(device, pad, align, di
         for got, want in zip(*outs):
             assert torch.equal(got, want)
         assert not torch.isnan(outs[0][0]).any() and outs[0][2].abs().sum() > 0
-        from torchtitan_amd.mx_tensor import grouped_feed_forward_fusable as fusable
+        from torchtitan_amd.mx_blocks import grouped_feed_forward_fusable as fusable
         assert fusable(x, blocks[0].w1, blocks[0].w2, blocks[0].w3)
         assert not fusable(x, blocks[1].w1, blocks[1].w2, blocks[1].w3)
     finally:

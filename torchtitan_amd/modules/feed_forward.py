@@ -4,7 +4,7 @@ from dataclasses import dataclass, field
 import torch
 import torch.nn.functional as F
 
-from ..mx_tensor import feed_forward_fusable, mx_feed_forward, mx_swiglu_linear, swiglu_fusable
+from ..mx_blocks import feed_forward_fusable, mx_feed_forward, mx_swiglu_linear, swiglu_fusable
 from ..protocols import Module
 from .linear import Linear
 

@@ -17,7 +17,7 @@ from torch import nn
 
 from dataclasses import dataclass
 
-from ..mx_tensor import grouped_feed_forward_fusable, mx_grouped_feed_forward, mx_routed_experts
+from ..mx_blocks import grouped_feed_forward_fusable, mx_grouped_feed_forward, mx_routed_experts
 from ..protocols import Module
 from .feed_forward import FeedForward
 from .linear import Linear

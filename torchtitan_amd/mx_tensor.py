@@ -259,188 +259,6 @@ def mx_linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, 
     return y
 
 
-# ----------------------------------------------------------------------------- SwiGLU + linear
-class _MXSwiGLULinear(torch.autograd.Function):
-    """y = (silu(h1) * h3) W^T with the gate formed inside the cast kernel: g is never written
-    to memory in forward and only its column-wise MXFP8 form is kept for wgrad.  Backward
-    returns the gradients the unfused bf16 ops would (silu and the products rounded to bf16
-    tensor by tensor, torchtitan/models/common/feed_forward.py:61-62 under autograd)."""
-
-    @staticmethod
-    def forward(ctx, h1, h3, weight, cfg: MXFP8Config):
-        mode = cfg.scale_mode
-        H, N = h1.shape[-1], weight.shape[0]
-        a, b = h1.reshape(-1, H), h3.reshape(-1, H)
-        w = weight if weight.dtype == torch.bfloat16 else weight.to(torch.bfloat16)
-        gq0, gq1, _ = ops.swiglu_to_mx_dim0_dim1(a, b, mode, MX_SCALES_MFMA)
-        need_dh = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
-        wq0, wq1 = _cast_weight(weight, mode, need_dh, cfg)
-        y = ops.mx_gemm_nt(gq0, wq0)
-        ctx.cfg, ctx.w_dtype, ctx.have_wq1 = cfg, weight.dtype, wq1 is not None
-        saved = [h1, h3]
-        if ctx.needs_input_grad[2]:
-            saved += [gq1.codes, gq1.scales]
-        if need_dh:
-            saved += [wq1.codes, wq1.scales] if wq1 is not None else [w]
-        ctx.save_for_backward(*saved)
-        return y.view(*h1.shape[:-1], N)
-
-    @staticmethod
-    def backward(ctx, dy):
-        mode = ctx.cfg.scale_mode
-        need_dh = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
-        need_dw = ctx.needs_input_grad[2]
-        saved = list(ctx.saved_tensors)
-        h1, h3 = saved.pop(0), saved.pop(0)
-        N = dy.shape[-1]
-        dy2 = dy.reshape(-1, N)
-        if dy2.dtype != torch.bfloat16:
-            dy2 = dy2.to(torch.bfloat16)
-        dy2 = dy2.contiguous()
-        gq1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA) if need_dw else None
-        wq1 = None
-        if need_dh:
-            if ctx.have_wq1:
-                wq1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
-            else:
-                wq1 = _cast_cols_padded(saved.pop(0), mode)
-        if need_dh and need_dw and N % ops.BLOCK == 0:
-            dyq0, dyq1 = ops.to_mx_dim0_dim1(dy2, mode, MX_SCALES_MFMA)
-        else:
-            dyq0 = _cast_rows_padded(dy2, mode) if need_dh else None
-            dyq1 = ops.to_mx_dim1(dy2, mode, MX_SCALES_MFMA) if need_dw else None
-        dh1 = dh3 = dw = None
-        if need_dh:
-            dg = ops.mx_gemm_nt(dyq0, wq1).view(h1.shape)
-            if ctx.needs_input_grad[1]:
-                dh3 = dg * F.silu(h1)
-            if ctx.needs_input_grad[0]:
-                dh1 = torch.ops.aten.silu_backward(dg * h3, h1)
-        if need_dw:
-            dw = ops.mx_gemm_nt(dyq1, gq1)
-            if dw.dtype != ctx.w_dtype:
-                dw = dw.to(ctx.w_dtype)
-        return dh1, dh3, dw, None
-
-
-def swiglu_fusable(h1: torch.Tensor, h3: torch.Tensor, weight: torch.Tensor) -> bool:
-    """The fused gate + cast needs bf16 row-contiguous inputs of one shape with 32-aligned token
-    and hidden counts (what a converted SwiGLU block produces) and a converted weight."""
-    if not isinstance(weight, MXFP8TrainingWeight) or not weight.mx_config.fuse_swiglu_cast:
-        return False
-    if h1.dtype != torch.bfloat16 or h3.dtype != torch.bfloat16 or h1.shape != h3.shape:
-        return False
-    H = h1.shape[-1]
-    return (h1.is_contiguous() and h3.is_contiguous() and h1.is_cuda and H % ops.BLOCK == 0
-            and h1.numel() // max(H, 1) % ops.BLOCK == 0 and h1.numel() > 0)
-
-
-def mx_swiglu_linear(h1: torch.Tensor, h3: torch.Tensor, weight: torch.Tensor,
-                     bias: torch.Tensor | None = None):
-    """``F.linear(F.silu(h1) * h3, weight, bias)`` for a converted weight, with the gate computed
-    inside the MXFP8 cast.  Callers check `swiglu_fusable` first."""
-    y = _MXSwiGLULinear.apply(h1, h3, _unwrap(weight), weight.mx_config)
-    if bias is not None:
-        y = y + _unwrap(bias).to(y.dtype)
-    return y
-
-
-# ----------------------------------------------------------------------------- whole SwiGLU block
-def _bf16(t: torch.Tensor) -> torch.Tensor:
-    return t if t.dtype == torch.bfloat16 else t.to(torch.bfloat16)
-
-
-class _MXFeedForward(torch.autograd.Function):
-    """y = (silu(x W1^T) * (x W3^T)) W2^T with every elementwise step folded into a cast kernel.
-
-    Forward: one cast of x, the gate inside the cast that feeds W2.  Backward: the gate's
-    gradients inside the cast that feeds the dgrad / wgrad GEMMs of W1 and W3.  Neither g nor
-    dh1 / dh3 is written to memory; kept for backward are h1, h3 and the column-wise MXFP8 forms
-    of x, g and the weights.  Results are bit-identical to the three converted linears around
-    bf16 ``F.silu`` and ``*`` (torchtitan/models/common/feed_forward.py:61-62)."""
-
-    @staticmethod
-    def forward(ctx, x, w1, w2, w3, cfg: MXFP8Config):
-        mode = cfg.scale_mode
-        D, H = x.shape[-1], w1.shape[0]
-        x2 = x.reshape(-1, D)
-        need_dx = ctx.needs_input_grad[0]
-        need_dw = any(ctx.needs_input_grad[1:4])
-        xq0, xq1 = _cast_activation(x2, x, mode, need_cols=need_dw)
-        w1q0, w1q1 = _cast_weight(w1, mode, need_dx, cfg)
-        w3q0, w3q1 = _cast_weight(w3, mode, need_dx, cfg)
-        w2q0, w2q1 = _cast_weight(w2, mode, need_dx or need_dw, cfg)
-        h1 = ops.mx_gemm_nt(xq0, w1q0)
-        h3 = ops.mx_gemm_nt(xq0, w3q0)
-        gq0, gq1, _ = ops.swiglu_to_mx_dim0_dim1(h1, h3, mode, MX_SCALES_MFMA)
-        y = ops.mx_gemm_nt(gq0, w2q0)
-        ctx.cfg, ctx.x_shape = cfg, x.shape
-        ctx.w_dtypes = (w1.dtype, w2.dtype, w3.dtype)
-        ctx.need_dx, ctx.need_dw = need_dx, need_dw
-        saved = []
-        if need_dx or need_dw:
-            saved += [h1, h3, w2q1.codes, w2q1.scales]
-        if need_dw:
-            saved += [xq1.codes, xq1.scales, gq1.codes, gq1.scales]
-        if need_dx:
-            saved += [w1q1.codes, w1q1.scales, w3q1.codes, w3q1.scales]
-        ctx.save_for_backward(*saved)
-        return y.view(*x.shape[:-1], w2.shape[0])
-
-    @staticmethod
-    def backward(ctx, dy):
-        mode = ctx.cfg.scale_mode
-        saved = list(ctx.saved_tensors)
-        take = lambda: MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
-        h1, h3 = saved.pop(0), saved.pop(0)
-        w2q1 = take()
-        dy2 = _bf16(dy.reshape(-1, dy.shape[-1])).contiguous()
-        if ctx.needs_input_grad[2]:
-            dyq0, dyq1 = ops.to_mx_dim0_dim1(dy2, mode, MX_SCALES_MFMA)
-        else:
-            dyq0, dyq1 = ops.to_mx_dim0(dy2, mode, MX_SCALES_MFMA), None
-        dg = ops.mx_gemm_nt(dyq0, w2q1)
-        (da0, da1), (db0, db1), _ = ops.swiglu_bwd_to_mx_dim0_dim1(dg, h1, h3, mode, MX_SCALES_MFMA)
-        dx = dw1 = dw2 = dw3 = None
-        if ctx.need_dw:
-            xq1, gq1 = take(), take()
-            cast_back = lambda g, dt: g if g.dtype == dt else g.to(dt)
-            if ctx.needs_input_grad[1]:
-                dw1 = cast_back(ops.mx_gemm_nt(da1, xq1), ctx.w_dtypes[0])
-            if ctx.needs_input_grad[2]:
-                dw2 = cast_back(ops.mx_gemm_nt(dyq1, gq1), ctx.w_dtypes[1])
-            if ctx.needs_input_grad[3]:
-                dw3 = cast_back(ops.mx_gemm_nt(db1, xq1), ctx.w_dtypes[2])
-        if ctx.need_dx:
-            w1q1, w3q1 = take(), take()
-            dx = (ops.mx_gemm_nt(da0, w1q1) + ops.mx_gemm_nt(db0, w3q1)).view(ctx.x_shape)
-        return dx, dw1, dw2, dw3, None
-
-
-def feed_forward_fusable(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, w3: torch.Tensor) -> bool:
-    """The whole-block function needs all three weights converted with gate fusion on, a bf16
-    GPU activation and 32-aligned token, model and hidden sizes."""
-    ws = (w1, w2, w3)
-    if not all(isinstance(w, MXFP8TrainingWeight) and w.mx_config.fuse_swiglu_cast for w in ws):
-        return False
-    if w1.mx_config.scale_mode != w2.mx_config.scale_mode or w1.mx_config.scale_mode != w3.mx_config.scale_mode:
-        return False
-    if x.dtype != torch.bfloat16 or not x.is_cuda or x.numel() == 0 or w1.shape != w3.shape:
-        return False
-    D, H = x.shape[-1], w1.shape[0]
-    return D % ops.BLOCK == 0 and H % ops.BLOCK == 0 and (x.numel() // D) % ops.BLOCK == 0
-
-
-def mx_feed_forward(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, w3: torch.Tensor,
-                    bias2: torch.Tensor | None = None):
-    """``F.linear(F.silu(F.linear(x, w1)) * F.linear(x, w3), w2, bias2)`` for converted weights.
-    Callers check `feed_forward_fusable` first."""
-    y = _MXFeedForward.apply(x, _unwrap(w1), _unwrap(w2), _unwrap(w3), w2.mx_config)
-    if bias2 is not None:
-        y = y + _unwrap(bias2).to(y.dtype)
-    return y
-
-
 # ----------------------------------------------------------------------------- grouped GEMM
 def _pad_plan(offs: torch.Tensor, T: int, align: int = 32):
     """Device-side plan that moves rows of variable-size groups into `align`-aligned groups.
@@ -559,230 +377,6 @@ class _MXGroupedMM(torch.autograd.Function):
             if dw.dtype != ctx.dtypes[1]:
                 dw = dw.to(ctx.dtypes[1])
         return dx, dw, None, None
-
-
-class _MXGroupedFeedForward(torch.autograd.Function):
-    """The expert block ``grouped_mm(silu(grouped_mm(x, w1)) * grouped_mm(x, w3), w2)`` as one
-    function (torchtitan/models/common/moe/moe.py:59-76): tokens are moved into aligned groups
-    once instead of once per GEMM, x is cast once for w1 and w3, and the gate and its backward
-    run inside the cast kernels as in `_MXFeedForward`.  Bit-identical to the three converted
-    grouped GEMMs around bf16 ``F.silu`` and ``*``."""
-
-    @staticmethod
-    def forward(ctx, x, w1, w2, w3, offs, cfg: MXFP8Config):
-        mode = cfg.scale_mode
-        T, D = x.shape
-        G, H, _ = w1.shape
-        xb = _bf16(x)
-        pad = cfg.pad_token_groups_for_grouped_mm
-        fast = D % 128 == 0 and H % 128 == 0 and G <= 638  # 128-row groups: persistent kernel
-        order = MX_SCALES_MFMA if fast else MX_SCALES_ROWMAJOR
-        plan = perm = back = None
-        if pad or fast:
-            plan = _pad_plan(offs, T, 128 if fast else ops.BLOCK)
-            perm, offs_p, back = plan
-        else:
-            offs_p = offs
-            if T % ops.BLOCK:
-                raise ValueError("without padding the token dimension must be a multiple of 32")
-        xb = xb.contiguous()
-        need_dx = ctx.needs_input_grad[0]
-        need_dw = any(ctx.needs_input_grad[1:4])
-        xq0, xq1 = _cast_into_groups(xb, perm, mode, order, need_dw)
-        w1q0, w1q1 = _cast_weight(w1, mode, need_dx, cfg)
-        w3q0, w3q1 = _cast_weight(w3, mode, need_dx, cfg)
-        w2q0, w2q1 = _cast_weight(w2, mode, need_dx or need_dw, cfg)
-        h1 = ops.mx_grouped_gemm_2d3d(xq0, w1q0, offs_p)
-        h3 = ops.mx_grouped_gemm_2d3d(xq0, w3q0, offs_p)
-        gq0, gq1, _ = ops.swiglu_to_mx_dim0_dim1(h1, h3, mode, order)
-        y = _grouped_2d3d_padded(gq0, w2q0, offs_p, back)
-        ctx.cfg, ctx.order, ctx.padded, ctx.D = cfg, order, plan is not None, D
-        ctx.dtypes = (x.dtype, w1.dtype, w2.dtype, w3.dtype)
-        ctx.need_dx, ctx.need_dw = need_dx, need_dw
-        saved = [offs_p]
-        if plan is not None:
-            saved += [plan[0], plan[2]]
-        if need_dx or need_dw:
-            saved += [h1, h3, w2q1.codes, w2q1.scales]
-        if need_dw:
-            saved += [xq1.codes, xq1.scales, gq1.codes, gq1.scales]
-        if need_dx:
-            saved += [w1q1.codes, w1q1.scales, w3q1.codes, w3q1.scales]
-        ctx.save_for_backward(*saved)
-        return y
-
-    @staticmethod
-    def backward(ctx, dy):
-        mode, order = ctx.cfg.scale_mode, ctx.order
-        saved = list(ctx.saved_tensors)
-        offs_p = saved.pop(0)
-        dyb = _bf16(dy).contiguous()
-        perm = back = None
-        if ctx.padded:
-            perm, back = saved.pop(0), saved.pop(0)
-        h1, h3 = saved.pop(0), saved.pop(0)
-        w2q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
-        dyq0, dyq1 = _cast_into_groups(dyb, perm, mode, order, ctx.needs_input_grad[2])
-        dg = ops.mx_grouped_gemm_2d3d(dyq0, w2q1, offs_p)
-        (da0, da1), (db0, db1), _ = ops.swiglu_bwd_to_mx_dim0_dim1(dg, h1, h3, mode, order)
-        dx = dw1 = dw2 = dw3 = None
-        cast_back = lambda g, dt: g if g.dtype == dt else g.to(dt)
-        if ctx.need_dw:
-            xq1 = MXData(saved.pop(0), saved.pop(0), order)
-            gq1 = MXData(saved.pop(0), saved.pop(0), order)
-            if ctx.needs_input_grad[1]:
-                dw1 = cast_back(ops.mx_grouped_gemm_2d2d(da1, xq1, offs_p), ctx.dtypes[1])
-            if ctx.needs_input_grad[2]:
-                dw2 = cast_back(ops.mx_grouped_gemm_2d2d(dyq1, gq1, offs_p), ctx.dtypes[2])
-            if ctx.needs_input_grad[3]:
-                dw3 = cast_back(ops.mx_grouped_gemm_2d2d(db1, xq1, offs_p), ctx.dtypes[3])
-        if ctx.need_dx:
-            w1q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
-            w3q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
-            dx = _grouped_2d3d_padded(da0, w1q1, offs_p, back) + _grouped_2d3d_padded(db0, w3q1, offs_p, back)
-            dx = cast_back(dx, ctx.dtypes[0])
-        return dx, dw1, dw2, dw3, None, None
-
-
-def grouped_feed_forward_fusable(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
-                                 w3: torch.Tensor) -> bool:
-    """All three expert parameters converted with gate fusion on, a 2-D GPU activation, model
-    and hidden sizes multiples of 32."""
-    ws = (w1, w2, w3)
-    if not all(isinstance(w, MXFP8TrainingWeight) and w.mx_config.fuse_swiglu_cast and w.dim() == 3 for w in ws):
-        return False
-    if x.dim() != 2 or not x.is_cuda or x.numel() == 0 or w1.shape != w3.shape:
-        return False
-    if w1.mx_config.scale_mode != w2.mx_config.scale_mode or w1.mx_config.scale_mode != w3.mx_config.scale_mode:
-        return False
-    return x.shape[-1] % ops.BLOCK == 0 and w1.shape[1] % ops.BLOCK == 0
-
-
-def mx_grouped_feed_forward(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, w3: torch.Tensor,
-                            offs: torch.Tensor):
-    """The SwiGLU expert block for converted 3-D parameters w1, w3 [G, hidden, dim] and
-    w2 [G, dim, hidden]; offs = inclusive cumulative group sizes.  Returns bf16.
-    Callers check `grouped_feed_forward_fusable` first."""
-    return _MXGroupedFeedForward.apply(x, _unwrap(w1), _unwrap(w2), _unwrap(w3), offs.to(torch.int32),
-                                       w2.mx_config)
-
-
-class _MXRoutedExperts(torch.autograd.Function):
-    """The routed half of an MoE layer as one function (torchtitan/models/common/moe/moe.py:519-555):
-
-        out[t] = sum_j  c[t, j] * experts(x[t] * r[t, j])        j over the token's top_k experts
-
-    with r = scores, c = 1 when the scores multiply the expert inputs (`score_before_experts`)
-    and r = 1, c = scores otherwise.  The token gather, the score multiply and the move into
-    aligned expert groups happen inside the cast kernel (no routed copy of x exists); the
-    un-sort and the weighted sum over top_k are one kernel over the padded expert outputs; in
-    backward the same two kernels swap roles and the score gradients are row dot products."""
-
-    @staticmethod
-    def forward(ctx, x, top_scores, w1, w2, w3, tok_sorted, counts, score_before: bool, cfg: MXFP8Config):
-        mode = cfg.scale_mode
-        T, D = x.shape
-        k = top_scores.shape[1]
-        R = T * k
-        G, H, _ = w1.shape
-        xb = _bf16(x).contiguous()
-        scores = top_scores.float().contiguous()
-        fast = D % 128 == 0 and H % 128 == 0 and G <= 638
-        order = MX_SCALES_MFMA if fast else MX_SCALES_ROWMAJOR
-        offs = torch.cumsum(counts, dim=0, dtype=torch.int32)
-        perm, offs_p, back = _pad_plan(offs, R, 128 if fast else ops.BLOCK)
-        slot = tok_sorted[perm.clamp_min(0)]              # (token, j) pair of every padded row
-        src_row = torch.where(perm >= 0, slot // k, -1)   # its token, -1 for padding
-        row_score = scores.view(-1)[slot]
-        pos = torch.empty(R, dtype=torch.int64, device=x.device)
-        pos[tok_sorted] = back                            # padded row of pair (t, j)
-        pos = pos.view(T, k)
-        need_dx = ctx.needs_input_grad[0]
-        need_ds = ctx.needs_input_grad[1]
-        need_dw = any(ctx.needs_input_grad[2:5])
-        xq0, xq1 = ops.to_mx_rows_gathered(xb, src_row, mode, order, need_dw,
-                                           row_score if score_before else None)
-        need_dg = need_dx or need_ds or need_dw
-        w1q0, w1q1 = _cast_weight(w1, mode, need_dx or need_ds, cfg)
-        w3q0, w3q1 = _cast_weight(w3, mode, need_dx or need_ds, cfg)
-        w2q0, w2q1 = _cast_weight(w2, mode, need_dg, cfg)
-        h1 = ops.mx_grouped_gemm_2d3d(xq0, w1q0, offs_p)
-        h3 = ops.mx_grouped_gemm_2d3d(xq0, w3q0, offs_p)
-        gq0, gq1, _ = ops.swiglu_to_mx_dim0_dim1(h1, h3, mode, order)
-        yp = ops.mx_grouped_gemm_2d3d(gq0, w2q0, offs_p)
-        out = ops.moe_combine(yp, pos, None if score_before else scores)
-        ctx.cfg, ctx.order, ctx.score_before = cfg, order, score_before
-        ctx.dtypes = (x.dtype, top_scores.dtype, w1.dtype, w2.dtype, w3.dtype)
-        ctx.flags = (need_dx, need_ds, need_dw)
-        saved = [offs_p, src_row, row_score, pos, scores]
-        if need_dg:
-            saved += [h1, h3, w2q1.codes, w2q1.scales]
-        if need_dw:
-            saved += [xq1.codes, xq1.scales, gq1.codes, gq1.scales]
-        if need_dx or need_ds:
-            saved += [w1q1.codes, w1q1.scales, w3q1.codes, w3q1.scales]
-        if need_ds:
-            saved += [xb if score_before else yp]
-        ctx.save_for_backward(*saved)
-        return out
-
-    @staticmethod
-    def backward(ctx, dout):
-        mode, order, score_before = ctx.cfg.scale_mode, ctx.order, ctx.score_before
-        need_dx, need_ds, need_dw = ctx.flags
-        saved = list(ctx.saved_tensors)
-        offs_p, src_row, row_score, pos, scores = (saved.pop(0) for _ in range(5))
-        T, k = pos.shape
-        dob = _bf16(dout).contiguous()
-        h1, h3 = saved.pop(0), saved.pop(0)
-        w2q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
-        # gradient of the padded expert outputs: dout of the row's token (times its score)
-        dyq0, dyq1 = ops.to_mx_rows_gathered(dob, src_row, mode, order, ctx.needs_input_grad[3],
-                                             None if score_before else row_score)
-        dg = ops.mx_grouped_gemm_2d3d(dyq0, w2q1, offs_p)
-        (da0, da1), (db0, db1), _ = ops.swiglu_bwd_to_mx_dim0_dim1(dg, h1, h3, mode, order)
-        dx = ds = dw1 = dw2 = dw3 = None
-        cast_back = lambda g, dt: g if g.dtype == dt else g.to(dt)
-        if need_dw:
-            xq1 = MXData(saved.pop(0), saved.pop(0), order)
-            gq1 = MXData(saved.pop(0), saved.pop(0), order)
-            if ctx.needs_input_grad[2]:
-                dw1 = cast_back(ops.mx_grouped_gemm_2d2d(da1, xq1, offs_p), ctx.dtypes[2])
-            if ctx.needs_input_grad[3]:
-                dw2 = cast_back(ops.mx_grouped_gemm_2d2d(dyq1, gq1, offs_p), ctx.dtypes[3])
-            if ctx.needs_input_grad[4]:
-                dw3 = cast_back(ops.mx_grouped_gemm_2d2d(db1, xq1, offs_p), ctx.dtypes[4])
-        if need_dx or need_ds:
-            w1q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
-            w3q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
-            need_dxp = need_dx or (need_ds and score_before)
-            if need_dxp:
-                # gradient of the (scaled) routed inputs, padded layout: the two halves from w1
-                # and w3; their bf16 sum is formed inside the kernels that consume it
-                dxp1 = ops.mx_grouped_gemm_2d3d(da0, w1q1, offs_p)
-                dxp3 = ops.mx_grouped_gemm_2d3d(db0, w3q1, offs_p)
-            if need_dx:
-                dx = cast_back(ops.moe_combine(dxp1, pos, scores if score_before else None, dxp3), ctx.dtypes[0])
-            if need_ds:
-                other = saved.pop(0)  # x (scores in front of the experts) or the expert outputs
-                token = torch.arange(T * k, device=pos.device, dtype=torch.int64).div_(k, rounding_mode="floor")
-                if score_before:
-                    ds = ops.moe_row_dot(dxp1, pos.view(-1), other, token, dxp3)
-                else:
-                    ds = ops.moe_row_dot(other, pos.view(-1), dob, token)
-                ds = cast_back(ds.view(T, k), ctx.dtypes[1])
-        return dx, ds, dw1, dw2, dw3, None, None, None, None
-
-
-def mx_routed_experts(x: torch.Tensor, top_scores: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
-                      w3: torch.Tensor, token_indices_experts_sorted: torch.Tensor,
-                      num_tokens_per_expert: torch.Tensor, score_before_experts: bool) -> torch.Tensor:
-    """Gather, score, run the SwiGLU experts and combine, for converted expert parameters.
-    x [T, dim] bf16, top_scores [T, top_k]; the index tensor is the stable argsort of the
-    flattened expert choices.  Callers check `grouped_feed_forward_fusable` first."""
-    return _MXRoutedExperts.apply(x, top_scores, _unwrap(w1), _unwrap(w2), _unwrap(w3),
-                                  token_indices_experts_sorted, num_tokens_per_expert,
-                                  bool(score_before_experts), w2.mx_config)
 
 
 def _cast_w_rows(w: torch.Tensor, mode: str) -> MXData:
