@@ -101,6 +101,21 @@ int mx_cast_rows_gathered(const void* x, const int64_t* row_index, const float* 
                           uint8_t* codes, uint8_t* scales, uint8_t* codes_t, uint8_t* scales_t,
                           int scale_mode, int scale_order, void* stream);
 
+/* Routing plan of an MoE layer, one launch, no host round trip.  counts int32 [experts] (pairs
+ * per expert), order int64 [pairs] (the (token, choice) pair = token * top_k + choice at every
+ * position of the expert-sorted order: `token_indices_experts_sorted` of
+ * torchtitan/models/common/moe/moe.py:355-362), scores float32 [pairs] by pair (may be NULL).
+ * Every expert's group is padded to a multiple of `alignment` rows (at least one multiple, as in
+ * moe/kernels.py:183-191).  Outputs: m_offsets int32 [experts] inclusive padded group ends;
+ * src_row int64 [max_len] token of every padded row, -1 for padding and for rows behind the last
+ * group; row_score float32 [max_len] that pair's score (0 for padding); pos int64 [pairs] padded
+ * row of every pair (entries of pairs that no count covers are left untouched).
+ * max_len >= sum of the padded sizes is the caller's static bound. */
+int mx_moe_route_plan(const int32_t* counts, int64_t experts, const int64_t* order,
+                      const float* scores, int64_t pairs, int64_t top_k, int64_t max_len,
+                      int64_t alignment, int32_t* m_offsets, int64_t* src_row, float* row_score,
+                      int64_t* pos, void* stream);
+
 /* Combine of the routed expert outputs: out[t, :] = sum_j weights[t, j] * y[pos[t, j], :] for
  * j = 0 .. top_k-1 in that order, in float32 (product and sum rounded separately), result
  * rounded to bf16; weights == NULL gives the plain sum.  y: bf16 [y_rows, cols] (row stride

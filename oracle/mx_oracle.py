@@ -40,6 +40,8 @@ Pinning status (what fixes each function independently of its own formula):
                                         float32 evaluation is PARITY UNPINNED (see its docstring)
   swiglu_backward_bf16       pinned  -- closed form vs a central difference and torch's CPU op;
                                         last bf16 ulp of da PARITY UNPINNED (see its docstring)
+  moe_route_plan             pinned  -- composition of generate_permute_indices (pinned) with index
+                                        arithmetic; checked against torch indexing in the tests
   gather_rows                pinned  -- index semantics vs torch indexing; score product exact
                                         before its bf16 rounding (torch CPU ops)
   moe_combine                pinned  -- vs an exact float64 sum (within one bf16 step) and torch's
@@ -410,6 +412,28 @@ def swiglu_backward_bf16(dg_bits: np.ndarray, a_bits: np.ndarray, b_bits: np.nda
         s = 1.0 / (1.0 + e)
         da = t * s * (1.0 + a * (1.0 - s))
         return f32_to_bf16_bits(da.astype(np.float32)), db
+
+
+def moe_route_plan(counts: np.ndarray, order: np.ndarray, scores: np.ndarray | None, top_k: int,
+                   alignment: int):
+    """Aligned group layout of an MoE layer's routed pairs, composed from the padding rule of
+    `generate_permute_indices` (moe/kernels.py:145-218) and the expert-sorted pair order
+    (moe.py:355-362): (padded inclusive ends, token per padded row or -1, score per padded row,
+    padded row per pair)."""
+    E, R = len(counts), len(order)
+    max_len = round_up(R + alignment * E, alignment)
+    perm, _, m_offsets = generate_permute_indices(np.asarray(counts), E, 1, max_len, alignment)
+    src_row = np.full(max_len, -1, dtype=np.int64)
+    row_score = np.zeros(max_len, dtype=np.float32)
+    pos = np.full(R, -1, dtype=np.int64)
+    for p, i in enumerate(perm):
+        if i >= 0:
+            pair = order[i]
+            src_row[p] = pair // top_k
+            if scores is not None:
+                row_score[p] = scores[pair]
+            pos[pair] = p
+    return m_offsets, src_row, row_score, pos
 
 
 def gather_rows(x_bits: np.ndarray, row_index: np.ndarray, row_scale: np.ndarray | None = None) -> np.ndarray:

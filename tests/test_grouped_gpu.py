@@ -251,3 +251,30 @@ def test_pad_then_grouped_gemm_moe_like(device):
     xp_bits = np.vstack((x_bits, np.zeros((1, dim), np.uint16)))[rp]
     ref = mo.grouped_fwd(xp_bits, w_bits, ro, mo.RCEIL)
     assert rel_l2(_f32(bits_of(y)), _f32(ref)) <= TOL
+
+
+@pytest.mark.parametrize("experts,top_k,tokens,align", [(4, 2, 50, 32), (16, 4, 300, 128), (128, 8, 2048, 128)])
+def test_moe_route_plan_matches_the_oracle(device, experts, top_k, tokens, align):
+    """One-launch routing plan (padded group ends, token and score of every padded row, padded
+    row of every pair) against the oracle's composition of the padding rule with the sorted
+    order; integer outputs and copied scores: exact.  One expert left without tokens."""
+    rng = np.random.default_rng(experts + tokens)
+    choice = rng.integers(0, experts - 1, (tokens, top_k))     # the last expert stays empty
+    order = np.argsort(choice.reshape(-1), kind="stable").astype(np.int64)
+    counts = np.bincount(choice.reshape(-1), minlength=experts).astype(np.int32)
+    scores = rng.random(tokens * top_k).astype(np.float32)
+    offs, src_row, row_score, pos = ops.moe_route_plan(
+        torch.from_numpy(counts).to(device), torch.from_numpy(order).to(device),
+        torch.from_numpy(scores).to(device), top_k, align)
+    o_offs, o_src, o_score, o_pos = mo.moe_route_plan(counts, order, scores, top_k, align)
+    assert np.array_equal(offs.cpu().numpy(), o_offs)
+    assert np.array_equal(src_row.cpu().numpy(), o_src)
+    assert np.array_equal(row_score.cpu().numpy(), o_score)
+    assert np.array_equal(pos.cpu().numpy(), o_pos)
+    # the plan is a bijection between pairs and non-padding rows, grouped by expert
+    valid = o_src >= 0
+    assert valid.sum() == tokens * top_k and np.array_equal(np.sort(o_pos), np.nonzero(valid)[0])
+    ends = np.concatenate(([0], o_offs))
+    for e in range(experts):
+        rows = np.nonzero(valid[ends[e]:ends[e + 1]])[0]
+        assert len(rows) == counts[e] and (len(rows) == 0 or rows[-1] == len(rows) - 1)

@@ -33,6 +33,7 @@ SIGNATURES = {
     "mx_dequant": (c_int, [_P, _P, _I, _I, c_int, _P, _I, _P]),
     "mx_token_logprob_fwd": (c_int, [_P, _I, _I, _I, _P, _P, _P, _P]),
     "mx_token_logprob_bwd": (c_int, [_P, _I, _I, _I, _P, _P, _P, _P, _I, _P]),
+    "mx_moe_route_plan": (c_int, [_P, _I, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P]),
     "mx_moe_combine": (c_int, [_P, _P, _I, _I, _P, _P, _I, _I, _I, _P, _I, _P]),
     "mx_moe_row_dot": (c_int, [_P, _P, _I, _I, _P, _P, _I, _I, _P, _I, _I, _P, _P]),
     "mx_swiglu_cast_dim0_dim1": (c_int, [_P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, c_int, c_int, _P]),

@@ -326,13 +326,9 @@ class _MXRoutedExperts(torch.autograd.Function):
         scores = top_scores.float().contiguous()
         fast = D % 128 == 0 and H % 128 == 0 and G <= 638
         order = MX_SCALES_MFMA if fast else MX_SCALES_ROWMAJOR
-        offs = torch.cumsum(counts, dim=0, dtype=torch.int32)
-        perm, offs_p, back = _pad_plan(offs, R, 128 if fast else ops.BLOCK)
-        slot = tok_sorted[perm.clamp_min(0)]              # (token, j) pair of every padded row
-        src_row = torch.where(perm >= 0, slot // k, -1)   # its token, -1 for padding
-        row_score = scores.view(-1)[slot]
-        pos = torch.empty(R, dtype=torch.int64, device=x.device)
-        pos[tok_sorted] = back                            # padded row of pair (t, j)
+        # aligned group layout and the maps between padded rows, tokens and (token, j) pairs
+        offs_p, src_row, row_score, pos = ops.moe_route_plan(counts, tok_sorted, scores.view(-1), k,
+                                                             128 if fast else ops.BLOCK)
         pos = pos.view(T, k)
         need_dx = ctx.needs_input_grad[0]
         need_ds = ctx.needs_input_grad[1]

@@ -179,6 +179,35 @@ def to_mx_rows_gathered(x: torch.Tensor, row_index: torch.Tensor, mode="floor",
     return MXData(codes, scales, order), (MXData(codes_t, scales_t, order) if want_cols else None)
 
 
+def moe_route_plan(counts: torch.Tensor, order: torch.Tensor, scores: torch.Tensor | None, top_k: int,
+                   alignment: int):
+    """(padded inclusive group ends int32 [E], token of every padded row int64 [max_len] (-1 =
+    padding), score of every padded row float32 [max_len], padded row of every (token, choice)
+    pair int64 [pairs]) for tokens-per-expert `counts` and the expert-sorted pair order; the
+    padded length is the static bound round_up(pairs + alignment * E, alignment)."""
+    if not counts.is_cuda:
+        raise _lib.MXLibraryError("moe_route_plan runs on the GPU only")
+    dev = counts.device
+    c32 = counts.to(torch.int32).contiguous()
+    E, R = c32.numel(), order.numel()
+    if order.dtype != torch.int64 or order.device != dev:
+        raise TypeError("order must be int64 on the counts' device")
+    order = order.contiguous()
+    if scores is not None:
+        if scores.dtype != torch.float32 or scores.numel() != R or scores.device != dev:
+            raise TypeError("scores must be float32 with one entry per pair")
+        scores = scores.contiguous()
+    max_len = -(-(R + alignment * E) // alignment) * alignment
+    offs = torch.empty(E, dtype=torch.int32, device=dev)
+    src_row = torch.empty(max_len, dtype=torch.int64, device=dev)
+    row_score = torch.empty(max_len, dtype=torch.float32, device=dev)
+    pos = torch.full((R,), -1, dtype=torch.int64, device=dev)
+    _call("mx_moe_route_plan", "moe_route_plan", dev, _ptr(c32), E, _ptr(order),
+          _ptr(scores) if scores is not None else None, R, top_k, max_len, alignment, _ptr(offs),
+          _ptr(src_row), _ptr(row_score), _ptr(pos), _stream(counts))
+    return offs, src_row, row_score, pos
+
+
 def moe_combine(y: torch.Tensor, pos: torch.Tensor, weights: torch.Tensor | None = None,
                 y2: torch.Tensor | None = None) -> torch.Tensor:
     """out[t] = sum_j weights[t, j] * y[pos[t, j]] (float32, j in order; plain sum without
