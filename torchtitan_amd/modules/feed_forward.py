@@ -1,4 +1,11 @@
-"""SwiGLU feed-forward ``w2(silu(w1 x) * w3 x)`` (torchtitan/models/common/feed_forward.py:18-67)."""
+"""SwiGLU feed-forward block ``w2(silu(w1 x) * w3 x)``.
+
+Mirror of the reference's shared block (torchtitan/models/common/feed_forward.py:18-67): the
+config carries the final hidden size, the model size arrives through ``build(dim=...)``, and the
+three projections are ``Linear`` modules named w1 (gate), w3 (up) and w2 (down) so that the
+converter's FQN filters and checkpoints line up.  When the converter has wrapped the weights,
+``forward`` hands the block to the fused MXFP8 functions instead of three separate linears.
+"""
 from dataclasses import dataclass, field
 
 import torch
@@ -11,8 +18,10 @@ from .linear import Linear
 
 def compute_ffn_hidden_dim(dim: int, *, multiple_of: int = 1,
                            ffn_dim_multiplier: float | None = None) -> int:
-    """2/3 * 4 * dim, optional multiplier, rounded up to `multiple_of` (Llama-3 8B: 14336)."""
-    hidden = int(2 * 4 * dim / 3)
+    """Hidden size of a Llama-style SwiGLU block: two thirds of 4 * dim, times the optional
+    multiplier, rounded up to a multiple of `multiple_of` (dim 4096, multiplier 1.3, multiple
+    1024 -> 14336)."""
+    hidden = int(8 * dim / 3)
     if ffn_dim_multiplier is not None:
         hidden = int(ffn_dim_multiplier * hidden)
     return -(-hidden // multiple_of) * multiple_of
@@ -23,26 +32,27 @@ class FeedForward(Module):
     class Config(Module.Config):
         hidden_dim: int
         linear_bias: bool = False
-        dim: int = field(init=False)
+        dim: int = field(init=False)  # supplied by build(dim=...)
 
     def __init__(self, config: Config):
         super().__init__()
-        lin = Linear.Config(bias=config.linear_bias)
-        self.w1 = lin.build(in_features=config.dim, out_features=config.hidden_dim)
-        self.w2 = lin.build(in_features=config.hidden_dim, out_features=config.dim)
-        self.w3 = lin.build(in_features=config.dim, out_features=config.hidden_dim)
+        make = Linear.Config(bias=config.linear_bias).build
+        up = dict(in_features=config.dim, out_features=config.hidden_dim)
+        self.w1 = make(**up)
+        self.w2 = make(in_features=config.hidden_dim, out_features=config.dim)
+        self.w3 = make(**up)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        if (self.w1.bias is None and self.w3.bias is None
-                and feed_forward_fusable(x, self.w1.weight, self.w2.weight, self.w3.weight)):
+        w1, w2, w3 = self.w1, self.w2, self.w3
+        if w1.bias is None and w3.bias is None and feed_forward_fusable(x, w1.weight, w2.weight, w3.weight):
             # all three converted: gate and its backward inside the MXFP8 cast kernels
-            return mx_feed_forward(x, self.w1.weight, self.w2.weight, self.w3.weight, self.w2.bias)
-        h1, h3 = self.w1(x), self.w3(x)
-        if swiglu_fusable(h1, h3, self.w2.weight):  # converted w2: gate inside the MXFP8 cast
-            return mx_swiglu_linear(h1, h3, self.w2.weight, self.w2.bias)
-        return self.w2(F.silu(h1) * h3)
+            return mx_feed_forward(x, w1.weight, w2.weight, w3.weight, w2.bias)
+        gate, up = w1(x), w3(x)
+        if swiglu_fusable(gate, up, w2.weight):  # converted w2 only: gate inside the cast feeding it
+            return mx_swiglu_linear(gate, up, w2.weight, w2.bias)
+        return w2(F.silu(gate) * up)
 
     def init_weights(self, init_std: float = 0.02, **kwargs):
-        self.w1.init_weights()
-        self.w2.init_weights(init_std=init_std)
-        self.w3.init_weights(init_std=init_std)
+        # the down projection takes the depth-scaled std, gate and up their configured default
+        for proj, std in ((self.w1, None), (self.w2, init_std), (self.w3, init_std)):
+            proj.init_weights(**({} if std is None else {"init_std": std}))
