@@ -133,6 +133,35 @@ def test_feed_forward_fused_gate_matches_separate_ops(device, recipe, tokens, di
     assert type(y.grad_fn).__name__ == "_MXFeedForwardBackward"
 
 
+def test_feed_forward_fused_with_float32_master_weights(device):
+    """float32 parameters, bf16 activations: the fused block casts the weights to bf16 on the
+    way in and returns float32 weight gradients, bit-identical to the separate-op form."""
+    torch.manual_seed(13)
+    blocks = []
+    for fuse in (True, False):
+        ff = FeedForward.Config(hidden_dim=256).build(dim=128).to(device)
+        if blocks:
+            ff.load_state_dict(blocks[0].state_dict())
+        else:
+            ff.init_weights(init_std=0.05)
+        holder = nn.Module()
+        holder.feed_forward = ff
+        _convert(holder, ["feed_forward"], fuse=fuse)
+        blocks.append(ff)
+    x = torch.randn(96, 128, device=device, dtype=torch.bfloat16)
+    dy = torch.randn(96, 128, device=device, dtype=torch.bfloat16)
+    outs = []
+    for ff in blocks:
+        xi = x.clone().requires_grad_(True)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            y = ff(xi)
+        y.backward(dy)
+        assert y.dtype == torch.bfloat16 and ff.w1.weight.grad.dtype == torch.float32
+        outs.append([y.detach(), xi.grad, ff.w1.weight.grad, ff.w2.weight.grad, ff.w3.weight.grad])
+    for got, want in zip(*outs):
+        assert torch.equal(got, want)
+
+
 def test_feed_forward_with_only_w2_converted_fuses_the_gate(device):
     """w1 / w3 left in bf16, w2 converted: the gate still runs inside the cast that feeds w2 and
     the block matches the same block built from separate ops bit for bit."""
