@@ -162,6 +162,33 @@ def test_feed_forward_fused_with_float32_master_weights(device):
         assert torch.equal(got, want)
 
 
+@pytest.mark.parametrize("fuse", [True, False])
+def test_converted_blocks_under_activation_checkpointing(device, fuse):
+    """torch.utils.checkpoint around a converted block (full activation checkpointing, as
+    torchtitan applies per layer): the forward is re-run in backward through the same kernels and
+    every gradient equals the one without checkpointing."""
+    from torch.utils.checkpoint import checkpoint
+
+    torch.manual_seed(17)
+    ff = FeedForward.Config(hidden_dim=256).build(dim=128).to(device).to(torch.bfloat16)
+    ff.init_weights(init_std=0.05)
+    holder = nn.Module()
+    holder.feed_forward = ff
+    _convert(holder, ["feed_forward"], fuse=fuse)
+    x = torch.randn(2, 64, 128, device=device, dtype=torch.bfloat16)
+    dy = torch.randn(2, 64, 128, device=device, dtype=torch.bfloat16)
+    grads = []
+    for use_ckpt in (False, True):
+        for p in ff.parameters():
+            p.grad = None
+        xi = x.clone().requires_grad_(True)
+        y = checkpoint(ff, xi, use_reentrant=False) if use_ckpt else ff(xi)
+        y.backward(dy)
+        grads.append([y.detach(), xi.grad] + [p.grad.clone() for p in ff.parameters()])
+    for a, b in zip(*grads):
+        assert torch.equal(a, b)
+
+
 def test_feed_forward_with_only_w2_converted_fuses_the_gate(device):
     """w1 / w3 left in bf16, w2 converted: the gate still runs inside the cast that feeds w2 and
     the block matches the same block built from separate ops bit for bit."""
