@@ -151,6 +151,18 @@ int mx_swiglu_cast_dim0_dim1(const void* a, const void* b, int64_t rows, int64_t
                              uint8_t* codes_t, uint8_t* scales_t, void* g, int scale_mode,
                              int scale_order, void* stream);
 
+/* RMSNorm fused in front of the casts: rstd[r] = 1 / sqrt(mean_c x[r, c]^2 + eps) (float32, also
+ * an output: the norm's backward needs it), y[r, c] = bf16(weight[c] * (rstd[r] * x[r, c])) in
+ * float32, then both casts of y as mx_cast_dim0_dim1 produces them.  x bf16 [rows, cols] (row
+ * stride ldx), weight bf16 [cols], y bf16 [rows, cols] dense or NULL (then the normalised
+ * activation never reaches memory).  rows % 32 == 0, cols % 32 == 0, ldx % 8 == 0, 16-byte aligned.
+ * Stands in for the RMSNorm in front of wq / wk / wv and of w1 / w3
+ * (torchtitan/models/common/rmsnorm.py:14-50) followed by the cast of its output. */
+int mx_rmsnorm_cast_dim0_dim1(const void* x, const void* weight, float eps, int64_t rows,
+                              int64_t cols, int64_t ldx, float* rstd, void* y, uint8_t* codes,
+                              uint8_t* scales, uint8_t* codes_t, uint8_t* scales_t, int scale_mode,
+                              int scale_order, void* stream);
+
 /* Backward of that gate fused into the casts that feed the dgrad and wgrad GEMMs of w1 and w3:
  * from dg, a, b (bf16 [rows, cols], row strides lddg, lda, ldb) forms, as bf16 autograd does
  * tensor op by tensor op,

@@ -36,6 +36,8 @@ Pinning status (what fixes each function independently of its own formula):
   grouped variants           pinned  -- loop of mx_matmul over groups, the shape of the
                                         reference's own per-expert loop
                                         (torchtitan/models/common/moe/moe.py:24-56)
+  rms_norm_bf16              pinned  -- textbook form in float64 vs torch's CPU rms_norm; last bf16
+                                        step under a float32 reduction PARITY UNPINNED
   swiglu_bf16                pinned  -- closed form in float64; the last bf16 ulp of a
                                         float32 evaluation is PARITY UNPINNED (see its docstring)
   swiglu_backward_bf16       pinned  -- closed form vs a central difference and torch's CPU op;
@@ -368,6 +370,18 @@ def padded_max_len(num_tokens: int, num_experts: int, alignment: int) -> int:
 
 
 # --------------------------------------------------------------------------- inputs
+def rms_norm_bf16(x_bits: np.ndarray, w_bits: np.ndarray, eps: float):
+    """(y, rstd): y = bf16(w * (x * rstd)), rstd = 1 / sqrt(mean(x^2) + eps) per row, in float64
+    from bf16 inputs (nn.RMSNorm with a weight, torchtitan/models/common/rmsnorm.py:14-50).
+    A float32 reduction gives rstd to a few 1e-7 relative, which moves y to the neighbouring
+    bf16 value at a few elements in a thousand: PARITY UNPINNED to that extent (tests bound it)."""
+    x = bf16_bits_to_f32(x_bits).astype(np.float64)
+    w = bf16_bits_to_f32(w_bits).astype(np.float64)
+    rstd = 1.0 / np.sqrt((x * x).mean(axis=1) + eps)
+    y = w[None, :] * (x * rstd[:, None])
+    return f32_to_bf16_bits(y.astype(np.float32)), rstd
+
+
 def silu_bf16(a_bits: np.ndarray) -> np.ndarray:
     """bf16 silu as one tensor op: x / (1 + exp(-x)) evaluated in float64 with float32's range
     (exp(-x) beyond float32 is infinite, so x below about -88.7 gives -0), rounded to bf16."""

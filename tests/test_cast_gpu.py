@@ -405,3 +405,32 @@ def test_fused_casts_at_benchmark_sizes_equal_separate_kernels(device):
     r0, r1 = ops.to_mx_dim0_dim1(gathered, "rceil", L)
     for got, want in ((q0, r0), (q1, r1)):
         assert torch.equal(got.codes, want.codes) and torch.equal(got.scales, want.scales)
+
+
+@pytest.mark.parametrize("mode_name,mode", MODES)
+@pytest.mark.parametrize("shape", [(32, 64), (160, 224), (512, 4096)])
+def test_rms_norm_fused_cast(device, mode_name, mode, shape):
+    """RMSNorm in front of both casts: rstd to 1e-6 of the float64 oracle; y equal to the oracle's
+    or the neighbouring bf16 value (float32 reduction), and likewise against torch's GPU
+    rms_norm; codes and scales exact for the y that was formed."""
+    rng = np.random.default_rng(shape[0] + shape[1])
+    x_bits = randn_bits(rng, shape, std=2.0, outliers=1e-3)
+    w_bits = mo.f32_to_bf16_bits((1 + 0.2 * rng.standard_normal(shape[1])).astype(np.float32))
+    x, w = bf16_from_bits(x_bits, device), bf16_from_bits(w_bits, device)
+    y_o, rstd_o = mo.rms_norm_bf16(x_bits, w_bits, 1e-5)
+    y_t = bits_of(torch.nn.functional.rms_norm(x, (shape[1],), w, 1e-5))
+    for order in (ops.MX_SCALES_ROWMAJOR, ops.MX_SCALES_MFMA):
+        q0, q1, rstd, y = ops.rms_norm_to_mx(x, w, 1e-5, mode_name, order, want_y=True)
+        assert np.allclose(rstd.cpu().numpy(), rstd_o, rtol=2e-6)
+        y_bits = bits_of(y)
+        for ref in (y_o, y_t):
+            off = y_bits != ref
+            assert off.mean() < 0.02 and (np.abs(y_bits[off].astype(np.int32) - ref[off].astype(np.int32)) <= 1).all()
+        c0, s0 = mo.cast_dim0(y_bits, mode)
+        c1, s1 = mo.cast_dim1(y_bits, mode)
+        if order == ops.MX_SCALES_MFMA:
+            s0, s1 = mo.scale_layout(s0), mo.scale_layout(s1)
+        assert np.array_equal(u8(q0.codes), c0) and np.array_equal(u8(q0.scales).reshape(-1), s0.reshape(-1))
+        assert np.array_equal(u8(q1.codes), c1) and np.array_equal(u8(q1.scales).reshape(-1), s1.reshape(-1))
+        p0, p1, _, none = ops.rms_norm_to_mx(x, w, 1e-5, mode_name, order)
+        assert none is None and torch.equal(p0.codes, q0.codes) and torch.equal(p1.scales, q1.scales)

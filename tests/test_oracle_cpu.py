@@ -56,6 +56,22 @@ def test_bf16_conversions_vs_torch():
     assert np.array_equal(mo.f32_to_bf16_bits(x), ref)
 
 
+def test_rms_norm_vs_torch_cpu():
+    """Oracle RMSNorm against torch's CPU op on bf16 tensors: equal except where float32
+    arithmetic lands on the neighbouring bf16 value."""
+    rng = np.random.default_rng(12)
+    x = mo.f32_to_bf16_bits((rng.standard_normal((64, 512)) * 3).astype(np.float32))
+    w = mo.f32_to_bf16_bits((1 + 0.1 * rng.standard_normal(512)).astype(np.float32))
+    t = lambda bits: torch.from_numpy(bits.view(np.int16)).view(torch.bfloat16)
+    ref = torch.nn.functional.rms_norm(t(x), (512,), t(w), 1e-5).view(torch.int16).numpy().view(np.uint16)
+    got, rstd = mo.rms_norm_bf16(x, w, 1e-5)
+    off = got != ref
+    assert off.mean() < 0.02
+    assert (np.abs(got[off].astype(np.int32) - ref[off].astype(np.int32)) <= 1).all()
+    xf = mo.bf16_bits_to_f32(x).astype(np.float64)
+    assert np.allclose(rstd, 1 / np.sqrt((xf ** 2).mean(1) + 1e-5))
+
+
 def test_swiglu_vs_torch_bf16_ops_every_gate_input():
     """silu over every bf16 bit pattern, and the gate product on a random pairing, against
     torch's CPU bf16 tensor ops (the ops feed_forward.py:61-62 runs)."""

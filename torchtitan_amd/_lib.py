@@ -36,6 +36,7 @@ SIGNATURES = {
     "mx_moe_route_plan": (c_int, [_P, _I, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P]),
     "mx_moe_combine": (c_int, [_P, _P, _I, _I, _P, _P, _I, _I, _I, _P, _I, _P]),
     "mx_moe_row_dot": (c_int, [_P, _P, _I, _I, _P, _P, _I, _I, _P, _I, _I, _P, _P]),
+    "mx_rmsnorm_cast_dim0_dim1": (c_int, [_P, _P, ctypes.c_float, _I, _I, _I, _P, _P, _P, _P, _P, _P, c_int, c_int, _P]),
     "mx_swiglu_cast_dim0_dim1": (c_int, [_P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, c_int, c_int, _P]),
     "mx_swiglu_bwd_cast_dim0_dim1": (c_int, [_P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, c_int, c_int, _P]),
     "mx_scale_layout": (c_int, [_P, _I, _I, _P, _P]),

@@ -643,7 +643,7 @@ __device__ __forceinline__ void load_patch_rows(u32x4 (&v)[8], const uint16_t* x
 
 // Operands of the tile kernel's variants beyond the plain cast.
 struct TileExtras {
-  const uint16_t* x3 = nullptr;  // GATE 1, 2: second gate input b
+  const uint16_t* x3 = nullptr;  // GATE 1, 2: second gate input b; GATE 3: norm weight [cols]
   int64_t ldx3 = 0;
   uint16_t* g_out = nullptr;     // GATE 1: g; GATE 2: stacked da, db (optional)
   const uint16_t* x4 = nullptr;  // GATE 2: dg
@@ -651,7 +651,7 @@ struct TileExtras {
   const int64_t* row_idx = nullptr;  // GATHER: source row of every output row
   int64_t src_rows = 0;
   uint32_t batch = 1;  // stacked independent matrices
-  const float* row_scale = nullptr;  // GATHER: optional multiplier of every output row
+  const float* row_scale = nullptr;  // GATHER: optional multiplier of every output row; GATE 3: rstd
 };
 
 // The gate-backward variant is bound by vector ALU work: four workgroups per CU (128 VGPRs).
@@ -713,6 +713,28 @@ __global__ __launch_bounds__(64 * WAVES, GATE == 2 ? 4 : 1) void cast_tile_kerne
                    swiglu2(v[k].w, b[k].w)};
       if (g_out && col_ok && k < rows_left)
         *reinterpret_cast<u32x4*>(g_out + (r0 + rl0 + k) * cols + c) = v[k];
+    }
+  }
+  if constexpr (GATE == 3) {
+    // RMSNorm in front of the cast: y = bf16(w[c] * (rstd[r] * x)), x3 = the norm weight [cols],
+    // row_scale = rstd [rows]
+    u32x4 wv = u32x4{0, 0, 0, 0};
+    if (col_ok) wv = *reinterpret_cast<const u32x4*>(x3 + c);
+    const float w8[8] = {bf16_lo(wv.x), bf16_hi(wv.x), bf16_lo(wv.y), bf16_hi(wv.y),
+                         bf16_lo(wv.z), bf16_hi(wv.z), bf16_lo(wv.w), bf16_hi(wv.w)};
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      if (col_ok && k < rows_left) {
+        const float rs = ex.row_scale[r0 + rl0 + k];
+        const uint32_t d[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+        uint32_t o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          o[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(
+                     v2f_t{w8[2 * e] * (rs * bf16_lo(d[e])), w8[2 * e + 1] * (rs * bf16_hi(d[e]))}, v2bf_t));
+        v[k] = u32x4{o[0], o[1], o[2], o[3]};
+        if (g_out) *reinterpret_cast<u32x4*>(g_out + (r0 + rl0 + k) * cols + c) = v[k];
+      }
     }
   }
   if constexpr (GATE == 2) {
@@ -1064,6 +1086,63 @@ extern "C" int mx_cast_rows_gathered(const void* x, const int64_t* row_index,
     MX_DISPATCH_TILE(true, false, 0, true, (const uint16_t*)x, rows, cols, ldx, codes, scales, nblk,
                      ks_n, (uint8_t*)nullptr, (uint8_t*)nullptr, (int64_t)0, (int64_t)0, (int64_t)0,
                      (int64_t)0, (int64_t)0, (uint32_t)gx, (uint32_t)tgy, ex);
+  return launch_status();
+}
+
+namespace mx {
+// rstd[r] = 1 / sqrt(mean_c x[r, c]^2 + eps) in float32; one wave per row, lanes stride over
+// 8-column chunks, butterfly over the 64 lanes.
+__global__ __launch_bounds__(256) void rms_rstd_kernel(const uint16_t* __restrict__ x, int64_t rows,
+                                                       int64_t cols, int64_t ldx, float eps,
+                                                       float* __restrict__ rstd) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 6;
+  if (r >= rows) return;
+  const uint16_t* row = x + r * ldx;
+  float acc = 0.f;
+  for (int64_t c = lane * 8; c < cols; c += 64 * 8) {
+    const u32x4 v = *reinterpret_cast<const u32x4*>(row + c);
+    const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float lo = bf16_lo(d[e]), hi = bf16_hi(d[e]);
+      acc = __builtin_fmaf(lo, lo, acc);
+      acc = __builtin_fmaf(hi, hi, acc);
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+  if (lane == 0) rstd[r] = rsqrtf(acc / (float)cols + eps);
+}
+}  // namespace mx
+
+extern "C" int mx_rmsnorm_cast_dim0_dim1(const void* x, const void* weight, float eps, int64_t rows,
+                                         int64_t cols, int64_t ldx, float* rstd, void* y,
+                                         uint8_t* codes, uint8_t* scales, uint8_t* codes_t,
+                                         uint8_t* scales_t, int scale_mode, int scale_order,
+                                         void* stream) {
+  if (rows < 0 || cols < 0 || ldx < cols || bad_enums(scale_mode, scale_order)) return MX_ERR_INVALID_ARG;
+  if (rows == 0 || cols == 0) return MX_OK;
+  if (!x || !weight || !rstd || !codes || !scales || !codes_t || !scales_t) return MX_ERR_INVALID_ARG;
+  if (rows % 32 || cols % 32 || ldx % 8 || ((uintptr_t)x & 15) || ((uintptr_t)weight & 15) ||
+      ((uintptr_t)y & 15) || ((uintptr_t)rstd & 3) || ((uintptr_t)codes & 7) ||
+      ((uintptr_t)codes_t & 15) || ((uintptr_t)scales & 3) || ((uintptr_t)scales_t & 3))
+    return MX_ERR_ALIGNMENT;
+  const int64_t nblk = cols / 32, ks_n = (nblk + 1) / 2;
+  const int64_t nblk_t = rows / 32, ks_n_t = (nblk_t + 1) / 2;
+  const int64_t gx = (cols + kT - 1) / kT, tgy = (rows + kTileRows - 1) / kTileRows;
+  if (tile_grid_x(gx, tgy, true) > 0x7FFFFFFF || (rows + 3) / 4 > 0x7FFFFFFF) return MX_ERR_UNSUPPORTED;
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(rms_rstd_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st,
+                     (const uint16_t*)x, rows, cols, ldx, eps, rstd);
+  dim3 grid = tile_grid(gx, tgy, 1, true), block(64 * MX_CAST_WAVES);
+  TileExtras ex;
+  ex.x3 = (const uint16_t*)weight;
+  ex.g_out = (uint16_t*)y;
+  ex.row_scale = rstd;
+  MX_DISPATCH_TILE(true, true, 3, false, (const uint16_t*)x, rows, cols, ldx, codes, scales, nblk, ks_n,
+                   codes_t, scales_t, nblk_t, ks_n_t, (int64_t)0, (int64_t)0, (int64_t)0,
+                   (uint32_t)gx, (uint32_t)tgy, ex);
   return launch_status();
 }
 

@@ -320,6 +320,30 @@ def token_logprob_bwd(logits: torch.Tensor, target: torch.Tensor, lse: torch.Ten
     return out
 
 
+def rms_norm_to_mx(x: torch.Tensor, weight: torch.Tensor, eps: float, mode="floor",
+                   order: int = MX_SCALES_ROWMAJOR, want_y: bool = False):
+    """Both casts of y = rms_norm(x) * weight (float32 arithmetic, one rounding to bf16) without
+    y passing through memory; returns (row-wise MXData, column-wise MXData, rstd float32 [rows],
+    y or None)."""
+    x = _check_hp(x)
+    if weight.dtype != torch.bfloat16 or weight.shape != (x.shape[1],) or weight.device != x.device:
+        raise TypeError("the norm weight must be bf16 [cols] on x's device")
+    weight = weight.contiguous()
+    R, C = x.shape
+    if R % BLOCK or C % BLOCK:
+        raise ValueError(f"both dims of {tuple(x.shape)} must be multiples of {BLOCK}")
+    codes = torch.empty((R, C), dtype=torch.uint8, device=x.device)
+    scales = _alloc_scales(R, C // BLOCK, order, x.device)
+    codes_t = torch.empty((C, R), dtype=torch.uint8, device=x.device)
+    scales_t = _alloc_scales(C, R // BLOCK, order, x.device)
+    rstd = torch.empty(R, dtype=torch.float32, device=x.device)
+    y = torch.empty((R, C), dtype=torch.bfloat16, device=x.device) if want_y else None
+    _call("mx_rmsnorm_cast_dim0_dim1", "rmsnorm_cast_dim0_dim1", x.device, _ptr(x), _ptr(weight),
+          ctypes.c_float(eps), R, C, x.stride(0), _ptr(rstd), _ptr(y) if y is not None else None,
+          _ptr(codes), _ptr(scales), _ptr(codes_t), _ptr(scales_t), _mode(mode), order, _stream(x))
+    return MXData(codes, scales, order), MXData(codes_t, scales_t, order), rstd, y
+
+
 def swiglu_to_mx_dim0_dim1(a: torch.Tensor, b: torch.Tensor, mode="floor",
                            order: int = MX_SCALES_ROWMAJOR, want_g: bool = False):
     """Both casts of g = silu(a) * b (bf16, every step rounded to bf16) without g passing through
