@@ -20,10 +20,11 @@ def _f32(bits):
     return mo.bf16_bits_to_f32(bits)
 
 
-def _convert(model, fqns, recipe="mxfp8_rceil", pad=True, fuse=True, cache=False):
+def _convert(model, fqns, recipe="mxfp8_rceil", pad=True, fuse=True, cache=False, norm=False):
     box = ModelConvertersContainer.Config(
         converters=[MXFP8Converter.Config(fqns=fqns, recipe_name=recipe, pad_token_groups_for_grouped_mm=pad,
-                                          fuse_swiglu_cast=fuse, cache_weight_casts=cache)]
+                                          fuse_swiglu_cast=fuse, cache_weight_casts=cache,
+                                          fuse_rmsnorm_cast=norm)]
     ).build(parallel_dims=None, model_compile_enabled=False)
     box.convert(model)
     return box
@@ -187,6 +188,77 @@ def test_converted_blocks_under_activation_checkpointing(device, fuse):
         grads.append([y.detach(), xi.grad] + [p.grad.clone() for p in ff.parameters()])
     for a, b in zip(*grads):
         assert torch.equal(a, b)
+
+
+class _NormedBlock(nn.Module):
+    """RMSNorm -> three projections sharing the normalised input, and RMSNorm -> SwiGLU block,
+    with the norms inside the casts when the converter allows it."""
+
+    def __init__(self, dim, inner, ffn):
+        super().__init__()
+        mk = lambda i, o: Linear.Config().build(in_features=i, out_features=o)
+        self.attention = nn.Module()
+        self.attention.wq, self.attention.wk, self.attention.wv = mk(dim, dim), mk(dim, inner), mk(dim, inner)
+        self.feed_forward = FeedForward.Config(hidden_dim=ffn).build(dim=dim)
+        self.attention_norm = nn.RMSNorm(dim, eps=1e-5)
+        self.ffn_norm = nn.RMSNorm(dim, eps=1e-5)
+
+    def forward(self, x):
+        from torchtitan_amd.mx_blocks import (feed_forward_fusable, mx_norm_feed_forward, mx_norm_linears,
+                                              norm_fusable)
+
+        a, ff = self.attention, self.feed_forward
+        qkv_w = (a.wq.weight, a.wk.weight, a.wv.weight)
+        if norm_fusable(x, self.attention_norm.weight, *qkv_w):
+            q, k, v = mx_norm_linears(x, self.attention_norm.weight, self.attention_norm.eps, qkv_w)
+        else:
+            h = self.attention_norm(x)
+            q, k, v = a.wq(h), a.wk(h), a.wv(h)
+        mixed = q + torch.cat((k, v), dim=-1)[..., : q.shape[-1]]      # stands in for attention
+        w = (ff.w1.weight, ff.w2.weight, ff.w3.weight)
+        if norm_fusable(mixed, self.ffn_norm.weight, w[0], w[2]) and feed_forward_fusable(mixed, *w):
+            return mixed + mx_norm_feed_forward(mixed, self.ffn_norm.weight, self.ffn_norm.eps, *w)
+        return mixed + ff(self.ffn_norm(mixed))
+
+
+def test_rms_norm_inside_the_casts_matches_separate_norms(device):
+    """Opt-in fusion of the two RMSNorms of a block into the casts that follow them: output and
+    all gradients (inputs, seven weights, both norm weights) agree with the separate-norm form:
+    to 2e-3 where only the norm differs (the normalised activation moves by one bf16 step at a
+    few elements in a million, which can flip an e4m3 code), to 5e-3 where bf16 sums of three
+    partial gradients are formed in a different order (dx and the first norm's weight)."""
+    torch.manual_seed(19)
+    blocks = []
+    for norm in (True, False):
+        blk = _NormedBlock(256, 128, 512).to(device).to(torch.bfloat16)
+        if blocks:
+            blk.load_state_dict(blocks[0].state_dict())
+        else:
+            for m in blk.modules():
+                if isinstance(m, nn.Linear):
+                    nn.init.normal_(m.weight, std=0.05)
+            with torch.no_grad():
+                blk.attention_norm.weight.add_(0.1 * torch.randn_like(blk.attention_norm.weight))
+                blk.ffn_norm.weight.add_(0.1 * torch.randn_like(blk.ffn_norm.weight))
+        _convert(blk, ["attention", "feed_forward"], norm=norm)
+        blocks.append(blk)
+    x = torch.randn(2, 128, 256, device=device, dtype=torch.bfloat16)
+    dy = torch.randn(2, 128, 256, device=device, dtype=torch.bfloat16)
+    outs = []
+    for blk in blocks:
+        xi = x.clone().requires_grad_(True)
+        y = blk(xi)
+        y.backward(dy)
+        outs.append({"y": y.detach(), "dx": xi.grad, **{n: p.grad for n, p in blk.named_parameters()}})
+    fused, plain = outs
+    assert set(fused) == set(plain) and len(fused) == 2 + 8
+    for name in fused:
+        assert fused[name] is not None, name
+        tol = 5e-3 if name in ("dx", "attention_norm.weight") else 2e-3
+        assert rel_l2(fused[name].float().cpu().numpy(), plain[name].float().cpu().numpy()) <= tol, name
+    from torchtitan_amd.mx_blocks import norm_fusable
+    assert norm_fusable(x, blocks[0].attention_norm.weight, blocks[0].attention.wq.weight)
+    assert not norm_fusable(x, blocks[1].attention_norm.weight, blocks[1].attention.wq.weight)
 
 
 def test_feed_forward_with_only_w2_converted_fuses_the_gate(device):

@@ -117,13 +117,18 @@ class _MXFeedForward(torch.autograd.Function):
     bf16 ``F.silu`` and ``*`` (torchtitan/models/common/feed_forward.py:61-62)."""
 
     @staticmethod
-    def forward(ctx, x, w1, w2, w3, cfg: MXFP8Config):
+    def forward(ctx, x, w1, w2, w3, cfg: MXFP8Config, norm_weight=None, eps: float = 0.0):
         mode = cfg.scale_mode
         D, H = x.shape[-1], w1.shape[0]
         x2 = x.reshape(-1, D)
-        need_dx = ctx.needs_input_grad[0]
+        need_dx = ctx.needs_input_grad[0] or ctx.needs_input_grad[5]
         need_dw = any(ctx.needs_input_grad[1:4])
-        xq0, xq1 = _cast_activation(x2, x, mode, need_cols=need_dw)
+        ctx.normed = norm_weight is not None
+        if ctx.normed:  # RMSNorm in front: normalised inside the cast, rstd kept for its backward
+            x2 = x2.contiguous()
+            xq0, xq1, rstd, _ = ops.rms_norm_to_mx(x2, _bf16(norm_weight), eps, mode, MX_SCALES_MFMA)
+        else:
+            xq0, xq1 = _cast_activation(x2, x, mode, need_cols=need_dw)
         w1q0, w1q1 = _cast_weight(w1, mode, need_dx, cfg)
         w3q0, w3q1 = _cast_weight(w3, mode, need_dx, cfg)
         w2q0, w2q1 = _cast_weight(w2, mode, need_dx or need_dw, cfg)
@@ -141,6 +146,8 @@ class _MXFeedForward(torch.autograd.Function):
             saved += [xq1.codes, xq1.scales, gq1.codes, gq1.scales]
         if need_dx:
             saved += [w1q1.codes, w1q1.scales, w3q1.codes, w3q1.scales]
+            if ctx.normed:
+                saved += [x2, rstd, norm_weight]
         ctx.save_for_backward(*saved)
         return y.view(*x.shape[:-1], w2.shape[0])
 
@@ -168,10 +175,15 @@ class _MXFeedForward(torch.autograd.Function):
                 dw2 = cast_back(ops.mx_gemm_nt(dyq1, gq1), ctx.w_dtypes[1])
             if ctx.needs_input_grad[3]:
                 dw3 = cast_back(ops.mx_gemm_nt(db1, xq1), ctx.w_dtypes[2])
+        dnw = None
         if ctx.need_dx:
             w1q1, w3q1 = take(), take()
-            dx = (ops.mx_gemm_nt(da0, w1q1) + ops.mx_gemm_nt(db0, w3q1)).view(ctx.x_shape)
-        return dx, dw1, dw2, dw3, None
+            dx = ops.mx_gemm_nt(da0, w1q1) + ops.mx_gemm_nt(db0, w3q1)
+            if ctx.normed:
+                dx, dnw = _rms_norm_backward(dx, *saved[:3], ctx.needs_input_grad[0], ctx.needs_input_grad[5])
+            if dx is not None:
+                dx = dx.view(ctx.x_shape)
+        return dx, dw1, dw2, dw3, None, dnw, None
 
 
 def feed_forward_fusable(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, w3: torch.Tensor) -> bool:
@@ -192,7 +204,110 @@ def mx_feed_forward(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, w3: tor
                     bias2: torch.Tensor | None = None):
     """``F.linear(F.silu(F.linear(x, w1)) * F.linear(x, w3), w2, bias2)`` for converted weights.
     Callers check `feed_forward_fusable` first."""
-    y = _MXFeedForward.apply(x, _unwrap(w1), _unwrap(w2), _unwrap(w3), w2.mx_config)
+    y = _MXFeedForward.apply(x, _unwrap(w1), _unwrap(w2), _unwrap(w3), w2.mx_config, None, 0.0)
+    if bias2 is not None:
+        y = y + _unwrap(bias2).to(y.dtype)
+    return y
+
+
+# ----------------------------------------------------------------------------- RMSNorm in front
+def _rms_norm_backward(dh, x2, rstd, norm_weight, need_dx: bool, need_dw: bool):
+    """(dx, dweight) of y = rms_norm(x) * weight from dy = dh, with torch's own fused backward
+    kernel fed the rstd the forward kernel produced."""
+    gx, gw = torch.ops.aten._fused_rms_norm_backward(dh, x2, [x2.shape[-1]], rstd.view(-1, 1), norm_weight,
+                                                     [need_dx, need_dw])
+    return (gx if need_dx else None), (gw if need_dw else None)
+
+
+class _MXNormLinears(torch.autograd.Function):
+    """(rms_norm(x) W_0^T, rms_norm(x) W_1^T, ...) for linears that share one normalised input
+    (wq / wk / wv behind the attention norm): the norm runs inside the one cast that feeds all of
+    them; the normalised activation is never written.  Not bit-identical to a separate norm: the
+    float32 row reduction differs from torch's in its last bits (a few bf16 values in a million
+    move by one step)."""
+
+    @staticmethod
+    def forward(ctx, x, norm_weight, eps, cfg: MXFP8Config, *weights):
+        mode = cfg.scale_mode
+        D = x.shape[-1]
+        x2 = x.reshape(-1, D).contiguous()
+        hq0, hq1, rstd, _ = ops.rms_norm_to_mx(x2, _bf16(norm_weight), eps, mode, MX_SCALES_MFMA)
+        need_dh = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
+        outs, saved = [], [x2, rstd, norm_weight, hq1.codes, hq1.scales]
+        for w in weights:
+            wq0, wq1 = _cast_weight(w, mode, need_dh, cfg)
+            outs.append(ops.mx_gemm_nt(hq0, wq0).view(*x.shape[:-1], w.shape[0]))
+            if need_dh:
+                saved += [wq1.codes, wq1.scales]
+        ctx.cfg, ctx.x_shape, ctx.need_dh = cfg, x.shape, need_dh
+        ctx.w_dtypes = tuple(w.dtype for w in weights)
+        ctx.save_for_backward(*saved)
+        return tuple(outs)
+
+    @staticmethod
+    def backward(ctx, *dys):
+        mode = ctx.cfg.scale_mode
+        saved = list(ctx.saved_tensors)
+        x2, rstd, norm_weight = saved[:3]
+        hq1 = MXData(saved[3], saved[4], MX_SCALES_MFMA)
+        rest = saved[5:]
+        dh, dws = None, []
+        for i, dy in enumerate(dys):
+            need_dw = ctx.needs_input_grad[4 + i]
+            if dy is None or not (ctx.need_dh or need_dw):
+                dws.append(None)
+                continue
+            dy2 = _bf16(dy.reshape(-1, dy.shape[-1])).contiguous()
+            if ctx.need_dh and need_dw:
+                dyq0, dyq1 = ops.to_mx_dim0_dim1(dy2, mode, MX_SCALES_MFMA)
+            else:
+                dyq0 = ops.to_mx_dim0(dy2, mode, MX_SCALES_MFMA) if ctx.need_dh else None
+                dyq1 = ops.to_mx_dim1(dy2, mode, MX_SCALES_MFMA) if need_dw else None
+            if ctx.need_dh:
+                part = ops.mx_gemm_nt(dyq0, MXData(rest[2 * i], rest[2 * i + 1], MX_SCALES_MFMA))
+                dh = part if dh is None else dh + part
+            dw = None
+            if need_dw:
+                dw = ops.mx_gemm_nt(dyq1, hq1)
+                if dw.dtype != ctx.w_dtypes[i]:
+                    dw = dw.to(ctx.w_dtypes[i])
+            dws.append(dw)
+        dx = dnw = None
+        if ctx.need_dh and dh is not None:
+            dx, dnw = _rms_norm_backward(dh, x2, rstd, norm_weight, ctx.needs_input_grad[0], ctx.needs_input_grad[1])
+            if dx is not None:
+                dx = dx.view(ctx.x_shape)
+        return (dx, dnw, None, None, *dws)
+
+
+def norm_fusable(x: torch.Tensor, norm_weight: torch.Tensor | None, *weights: torch.Tensor) -> bool:
+    """RMSNorm can move into the cast when the converter was built with `fuse_rmsnorm_cast`, the
+    norm has a bf16 weight, every linear behind it is converted with in_features % 32 == 0 and
+    out_features % 32 == 0, and x is a bf16 GPU tensor with a multiple of 32 tokens."""
+    if norm_weight is None or norm_weight.dtype != torch.bfloat16 or not weights:
+        return False
+    if not all(isinstance(w, MXFP8TrainingWeight) and w.mx_config.fuse_rmsnorm_cast and w.dim() == 2 for w in weights):
+        return False
+    if x.dtype != torch.bfloat16 or not x.is_cuda or x.numel() == 0:
+        return False
+    D = x.shape[-1]
+    if any(w.shape[1] != D or w.shape[0] % ops.BLOCK for w in weights):
+        return False
+    return D % ops.BLOCK == 0 and (x.numel() // D) % ops.BLOCK == 0 and norm_weight.shape == (D,)
+
+
+def mx_norm_linears(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, weights) -> tuple:
+    """``tuple(F.linear(F.rms_norm(x, (dim,), norm_weight, eps), w) for w in weights)`` for
+    converted weights without biases.  Callers check `norm_fusable` first."""
+    weights = list(weights)
+    return _MXNormLinears.apply(x, norm_weight, float(eps), weights[0].mx_config, *[_unwrap(w) for w in weights])
+
+
+def mx_norm_feed_forward(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w1: torch.Tensor,
+                         w2: torch.Tensor, w3: torch.Tensor, bias2: torch.Tensor | None = None):
+    """The SwiGLU block applied to ``F.rms_norm(x, (dim,), norm_weight, eps)``, norm inside the
+    cast.  Callers check `norm_fusable(x, norm_weight, w1, w3)` and `feed_forward_fusable`."""
+    y = _MXFeedForward.apply(x, _unwrap(w1), _unwrap(w2), _unwrap(w3), w2.mx_config, norm_weight, float(eps))
     if bias2 is not None:
         y = y + _unwrap(bias2).to(y.dtype)
     return y

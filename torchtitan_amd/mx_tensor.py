@@ -28,16 +28,19 @@ from .ops import MX_SCALES_MFMA, MX_SCALES_ROWMAJOR, MXData
 class MXFP8Config:
     """Per-weight recipe: scale mode and whether grouped GEMMs pad token groups to 32."""
 
-    __slots__ = ("scale_mode", "pad_token_groups_for_grouped_mm", "fuse_swiglu_cast", "cache_weight_casts")
+    __slots__ = ("scale_mode", "pad_token_groups_for_grouped_mm", "fuse_swiglu_cast", "cache_weight_casts",
+                 "fuse_rmsnorm_cast")
 
     def __init__(self, scale_mode: str = "rceil", pad_token_groups_for_grouped_mm: bool = True,
-                 fuse_swiglu_cast: bool = True, cache_weight_casts: bool = False):
+                 fuse_swiglu_cast: bool = True, cache_weight_casts: bool = False,
+                 fuse_rmsnorm_cast: bool = False):
         if scale_mode not in ops.SCALE_MODES:
             raise ValueError(f"unknown scale mode {scale_mode!r}")
         self.scale_mode = scale_mode
         self.pad_token_groups_for_grouped_mm = pad_token_groups_for_grouped_mm
         self.fuse_swiglu_cast = fuse_swiglu_cast
         self.cache_weight_casts = cache_weight_casts
+        self.fuse_rmsnorm_cast = fuse_rmsnorm_cast
 
     def __repr__(self):
         return (f"MXFP8Config(scale_mode={self.scale_mode!r}, "

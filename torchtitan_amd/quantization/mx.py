@@ -76,6 +76,12 @@ class MXFP8Converter(QuantizationConverter):
         next step (gradient accumulation, evaluation, several micro-batches) and
         `export_mxfp8_state_dict` reuse those codes."""
 
+        fuse_rmsnorm_cast: bool = False
+        """Not in the reference's Config.  Lets blocks that call `mx_norm_linears` /
+        `mx_norm_feed_forward` run the RMSNorm in front of converted linears inside the cast
+        kernel.  Off by default because the result is not bit-identical to a separate norm (the
+        float32 row reduction differs from torch's in its last bits)."""
+
     def __init__(self, config: Config, *, parallel_dims: Any, model_compile_enabled: bool):
         self.enabled = False
         if not _lib.LIB_PATH.exists():
@@ -104,7 +110,8 @@ class MXFP8Converter(QuantizationConverter):
         saved = capture_module_attrs(model, ["_init_mean", "_init_std"], nn_module_cls=nn.Linear)
         cfg = MXFP8Config(_RECIPES[self.config.recipe_name],
                           self.config.pad_token_groups_for_grouped_mm,
-                          self.config.fuse_swiglu_cast, self.config.cache_weight_casts)
+                          self.config.fuse_swiglu_cast, self.config.cache_weight_casts,
+                          self.config.fuse_rmsnorm_cast)
         n_linear = n_grouped = 0
         for fqn, mod in model.named_modules():
             if not self._matches(fqn):
