@@ -336,6 +336,26 @@ def time_ffn_block(dev, recipe):
         sec = s.elapsed_time(e) * 1e-4
         out[name] = {"us": round(sec * 1e6, 1), "GB/s": round(el * bpe / sec / 1e9, 1),
                      "frac_hbm": round(el * bpe / sec / 1e9 / PEAK_HBM_GBPS, 3)}
+    del a, b, dg
+    # RMSNorm inside the cast (opt-in) against torch's rms_norm followed by the cast, X M x DIM,
+    # over four inputs in turn so that neither form finds its input in the last-level cache
+    import torch.nn.functional as F
+    xs = [torch.randn((M, DIM), device=dev, dtype=torch.bfloat16) for _ in range(4)]
+    w = torch.ones(DIM, device=dev, dtype=torch.bfloat16)
+    for name, fn in (("rmsnorm_cast_dim0_dim1", lambda t: ops.rms_norm_to_mx(t, w, 1e-5, mode, L)),
+                     ("torch_rms_norm_then_cast",
+                      lambda t: ops.to_mx_dim0_dim1(F.rms_norm(t, (DIM,), w, 1e-5), mode, L))):
+        for t in xs[:2]:
+            fn(t)
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for i in range(12):
+            fn(xs[i % 4])
+        e.record()
+        torch.cuda.synchronize()
+        sec = s.elapsed_time(e) * 1e-3 / 12
+        out[name] = {"us": round(sec * 1e6, 1), "GB/s": round(M * DIM * 4.0625 / sec / 1e9, 1)}
     return out
 
 

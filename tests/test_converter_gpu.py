@@ -7,6 +7,7 @@ import torch.nn as nn
 from oracle import mx_oracle as mo
 from tests.helpers import bf16_from_bits, bits_of, randn_bits, rel_l2
 from torchtitan_amd.modules import FeedForward, GroupedExperts, Linear, MoE
+from torchtitan_amd import ops
 from torchtitan_amd.modules import moe as moe_mod
 from torchtitan_amd.mx_tensor import MXFP8TrainingWeight
 from torchtitan_amd.protocols import ModelConvertersContainer
@@ -188,6 +189,103 @@ def test_converted_blocks_under_activation_checkpointing(device, fuse):
         grads.append([y.detach(), xi.grad] + [p.grad.clone() for p in ff.parameters()])
     for a, b in zip(*grads):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("fuse", [True, False])
+def test_per_op_checkpoint_policy_can_keep_gemm_outputs(device, fuse, monkeypatch):
+    """Selective activation checkpointing by op (the policy shape of
+    torchtitan/distributed/activation_checkpoint.py:105-141 over a save list like
+    torchtitan/models/llama3/parallelize.py:44-60): with this package's dispatcher ops in the save
+    list the three forward GEMMs of a block are not run again in the recomputation (9 GEMM
+    launches instead of 12), and every result equals the one without checkpointing."""
+    from torch.utils.checkpoint import CheckpointPolicy, checkpoint, create_selective_checkpoint_contexts
+
+    save = ops.op_sac_save_list() | {torch.ops.aten.mm.default}
+
+    def policy(ctx, func, *args, **kwargs):
+        return CheckpointPolicy.MUST_SAVE if func in save else CheckpointPolicy.PREFER_RECOMPUTE
+
+    launches = []
+    real_call = ops._call
+    monkeypatch.setattr(ops, "_call", lambda name, *a: (launches.append(name), real_call(name, *a))[1])
+
+    torch.manual_seed(23)
+    ff = FeedForward.Config(hidden_dim=256).build(dim=128).to(device).to(torch.bfloat16)
+    ff.init_weights(init_std=0.05)
+    holder = nn.Module()
+    holder.feed_forward = ff
+    _convert(holder, ["feed_forward"], fuse=fuse)
+    x = torch.randn(2, 64, 128, device=device, dtype=torch.bfloat16)
+    dy = torch.randn(2, 64, 128, device=device, dtype=torch.bfloat16)
+    runs = {}
+    for how in ("plain", "full", "per_op"):
+        for p in ff.parameters():
+            p.grad = None
+        xi = x.clone().requires_grad_(True)
+        launches.clear()
+        if how == "plain":
+            y = ff(xi)
+        elif how == "full":
+            y = checkpoint(ff, xi, use_reentrant=False)
+        else:
+            y = checkpoint(ff, xi, use_reentrant=False,
+                           context_fn=lambda: create_selective_checkpoint_contexts(policy))
+        y.backward(dy)
+        runs[how] = (launches.count("mx_gemm_nt"),
+                     [y.detach(), xi.grad] + [p.grad.clone() for p in ff.parameters()])
+    assert [runs[h][0] for h in ("plain", "full", "per_op")] == [9, 12, 9]
+    for how in ("full", "per_op"):
+        for a, b in zip(runs["plain"][1], runs[how][1]):
+            assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("fuse", [True, False])
+def test_per_op_checkpoint_policy_keeps_grouped_gemm_outputs(device, fuse, monkeypatch):
+    """As above for the expert block: three forward grouped GEMMs kept, 6 launches of the 2d3d
+    kernel per step instead of 9, results unchanged."""
+    from torch.utils.checkpoint import CheckpointPolicy, checkpoint, create_selective_checkpoint_contexts
+
+    save = ops.op_sac_save_list()
+
+    def policy(ctx, func, *args, **kwargs):
+        return CheckpointPolicy.MUST_SAVE if func in save else CheckpointPolicy.PREFER_RECOMPUTE
+
+    launches = []
+    real_call = ops._call
+    monkeypatch.setattr(ops, "_call", lambda name, *a: (launches.append(name), real_call(name, *a))[1])
+    torch.manual_seed(29)
+    moe_mod.set_token_group_alignment_size_m(32)
+    try:
+        counts = torch.tensor([40, 0, 200, 16, 7, 130], device=device)
+        ex = GroupedExperts(dim=128, hidden_dim=256, num_experts=6, use_grouped_mm=True).to(device).to(torch.bfloat16)
+        ex.init_weights(init_std=0.05)
+        holder = nn.Module()
+        holder.experts = ex
+        _convert(holder, ["experts"], pad=True, fuse=fuse)
+        x = torch.randn(int(counts.sum()), 128, device=device, dtype=torch.bfloat16)
+        dy = torch.randn(int(counts.sum()), 128, device=device, dtype=torch.bfloat16)
+        runs = {}
+        for how in ("plain", "full", "per_op"):
+            for p in ex.parameters():
+                p.grad = None
+            xi = x.clone().requires_grad_(True)
+            launches.clear()
+            if how == "plain":
+                y = ex(xi, counts)
+            elif how == "full":
+                y = checkpoint(ex, xi, counts, use_reentrant=False)
+            else:
+                y = checkpoint(ex, xi, counts, use_reentrant=False,
+                               context_fn=lambda: create_selective_checkpoint_contexts(policy))
+            y.backward(dy)
+            runs[how] = (launches.count("mx_grouped_gemm_2d3d"),
+                         [y.detach(), xi.grad, ex.w1.grad.clone(), ex.w2.grad.clone(), ex.w3.grad.clone()])
+        assert [runs[h][0] for h in ("plain", "full", "per_op")] == [6, 9, 6]
+        for how in ("full", "per_op"):
+            for a, b in zip(runs["plain"][1], runs[how][1]):
+                assert torch.equal(a, b)
+    finally:
+        moe_mod.set_token_group_alignment_size_m(8)
 
 
 class _NormedBlock(nn.Module):

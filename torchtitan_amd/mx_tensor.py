@@ -295,6 +295,9 @@ def _grouped_2d3d_padded(a: MXData, b: MXData, offs_p: torch.Tensor, back):
     Tp, N = a.codes.shape[0], b.codes.shape[1]
     if back is None:
         return ops.mx_grouped_gemm_2d3d(a, b, offs_p)
+    if ops._watched():  # the dispatcher form of the GEMM allocates its own output
+        y = ops.mx_grouped_gemm_2d3d(a, b, offs_p)
+        return torch.cat((y, y.new_zeros(1, N)))[back]
     buf = torch.empty((Tp + 1, N), dtype=torch.bfloat16, device=a.codes.device)
     buf[Tp].zero_()
     ops.mx_grouped_gemm_2d3d(a, b, offs_p, buf[:Tp])

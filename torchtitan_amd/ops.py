@@ -420,19 +420,72 @@ def _as_mfma(d: MXData) -> torch.Tensor:
     return d.scales if d.scale_order == MX_SCALES_MFMA else scale_layout(d.scales)
 
 
+def _gemm_nt_into(a_codes, a_scales, b_codes, b_scales, out):
+    M, K = a_codes.shape
+    _call("mx_gemm_nt", "gemm_nt", out.device, _ptr(a_codes), _ptr(a_scales), _ptr(b_codes),
+          _ptr(b_scales), _ptr(out), M, b_codes.shape[0], K, out.stride(0), _stream(out))
+    return out
+
+
+def _gemm_nt_op(a_codes, a_scales, b_codes, b_scales):
+    out = torch.empty((a_codes.shape[0], b_codes.shape[0]), dtype=torch.bfloat16, device=a_codes.device)
+    return _gemm_nt_into(a_codes, a_scales, b_codes, b_scales, out)
+
+
+def _grouped_2d3d_into(a_codes, a_scales, a_order, b_codes, b_scales, offs, out):
+    T, K = a_codes.shape
+    G, N, _ = b_codes.shape
+    _call("mx_grouped_gemm_2d3d", "grouped_gemm_2d3d", out.device, _ptr(a_codes), _ptr(a_scales),
+          _ptr(b_codes), _ptr(b_scales), _ptr(offs), _ptr(out), T, N, K, G, out.stride(0), a_order,
+          _stream(out))
+    return out
+
+
+def _grouped_2d3d_op(a_codes, a_scales, a_order, b_codes, b_scales, offs):
+    out = torch.empty((a_codes.shape[0], b_codes.shape[1]), dtype=torch.bfloat16, device=a_codes.device)
+    return _grouped_2d3d_into(a_codes, a_scales, a_order, b_codes, b_scales, offs, out)
+
+
+# The GEMMs whose output a forward pass hands on are also registered with torch's dispatcher, so
+# that a per-op activation-checkpoint policy (torch.utils.checkpoint's selective contexts, which
+# watch dispatched ops) can name them and keep their outputs instead of running them again in
+# the recomputation.  The registered form is only taken while some dispatch mode is active; the
+# plain eager path keeps calling the library directly.
+_dispatcher_ops = torch.library.Library("torchtitan_amd", "DEF")
+_dispatcher_ops.define("mx_gemm_nt(Tensor a_codes, Tensor a_scales, Tensor b_codes, Tensor b_scales) -> Tensor")
+_dispatcher_ops.define("mx_grouped_gemm_2d3d(Tensor a_codes, Tensor a_scales, int a_order, Tensor b_codes, "
+                       "Tensor b_scales, Tensor offs) -> Tensor")
+_dispatcher_ops.impl("mx_gemm_nt", _gemm_nt_op, "CUDA")
+_dispatcher_ops.impl("mx_grouped_gemm_2d3d", _grouped_2d3d_op, "CUDA")
+
+
+def _watched() -> bool:
+    return torch._C._len_torch_dispatch_stack() > 0
+
+
+def op_sac_save_list() -> set:
+    """The dispatcher ops of this package whose outputs a per-op activation-checkpoint policy may
+    save (the forward GEMMs): add them to the model's save list
+    (torchtitan/models/llama3/parallelize.py:44-60) to keep MXFP8 GEMM outputs through the
+    recomputation, as the bf16 path keeps its `aten.mm` outputs.  Casts stay recomputed."""
+    return {torch.ops.torchtitan_amd.mx_gemm_nt.default,
+            torch.ops.torchtitan_amd.mx_grouped_gemm_2d3d.default}
+
+
 def mx_gemm_nt(a: MXData, b: MXData, out: torch.Tensor | None = None) -> torch.Tensor:
     """bf16 D[M,N] = deq(a)[M,K] @ deq(b)[N,K]^T with fp32 accumulation."""
     M, K = a.codes.shape
     N, Kb = b.codes.shape
     if K != Kb:
         raise ValueError(f"contraction mismatch: {K} vs {Kb}")
-    if out is None:
-        out = torch.empty((M, N), dtype=torch.bfloat16, device=a.codes.device)
-    elif out.shape != (M, N) or out.dtype != torch.bfloat16 or out.stride(1) != 1:
-        raise ValueError("out must be a bf16 [M, N] tensor with unit inner stride")
     sa, sb = _as_mfma(a), _as_mfma(b)
-    _call("mx_gemm_nt", f"gemm_nt", out.device, _ptr(a.codes), _ptr(sa), _ptr(b.codes), _ptr(sb), _ptr(out), M, N, K, out.stride(0), _stream(out))
-    return out
+    if out is None:
+        if _watched():
+            return torch.ops.torchtitan_amd.mx_gemm_nt(a.codes, sa, b.codes, sb)
+        return _gemm_nt_op(a.codes, sa, b.codes, sb)
+    if out.shape != (M, N) or out.dtype != torch.bfloat16 or out.stride(1) != 1:
+        raise ValueError("out must be a bf16 [M, N] tensor with unit inner stride")
+    return _gemm_nt_into(a.codes, sa, b.codes, sb, out)
 
 
 # --------------------------------------------------------------------------- 3-D weights
@@ -511,9 +564,11 @@ def mx_grouped_gemm_2d3d(a: MXData, b: MXData, offs: torch.Tensor,
     if offs.dtype != torch.int32 or offs.numel() != G:
         raise ValueError("offs must be int32 with one entry per group")
     if out is None:
-        out = torch.empty((T, N), dtype=torch.bfloat16, device=a.codes.device)
-    _call("mx_grouped_gemm_2d3d", "grouped_gemm_2d3d", out.device, _ptr(a.codes), _ptr(a.scales), _ptr(b.codes), _ptr(b.scales), _ptr(offs), _ptr(out), T, N, K, G, out.stride(0), a.scale_order, _stream(out))
-    return out
+        if _watched():
+            return torch.ops.torchtitan_amd.mx_grouped_gemm_2d3d(a.codes, a.scales, a.scale_order,
+                                                                 b.codes, b.scales, offs)
+        return _grouped_2d3d_op(a.codes, a.scales, a.scale_order, b.codes, b.scales, offs)
+    return _grouped_2d3d_into(a.codes, a.scales, a.scale_order, b.codes, b.scales, offs, out)
 
 
 def mx_grouped_gemm_2d2d(at: MXData, bt: MXData, offs: torch.Tensor,
