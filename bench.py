@@ -178,13 +178,16 @@ def time_decoder_block(dev, recipe):
     """BASELINE configs[2] for scale (not the headline): one Llama-3-8B-style decoder block (dim
     4096, 32 heads / 8 KV heads, FFN 14336, RMSNorm eps 1e-5, RoPE theta 5e5, init N(0, 0.02)),
     forward + backward at batch 1 x seq 8192, with all seven linears converted to MXFP8
-    (attention itself in bf16 through torch's SDPA) and unconverted in bf16."""
+    (attention itself in bf16 through torch's SDPA), the same with the two RMSNorms inside the casts
+    (opt-in), and unconverted in bf16."""
     import torch
     import torch.nn as nn
     import torch.nn.functional as F
 
     from torchtitan_amd import mx_tensor
     from torchtitan_amd.modules import FeedForward, Linear
+    from torchtitan_amd.mx_blocks import (feed_forward_fusable, mx_norm_feed_forward, mx_norm_linears,
+                                          norm_fusable)
     from torchtitan_amd.protocols import ModelConvertersContainer
     from torchtitan_amd.quantization.mx import MXFP8Converter
 
@@ -197,11 +200,15 @@ def time_decoder_block(dev, recipe):
             mk = lambda i, o: Linear.Config().build(in_features=i, out_features=o)
             self.wq, self.wk, self.wv, self.wo = mk(dim, dim), mk(dim, kv_heads * hd), mk(dim, kv_heads * hd), mk(dim, dim)
 
-        def forward(self, x, rope):
+        def forward(self, x, rope, norm):
             B, S, _ = x.shape
-            q = self.wq(x).view(B, S, heads, hd)
-            k = self.wk(x).view(B, S, kv_heads, hd)
-            v = self.wv(x).view(B, S, kv_heads, hd)
+            qkv_w = (self.wq.weight, self.wk.weight, self.wv.weight)
+            if norm_fusable(x, norm.weight, *qkv_w):  # opt-in: the norm inside the cast of x
+                q, k, v = mx_norm_linears(x, norm.weight, norm.eps, qkv_w)
+            else:
+                h = norm(x)
+                q, k, v = self.wq(h), self.wk(h), self.wv(h)
+            q, k, v = q.view(B, S, heads, hd), k.view(B, S, kv_heads, hd), v.view(B, S, kv_heads, hd)
             cos, sin = rope
 
             def rot(t):  # rotate pairs (even, odd) of the head dimension
@@ -223,8 +230,12 @@ def time_decoder_block(dev, recipe):
             self.ffn_norm = nn.RMSNorm(dim, eps=1e-5)
 
         def forward(self, x, rope):
-            h = x + self.attention(self.attention_norm(x), rope)
-            return h + self.feed_forward(self.ffn_norm(h))
+            h = x + self.attention(x, rope, self.attention_norm)
+            ff = self.feed_forward
+            w = (ff.w1.weight, ff.w2.weight, ff.w3.weight)
+            if norm_fusable(h, self.ffn_norm.weight, w[0], w[2]) and feed_forward_fusable(h, *w):
+                return h + mx_norm_feed_forward(h, self.ffn_norm.weight, self.ffn_norm.eps, *w)
+            return h + ff(self.ffn_norm(h))
 
     pos = torch.arange(seq, device=dev, dtype=torch.float32)
     freqs = 1.0 / (500000.0 ** (torch.arange(0, hd, 2, device=dev, dtype=torch.float32) / hd))
@@ -234,12 +245,14 @@ def time_decoder_block(dev, recipe):
     dy = torch.randn((1, seq, dim), device=dev, dtype=torch.bfloat16) * 1e-3
     flops = 3 * 2.0 * seq * (2 * dim * dim + 2 * dim * kv_heads * hd + 3 * dim * ffn)  # the seven linears
     out = {}
-    for name, convert in (("mxfp8_linears", True), ("bf16", False)):
+    for name, convert, norms in (("mxfp8_linears", True, False), ("mxfp8_linears_norms_in_casts", True, True),
+                                 ("bf16", False, False)):
         torch.manual_seed(0)
         blk = Block()
         if convert:
             ModelConvertersContainer.Config(
-                converters=[MXFP8Converter.Config(fqns=["attention", "feed_forward"], recipe_name=recipe)]
+                converters=[MXFP8Converter.Config(fqns=["attention", "feed_forward"], recipe_name=recipe,
+                                                  fuse_rmsnorm_cast=norms)]
             ).build(parallel_dims=None, model_compile_enabled=False).convert(blk)
         blk.to(dev).to(torch.bfloat16)
         with torch.no_grad():
@@ -259,11 +272,11 @@ def time_decoder_block(dev, recipe):
         torch.cuda.synchronize()
         s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         s.record()
-        for _ in range(4):
+        for _ in range(10):
             step()
         e.record()
         torch.cuda.synchronize()
-        ms = s.elapsed_time(e) / 4
+        ms = s.elapsed_time(e) / 10
         out[name] = {"ms": round(ms, 3), "linear_TFLOP/s_over_block_time": round(flops / ms / 1e9, 1)}
         del blk
         torch.cuda.empty_cache()

@@ -296,18 +296,25 @@ def norm_fusable(x: torch.Tensor, norm_weight: torch.Tensor | None, *weights: to
     return D % ops.BLOCK == 0 and (x.numel() // D) % ops.BLOCK == 0 and norm_weight.shape == (D,)
 
 
-def mx_norm_linears(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, weights) -> tuple:
+def _norm_eps(x: torch.Tensor, eps: float | None) -> float:
+    # nn.RMSNorm(eps=None) means the machine epsilon of the input's dtype
+    return float(torch.finfo(x.dtype).eps if eps is None else eps)
+
+
+def mx_norm_linears(x: torch.Tensor, norm_weight: torch.Tensor, eps: float | None, weights) -> tuple:
     """``tuple(F.linear(F.rms_norm(x, (dim,), norm_weight, eps), w) for w in weights)`` for
     converted weights without biases.  Callers check `norm_fusable` first."""
     weights = list(weights)
-    return _MXNormLinears.apply(x, norm_weight, float(eps), weights[0].mx_config, *[_unwrap(w) for w in weights])
+    return _MXNormLinears.apply(x, norm_weight, _norm_eps(x, eps), weights[0].mx_config,
+                                *[_unwrap(w) for w in weights])
 
 
-def mx_norm_feed_forward(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w1: torch.Tensor,
+def mx_norm_feed_forward(x: torch.Tensor, norm_weight: torch.Tensor, eps: float | None, w1: torch.Tensor,
                          w2: torch.Tensor, w3: torch.Tensor, bias2: torch.Tensor | None = None):
     """The SwiGLU block applied to ``F.rms_norm(x, (dim,), norm_weight, eps)``, norm inside the
     cast.  Callers check `norm_fusable(x, norm_weight, w1, w3)` and `feed_forward_fusable`."""
-    y = _MXFeedForward.apply(x, _unwrap(w1), _unwrap(w2), _unwrap(w3), w2.mx_config, norm_weight, float(eps))
+    y = _MXFeedForward.apply(x, _unwrap(w1), _unwrap(w2), _unwrap(w3), w2.mx_config, norm_weight,
+                             _norm_eps(x, eps))
     if bias2 is not None:
         y = y + _unwrap(bias2).to(y.dtype)
     return y
