@@ -372,6 +372,41 @@ def time_ffn_block(dev, recipe):
     return out
 
 
+def time_split_k(dev, recipe_mode):
+    """Beyond the headline: the weight gradient of a small weight over many tokens, where the
+    library splits the contraction (Qwen3-1.7B's wq, 2048 x 2048, over the 147 456 packed tokens
+    of the RL config), against the same GEMM through the entry point that does not split."""
+    import torch
+
+    from torchtitan_amd import _lib, ops
+
+    N, K, T = 2048, 2048, 147456
+    dyt = ops.to_mx_dim1(torch.randn((T, N), device=dev, dtype=torch.bfloat16) * 1e-3, recipe_mode, ops.MX_SCALES_MFMA)
+    xt = ops.to_mx_dim1(torch.randn((T, K), device=dev, dtype=torch.bfloat16), recipe_mode, ops.MX_SCALES_MFMA)
+    out = torch.empty((N, K), device=dev, dtype=torch.bfloat16)
+    lib = _lib.load()
+
+    def unsplit():
+        lib.mx_gemm_nt(ops._ptr(dyt.codes), ops._ptr(dyt.scales), ops._ptr(xt.codes), ops._ptr(xt.scales),
+                       ops._ptr(out), N, K, T, K, ops._stream(out))
+
+    res = {"shape": f"dW[{N},{K}] over {T} tokens",
+           "slices": int(lib.mx_gemm_nt_workspace_bytes(N, K, T)) // (N * K * 4) or 1}
+    for name, fn in (("split", lambda: ops.mx_gemm_nt(dyt, xt, out=out)), ("unsplit", unsplit)):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(5):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        us = s.elapsed_time(e) * 1e3 / 5
+        res[name] = {"us": round(us, 1), "TFLOP/s": round(2.0 * N * K * T / us / 1e6, 1)}
+    return res
+
+
 def time_policy_loss(dev):
     """Beyond the headline: the log-probabilities of one 2048-token completion over the RL
     config's vocabulary (151 936) from bf16 logits, forward + backward: fused kernels against
@@ -709,6 +744,8 @@ def main():
         del ffn, x, h, dy_h, dy_o
         torch.cuda.empty_cache()
         line["swiglu_block"] = time_ffn_block(dev, args.recipe)
+        torch.cuda.empty_cache()
+        line["wgrad_split_along_k"] = time_split_k(dev, recipe_mode)
         torch.cuda.empty_cache()
         line["policy_loss_logprobs"] = time_policy_loss(dev)
         torch.cuda.empty_cache()

@@ -217,6 +217,20 @@ int mx_gemm_nt(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b
                const uint8_t* b_scales, void* d, int64_t M, int64_t N, int64_t K, int64_t ldd,
                void* stream);
 
+/* The same GEMM for a caller that can lend scratch memory: shapes with few 256x256 output
+ * tiles and a long contraction (the wgrad of a small weight over many tokens,
+ * dW[N,K] = dY^T X with M in the tens of thousands) are then split along the contraction over
+ * several workgroups per tile, float32 partial sums in `workspace`, one reduction pass.
+ * mx_gemm_nt_workspace_bytes: bytes with which the shape would be split on the current device
+ * (0: mx_gemm_nt_ws runs exactly what mx_gemm_nt runs).  workspace: device memory, 16-byte
+ * aligned, contents undefined before and after; with less than the stated size (or NULL) the
+ * call falls back to mx_gemm_nt.  Results differ from mx_gemm_nt's only by the order of the
+ * float32 summation.  Same reference anchor as mx_gemm_nt. */
+int64_t mx_gemm_nt_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int mx_gemm_nt_ws(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                  const uint8_t* b_scales, void* d, int64_t M, int64_t N, int64_t K, int64_t ldd,
+                  void* workspace, int64_t workspace_bytes, void* stream);
+
 /* Grouped GEMM, 2D x 3D: for group g with rows [offs[g-1], offs[g]) of A:
  * D[rows, :] = deq(A[rows, :]) * deq(B[g])^T.  a_codes [T,K]; b_codes [G,N,K];
  * b_scales G consecutive MFMA-order blocks, each for [N, K/32].

@@ -194,3 +194,44 @@ def test_output_row_stride(device, M, N, K):
     ops.mx_gemm_nt(a, b, out=wide[:, 24:24 + N])
     assert rel_l2(_f32(bits_of(wide[:, 24:24 + N].contiguous())), _f32(ref)) <= TOL
     assert torch.all(wide[:, :24] == 7.0) and torch.all(wide[:, 24 + N:] == 7.0)
+
+
+@pytest.mark.parametrize("M,N,K", [(512, 512, 16384),    # 4 tiles, 128 K blocks
+                                   (700, 520, 16384),    # ragged tile edges
+                                   (768, 256, 12288 + 128)])  # 97 blocks: slices of unequal length
+def test_gemm_split_along_k_matches_oracle(device, M, N, K):
+    """Few output tiles and a long contraction: the library splits K over several workgroups per
+    tile (float32 partial sums in a workspace, one reduction).  Against the oracle, and against
+    the unsplit call: the two differ only by float32 summation order."""
+    from torchtitan_amd import _lib
+
+    lib = _lib.load()
+    with torch.cuda.device(device):
+        need = int(lib.mx_gemm_nt_workspace_bytes(M, N, K))
+    assert need > 0 and need % (M * N * 4) == 0, "the shape is meant to be split"
+    rng = np.random.default_rng(M + N + K)
+    a_bits = randn_bits(rng, (M, K), outliers=1e-3)
+    b_bits = randn_bits(rng, (N, K), std=0.02)
+    ac, asc = mo.cast_dim0(a_bits, mo.FLOOR)
+    bc, bsc = mo.cast_dim0(b_bits, mo.FLOOR)
+    ref = _f32(mo.mx_matmul_q(ac, asc, bc, bsc))
+    a = ops.MXData(torch.from_numpy(ac).to(device), torch.from_numpy(asc).to(device), ops.MX_SCALES_ROWMAJOR)
+    b = ops.MXData(torch.from_numpy(bc).to(device), torch.from_numpy(bsc).to(device), ops.MX_SCALES_ROWMAJOR)
+    launches = []
+    real_call = ops._call
+    ops._call = lambda name, *rest: (launches.append(name), real_call(name, *rest))[1]
+    try:
+        got = ops.mx_gemm_nt(a, b)
+        wide = torch.full((M, N + 24), 7.0, dtype=torch.bfloat16, device=device)
+        ops.mx_gemm_nt(a, b, out=wide[:, :N])  # row stride larger than N
+    finally:
+        ops._call = real_call
+    assert launches.count("mx_gemm_nt_ws") == 2
+    assert rel_l2(_f32(bits_of(got)), ref) <= TOL
+    assert torch.equal(wide[:, :N], got) and bool((wide[:, N:] == 7.0).all())
+    # the unsplit kernel on the same operands
+    sa, sb = ops._as_mfma(a), ops._as_mfma(b)
+    plain = torch.empty_like(got)
+    real_call("mx_gemm_nt", "gemm_nt", got.device, ops._ptr(a.codes), ops._ptr(sa), ops._ptr(b.codes),
+              ops._ptr(sb), ops._ptr(plain), M, N, K, N, ops._stream(plain))
+    assert rel_l2(got.float().cpu().numpy(), plain.float().cpu().numpy()) <= 3e-4

@@ -55,6 +55,12 @@ int launch_gemm_nt32(const uint8_t* a_codes, const uint8_t* a_scales, const uint
                      const uint8_t* b_scales, void* d, int64_t M, int64_t N, int64_t K,
                      int64_t ldd, hipStream_t st);
 }
+namespace mx {
+int splitk_slices(int64_t M, int64_t N, int64_t K);
+int launch_gemm_nt32_splitk(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                            const uint8_t* b_scales, void* d, int64_t M, int64_t N, int64_t K,
+                            int64_t ldd, int slices, void* workspace, hipStream_t st);
+}
 // 0: pick by shape; 1 / 2: the 16x16x128 tile kernel with 256x256 / 128x128 tiles for every
 // shape; 3: the persistent kernel wherever it is legal (comparison runs and tests)
 static int force_kernel = 0;
@@ -65,9 +71,9 @@ namespace mx { void set_debug_prof(uint64_t* buf); }
 // device buffer of 256*4*4 uint64 receiving per-wave cycle counts; nullptr switches timing off
 extern "C" void mx_debug_set_prof(void* buf) { mx::set_debug_prof((uint64_t*)buf); }
 
-extern "C" int mx_gemm_nt(const uint8_t* a_codes, const uint8_t* a_scales,
-                          const uint8_t* b_codes, const uint8_t* b_scales, void* d, int64_t M,
-                          int64_t N, int64_t K, int64_t ldd, void* stream) {
+static int check_dense(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                       const uint8_t* b_scales, const void* d, int64_t M, int64_t N, int64_t K,
+                       int64_t ldd) {
   if (M < 0 || N < 0 || K < 0 || ldd < N) return MX_ERR_INVALID_ARG;
   if (M == 0 || N == 0) return MX_OK;
   if (!a_codes || !a_scales || !b_codes || !b_scales || !d) return MX_ERR_INVALID_ARG;
@@ -76,11 +82,25 @@ extern "C" int mx_gemm_nt(const uint8_t* a_codes, const uint8_t* a_scales,
       ((uintptr_t)b_scales & 3) || ((uintptr_t)d & 1) || (K % 16))
     return MX_ERR_ALIGNMENT;
   if (256 * K > 0x7FFFFFFFll) return MX_ERR_UNSUPPORTED;
+  return MX_OK;
+}
+
+// What the persistent 32x32x64 kernel needs beyond the general checks.
+static bool persistent_ok(const void* d, int64_t N, int64_t K, int64_t ldd) {
+  return !(K % 128 || (uint64_t)K * 256 > 0x7FFFFFFFull || N % 8 || ldd % 8 || ((uintptr_t)d & 15) ||
+           (uint64_t)ldd * 512 > 0x7FFFFFFFull);
+}
+
+extern "C" int mx_gemm_nt(const uint8_t* a_codes, const uint8_t* a_scales,
+                          const uint8_t* b_codes, const uint8_t* b_scales, void* d, int64_t M,
+                          int64_t N, int64_t K, int64_t ldd, void* stream) {
+  const int rc = check_dense(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd);
+  if (rc != MX_OK || M == 0 || N == 0) return rc;
   DenseArgs p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, M, N, K, ldd};
   hipStream_t st = (hipStream_t)stream;
   if (M <= 128 || N <= 128 || force_kernel == 2) return launch_dense<128, 128>(p, st);
-  // Few 256x256 tiles leave most CUs of the persistent kernel idle (it has no split along K):
-  // up to 3/8 of the CUs' worth of tiles, four times as many 128x128 tiles finish sooner
+  // Few 256x256 tiles leave most CUs of the persistent kernel idle when the contraction is not
+  // split: up to 3/8 of the CUs' worth of tiles, four times as many 128x128 tiles finish sooner
   // (measured: 64 tiles 58 vs 71 us at K = 8192; 128 tiles 46 vs 43 us).
   static int num_cus = 0;
   if (num_cus == 0) {
@@ -91,7 +111,26 @@ extern "C" int mx_gemm_nt(const uint8_t* a_codes, const uint8_t* a_scales,
   }
   const int64_t tiles256 = ((M + 255) / 256) * ((N + 255) / 256);
   if (force_kernel == 0 && tiles256 * 8 <= (int64_t)num_cus * 3) return launch_dense<128, 128>(p, st);
-  if (force_kernel == 1 || K % 128 || (uint64_t)K * 256 > 0x7FFFFFFFull || N % 8 || ldd % 8 ||
-      ((uintptr_t)d & 15) || (uint64_t)ldd * 512 > 0x7FFFFFFFull) return launch_dense<256, 256>(p, st);
+  if (force_kernel == 1 || !persistent_ok(d, N, K, ldd)) return launch_dense<256, 256>(p, st);
   return launch_gemm_nt32(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd, st);
+}
+
+extern "C" int64_t mx_gemm_nt_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (M <= 128 || N <= 128 || K <= 0 || N % 8 || (uint64_t)N * 1024 > 0x7FFFFFFFull) return 0;
+  const int s = splitk_slices(M, N, K);
+  return s > 1 ? (int64_t)s * M * N * 4 : 0;
+}
+
+extern "C" int mx_gemm_nt_ws(const uint8_t* a_codes, const uint8_t* a_scales,
+                             const uint8_t* b_codes, const uint8_t* b_scales, void* d, int64_t M,
+                             int64_t N, int64_t K, int64_t ldd, void* workspace,
+                             int64_t workspace_bytes, void* stream) {
+  const int rc = check_dense(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd);
+  if (rc != MX_OK || M == 0 || N == 0) return rc;
+  const int64_t need = force_kernel == 0 ? mx_gemm_nt_workspace_bytes(M, N, K) : 0;
+  if (need == 0 || !workspace || workspace_bytes < need || ((uintptr_t)workspace & 15) ||
+      !persistent_ok(d, N, K, ldd))
+    return mx_gemm_nt(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd, stream);
+  return launch_gemm_nt32_splitk(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd,
+                                 (int)(need / (M * N * 4)), workspace, (hipStream_t)stream);
 }

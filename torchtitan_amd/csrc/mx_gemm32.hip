@@ -30,6 +30,7 @@
 namespace mx {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr int kT32 = 256;                        // tile edge (M and N)
 constexpr int kK32 = 64;                         // K per compute step
@@ -45,7 +46,9 @@ constexpr int kRing32 = 2 * kBlock32;            // 132 KB
 //   kGrouped2d3d  rows of A in groups (inclusive ends offs[g], all multiples of 128), group g
 //                 against B[g][N,K]; rows from offs[G-1] to M are written as zeros
 //   kGrouped2d2d  D[g][M,N] = A[M, lo_g:hi_g] B[N, lo_g:hi_g]^T, K = row length of A and B
-enum Gemm32Mode { kDense = 0, kGrouped2d3d = 1, kGrouped2d2d = 2 };
+//   kSplitK       as kGrouped2d2d with G equal slices of the K blocks worked out in the kernel
+//                 and float32 output: D[g][M,N] are partial sums for a reduction pass
+enum Gemm32Mode { kDense = 0, kGrouped2d3d = 1, kGrouped2d2d = 2, kSplitK = 3 };
 struct Gemm32Args {
   const uint8_t* a_codes;
   const uint8_t* a_scales;
@@ -159,6 +162,8 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   };
   if constexpr (MODE == kDense) {
     nb = (uint32_t)((p.M + kT32 - 1) / kT32) * tiles_n;
+  } else if constexpr (MODE == kSplitK) {
+    nb = G * (uint32_t)((p.M + kT32 - 1) / kT32) * tiles_n;
   } else if constexpr (MODE == kGrouped2d2d) {
     nb = G * (uint32_t)((p.M + kT32 - 1) / kT32) * tiles_n;
     int bad = 0;
@@ -249,6 +254,25 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       r.rows_b = p.N - (int64_t)tn * kT32;
       r.nblocks = g < G ? K / kKB : 1;
       r.empty = g >= G;
+    } else if (MODE == kSplitK) {
+      // slice g of the K blocks: ceil(blocks / G) each, the host picks G so that none is empty
+      const uint32_t tiles_m = (uint32_t)((p.M + kT32 - 1) / kT32), per_g = tiles_m * tiles_n;
+      const uint32_t g = t / per_g;
+      tile_coords(t - g * per_g, tiles_m, tiles_n, tm, tn);
+      const uint32_t blocks = K / kKB, per = (blocks + G - 1) / G;
+      const uint32_t b_lo = g * per, b_hi = b_lo + per < blocks ? b_lo + per : blocks;
+      const uint32_t lo = b_lo * kKB;
+      r.a = p.a_codes + (int64_t)tm * kT32 * K + lo;
+      r.b = p.b_codes + (int64_t)tn * kT32 * K + lo;
+      r.sa = p.a_scales + ((int64_t)(tm * 2) * ks_n + (lo >> 6)) * 256;
+      r.sb = p.b_scales + ((int64_t)(tn * 2) * ks_n + (lo >> 6)) * 256;
+      float* part = reinterpret_cast<float*>(p.d) +
+                    ((int64_t)g * p.M + (int64_t)tm * kT32) * p.ldd + (int64_t)tn * kT32;
+      r.d = reinterpret_cast<uint16_t*>(part);
+      r.rows_a = p.M - (int64_t)tm * kT32;
+      r.rows_b = p.N - (int64_t)tn * kT32;
+      r.koff = lo;
+      r.nblocks = b_hi - b_lo;
     } else {
       const uint32_t tiles_m = (uint32_t)((p.M + kT32 - 1) / kT32), per_g = tiles_m * tiles_n;
       const uint32_t g = t / per_g;
@@ -601,6 +625,26 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   auto epilogue = [&](const Tile32& t) {
     const int64_t rows_valid = t.rows_a;
     const uint32_t cols_valid = (uint32_t)(t.rows_b < kT32 ? t.rows_b : kT32);
+    if constexpr (MODE == kSplitK) {
+      // float32 partial sums straight from the accumulators: a lane stores 16 bytes of row li
+      // per sub-tile and q; short pieces, but the partial tiles are few and are read back at once
+      const uint32_t ld_b = (uint32_t)p.ldd * 4;
+      const __amdgpu_buffer_rsrc_t rp = make_rsrc(t.d, rows_valid * ld_b);
+      const uint32_t row_b = (wm * 128 + li) * ld_b;
+      static_for<0, 16>([&](auto i_) {
+        constexpr int m = decltype(i_)::value >> 2, n = decltype(i_)::value & 3;
+        const v16f a = acc[m][n];
+        static_for<0, 4>([&](auto q_) {
+          constexpr int q = decltype(q_)::value;
+          const uint32_t col = wn * 128 + n * 32 + 8 * q + 4 * lj;
+          const uint32_t v = col < cols_valid ? row_b + col * 4 : 0x80000000u;
+          const u32x4 w = {__float_as_uint(a[4 * q + 0]), __float_as_uint(a[4 * q + 1]),
+                           __float_as_uint(a[4 * q + 2]), __float_as_uint(a[4 * q + 3])};
+          __builtin_amdgcn_raw_buffer_store_b128(w, rp, v, m * 32 * ld_b, MX_STORE_AUX);
+        });
+      });
+      return;
+    }
     const uint32_t ldd_b = (uint32_t)p.ldd * 2;
     const __amdgpu_buffer_rsrc_t rd = make_rsrc(t.d, rows_valid * ldd_b);
     // lane's place in a stored piece: row (lane >> 3) + 8*pass, columns (lane & 7)*8 .. +7
@@ -756,6 +800,89 @@ int launch_gemm_nt32(const uint8_t* a_codes, const uint8_t* a_scales, const uint
   const int64_t nb = ((M + kT32 - 1) / kT32) * ((N + kT32 - 1) / kT32);
   if (debug_prof) return launch32<kDense, true>(p, nb, st);
   return launch32<kDense, false>(p, nb, st);
+}
+
+// ---- split along K for shapes whose 256x256 tiles do not fill the CUs ----------------------
+// Sum of the S float32 partial matrices [S][M][N], in slice order, rounded once to bf16.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ part, int S,
+                                                            int64_t M, int64_t N,
+                                                            uint16_t* __restrict__ d, int64_t ldd) {
+  const int64_t per_row = N / 8, i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= M * per_row) return;
+  const int64_t r = i / per_row, c = (i - r * per_row) * 8;
+  const float* src = part + r * N + c;
+  float acc[8];
+  {
+    const v4f lo = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(src));
+    const v4f hi = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(src) + 1);
+    acc[0] = lo.x; acc[1] = lo.y; acc[2] = lo.z; acc[3] = lo.w;
+    acc[4] = hi.x; acc[5] = hi.y; acc[6] = hi.z; acc[7] = hi.w;
+  }
+  for (int s = 1; s < S; ++s) {
+    const float* q = src + (int64_t)s * M * N;
+    const v4f lo = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(q));
+    const v4f hi = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(q) + 1);
+    acc[0] += lo.x; acc[1] += lo.y; acc[2] += lo.z; acc[3] += lo.w;
+    acc[4] += hi.x; acc[5] += hi.y; acc[6] += hi.z; acc[7] += hi.w;
+  }
+  const u32x4 w = {pack_bf16(acc[0], acc[1]), pack_bf16(acc[2], acc[3]), pack_bf16(acc[4], acc[5]),
+                   pack_bf16(acc[6], acc[7])};
+  *reinterpret_cast<u32x4*>(d + r * ldd + c) = w;
+}
+
+// Number of K slices for a dense shape on the persistent kernel (1: no split), from a cost model
+// in microseconds fitted to measurements on MI355X:
+//   one 128-deep block of a 256x256 tile takes a CU 1.6 us with the whole chip busy (about 10 %
+//   less with idle CUs: the clock is power-bound);
+//   unsplit, up to 3/8 of the CUs' worth of tiles go to the 128x128-tile kernel, 1.3 PFLOP/s
+//   times the share of the CUs its tiles cover;
+//   split, S slices run ceil(tiles * S / CUs) rounds of blocks / S each, then the float32
+//   partial tiles make a round trip through memory (8 bytes per element and slice at 3 TB/s)
+//   plus a second launch.
+// The split is taken when the model promises at least a fifth less time: a 2048 x 2048 weight
+// gradient over 147 456 tokens 1265 -> 559 us, over 32 768 tokens 198 -> 154 us; over 16 384
+// tokens it stays unsplit (105 vs 110 us).
+int splitk_slices(int64_t M, int64_t N, int64_t K) {
+  const int64_t grid = persistent_grid();
+  if (grid == 0 || K % kKB) return 1;
+  const int64_t tiles = ((M + kT32 - 1) / kT32) * ((N + kT32 - 1) / kT32), blocks = K / kKB;
+  if (tiles >= 2 * grid) return 1;
+  const double block_us = 1.6, flops = 2.0 * (double)M * (double)N * (double)K;
+  double plain;
+  if (tiles * 8 <= grid * 3) {
+    const double share = 4.0 * tiles / grid;
+    plain = flops / (1.3e9 * (share < 1.0 ? share : 1.0));  // 1.3e9 flop per microsecond
+  } else {
+    plain = (double)((tiles + grid - 1) / grid) * blocks * block_us * (tiles < grid ? 0.9 : 1.0);
+  }
+  int best = 1;
+  double best_us = plain;
+  for (int s = 2; s <= 8; ++s) {
+    const int64_t per = (blocks + s - 1) / s;
+    if (per < 16 || (int64_t)(s - 1) * per >= blocks) continue;
+    const double us = (double)((tiles * s + grid - 1) / grid) * per * block_us +
+                      (double)s * M * N * 8.0 / 3.0e6 + 8.0;
+    if (us < best_us) {
+      best = s;
+      best_us = us;
+    }
+  }
+  return best_us <= 0.8 * plain ? best : 1;
+}
+
+// D = sum over slices, through `workspace` (S * M * N floats).
+int launch_gemm_nt32_splitk(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                            const uint8_t* b_scales, void* d, int64_t M, int64_t N, int64_t K,
+                            int64_t ldd, int slices, void* workspace, hipStream_t st) {
+  const int64_t tiles_n = (N + kT32 - 1) / kT32, tiles = ((M + kT32 - 1) / kT32) * tiles_n;
+  Gemm32Args p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)workspace, M, N, K, N, nullptr,
+               slices, 0, (int32_t)tiles_n, nullptr};
+  const int rc = launch32<kSplitK, false>(p, tiles * slices, st);
+  if (rc != MX_OK) return rc;
+  const int64_t threads = M * (N / 8);
+  hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st,
+                     (const float*)workspace, slices, M, N, (uint16_t*)d, ldd);
+  return hipGetLastError() == hipSuccess ? MX_OK : MX_ERR_LAUNCH;
 }
 
 // Grouped forms with every group end a multiple of 128 and all scales in MFMA order

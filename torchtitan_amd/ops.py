@@ -420,10 +420,24 @@ def _as_mfma(d: MXData) -> torch.Tensor:
     return d.scales if d.scale_order == MX_SCALES_MFMA else scale_layout(d.scales)
 
 
+_gemm_workspace: dict = {}  # (device index, M, N, K) -> bytes the library would split with
+
+
 def _gemm_nt_into(a_codes, a_scales, b_codes, b_scales, out):
     M, K = a_codes.shape
+    N = b_codes.shape[0]
+    key = (out.device.index, M, N, K)
+    need = _gemm_workspace.get(key)
+    if need is None:
+        with torch.cuda.device(out.device):
+            need = _gemm_workspace[key] = int(_lib.load().mx_gemm_nt_workspace_bytes(M, N, K))
+    if need:  # few output tiles, long contraction: split over the CUs through float32 partial sums
+        ws = torch.empty(need, dtype=torch.uint8, device=out.device)
+        _call("mx_gemm_nt_ws", "gemm_nt_splitk", out.device, _ptr(a_codes), _ptr(a_scales), _ptr(b_codes),
+              _ptr(b_scales), _ptr(out), M, N, K, out.stride(0), _ptr(ws), need, _stream(out))
+        return out
     _call("mx_gemm_nt", "gemm_nt", out.device, _ptr(a_codes), _ptr(a_scales), _ptr(b_codes),
-          _ptr(b_scales), _ptr(out), M, b_codes.shape[0], K, out.stride(0), _stream(out))
+          _ptr(b_scales), _ptr(out), M, N, K, out.stride(0), _stream(out))
     return out
 
 
