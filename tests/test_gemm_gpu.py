@@ -235,3 +235,39 @@ def test_gemm_split_along_k_matches_oracle(device, M, N, K):
     real_call("mx_gemm_nt", "gemm_nt", got.device, ops._ptr(a.codes), ops._ptr(sa), ops._ptr(b.codes),
               ops._ptr(sb), ops._ptr(plain), M, N, K, N, ops._stream(plain))
     assert rel_l2(got.float().cpu().numpy(), plain.float().cpu().numpy()) <= 3e-4
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 256, 512), (1024, 768, 4096), (4096, 1024, 1024)])
+def test_gemm_agrees_with_the_vendor_block_scaled_gemm(device, M, N, K):
+    """An implementation of the same contract that shares nothing with this repository: the
+    vendor library's MX block-scaled GEMM behind torch._scaled_mm (e4m3 operands, one E8M0 scale
+    per 32 elements along K, row-major scale matrices) -- the call the reference's path ends in
+    (docs/mxfp8.md:36).  Operands with block scales spread over 2^-6 .. 2^5, so a scale applied
+    to the wrong block or read from the wrong byte would be far off.  The vendor kernel is asked
+    for fp16 output (it rounds that to nearest; its bf16 output is truncated, one step below
+    round-to-nearest on half of the elements).  Against that finer result this kernel's bf16
+    output may be off by its own rounding only: rel-L2 <= 2.5e-3 (bf16 rounding noise is about
+    1.5e-3); rounded on to bf16 the vendor result is the same number at more than 9 elements in
+    10 and never more than one bf16 step away (double rounding and summation order)."""
+    torch.manual_seed(M + K)
+
+    def spread(rows, lo, hi):  # one power of two per 32-element block
+        e = torch.randint(lo, hi, (rows, K // 32), device=device).repeat_interleave(32, 1)
+        return torch.exp2(e.float()).to(torch.bfloat16)
+
+    x = torch.randn(M, K, device=device, dtype=torch.bfloat16) * spread(M, -6, 6)
+    w = torch.randn(N, K, device=device, dtype=torch.bfloat16) * 0.02 * spread(N, -4, 4)
+    xq = ops.to_mx_dim0(x, "rceil", ops.MX_SCALES_ROWMAJOR)
+    wq = ops.to_mx_dim0(w, "rceil", ops.MX_SCALES_ROWMAJOR)
+    mine = ops.mx_gemm_nt(xq, wq)
+    try:
+        vendor = torch._scaled_mm(xq.codes.view(torch.float8_e4m3fn), wq.codes.view(torch.float8_e4m3fn).t(),
+                                  scale_a=xq.scales.view(torch.float8_e8m0fnu),
+                                  scale_b=wq.scales.view(torch.float8_e8m0fnu), out_dtype=torch.float16)
+    except (RuntimeError, ValueError, NotImplementedError) as ex:
+        pytest.skip(f"this torch build has no MX block-scaled GEMM: {ex}")
+    want = vendor.float().to(torch.bfloat16)
+    assert rel_l2(mine.float().cpu().numpy(), vendor.float().cpu().numpy()) <= 2.5e-3
+    steps = (mine.view(torch.int16).int() - want.view(torch.int16).int()).abs()
+    normal = vendor.abs() >= 2.0 ** -13  # below that fp16 itself is coarser than bf16
+    assert int(steps[normal].max()) <= 1 and float((steps == 0).float().mean()) > 0.9
