@@ -407,6 +407,70 @@ def time_split_k(dev, recipe_mode):
     return res
 
 
+def time_policy_layer_linears(dev, recipe):
+    """BASELINE configs[4] for scale (not the headline): the seven linears of one layer of the
+    Qwen3-1.7B-shaped policy (dim 2048, 16 heads / 8 KV heads of 128, FFN 6144) over the packed
+    tokens of one policy step (128 sequences, lengths uniform in [256, 2048]: 147 456 tokens),
+    each forward + backward through a converted module on inputs of the config's distributions,
+    then the hand-over of the layer's weights in MXFP8 form.  The weight gradients of the small
+    weights (64 to 192 output tiles over 147 456 tokens) are where the split along K acts."""
+    import torch
+    import torch.nn as nn
+
+    from torchtitan_amd import mx_tensor
+    from torchtitan_amd.modules import Linear
+    from torchtitan_amd.protocols import ModelConvertersContainer
+    from torchtitan_amd.quantization.mx import MXFP8Converter, export_mxfp8_state_dict
+
+    T, dim, kv, ffn = 147456, 2048, 1024, 6144
+    shapes = {"wq": (dim, dim), "wk": (dim, kv), "wv": (dim, kv), "wo": (dim, dim),
+              "w1": (dim, ffn), "w3": (dim, ffn), "w2": (ffn, dim)}
+    layer = nn.Module()
+    for name, (i, o) in shapes.items():
+        setattr(layer, name, Linear.Config().build(in_features=i, out_features=o))
+    holder = nn.Module()
+    holder.layer = layer
+    box = ModelConvertersContainer.Config(
+        converters=[MXFP8Converter.Config(fqns=["layer"], recipe_name=recipe)]
+    ).build(parallel_dims=None, model_compile_enabled=False)
+    box.convert(holder)
+    holder.to(dev).to(torch.bfloat16)
+    with torch.no_grad():
+        for lin in layer.children():
+            lin.weight.normal_(0.0, 0.02)
+    acts = {w: torch.randn((T, w), device=dev, dtype=torch.bfloat16).requires_grad_(True) for w in (dim, ffn)}
+    grads = {w: torch.randn((T, w), device=dev, dtype=torch.bfloat16) * 1e-3 for w in (dim, kv, ffn)}
+    flops = 3 * 2.0 * T * sum(i * o for i, o in shapes.values())
+
+    def step():
+        mx_tensor._cast_cache.clear()
+        for name, (i, o) in shapes.items():
+            lin = getattr(layer, name)
+            lin.weight.grad = None
+            acts[i].grad = None
+            lin(acts[i]).backward(grads[o])
+
+    for _ in range(2):
+        step()
+    torch.cuda.synchronize()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(4):
+        step()
+    e.record()
+    torch.cuda.synchronize()
+    ms = s.elapsed_time(e) / 4
+    export_mxfp8_state_dict(holder)
+    torch.cuda.synchronize()
+    s.record()
+    for _ in range(4):
+        export_mxfp8_state_dict(holder)
+    e.record()
+    torch.cuda.synchronize()
+    return {"tokens": T, "seven_linears_fwd_bwd": {"ms": round(ms, 3), "TFLOP/s": round(flops / ms / 1e9, 1)},
+            "weights_to_mxfp8_for_hand_over_us": round(s.elapsed_time(e) * 1e3 / 4, 1)}
+
+
 def time_policy_loss(dev):
     """Beyond the headline: the log-probabilities of one 2048-token completion over the RL
     config's vocabulary (151 936) from bf16 logits, forward + backward: fused kernels against
@@ -746,6 +810,8 @@ def main():
         line["swiglu_block"] = time_ffn_block(dev, args.recipe)
         torch.cuda.empty_cache()
         line["wgrad_split_along_k"] = time_split_k(dev, recipe_mode)
+        torch.cuda.empty_cache()
+        line["qwen3_1p7b_layer_linears"] = time_policy_layer_linears(dev, args.recipe)
         torch.cuda.empty_cache()
         line["policy_loss_logprobs"] = time_policy_loss(dev)
         torch.cuda.empty_cache()
