@@ -278,3 +278,51 @@ def test_moe_route_plan_matches_the_oracle(device, experts, top_k, tokens, align
     for e in range(experts):
         rows = np.nonzero(valid[ends[e]:ends[e + 1]])[0]
         assert len(rows) == counts[e] and (len(rows) == 0 or rows[-1] == len(rows) - 1)
+
+
+def test_moe_config_full_size_groups_equal_dense_gemms(device):
+    """The MoE configuration at full size (128 experts, dim 2048, expert FFN 768, 16384 tokens x
+    top-8 = 131 072 routed rows, group sizes from a softmax over seeded Gumbel-perturbed logits,
+    groups padded to the persistent kernels' 128 rows): no oracle at this size, but a grouped
+    GEMM is a stack of dense ones.  For the smallest, the largest and two other experts the
+    group's rows of the forward and dgrad outputs and its weight gradient are bit-identical to
+    the dense kernel on that group's operands alone (same codes, same K order); rows behind the
+    last group are zero."""
+    E, D, H, tokens, top_k = 128, 2048, 768, 16384, 8
+    torch.manual_seed(4)
+    logits = torch.randn(tokens, E, device=device) + 0.5 * torch.randn(E, device=device)
+    gumbel = -torch.log(-torch.log(torch.rand(tokens, E, device=device).clamp_min(1e-9)))
+    picked = torch.topk(torch.softmax(logits + gumbel, dim=-1), top_k, dim=-1).indices
+    counts = torch.bincount(picked.flatten(), minlength=E)
+    sizes = ((counts + 127) // 128 * 128).cpu().numpy()
+    assert counts.sum() == tokens * top_k and sizes.min() != sizes.max()
+    ends = np.cumsum(sizes)
+    Tp = int(ends[-1]) + 256  # two tiles' worth of rows that belong to no expert
+    offs = _sizes_to_offs(sizes, device)
+    x = torch.randn(Tp, D, device=device, dtype=torch.bfloat16)
+    dy = torch.randn(Tp, H, device=device, dtype=torch.bfloat16) * 1e-3
+    w = torch.randn(E, H, D, device=device, dtype=torch.bfloat16) * 0.02
+    xq0, xq1 = ops.to_mx_dim0_dim1(x, "rceil", L)
+    dyq0, dyq1 = ops.to_mx_dim0_dim1(dy, "rceil", L)
+    wq0, wq1 = ops.to_mx_dim0_dim1_batched(w, "rceil", L)
+    y = ops.mx_grouped_gemm_2d3d(xq0, wq0, offs)        # [Tp, H]
+    dx = ops.mx_grouped_gemm_2d3d(dyq0, wq1, offs)      # [Tp, D]
+    dw = ops.mx_grouped_gemm_2d2d(dyq1, xq1, offs)      # [E, H, D]
+    assert not bool(y[int(ends[-1]):].any()) and not bool(dx[int(ends[-1]):].any())
+    assert not bool(torch.isnan(y).any() | torch.isnan(dx).any()) and not bool(torch.isnan(dw).any())
+    from torchtitan_amd import _lib
+
+    order = np.argsort(sizes)
+    _lib.load().mx_debug_force_kernel(3)  # the dense calls on the same (persistent) kernel
+    try:
+        for g in (int(order[0]), int(order[-1]), int(order[E // 2]), E - 1):
+            lo, hi = int(ends[g] - sizes[g]), int(ends[g])
+            xg, dyg = x[lo:hi].contiguous(), dy[lo:hi].contiguous()
+            xg0, xg1 = ops.to_mx_dim0_dim1(xg, "rceil", L)
+            dyg0, dyg1 = ops.to_mx_dim0_dim1(dyg, "rceil", L)
+            wg0, wg1 = ops.to_mx_dim0_dim1(w[g].contiguous(), "rceil", L)
+            assert torch.equal(y[lo:hi], ops.mx_gemm_nt(xg0, wg0)), g
+            assert torch.equal(dx[lo:hi], ops.mx_gemm_nt(dyg0, wg1)), g
+            assert torch.equal(dw[g], ops.mx_gemm_nt(dyg1, xg1)), g
+    finally:
+        _lib.load().mx_debug_force_kernel(0)
