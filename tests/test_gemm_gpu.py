@@ -271,3 +271,36 @@ def test_gemm_agrees_with_the_vendor_block_scaled_gemm(device, M, N, K):
     steps = (mine.view(torch.int16).int() - want.view(torch.int16).int()).abs()
     normal = vendor.abs() >= 2.0 ** -13  # below that fp16 itself is coarser than bf16
     assert int(steps[normal].max()) <= 1 and float((steps == 0).float().mean()) > 0.9
+
+
+def test_policy_step_token_count_row_blocks_equal_small_calls(device):
+    """147 456 packed tokens (the policy step of the RL config) against a 2048 -> 6144 projection:
+    far beyond what the oracle can do, but every block of rows of the cast and of the GEMM
+    depends on those rows only.  Blocks from the start, the middle and the very end of the token
+    axis must equal the same kernels run on that slice alone, bit for bit; the weight gradient
+    over all tokens (split along K) must equal the sum of the gradients over two halves to
+    float32-summation accuracy."""
+    T, K, N = 147456, 2048, 6144
+    torch.manual_seed(11)
+    x = torch.randn(T, K, device=device, dtype=torch.bfloat16)
+    w = torch.randn(N, K, device=device, dtype=torch.bfloat16) * 0.02
+    xq0, xq1 = ops.to_mx_dim0_dim1(x, "rceil", ops.MX_SCALES_MFMA)
+    wq0 = ops.to_mx_dim0(w, "rceil", ops.MX_SCALES_MFMA)
+    y = ops.mx_gemm_nt(xq0, wq0)
+    for r0 in (0, 73728 - 128, T - 512):
+        part = x[r0:r0 + 512].contiguous()
+        pq0, pq1 = ops.to_mx_dim0_dim1(part, "rceil", ops.MX_SCALES_MFMA)
+        assert torch.equal(xq0.codes[r0:r0 + 512], pq0.codes)
+        assert torch.equal(xq1.codes[:, r0:r0 + 512], pq1.codes)
+        assert torch.equal(y[r0:r0 + 512], ops.mx_gemm_nt(pq0, wq0)), r0
+    del y
+    dy = torch.randn(T, 1024, device=device, dtype=torch.bfloat16) * 1e-3
+    dyq1 = ops.to_mx_dim1(dy, "rceil", ops.MX_SCALES_MFMA)
+    dw = ops.mx_gemm_nt(dyq1, xq1)  # [1024, 2048] over 147 456 tokens: split along K
+    halves = torch.zeros_like(dw, dtype=torch.float32)
+    for r0 in (0, T // 2):
+        a = ops.to_mx_dim1(dy[r0:r0 + T // 2].contiguous(), "rceil", ops.MX_SCALES_MFMA)
+        b = ops.to_mx_dim1(x[r0:r0 + T // 2].contiguous(), "rceil", ops.MX_SCALES_MFMA)
+        halves += ops.mx_gemm_nt(a, b).float()
+    # each half is rounded to bf16 before the sum: two roundings of 2^-9 relative against one
+    assert rel_l2(dw.float().cpu().numpy(), halves.cpu().numpy()) <= 3e-3
