@@ -514,7 +514,14 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   // other instruction is placed in the shadow of an MFMA; the sequence is pinned with
   // scheduling fences.  (Waits are written as assembly: the compiler rewrites the immediates
   // of s_waitcnt builtins from its own, here too pessimistic, model of what is outstanding.)
-  constexpr int kReadSlots = 9;  // 18 fragment reads, two per MFMA slot
+#ifndef MX_READ_SLOTS_A
+#define MX_READ_SLOTS_A 9
+#endif
+#ifndef MX_READ_SLOTS_B
+#define MX_READ_SLOTS_B 9
+#endif
+  // the 18 fragment reads of a step are spread evenly over its first kReadSlots MFMA slots
+  constexpr int kReadSlotsA = MX_READ_SLOTS_A, kReadSlotsB = MX_READ_SLOTS_B;
 // Output stores carry the nontemporal policy bit: written once, never re-read by this kernel,
 // and without it the output lines displace operand panels in L2 and the copies of the next
 // tile's first blocks queue behind the draining stores.
@@ -550,9 +557,9 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
         }
         mfma_one(f0, first_, i_);
 #ifndef MX_ABL_NO_READ
-        if constexpr (i < kReadSlots) {
-          read_piece(f1, sbase, std::integral_constant<int, 1>{}, std::integral_constant<int, 2 * i>{});
-          read_piece(f1, sbase, std::integral_constant<int, 1>{}, std::integral_constant<int, 2 * i + 1>{});
+        if constexpr (i < kReadSlotsA) {
+          constexpr int r0 = i * 18 / kReadSlotsA, r1 = (i + 1) * 18 / kReadSlotsA;
+          static_for<r0, r1>([&](auto r_) { read_piece(f1, sbase, std::integral_constant<int, 1>{}, r_); });
         }
 #endif
 #ifndef MX_ABL_NO_DMA
@@ -592,9 +599,9 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
         if constexpr (!skip && kCopiesA + j < 17) issue_piece(std::integral_constant<int, kCopiesA + j>{});
 #endif
 #ifndef MX_ABL_NO_READ
-        if constexpr (i < kReadSlots) {
-          read_piece(f0, sbase, std::integral_constant<int, 0>{}, std::integral_constant<int, 2 * i>{});
-          read_piece(f0, sbase, std::integral_constant<int, 0>{}, std::integral_constant<int, 2 * i + 1>{});
+        if constexpr (i < kReadSlotsB) {
+          constexpr int r0 = i * 18 / kReadSlotsB, r1 = (i + 1) * 18 / kReadSlotsB;
+          static_for<r0, r1>([&](auto r_) { read_piece(f0, sbase, std::integral_constant<int, 0>{}, r_); });
         }
 #endif
         __builtin_amdgcn_sched_barrier(0);
