@@ -166,6 +166,17 @@ def time_yardsticks(dev):
         except Exception as ex:  # a build of torch without that kernel: say so, measure the rest
             out[name] = {"error": f"{type(ex).__name__}: {str(ex)[:120]}"}
     del a, b, sa, sb, xb, wb
+    # this library's GEMM kernel, same shape, on operands that do not toggle the data paths (all
+    # ones): the same instruction stream at whatever clock the power limit then allows
+    from torchtitan_amd import ops
+
+    ones_a = ops.to_mx_dim0(torch.ones((M, DIM), device=dev, dtype=torch.bfloat16), "rceil", ops.MX_SCALES_MFMA)
+    ones_b = ops.to_mx_dim0(torch.ones((HIDDEN, DIM), device=dev, dtype=torch.bfloat16), "rceil", ops.MX_SCALES_MFMA)
+    dst = torch.empty((M, HIDDEN), device=dev, dtype=torch.bfloat16)
+    sec = timed(lambda: ops.mx_gemm_nt(ones_a, ones_b, out=dst), reps=10)
+    out["this_gemm_kernel_on_constant_operands"] = {"TFLOP/s": round(flops / sec / 1e12, 1),
+                                                     "frac_of_peak": round(flops / sec / 1e12 / PEAK_MXFP8_TFLOPS, 3)}
+    del ones_a, ones_b, dst
     src = torch.empty(256 * 1024 * 1024, device=dev, dtype=torch.bfloat16).normal_()
     dst = torch.empty_like(src)
     sec = timed(lambda: dst.copy_(src), reps=10)
