@@ -827,6 +827,11 @@ def main():
         line["policy_loss_logprobs"] = time_policy_loss(dev)
         torch.cuda.empty_cache()
         line["yardsticks"] = time_yardsticks(dev)
+        same = line["yardsticks"].get("this_gemm_kernel_on_constant_operands", {})
+        if "frac_of_peak" in same:
+            line["roofline"]["frac_on_constant_operands"] = same["frac_of_peak"]
+            line["roofline"]["power_note"] = ("the same kernel and shape on all-ones operands, timed in this run: the "
+                                              "gap to `frac` is the shader clock the power limit grants under random data")
         torch.cuda.empty_cache()
         line["llama3_8b_decoder_block"] = time_decoder_block(dev, args.recipe)
     if not args.no_cpu_baseline:
