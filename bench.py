@@ -295,6 +295,33 @@ def time_decoder_block(dev, recipe):
     return out
 
 
+def time_graph_replay(step, reps=5):
+    """Capture `step` (forward + backward on static tensors) in a HIP graph after a warm-up on a
+    side stream and return the mean replay time in ms: the same kernels without the host in
+    between."""
+    import torch
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    graph.replay()
+    torch.cuda.synchronize()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(reps):
+        graph.replay()
+    e.record()
+    torch.cuda.synchronize()
+    ms = s.elapsed_time(e) / reps
+    del graph
+    return ms
+
+
 def time_ffn_block(dev, recipe):
     """Beyond the headline: the whole SwiGLU block w2(silu(w1 x) * w3 x), forward + backward, at
     the same shapes, with the gate (and its backward) inside the cast kernels and with silu and
@@ -339,6 +366,8 @@ def time_ffn_block(dev, recipe):
         torch.cuda.synchronize()
         ms = s.elapsed_time(e) / reps
         out[name] = {"ms": round(ms, 3), "TFLOP/s": round(18.0 * M * DIM * HIDDEN / ms / 1e9, 1)}
+        if fuse:
+            out[name]["ms_replayed_from_a_hip_graph"] = round(time_graph_replay(step), 3)
         del ff, holder
     el = M * HIDDEN
     a = torch.randn((M, HIDDEN), device=dev, dtype=torch.bfloat16)
@@ -620,6 +649,8 @@ def time_moe_layer(dev, recipe_mode):
         torch.cuda.synchronize()
         ms = s.elapsed_time(e) / 5
         out[name] = {"ms": round(ms, 3), "TFLOP/s": round(18.0 * 16384 * 8 * 2048 * 768 / ms / 1e9, 1)}
+        if fuse:  # no host synchronisation anywhere in the layer: it can be captured whole
+            out[name]["ms_replayed_from_a_hip_graph"] = round(time_graph_replay(step), 3)
         del moe, holder
     return out
 
