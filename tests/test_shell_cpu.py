@@ -283,3 +283,46 @@ def test_module_filter_fn_rules():
     assert not module_filter_fn(nn.Linear(32, 40), "w", [])
     assert not module_filter_fn(nn.Embedding(32, 48), "tok_embeddings", [])
     assert module_filter_fn(nn.Linear(16, 16), "output", ["router"])
+
+
+def test_converted_weights_survive_deepcopy_and_checkpoint_as_plain_tensors():
+    """A converted model can be deep-copied (independent storage, still converted, still
+    Parameters) and its state dict holds plain tensors: torch.save / weights-only torch.load
+    round-trips it, and it loads into an unconverted model (and back) -- the parameter stays an
+    ordinary high-precision one for everything but its GEMMs
+    (torchtitan/components/quantization/mx.py:98-134 leaves checkpointing untouched)."""
+    import copy
+    import io
+
+    import torch
+    import torch.nn as nn
+
+    from torchtitan_amd.modules import FeedForward
+    from torchtitan_amd.mx_tensor import MXFP8Config, MXFP8TrainingWeight, wrap_parameter
+    from torchtitan_amd.quantization.mx import _plain_state_dict_entries
+
+    ff = FeedForward.Config(hidden_dim=64).build(dim=32)
+    ff.init_weights(init_std=0.02)
+    cfg = MXFP8Config("floor", False)
+    for lin in (ff.w1, ff.w2, ff.w3):   # what MXFP8Converter.convert does per module (it needs a GPU)
+        lin.weight = wrap_parameter(lin.weight, cfg)
+        lin.register_state_dict_post_hook(_plain_state_dict_entries)
+    twin = copy.deepcopy(ff)
+    for a, b in zip(ff.parameters(), twin.parameters()):
+        assert isinstance(b, MXFP8TrainingWeight) and isinstance(b, nn.Parameter) and b.requires_grad
+        assert b.mx_config == cfg and b.data_ptr() != a.data_ptr()
+        assert torch.equal(a.as_subclass(torch.Tensor), b.as_subclass(torch.Tensor))
+    sd = ff.state_dict()
+    assert all(type(v) is torch.Tensor for v in sd.values())
+    buf = io.BytesIO()
+    torch.save(sd, buf)
+    buf.seek(0)
+    back = torch.load(buf, weights_only=True)
+    plain = FeedForward.Config(hidden_dim=64).build(dim=32)
+    plain.load_state_dict(back)
+    with torch.no_grad():
+        for p in twin.parameters():
+            p.zero_()
+    twin.load_state_dict(plain.state_dict())
+    for a, b in zip(ff.parameters(), twin.parameters()):
+        assert isinstance(b, MXFP8TrainingWeight) and torch.equal(a.as_subclass(torch.Tensor), b.as_subclass(torch.Tensor))

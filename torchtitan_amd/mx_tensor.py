@@ -449,9 +449,24 @@ class MXFP8TrainingWeight(torch.Tensor):
             out = func(*args, **kwargs)
         return _rewrap(out, cls, cfg, func)
 
-    # plain-tensor semantics for pickling / deepcopy of the storage
+    # pickling: the plain tensor plus the config
     def __reduce_ex__(self, proto):
         return (MXFP8TrainingWeight, (self.as_subclass(torch.Tensor), self.mx_config))
+
+    def __deepcopy__(self, memo):
+        """An independent copy that is still a converted weight (and still a Parameter if this
+        one is): what ``copy.deepcopy(model)`` needs, e.g. when a trainer clones a converted model
+        per pipeline stage."""
+        if id(self) in memo:
+            return memo[id(self)]
+        data = self.as_subclass(torch.Tensor).detach().clone(memory_format=torch.preserve_format)
+        out = MXFP8TrainingWeight(data, self.mx_config)
+        if getattr(self, "_is_param", False):
+            out = torch.nn.Parameter(out, requires_grad=self.requires_grad)
+        else:
+            out.requires_grad_(self.requires_grad)
+        memo[id(self)] = out
+        return out
 
 
 _KEEP_WRAPPED = {

@@ -41,6 +41,13 @@ def has_rocm_capability(major: int, minor: int) -> bool:
     return got >= (major, minor)
 
 
+def _plain_state_dict_entries(module, state_dict, prefix, local_metadata):
+    for name, _ in module.named_parameters(recurse=False):
+        v = state_dict.get(prefix + name)
+        if isinstance(v, MXFP8TrainingWeight):
+            state_dict[prefix + name] = v.as_subclass(torch.Tensor)
+
+
 class MXFP8Converter(QuantizationConverter):
     """Wraps the weights of target ``nn.Linear`` modules and 3-D ``nn.Parameter`` experts in a
     tensor subclass that overrides ``F.linear`` and ``torch._grouped_mm`` with dynamically
@@ -116,17 +123,22 @@ class MXFP8Converter(QuantizationConverter):
         for fqn, mod in model.named_modules():
             if not self._matches(fqn):
                 continue
+            before = n_linear + n_grouped
             if isinstance(mod, nn.Linear):
                 if mod.in_features % 32:
                     logger.warning("skipping %s: in_features %d is not a multiple of 32", fqn, mod.in_features)
                     continue
                 mod.weight = wrap_parameter(mod.weight, cfg)
                 n_linear += 1
-                continue
-            for name, p in list(mod.named_parameters(recurse=False)):
-                if p.dim() == 3 and not isinstance(p, MXFP8TrainingWeight):
-                    setattr(mod, name, wrap_parameter(p, cfg))
-                    n_grouped += 1
+            else:
+                for name, p in list(mod.named_parameters(recurse=False)):
+                    if p.dim() == 3 and not isinstance(p, MXFP8TrainingWeight):
+                        setattr(mod, name, wrap_parameter(p, cfg))
+                        n_grouped += 1
+            if n_linear + n_grouped > before and not getattr(mod, "_mx_plain_state_dict", False):
+                # checkpoints hold plain tensors: loadable without this package, also weights-only
+                mod.register_state_dict_post_hook(_plain_state_dict_entries)
+                mod._mx_plain_state_dict = True
         inject_module_protocol(model, Linear, saved)
         verify_module_protocol(model, nn.Linear, Linear)
         logger.info(
