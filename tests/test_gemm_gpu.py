@@ -235,6 +235,13 @@ def test_gemm_split_along_k_matches_oracle(device, M, N, K):
     real_call("mx_gemm_nt", "gemm_nt", got.device, ops._ptr(a.codes), ops._ptr(sa), ops._ptr(b.codes),
               ops._ptr(sb), ops._ptr(plain), M, N, K, N, ops._stream(plain))
     assert rel_l2(got.float().cpu().numpy(), plain.float().cpu().numpy()) <= 3e-4
+    # without the workspace (or with too little of it) the call is the unsplit one
+    for ws, nbytes in ((None, 0), (torch.empty(need // 2, dtype=torch.uint8, device=device), need // 2)):
+        again = torch.empty_like(got)
+        real_call("mx_gemm_nt_ws", "gemm_nt_ws", got.device, ops._ptr(a.codes), ops._ptr(sa), ops._ptr(b.codes),
+                  ops._ptr(sb), ops._ptr(again), M, N, K, N, ops._ptr(ws) if ws is not None else None, nbytes,
+                  ops._stream(again))
+        assert torch.equal(again, plain)
 
 
 @pytest.mark.parametrize("M,N,K", [(256, 256, 512), (1024, 768, 4096), (4096, 1024, 1024)])
