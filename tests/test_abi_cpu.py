@@ -94,3 +94,12 @@ def test_new_entry_points_validate_arguments_before_any_launch():
     assert lib.mx_token_logprob_fwd(a16, 4, 100, 100, a16, a16, a16, None) == 2
     assert lib.mx_token_logprob_bwd(a16, 70000, 104, 104, a16, a16, a16, a16, 104, None) == 4
     assert lib.mx_token_logprob_bwd(a16, 4, 104, 104, a16, a16, None, a16, 104, None) == 1
+    # the GEMM that may split its contraction: same checks as mx_gemm_nt, decided before any launch
+    assert lib.mx_gemm_nt_ws(a16, a16, a16, a16, a16, 0, 64, 64, 64, None, 0, None) == 0
+    assert lib.mx_gemm_nt_ws(None, a16, a16, a16, a16, 64, 64, 64, 64, None, 0, None) == 1
+    assert lib.mx_gemm_nt_ws(a16, a16, a16, a16, a16, 64, 64, 64, 32, None, 0, None) == 1   # ldd < N
+    assert lib.mx_gemm_nt_ws(a16, a16, a16, a16, a16, 64, 64, 48, 64, None, 0, None) == 2   # K % 32
+    assert lib.mx_gemm_nt_ws(odd, a16, a16, a16, a16, 64, 64, 64, 64, None, 0, None) == 2
+    # shapes that are never split need no device to say so
+    assert lib.mx_gemm_nt_workspace_bytes(64, 64, 4096) == 0
+    assert lib.mx_gemm_nt_workspace_bytes(4096, 4096, 0) == 0
