@@ -326,3 +326,28 @@ def test_moe_config_full_size_groups_equal_dense_gemms(device):
             assert torch.equal(dw[g], ops.mx_gemm_nt(dyg1, xg1)), g
     finally:
         _lib.load().mx_debug_force_kernel(0)
+
+
+@pytest.mark.parametrize("G,N,K", [(40, 256, 512), (33, 512, 256), (67, 384, 256)])
+def test_grouped_wgrad_many_uneven_groups(device, G, N, K):
+    """From 32 groups on the persistent wgrad kernel deals its tiles by group length (longest
+    first, back and forth over XCDs and workgroups) instead of in tile order: every group's
+    gradient against the oracle, with empty groups, one long group and a tail that belongs to
+    no group."""
+    rng = np.random.default_rng(G * 13 + N + K)
+    sizes = rng.choice([0, 128, 128, 256, 384, 640], size=G).tolist()
+    sizes[G // 2] = 1536
+    sizes[3] = 0
+    T = sum(sizes) + 256
+    x_bits = randn_bits(rng, (T, K), outliers=1e-3)
+    dy_bits = randn_bits(rng, (T, N), std=1e-3)
+    offs = _sizes_to_offs(sizes, device)
+    x, dy = bf16_from_bits(x_bits, device), bf16_from_bits(dy_bits, device)
+    dw = ops.mx_grouped_gemm_2d2d(ops.to_mx_dim1(dy, "rceil", L), ops.to_mx_dim1(x, "rceil", L), offs)
+    ref = mo.grouped_wgrad(dy_bits, x_bits, np.cumsum(sizes), mo.RCEIL)
+    got = bits_of(dw)
+    for g, s_ in enumerate(sizes):
+        if s_ == 0:
+            assert np.all(got[g] == 0), g
+        else:
+            assert rel_l2(_f32(got[g]), _f32(ref[g])) <= TOL, g

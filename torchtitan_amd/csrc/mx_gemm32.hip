@@ -149,6 +149,9 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   //      tile number of every group (G + 2 entries, the last group being the zero rows behind
   //      offs[G-1]) is kept in the 2.5 KB that wave 0's output patch leaves unused.
   bool poison = false;
+  bool dealt = false;  // kGrouped2d2d: tiles dealt by length (below) instead of in tile order
+  constexpr uint32_t kMaxDealt = 640;  // two uint16 per group in wave 0's 2.5 KB of spare patch LDS
+  constexpr uint32_t kMinDealt = 32;   // fewer groups than that cannot be spread evenly over 8 XCDs
   uint32_t nb;
   // "any thread saw a bad group end", through a word of wave 1's spare patch bytes (the
   // kernel's whole 160 KB are dynamic LDS: a library reduction would ask for more)
@@ -166,12 +169,34 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     nb = G * (uint32_t)((p.M + kT32 - 1) / kT32) * tiles_n;
   } else if constexpr (MODE == kGrouped2d2d) {
     nb = G * (uint32_t)((p.M + kT32 - 1) / kT32) * tiles_n;
+    // group lengths in K blocks, kept for the dealing below (up to kMaxDealt groups)
+    uint16_t* g_blocks = reinterpret_cast<uint16_t*>(smem + kRing32 + 4608);
     int bad = 0;
     for (uint32_t g = tid; g < G; g += 256) {
       const int32_t hi = p.offs[g], lo = g ? p.offs[g - 1] : 0;
       bad |= (hi & 127) | (hi < lo) | (hi > (int64_t)K) | (lo < 0);
+      if (G <= kMaxDealt && G >= kMinDealt) {
+        const int64_t len = hi > lo ? ((int64_t)hi - lo) >> 7 : 0;
+        g_blocks[g] = (uint16_t)(len > 0xFFFF ? 0xFFFF : len);
+      }
     }
     poison = any_bad(bad);
+    dealt = !poison && G <= kMaxDealt && G >= kMinDealt;
+    if (dealt) {
+      // position of every group in the order of falling length (ties by index): G^2 / 256
+      // comparisons per thread, far below one tile's worth of time
+      uint16_t* g_sorted = g_blocks + kMaxDealt;
+      for (uint32_t g = tid; g < G; g += 256) {
+        const uint32_t mine = g_blocks[g];
+        uint32_t rank = 0;
+        for (uint32_t h = 0; h < G; ++h) {
+          const uint32_t o = g_blocks[h];
+          rank += (o > mine) | ((o == mine) & (h < g));
+        }
+        g_sorted[rank] = (uint16_t)g;
+      }
+      __syncthreads();
+    }
   } else {
     uint32_t* first = reinterpret_cast<uint32_t*>(smem + kRing32 + 4608);
     int bad = 0;
@@ -209,7 +234,25 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   const uint32_t per_xcd = (nb + 7) / 8;
   const uint32_t t_lo = xcd * per_xcd + idx;
   const uint32_t t_hi = (xcd + 1) * per_xcd < nb ? (xcd + 1) * per_xcd : nb;
-  const uint32_t n_my = t_lo < t_hi ? (t_hi - t_lo + wgs_per_xcd - 1) / wgs_per_xcd : 0;
+  uint32_t n_my = t_lo < t_hi ? (t_hi - t_lo + wgs_per_xcd - 1) / wgs_per_xcd : 0;
+  // kGrouped2d2d with uneven groups: a tile's time goes with its group's length, so tiles taken
+  // in tile order leave the workgroups with sums that differ by a fifth and more.  Instead the
+  // groups, in order of falling length, are dealt to the XCDs back and forth (j-th group of XCD
+  // x = position 8j + x or 8j + 7 - x), which keeps the tiles of a group, and their operand
+  // panels, inside one L2; and the tiles of an XCD's groups, still in that order, are dealt to
+  // its workgroups back and forth in the same way: every workgroup gets one tile from each band
+  // of neighbouring lengths.
+  auto snake = [](uint32_t band, uint32_t k, uint32_t width) -> uint32_t {
+    return (band & 1) ? width - 1 - k : k;
+  };
+  const uint32_t per_g2 = (uint32_t)((p.M + kT32 - 1) / kT32) * tiles_n;  // tiles of one group
+  if (MODE == kGrouped2d2d && dealt) {
+    const uint32_t full = G / 8, rest = G % 8;
+    const uint32_t groups_x = full + (snake(full, xcd, 8) < rest ? 1 : 0);
+    const uint32_t tiles_x = groups_x * per_g2;
+    const uint32_t bands = tiles_x / wgs_per_xcd, tail = tiles_x % wgs_per_xcd;
+    n_my = bands + (snake(bands, idx, wgs_per_xcd) < tail ? 1 : 0);
+  }
   if (n_my == 0) return;
   if (MODE != kDense && n_my > 120) return;  // more tiles than records: the host never launches this
 
@@ -275,8 +318,15 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       r.nblocks = b_hi - b_lo;
     } else {
       const uint32_t tiles_m = (uint32_t)((p.M + kT32 - 1) / kT32), per_g = tiles_m * tiles_n;
-      const uint32_t g = t / per_g;
-      tile_coords(t - g * per_g, tiles_m, tiles_n, tm, tn);
+      uint32_t g = t / per_g, in_g = t - g * per_g;
+      if (dealt) {  // t counts this workgroup's tiles: the i-th tile it was dealt
+        const uint16_t* g_sorted = reinterpret_cast<const uint16_t*>(smem + kRing32 + 4608) + kMaxDealt;
+        const uint32_t q = wgs_per_xcd * t + snake(t, idx, wgs_per_xcd);  // place in the XCD's tile list
+        const uint32_t j = q / per_g;
+        in_g = q - j * per_g;
+        g = g_sorted[8 * j + snake(j, xcd, 8)];
+      }
+      tile_coords(in_g, tiles_m, tiles_n, tm, tn);
       tn += tn0;
       const int64_t lo = poison ? 0 : (g ? p.offs[g - 1] : 0), hi = poison ? 0 : p.offs[g];
       r.a = p.a_codes + (int64_t)tm * kT32 * K + lo;
@@ -306,7 +356,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   };
   if constexpr (MODE != kDense) {
     for (uint32_t i = tid; i < n_my; i += 256) {
-      const Tile32 t = describe(t_lo + i * wgs_per_xcd);
+      const Tile32 t = describe((MODE == kGrouped2d2d && dealt) ? i : t_lo + i * wgs_per_xcd);
       uint64_t* q = reinterpret_cast<uint64_t*>(smem + record_offset(i));
       q[0] = (uint64_t)(uintptr_t)t.a;
       q[1] = (uint64_t)(uintptr_t)t.b;
@@ -929,7 +979,9 @@ int launch_grouped32_2d2d(const uint8_t* at_codes, const uint8_t* at_scales,
                           const uint8_t* bt_codes, const uint8_t* bt_scales, const int32_t* offs,
                           void* d, int64_t T, int64_t N, int64_t K, int64_t G, hipStream_t st) {
   Gemm32Args p{at_codes, at_scales, bt_codes, bt_scales, (uint16_t*)d, N, K, T, K, offs, G, 0, 0, debug_prof};
-  return launch_grouped32<kGrouped2d2d>(p, G * ((N + kT32 - 1) / kT32), (K + kT32 - 1) / kT32, st);
+  // tiles per column counted with G rounded up to the 8 XCDs: the kernel deals whole groups to
+  // XCDs, and the busiest XCD's share must fit its workgroups' records
+  return launch_grouped32<kGrouped2d2d>(p, (G + 7) / 8 * 8 * ((N + kT32 - 1) / kT32), (K + kT32 - 1) / kT32, st);
 }
 
 }  // namespace mx
