@@ -473,8 +473,12 @@ _dispatcher_ops.impl("mx_gemm_nt", _gemm_nt_op, "CUDA")
 _dispatcher_ops.impl("mx_grouped_gemm_2d3d", _grouped_2d3d_op, "CUDA")
 
 
+_dispatch_depth = getattr(torch._C, "_len_torch_dispatch_stack", None)
+
+
 def _watched() -> bool:
-    return torch._C._len_torch_dispatch_stack() > 0
+    """True while some TorchDispatchMode is active (a selective-checkpoint context is one)."""
+    return _dispatch_depth is not None and _dispatch_depth() > 0
 
 
 def op_sac_save_list() -> set:
