@@ -231,6 +231,18 @@ int mx_gemm_nt_ws(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t
                   const uint8_t* b_scales, void* d, int64_t M, int64_t N, int64_t K, int64_t ldd,
                   void* workspace, int64_t workspace_bytes, void* stream);
 
+/* D = deq(A) deq(B)^T + deq(A2) deq(B2)^T in one pass, both operand sets of the shapes of
+ * mx_gemm_nt: every output tile accumulates the products of the first set and then of the second
+ * before it is rounded once to bf16 and written.  The input gradient of a SwiGLU block,
+ * dx = d(h1) W1 + d(h3) W3 (autograd of torchtitan/models/common/feed_forward.py:61-62), as one
+ * GEMM instead of two and a bf16 add.  Shapes the persistent kernel does not take (M or N <= 128,
+ * K % 128, N % 8, ldd % 8, D not 16-byte aligned) return MX_ERR_UNSUPPORTED: the caller then
+ * runs two mx_gemm_nt calls and adds. */
+int mx_gemm_nt_pair(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                    const uint8_t* b_scales, const uint8_t* a2_codes, const uint8_t* a2_scales,
+                    const uint8_t* b2_codes, const uint8_t* b2_scales, void* d, int64_t M,
+                    int64_t N, int64_t K, int64_t ldd, void* stream);
+
 /* Grouped GEMM, 2D x 3D: for group g with rows [offs[g-1], offs[g]) of A:
  * D[rows, :] = deq(A[rows, :]) * deq(B[g])^T.  a_codes [T,K]; b_codes [G,N,K];
  * b_scales G consecutive MFMA-order blocks, each for [N, K/32].
@@ -248,6 +260,17 @@ int mx_grouped_gemm_2d3d(const uint8_t* a_codes, const uint8_t* a_scales, const 
                          const uint8_t* b_scales, const int32_t* offs, void* d, int64_t T,
                          int64_t N, int64_t K, int64_t G, int64_t ldd, int a_scale_order,
                          void* stream);
+
+/* The grouped 2D x 3D GEMM over two operand sets of the same shapes, summed per output tile as
+ * in mx_gemm_nt_pair: the expert block's input gradient d(h1) W1[g] + d(h3) W3[g]
+ * (autograd of torchtitan/models/common/moe/moe.py:59-76) as one grouped GEMM.  MFMA-order
+ * scales and the contract of the MX_SCALES_MFMA form above only. */
+int mx_grouped_gemm_2d3d_pair(const uint8_t* a_codes, const uint8_t* a_scales,
+                              const uint8_t* b_codes, const uint8_t* b_scales,
+                              const uint8_t* a2_codes, const uint8_t* a2_scales,
+                              const uint8_t* b2_codes, const uint8_t* b2_scales,
+                              const int32_t* offs, void* d, int64_t T, int64_t N, int64_t K,
+                              int64_t G, int64_t ldd, void* stream);
 
 /* Grouped GEMM, 2D x 2D (wgrad): D[g][N,K] = deq(A^T[:, rows_g]) * deq(B^T[:, rows_g])^T,
  * contracting over the tokens of group g.  at_codes [N,T] and bt_codes [K,T] are the

@@ -106,7 +106,12 @@ def test_feed_forward_close_to_bf16_and_trains(device):
 @pytest.mark.parametrize("tokens,dim,hidden", [(256, 256, 512), (96, 128, 352)])
 def test_feed_forward_fused_gate_matches_separate_ops(device, recipe, tokens, dim, hidden):
     """The SwiGLU block with the gate inside the cast kernel against the same block with silu and
-    the product as separate bf16 ops: the output and every gradient are bit-identical."""
+    the product as separate bf16 ops: the output and the weight gradients are bit-identical.  The
+    input gradient d(h1) W1 + d(h3) W3 is one GEMM in the fused block where the kernel takes the
+    shape (summed in float32, rounded once; `test_pair_gemm_*` pins it against the oracle) against
+    two GEMMs and a bf16 add.  The two halves partly cancel, so the separate form's three
+    roundings weigh about 3e-3 of the result: rel-L2 <= 5e-3 there, bit-identical where the fused
+    block falls back to two GEMMs."""
     torch.manual_seed(7)
     blocks = []
     for fuse in (True, False):
@@ -128,8 +133,11 @@ def test_feed_forward_fused_gate_matches_separate_ops(device, recipe, tokens, di
         y.backward(dy)
         ff = holder.feed_forward
         outs.append([y.detach(), xi.grad, ff.w1.weight.grad, ff.w2.weight.grad, ff.w3.weight.grad])
-    for got, want in zip(*outs):
-        assert torch.equal(got, want)
+    for i, (got, want) in enumerate(zip(*outs)):
+        if i == 1 and hidden % 128 == 0 and tokens > 128 and dim > 128:
+            assert rel_l2(got.float().cpu().numpy(), want.float().cpu().numpy()) <= 5e-3
+        else:
+            assert torch.equal(got, want), i
     # the fused forward keeps no bf16 gate tensor: the graph node of y is the fused function
     y = blocks[0].feed_forward(x.clone().requires_grad_(True))
     assert type(y.grad_fn).__name__ == "_MXFeedForwardBackward"
@@ -241,8 +249,8 @@ def test_per_op_checkpoint_policy_can_keep_gemm_outputs(device, fuse, monkeypatc
 
 @pytest.mark.parametrize("fuse", [True, False])
 def test_per_op_checkpoint_policy_keeps_grouped_gemm_outputs(device, fuse, monkeypatch):
-    """As above for the expert block: three forward grouped GEMMs kept, 6 launches of the 2d3d
-    kernel per step instead of 9, results unchanged."""
+    """As above for the expert block: three forward grouped GEMMs kept, three launches of the 2d3d
+    kernel per step fewer than under full checkpointing, results unchanged."""
     from torch.utils.checkpoint import CheckpointPolicy, checkpoint, create_selective_checkpoint_contexts
 
     save = ops.op_sac_save_list()
@@ -280,7 +288,9 @@ def test_per_op_checkpoint_policy_keeps_grouped_gemm_outputs(device, fuse, monke
             y.backward(dy)
             runs[how] = (launches.count("mx_grouped_gemm_2d3d"),
                          [y.detach(), xi.grad, ex.w1.grad.clone(), ex.w2.grad.clone(), ex.w3.grad.clone()])
-        assert [runs[h][0] for h in ("plain", "full", "per_op")] == [6, 9, 6]
+        # forward 3; backward: d(g), and d(x) as two launches or as one of the paired form
+        base = 4 if fuse else 6
+        assert [runs[h][0] for h in ("plain", "full", "per_op")] == [base, base + 3, base]
         for how in ("full", "per_op"):
             for a, b in zip(runs["plain"][1], runs[how][1]):
                 assert torch.equal(a, b)
@@ -490,7 +500,10 @@ def test_grouped_experts_swiglu_block(device):
 def test_grouped_experts_fused_block_matches_separate_ops(device, pad, align, dim, hidden):
     """The expert block as one fused function (one padding pass, gate inside the casts) against
     three converted grouped GEMMs around separate bf16 silu / product ops: bit-identical output
-    and gradients, on the persistent kernels (pad on, dims % 128) and on the general ones."""
+    and weight gradients, on the persistent kernels (pad on, dims % 128) and on the general ones;
+    the input gradient (float32 sum of both halves inside one grouped GEMM on the persistent
+    kernel) within rel-L2 5e-3 of the separate form's bf16 sum of two rounded halves that partly
+    cancel."""
     torch.manual_seed(21)
     moe_mod.set_token_group_alignment_size_m(align)
     try:
@@ -514,8 +527,11 @@ def test_grouped_experts_fused_block_matches_separate_ops(device, pad, align, di
             y = ex(xi, counts)
             y.backward(dy)
             outs.append([y.detach(), xi.grad, ex.w1.grad, ex.w2.grad, ex.w3.grad])
-        for got, want in zip(*outs):
-            assert torch.equal(got, want)
+        for i, (got, want) in enumerate(zip(*outs)):
+            if i == 1:  # dx: one grouped GEMM over both halves (one rounding) against two and an add
+                assert rel_l2(got.float().cpu().numpy(), want.float().cpu().numpy()) <= 5e-3
+            else:
+                assert torch.equal(got, want), i
         assert not torch.isnan(outs[0][0]).any() and outs[0][2].abs().sum() > 0
         from torchtitan_amd.mx_blocks import grouped_feed_forward_fusable as fusable
         assert fusable(x, blocks[0].w1, blocks[0].w2, blocks[0].w3)
@@ -531,7 +547,10 @@ def test_moe_layer_fused_routing_matches_torch_ops(device, score_before, dim, hi
     layer built from torch's gather / scatter / bmm around the converted experts.  Expert weight
     gradients are bit-identical (the experts see bit-identical inputs and output gradients); the
     output, dx and the router's gradient differ only by float32 summation order over top_k and
-    over the row dot products: rel-L2 <= 2e-3 (bf16 rounding of a differently ordered sum)."""
+    over the row dot products: rel-L2 <= 2e-3 (bf16 rounding of a differently ordered sum); 5e-3
+    for dx and the router's gradient, where the fused form also sums the two halves of the
+    experts' input gradient in float32 inside one grouped GEMM and the other rounds each half
+    (halves that partly cancel, so their roundings weigh about 3e-3 of the sum)."""
     torch.manual_seed(5)
     layers = []
     for fuse in (True, False):
@@ -559,8 +578,8 @@ def test_moe_layer_fused_routing_matches_torch_ops(device, score_before, dim, hi
     assert torch.equal(a["counts"], b["counts"]) and a["counts"].sum() == 2 * 96 * top_k
     for name in ("w1", "w2", "w3"):
         assert torch.equal(a[name], b[name]), name
-    for name in ("y", "dx", "gate"):
-        assert rel_l2(a[name].float().cpu().numpy(), b[name].float().cpu().numpy()) <= 2e-3, name
+    for name, tol in (("y", 2e-3), ("dx", 5e-3), ("gate", 5e-3)):
+        assert rel_l2(a[name].float().cpu().numpy(), b[name].float().cpu().numpy()) <= tol, name
 
 
 def test_weight_cast_cache_and_mxfp8_hand_over(device):

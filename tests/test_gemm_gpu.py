@@ -311,3 +311,30 @@ def test_policy_step_token_count_row_blocks_equal_small_calls(device):
         halves += ops.mx_gemm_nt(a, b).float()
     # each half is rounded to bf16 before the sum: two roundings of 2^-9 relative against one
     assert rel_l2(dw.float().cpu().numpy(), halves.cpu().numpy()) <= 3e-3
+
+
+@pytest.mark.parametrize("M,N,K", [(512, 384, 256), (300, 264, 128), (1024, 1024, 1024), (2048, 4096, 512)])
+def test_pair_gemm_is_one_gemm_over_the_concatenated_contraction(device, M, N, K):
+    """D = A B^T + A2 B2^T in one pass equals the oracle's MX matmul of [A | A2] with [B | B2]
+    (one rounding to bf16), and is at least as close to it as two GEMMs and a bf16 add."""
+    rng = np.random.default_rng(M + 3 * N + K)
+    ops_q = []
+    for std in (1.0, 0.02, 0.5, 0.05):
+        rows = M if len(ops_q) % 2 == 0 else N
+        ops_q.append(mo.cast_dim0(randn_bits(rng, (rows, K), std=std), mo.RCEIL))
+    (ac, asc), (bc, bsc), (a2c, a2sc), (b2c, b2sc) = ops_q
+    ref = _f32(mo.mx_matmul_q(np.concatenate([ac, a2c], 1), np.concatenate([asc, a2sc], 1),
+                              np.concatenate([bc, b2c], 1), np.concatenate([bsc, b2sc], 1)))
+    dev = lambda c, s_: ops.MXData(torch.from_numpy(c).to(device), torch.from_numpy(s_).to(device), ops.MX_SCALES_ROWMAJOR)
+    a, b, a2, b2 = dev(ac, asc), dev(bc, bsc), dev(a2c, a2sc), dev(b2c, b2sc)
+    launches = []
+    real_call = ops._call
+    ops._call = lambda name, *rest: (launches.append(name), real_call(name, *rest))[1]
+    try:
+        got = ops.mx_gemm_nt_pair(a, b, a2, b2)
+    finally:
+        ops._call = real_call
+    assert launches.count("mx_gemm_nt_pair") == 1 and "mx_gemm_nt" not in launches
+    err = rel_l2(_f32(bits_of(got)), ref)
+    two = ops.mx_gemm_nt(a, b) + ops.mx_gemm_nt(a2, b2)
+    assert err <= TOL and err <= rel_l2(_f32(bits_of(two)), ref) + 1e-5, err

@@ -351,3 +351,28 @@ def test_grouped_wgrad_many_uneven_groups(device, G, N, K):
             assert np.all(got[g] == 0), g
         else:
             assert rel_l2(_f32(got[g]), _f32(ref[g])) <= TOL, g
+
+
+@pytest.mark.parametrize("sizes,N,K,tail", [([256, 0, 128, 640], 256, 256, 128), ([128] * 9 + [1024, 0, 384], 512, 384, 0)])
+def test_grouped_pair_gemm_matches_the_oracle_over_the_concatenated_contraction(device, sizes, N, K, tail):
+    """Two operand sets summed per output tile in the grouped 2D x 3D kernel: against the oracle's
+    grouped forward of [X | X2] with [W | W2] (contraction 2K), rows behind the last group zero."""
+    rng = np.random.default_rng(sum(sizes) + N + K)
+    T, G = sum(sizes) + tail, len(sizes)
+    x_bits, x2_bits = randn_bits(rng, (T, K)), randn_bits(rng, (T, K), std=0.3)
+    w_bits, w2_bits = randn_bits(rng, (G, N, K), std=0.02), randn_bits(rng, (G, N, K), std=0.05)
+    offs = _sizes_to_offs(sizes, device)
+    q = lambda bits: ops.to_mx_dim0(bf16_from_bits(bits, device), "rceil", L)
+    qb = lambda bits: ops.to_mx_dim0_batched(bf16_from_bits(bits, device), "rceil", L)
+    launches = []
+    real_call = ops._call
+    ops._call = lambda name, *rest: (launches.append(name), real_call(name, *rest))[1]
+    try:
+        y = ops.mx_grouped_gemm_2d3d_pair(q(x_bits), qb(w_bits), q(x2_bits), qb(w2_bits), offs)
+    finally:
+        ops._call = real_call
+    assert "mx_grouped_gemm_2d3d_pair" in launches
+    ref = mo.grouped_fwd(np.concatenate([x_bits, x2_bits], 1), np.concatenate([w_bits, w2_bits], 2),
+                         np.cumsum(sizes), mo.RCEIL)
+    assert rel_l2(_f32(bits_of(y)), _f32(ref)) <= TOL
+    assert np.all(bits_of(y)[sum(sizes):] == 0)

@@ -60,6 +60,13 @@ struct Gemm32Args {
   int64_t G;
   int32_t tn0, tn_cnt;  // grouped modes: this launch covers tile columns [tn0, tn0 + tn_cnt)
   uint64_t* prof;  // timing build only: per wave {vmcnt wait, barrier wait, step body} cycles
+  // PAIR kernels: a second operand set of the same shapes; D = A B^T + A2 B2^T in one pass, every
+  // output tile running the K blocks of the first set and then those of the second before it is
+  // written out (dx = da W1 + db W3 of a SwiGLU block's backward)
+  const uint8_t* a2_codes = nullptr;
+  const uint8_t* a2_scales = nullptr;
+  const uint8_t* b2_codes = nullptr;
+  const uint8_t* b2_scales = nullptr;
 };
 
 // Where one 256x256 tile lives.
@@ -130,7 +137,7 @@ struct Frags32 {
   uint32_t sa, sb;
 };
 
-template <int MODE, bool PROF>
+template <int MODE, bool PROF, bool PAIR = false>
 __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   const int tid = threadIdx.x;
@@ -254,22 +261,27 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     n_my = bands + (snake(bands, idx, wgs_per_xcd) < tail ? 1 : 0);
   }
   if (n_my == 0) return;
+  if (PAIR) n_my *= 2;  // from here on n_my counts segments: two per output tile
   if (MODE != kDense && n_my > 120) return;  // more tiles than records: the host never launches this
 
   // Tile number -> operands.
-  auto describe = [&](uint32_t t) -> Tile32 {
+  auto describe = [&](uint32_t t, uint32_t seg) -> Tile32 {
     Tile32 r;
     r.poison = poison;
     r.koff = 0;
     r.empty = false;
+    const uint8_t* const a_codes = (PAIR && seg) ? p.a2_codes : p.a_codes;
+    const uint8_t* const a_scales = (PAIR && seg) ? p.a2_scales : p.a_scales;
+    const uint8_t* const b_codes = (PAIR && seg) ? p.b2_codes : p.b_codes;
+    const uint8_t* const b_scales = (PAIR && seg) ? p.b2_scales : p.b_scales;
     uint32_t tm, tn;
     if (MODE == kDense || (MODE == kGrouped2d3d && poison)) {
       tile_coords(t, (uint32_t)((p.M + kT32 - 1) / kT32), tiles_n, tm, tn);
       tn += tn0;
-      r.a = p.a_codes + (int64_t)tm * kT32 * K;
-      r.b = p.b_codes + (int64_t)tn * kT32 * K;
-      r.sa = p.a_scales + (int64_t)(tm * 2) * ks_n * 256;
-      r.sb = p.b_scales + (int64_t)(tn * 2) * ks_n * 256;
+      r.a = a_codes + (int64_t)tm * kT32 * K;
+      r.b = b_codes + (int64_t)tn * kT32 * K;
+      r.sa = a_scales + (int64_t)(tm * 2) * ks_n * 256;
+      r.sb = b_scales + (int64_t)(tn * 2) * ks_n * 256;
       r.d = p.d + (int64_t)tm * kT32 * p.ldd + (int64_t)tn * kT32;
       r.rows_a = p.M - (int64_t)tm * kT32;
       r.rows_b = p.N - (int64_t)tn * kT32;
@@ -288,10 +300,10 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       tn += tn0;
       const int64_t row0 = lo + (int64_t)tm * kT32;
       const uint32_t gb = g < G ? g : 0;  // the zero rows have no expert: any valid address
-      r.a = p.a_codes + row0 * K;
-      r.b = p.b_codes + ((int64_t)gb * p.N + (int64_t)tn * kT32) * K;
-      r.sa = p.a_scales + (row0 >> 7) * ks_n * 256;
-      r.sb = p.b_scales + ((int64_t)gb * ((p.N + 127) >> 7) + tn * 2) * ks_n * 256;
+      r.a = a_codes + row0 * K;
+      r.b = b_codes + ((int64_t)gb * p.N + (int64_t)tn * kT32) * K;
+      r.sa = a_scales + (row0 >> 7) * ks_n * 256;
+      r.sb = b_scales + ((int64_t)gb * ((p.N + 127) >> 7) + tn * 2) * ks_n * 256;
       r.d = p.d + row0 * p.ldd + (int64_t)tn * kT32;
       r.rows_a = hi - row0;
       r.rows_b = p.N - (int64_t)tn * kT32;
@@ -305,10 +317,10 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       const uint32_t blocks = K / kKB, per = (blocks + G - 1) / G;
       const uint32_t b_lo = g * per, b_hi = b_lo + per < blocks ? b_lo + per : blocks;
       const uint32_t lo = b_lo * kKB;
-      r.a = p.a_codes + (int64_t)tm * kT32 * K + lo;
-      r.b = p.b_codes + (int64_t)tn * kT32 * K + lo;
-      r.sa = p.a_scales + ((int64_t)(tm * 2) * ks_n + (lo >> 6)) * 256;
-      r.sb = p.b_scales + ((int64_t)(tn * 2) * ks_n + (lo >> 6)) * 256;
+      r.a = a_codes + (int64_t)tm * kT32 * K + lo;
+      r.b = b_codes + (int64_t)tn * kT32 * K + lo;
+      r.sa = a_scales + ((int64_t)(tm * 2) * ks_n + (lo >> 6)) * 256;
+      r.sb = b_scales + ((int64_t)(tn * 2) * ks_n + (lo >> 6)) * 256;
       float* part = reinterpret_cast<float*>(p.d) +
                     ((int64_t)g * p.M + (int64_t)tm * kT32) * p.ldd + (int64_t)tn * kT32;
       r.d = reinterpret_cast<uint16_t*>(part);
@@ -329,10 +341,10 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       tile_coords(in_g, tiles_m, tiles_n, tm, tn);
       tn += tn0;
       const int64_t lo = poison ? 0 : (g ? p.offs[g - 1] : 0), hi = poison ? 0 : p.offs[g];
-      r.a = p.a_codes + (int64_t)tm * kT32 * K + lo;
-      r.b = p.b_codes + (int64_t)tn * kT32 * K + lo;
-      r.sa = p.a_scales + ((int64_t)(tm * 2) * ks_n + (lo >> 6)) * 256;
-      r.sb = p.b_scales + ((int64_t)(tn * 2) * ks_n + (lo >> 6)) * 256;
+      r.a = a_codes + (int64_t)tm * kT32 * K + lo;
+      r.b = b_codes + (int64_t)tn * kT32 * K + lo;
+      r.sa = a_scales + ((int64_t)(tm * 2) * ks_n + (lo >> 6)) * 256;
+      r.sb = b_scales + ((int64_t)(tn * 2) * ks_n + (lo >> 6)) * 256;
       r.d = p.d + ((int64_t)g * p.M + (int64_t)tm * kT32) * p.ldd + (int64_t)tn * kT32;
       r.rows_a = p.M - (int64_t)tm * kT32;
       r.rows_b = p.N - (int64_t)tn * kT32;
@@ -356,7 +368,8 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   };
   if constexpr (MODE != kDense) {
     for (uint32_t i = tid; i < n_my; i += 256) {
-      const Tile32 t = describe((MODE == kGrouped2d2d && dealt) ? i : t_lo + i * wgs_per_xcd);
+      const uint32_t ti = PAIR ? i >> 1 : i;  // PAIR: records 2t and 2t+1 are the two segments of tile t
+      const Tile32 t = describe((MODE == kGrouped2d2d && dealt) ? ti : t_lo + ti * wgs_per_xcd, PAIR ? i & 1 : 0);
       uint64_t* q = reinterpret_cast<uint64_t*>(smem + record_offset(i));
       q[0] = (uint64_t)(uintptr_t)t.a;
       q[1] = (uint64_t)(uintptr_t)t.b;
@@ -376,7 +389,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   // does not see an LDS read, see read_piece; every lane reads the same 64 bytes)
   auto get_tile = [&](uint32_t i) -> Tile32 {
     if constexpr (MODE == kDense) {
-      return describe(t_lo + i * wgs_per_xcd);
+      return describe(t_lo + (PAIR ? i >> 1 : i) * wgs_per_xcd, PAIR ? i & 1 : 0);
     } else {
       const uint32_t addr = lds_base + record_offset(i);
       v4i r0, r1, r2, r3;
@@ -773,11 +786,14 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   // ---- tiles; at the top of every tile f0 holds the fragments of its first half block (the
   // last step of a tile has already read them from the next tile's first block, which the
   // loader fetched like any other block).
-  for (uint32_t tile = 0; tile < n_my; ++tile) {
+  for (uint32_t tile = 0; tile < n_my; tile += PAIR ? 2 : 1) {
     const Tile32 t = get_tile(tile);
     {
+      // PAIR: the loader walks both segments of the tile one after the other (same K for both);
+      // for the compute stream they are one run of blocks
+      const uint32_t nblocks = PAIR ? 2 * t.nblocks : t.nblocks;
       block_steps(f0, f1, std::true_type{});
-      for (uint32_t i = 1; i < t.nblocks; ++i) block_steps(f0, f1, std::false_type{});
+      for (uint32_t i = 1; i < nblocks; ++i) block_steps(f0, f1, std::false_type{});
       // the next tile's first fragments were read in the last step: make them ordinary
       // values before anything else runs (a register the compiler moved or spilled while
       // its read was still in flight would lose the data)
@@ -828,9 +844,9 @@ static int64_t persistent_grid() {
   return grid;
 }
 
-template <int MODE, bool PROF>
+template <int MODE, bool PROF, bool PAIR = false>
 static int launch32(const Gemm32Args& p, int64_t nb, hipStream_t st) {
-  auto kern = gemm_nt32_kernel<MODE, PROF>;
+  auto kern = gemm_nt32_kernel<MODE, PROF, PAIR>;
   constexpr int lds = kRing32 + 4 * 7168;  // ring + one output patch per wave = all 160 KB
   static bool configured = false;
   if (!configured) {
@@ -948,19 +964,24 @@ int launch_gemm_nt32_splitk(const uint8_t* a_codes, const uint8_t* a_scales, con
 // launches over ranges of tile columns.
 constexpr int64_t kMaxRecords = 120;
 
-template <int MODE>
+template <int MODE, bool PAIR = false>
 static int launch_grouped32(Gemm32Args p, int64_t tiles_per_column, int64_t tiles_n, hipStream_t st) {
   const int64_t grid = persistent_grid();
   if (grid == 0) return MX_ERR_LAUNCH;
   // tiles of one launch <= grid * kMaxRecords - slack for the rounding of the per-XCD runs
-  int64_t cols = (grid * kMaxRecords - 8 * (grid / 8)) / tiles_per_column;
+  // (PAIR: two records per tile)
+  int64_t cols = (grid * (kMaxRecords / (PAIR ? 2 : 1)) - 8 * (grid / 8)) / tiles_per_column;
   if (cols < 1) return MX_ERR_UNSUPPORTED;
   if (cols > tiles_n) cols = tiles_n;
   for (int64_t tn0 = 0; tn0 < tiles_n; tn0 += cols) {
     p.tn0 = (int32_t)tn0;
     p.tn_cnt = (int32_t)(tiles_n - tn0 < cols ? tiles_n - tn0 : cols);
     const int64_t nb = tiles_per_column * p.tn_cnt;
-    const int rc = p.prof ? launch32<MODE, true>(p, nb, st) : launch32<MODE, false>(p, nb, st);
+    int rc;
+    if constexpr (PAIR)
+      rc = launch32<MODE, false, true>(p, nb, st);
+    else
+      rc = p.prof ? launch32<MODE, true>(p, nb, st) : launch32<MODE, false>(p, nb, st);
     if (rc != MX_OK) return rc;
   }
   return MX_OK;
@@ -972,6 +993,27 @@ int launch_grouped32_2d3d(const uint8_t* a_codes, const uint8_t* a_scales, const
   Gemm32Args p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, T, N, K, ldd, offs, G, 0, 0, debug_prof};
   // an upper bound of the tile rows: every group may add one partly filled tile
   return launch_grouped32<kGrouped2d3d>(p, (T + kT32 - 1) / kT32 + G + 1, (N + kT32 - 1) / kT32, st);
+}
+
+// D = A B^T + A2 B2^T (dense) and its grouped 2D x 3D form: both operand sets of the same shapes.
+int launch_gemm_nt32_pair(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                          const uint8_t* b_scales, const uint8_t* a2_codes, const uint8_t* a2_scales,
+                          const uint8_t* b2_codes, const uint8_t* b2_scales, void* d, int64_t M,
+                          int64_t N, int64_t K, int64_t ldd, hipStream_t st) {
+  Gemm32Args p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, M, N, K, ldd, nullptr, 0, 0, 0, nullptr,
+               a2_codes, a2_scales, b2_codes, b2_scales};
+  const int64_t nb = ((M + kT32 - 1) / kT32) * ((N + kT32 - 1) / kT32);
+  return launch32<kDense, false, true>(p, nb, st);
+}
+
+int launch_grouped32_2d3d_pair(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                               const uint8_t* b_scales, const uint8_t* a2_codes,
+                               const uint8_t* a2_scales, const uint8_t* b2_codes,
+                               const uint8_t* b2_scales, const int32_t* offs, void* d, int64_t T,
+                               int64_t N, int64_t K, int64_t G, int64_t ldd, hipStream_t st) {
+  Gemm32Args p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, T, N, K, ldd, offs, G, 0, 0, nullptr,
+               a2_codes, a2_scales, b2_codes, b2_scales};
+  return launch_grouped32<kGrouped2d3d, true>(p, (T + kT32 - 1) / kT32 + G + 1, (N + kT32 - 1) / kT32, st);
 }
 
 // D[g][N, K] = A^T[N, lo:hi] B^T[K, lo:hi]^T; operand rows are T long.

@@ -130,7 +130,34 @@ int launch_grouped32_2d3d(const uint8_t* a_codes, const uint8_t* a_scales, const
 int launch_grouped32_2d2d(const uint8_t* at_codes, const uint8_t* at_scales,
                           const uint8_t* bt_codes, const uint8_t* bt_scales, const int32_t* offs,
                           void* d, int64_t T, int64_t N, int64_t K, int64_t G, hipStream_t st);
+int launch_grouped32_2d3d_pair(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                               const uint8_t* b_scales, const uint8_t* a2_codes,
+                               const uint8_t* a2_scales, const uint8_t* b2_codes,
+                               const uint8_t* b2_scales, const int32_t* offs, void* d, int64_t T,
+                               int64_t N, int64_t K, int64_t G, int64_t ldd, hipStream_t st);
 }  // namespace mx
+
+extern "C" int mx_grouped_gemm_2d3d_pair(const uint8_t* a_codes, const uint8_t* a_scales,
+                                         const uint8_t* b_codes, const uint8_t* b_scales,
+                                         const uint8_t* a2_codes, const uint8_t* a2_scales,
+                                         const uint8_t* b2_codes, const uint8_t* b2_scales,
+                                         const int32_t* offs, void* d, int64_t T, int64_t N,
+                                         int64_t K, int64_t G, int64_t ldd, void* stream) {
+  if (T < 0 || N < 0 || K < 0 || G <= 0 || ldd < N) return MX_ERR_INVALID_ARG;
+  if (T == 0 || N == 0) return MX_OK;
+  if (!a_codes || !a_scales || !b_codes || !b_scales || !a2_codes || !a2_scales || !b2_codes ||
+      !b2_scales || !offs || !d)
+    return MX_ERR_INVALID_ARG;
+  if (K == 0 || K % 128 || N % 8 || ldd % 8 || T % 128) return MX_ERR_ALIGNMENT;
+  if (((uintptr_t)a_codes & 15) || ((uintptr_t)b_codes & 15) || ((uintptr_t)a2_codes & 15) ||
+      ((uintptr_t)b2_codes & 15) || ((uintptr_t)a_scales & 3) || ((uintptr_t)b_scales & 3) ||
+      ((uintptr_t)a2_scales & 3) || ((uintptr_t)b2_scales & 3) || ((uintptr_t)d & 15))
+    return MX_ERR_ALIGNMENT;
+  if (256 * K > 0x7FFFFFFFll || G > 638 || ldd * 512 > 0x7FFFFFFFll) return MX_ERR_UNSUPPORTED;
+  return launch_grouped32_2d3d_pair(a_codes, a_scales, b_codes, b_scales, a2_codes, a2_scales,
+                                    b2_codes, b2_scales, offs, d, T, N, K, G, ldd,
+                                    (hipStream_t)stream);
+}
 
 extern "C" int mx_grouped_gemm_2d3d(const uint8_t* a_codes, const uint8_t* a_scales,
                                     const uint8_t* b_codes, const uint8_t* b_scales,

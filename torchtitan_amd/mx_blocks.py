@@ -178,7 +178,8 @@ class _MXFeedForward(torch.autograd.Function):
         dnw = None
         if ctx.need_dx:
             w1q1, w3q1 = take(), take()
-            dx = ops.mx_gemm_nt(da0, w1q1) + ops.mx_gemm_nt(db0, w3q1)
+            # dx = d(h1) W1 + d(h3) W3 as one GEMM: summed in float32, rounded once
+            dx = ops.mx_gemm_nt_pair(da0, w1q1, db0, w3q1)
             if ctx.normed:
                 dx, dnw = _rms_norm_backward(dx, *saved[:3], ctx.needs_input_grad[0], ctx.needs_input_grad[5])
             if dx is not None:
@@ -398,7 +399,16 @@ class _MXGroupedFeedForward(torch.autograd.Function):
         if ctx.need_dx:
             w1q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
             w3q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
-            dx = _grouped_2d3d_padded(da0, w1q1, offs_p, back) + _grouped_2d3d_padded(db0, w3q1, offs_p, back)
+            # d(h1) W1[g] + d(h3) W3[g] as one grouped GEMM (summed in float32, rounded once); the
+            # spare zero row behind it serves rows that belong to no group
+            Tp, D = da0.codes.shape[0], w1q1.codes.shape[1]
+            if back is None:
+                dx = ops.mx_grouped_gemm_2d3d_pair(da0, w1q1, db0, w3q1, offs_p)
+            else:
+                buf = torch.empty((Tp + 1, D), dtype=torch.bfloat16, device=da0.codes.device)
+                buf[Tp].zero_()
+                ops.mx_grouped_gemm_2d3d_pair(da0, w1q1, db0, w3q1, offs_p, buf[:Tp])
+                dx = buf[back]
             dx = cast_back(dx, ctx.dtypes[0])
         return dx, dw1, dw2, dw3, None, None
 
@@ -512,17 +522,16 @@ class _MXRoutedExperts(torch.autograd.Function):
             w3q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
             need_dxp = need_dx or (need_ds and score_before)
             if need_dxp:
-                # gradient of the (scaled) routed inputs, padded layout: the two halves from w1
-                # and w3; their bf16 sum is formed inside the kernels that consume it
-                dxp1 = ops.mx_grouped_gemm_2d3d(da0, w1q1, offs_p)
-                dxp3 = ops.mx_grouped_gemm_2d3d(db0, w3q1, offs_p)
+                # gradient of the (scaled) routed inputs, padded layout: the halves from w1 and
+                # w3 summed inside one grouped GEMM (float32, one rounding)
+                dxp = ops.mx_grouped_gemm_2d3d_pair(da0, w1q1, db0, w3q1, offs_p)
             if need_dx:
-                dx = cast_back(ops.moe_combine(dxp1, pos, scores if score_before else None, dxp3), ctx.dtypes[0])
+                dx = cast_back(ops.moe_combine(dxp, pos, scores if score_before else None), ctx.dtypes[0])
             if need_ds:
                 other = saved.pop(0)  # x (scores in front of the experts) or the expert outputs
                 token = torch.arange(T * k, device=pos.device, dtype=torch.int64).div_(k, rounding_mode="floor")
                 if score_before:
-                    ds = ops.moe_row_dot(dxp1, pos.view(-1), other, token, dxp3)
+                    ds = ops.moe_row_dot(dxp, pos.view(-1), other, token)
                 else:
                     ds = ops.moe_row_dot(other, pos.view(-1), dob, token)
                 ds = cast_back(ds.view(T, k), ctx.dtypes[1])

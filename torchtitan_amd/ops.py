@@ -506,6 +506,23 @@ def mx_gemm_nt(a: MXData, b: MXData, out: torch.Tensor | None = None) -> torch.T
     return _gemm_nt_into(a.codes, sa, b.codes, sb, out)
 
 
+def mx_gemm_nt_pair(a: MXData, b: MXData, a2: MXData, b2: MXData) -> torch.Tensor:
+    """bf16 deq(a) @ deq(b)^T + deq(a2) @ deq(b2)^T: one GEMM whose output tiles accumulate both
+    products before they are rounded and written, where the persistent kernel takes the shape;
+    otherwise two GEMMs and a bf16 add."""
+    M, K = a.codes.shape
+    N = b.codes.shape[0]
+    if a2.codes.shape != (M, K) or b2.codes.shape != (N, K) or b.codes.shape[1] != K:
+        raise ValueError("both operand sets must have the same shapes")
+    if M <= 128 or N <= 128 or K % 128 or N % 8:
+        return mx_gemm_nt(a, b) + mx_gemm_nt(a2, b2)
+    out = torch.empty((M, N), dtype=torch.bfloat16, device=a.codes.device)
+    sa, sb, sa2, sb2 = _as_mfma(a), _as_mfma(b), _as_mfma(a2), _as_mfma(b2)  # kept alive over the launch
+    _call("mx_gemm_nt_pair", "gemm_nt_pair", out.device, _ptr(a.codes), _ptr(sa), _ptr(b.codes), _ptr(sb),
+          _ptr(a2.codes), _ptr(sa2), _ptr(b2.codes), _ptr(sb2), _ptr(out), M, N, K, N, _stream(out))
+    return out
+
+
 # --------------------------------------------------------------------------- 3-D weights
 def to_mx_dim0_batched(w: torch.Tensor, mode="floor", order: int = MX_SCALES_MFMA) -> MXData:
     """Row-wise cast of every matrix of w [G, R, C]: codes [G, R, C], one scale block each.
@@ -587,6 +604,29 @@ def mx_grouped_gemm_2d3d(a: MXData, b: MXData, offs: torch.Tensor,
                                                                  b.codes, b.scales, offs)
         return _grouped_2d3d_op(a.codes, a.scales, a.scale_order, b.codes, b.scales, offs)
     return _grouped_2d3d_into(a.codes, a.scales, a.scale_order, b.codes, b.scales, offs, out)
+
+
+def mx_grouped_gemm_2d3d_pair(a: MXData, b: MXData, a2: MXData, b2: MXData, offs: torch.Tensor,
+                              out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[rows of g] = deq(a[rows of g]) @ deq(b[g])^T + deq(a2[rows of g]) @ deq(b2[g])^T, both
+    sets with MFMA-order scales and 128-aligned groups (the persistent kernel); other layouts:
+    two grouped GEMMs and a bf16 add."""
+    T, K = a.codes.shape
+    G, N, _ = b.codes.shape
+    if a2.codes.shape != a.codes.shape or b2.codes.shape != b.codes.shape:
+        raise ValueError("both operand sets must have the same shapes")
+    fast = all(d.scale_order == MX_SCALES_MFMA for d in (a, b, a2, b2))
+    if not fast or K % 128 or N % 8 or T % 128 or G > 638:
+        both = mx_grouped_gemm_2d3d(a, b, offs) + mx_grouped_gemm_2d3d(a2, b2, offs)
+        return both if out is None else out.copy_(both)
+    if offs.dtype != torch.int32 or offs.numel() != G:
+        raise ValueError("offs must be int32 with one entry per group")
+    if out is None:
+        out = torch.empty((T, N), dtype=torch.bfloat16, device=a.codes.device)
+    _call("mx_grouped_gemm_2d3d_pair", "grouped_gemm_2d3d_pair", out.device, _ptr(a.codes), _ptr(a.scales),
+          _ptr(b.codes), _ptr(b.scales), _ptr(a2.codes), _ptr(a2.scales), _ptr(b2.codes), _ptr(b2.scales),
+          _ptr(offs), _ptr(out), T, N, K, G, out.stride(0), _stream(out))
+    return out
 
 
 def mx_grouped_gemm_2d2d(at: MXData, bt: MXData, offs: torch.Tensor,
