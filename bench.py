@@ -89,7 +89,7 @@ def build_linears(dev, recipe):
 def one_step(ffn, x, h, dy_h, dy_o):
     from torchtitan_amd import mx_tensor
 
-    mx_tensor._cast_cache.clear()  # a new step has new activations: nothing carries over
+    mx_tensor.clear_cast_cache()  # a new step has new activations: nothing carries over
     x.grad = None
     h.grad = None
     for lin, inp, dy in ((ffn.w1, x, dy_h), (ffn.w3, x, dy_h), (ffn.w2, h, dy_o)):
@@ -272,7 +272,7 @@ def time_decoder_block(dev, recipe):
                     m.weight.normal_(0.0, 0.02)
 
         def step():
-            mx_tensor._cast_cache.clear()
+            mx_tensor.clear_cast_cache()
             x.grad = None
             for p in blk.parameters():
                 p.grad = None
@@ -348,7 +348,7 @@ def time_ffn_block(dev, recipe):
         ff.init_weights(init_std=0.02)
 
         def step():
-            mx_tensor._cast_cache.clear()
+            mx_tensor.clear_cast_cache()
             x.grad = None
             for p in ff.parameters():
                 p.grad = None
@@ -483,7 +483,7 @@ def time_policy_layer_linears(dev, recipe):
     flops = 3 * 2.0 * T * sum(i * o for i, o in shapes.values())
 
     def step():
-        mx_tensor._cast_cache.clear()
+        mx_tensor.clear_cast_cache()
         for name, (i, o) in shapes.items():
             lin = getattr(layer, name)
             lin.weight.grad = None

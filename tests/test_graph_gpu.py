@@ -4,13 +4,14 @@ Nothing on the MXFP8 path synchronises with the host or clears memory with a mem
 sizes stay on the device, padded lengths are static bounds, flags are cleared by fill kernels),
 so a forward + backward through converted modules can be captured once and replayed.  Each test
 replays the graph several times on new inputs, with eager work and synchronisations between the
-replays, and checks every replay bit for bit against the eager run of the same step."""
+replays, and checks every replay bit for bit against the eager run of the same step.  No test
+clears the activation-cast reuse by hand: an entry made by the eager warm-up must not be taken
+under capture (the cast would be missing from the graph and every replay would reuse old codes)."""
 import pytest
 import torch
 import torch.nn as nn
 
-from torchtitan_amd import mx_tensor
-from torchtitan_amd.modules import FeedForward, MoE
+from torchtitan_amd.modules import FeedForward, Linear, MoE
 from torchtitan_amd.protocols import ModelConvertersContainer
 from torchtitan_amd.quantization.mx import MXFP8Converter
 
@@ -24,7 +25,6 @@ def _convert(model, fqns):
 
 
 def _step(module, x, dy):
-    mx_tensor._cast_cache.clear()
     for p in module.parameters():
         p.grad = None
     x.grad = None
@@ -56,11 +56,9 @@ def _check_graph_replays(module, shape, device):
     for p in module.parameters():
         p.grad = None
     x.grad = None
-    mx_tensor._cast_cache.clear()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         module(x).backward(dy)
-    mx_tensor._cast_cache.clear()
     for rep in range(2):
         for (xi, dyi), want in zip(inputs, eager):
             with torch.no_grad():
@@ -98,3 +96,36 @@ def test_moe_layer_in_a_captured_graph(device):
     holder.moe = moe
     _convert(holder, ["experts"])
     _check_graph_replays(moe, (2, 96, 256), device)
+
+
+def test_single_linear_captured_after_a_warm_up_on_the_same_static_input(device):
+    """The usual recipe, warm-up then capture, on a model whose only cast input is the static
+    input itself: the warm-up leaves that tensor's cast in the reuse slot, and the capture must
+    not take it."""
+    torch.manual_seed(41)
+    holder = nn.Module()
+    holder.proj = Linear.Config().build(in_features=256, out_features=384)
+    holder.to(device).to(torch.bfloat16)
+    holder.proj.init_weights(init_std=0.05)
+    _convert(holder, ["proj"])
+    shape = (4, 64, 256)
+    inputs = [torch.randn(shape, device=device, dtype=torch.bfloat16) for _ in range(3)]
+    x = torch.zeros(shape, device=device, dtype=torch.bfloat16)
+    with torch.no_grad():
+        eager = [holder.proj(xi).clone() for xi in inputs]
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            holder.proj(x)  # warm-up on the static input, no backward: the reuse slot now holds x's cast
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            y = holder.proj(x)
+        for rep in range(2):
+            for xi, want in zip(inputs, eager):
+                x.copy_(xi)
+                graph.replay()
+                torch.cuda.synchronize()
+                assert torch.equal(y, want), rep
+                # eager calls on the same static tensor between replays see its new contents too
+                assert torch.equal(holder.proj(x), want)

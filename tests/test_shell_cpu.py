@@ -285,6 +285,50 @@ def test_module_filter_fn_rules():
     assert module_filter_fn(nn.Linear(16, 16), "output", ["router"])
 
 
+def test_converter_applies_filter_fqns_and_the_dims_rule(monkeypatch):
+    """`filter_fqns` takes a module out of the selection `fqns` makes, and an nn.Linear with a
+    weight dimension that is not a multiple of 16 is never converted (the Config field and filter
+    of torchtitan/components/quantization/float8.py:51-56,176 with utils.py:10-27)."""
+    cfg = MXFP8Converter.Config()
+    assert cfg.filter_fqns == []
+
+    class Block(Module):
+        def __init__(self):
+            super().__init__()
+            self.wq = Linear.Config().build(in_features=64, out_features=64)
+            self.wk = Linear.Config().build(in_features=64, out_features=32)
+            self.narrow = Linear.Config().build(in_features=64, out_features=40)  # 40 % 16 != 0
+            self.experts = GroupedExperts(dim=64, hidden_dim=32, num_experts=4, use_grouped_mm=True)
+
+    class Model(Module):
+        def __init__(self):
+            super().__init__()
+            self.layers = nn.ModuleList([Block(), Block()])
+            self.output = Linear.Config().build(in_features=64, out_features=96)
+
+    with torch.device("meta"):
+        model = Model()
+    conv = _converter(monkeypatch, fqns=["layers", "output"], filter_fqns=["wk", "layers.1.experts", "output"]).build(
+        parallel_dims=None, model_compile_enabled=False)
+    conv.convert(model)
+    for i, blk in enumerate(model.layers):
+        assert isinstance(blk.wq.weight, MXFP8TrainingWeight)
+        assert not isinstance(blk.wk.weight, MXFP8TrainingWeight)       # excluded by name
+        assert not isinstance(blk.narrow.weight, MXFP8TrainingWeight)   # 40 is not a multiple of 16
+        assert isinstance(blk.experts.w1, MXFP8TrainingWeight) == (i == 0)
+    assert not isinstance(model.output.weight, MXFP8TrainingWeight)
+    assert conv.filter_fn(model.layers[0].wq, "layers.0.wq") and not conv.filter_fn(model.output, "output")
+    verify_module_protocol(model, nn.Linear, Linear)
+
+
+def test_capability_gate_wants_the_gfx95_family():
+    """Exactly the CDNA4 family passes: other AMD families are different instruction sets."""
+    ok = mx_mod._arch_has_capability
+    assert ok("gfx950", 9, 5) and ok("gfx950:sramecc+:xnack-", 9, 5)
+    for other in ("gfx942", "gfx90a", "gfx1100", "gfx1201", "gfx908", "sm_100", "", "gfx"):
+        assert not ok(other, 9, 5), other
+
+
 def test_converted_weights_survive_deepcopy_and_checkpoint_as_plain_tensors():
     """A converted model can be deep-copied (independent storage, still converted, still
     Parameters) and its state dict holds plain tensors: torch.save / weights-only torch.load
@@ -326,3 +370,35 @@ def test_converted_weights_survive_deepcopy_and_checkpoint_as_plain_tensors():
     twin.load_state_dict(plain.state_dict())
     for a, b in zip(ff.parameters(), twin.parameters()):
         assert isinstance(b, MXFP8TrainingWeight) and torch.equal(a.as_subclass(torch.Tensor), b.as_subclass(torch.Tensor))
+
+
+def test_optimizer_state_of_converted_weights_is_plain_and_pickling_keeps_parameters():
+    """AdamW's moments are made with zeros_like: they must be plain tensors, so that an optimizer
+    state dict round-trips through a weights-only load; and a pickled converted Parameter comes
+    back as a converted Parameter."""
+    import io
+    import pickle
+
+    import torch
+    import torch.nn as nn
+
+    from torchtitan_amd.mx_tensor import MXFP8Config, MXFP8TrainingWeight, wrap_parameter
+
+    lin = nn.Linear(32, 16, bias=False)
+    lin.weight = wrap_parameter(lin.weight, MXFP8Config("floor", False))
+    opt = torch.optim.AdamW(lin.parameters(), lr=1e-2)
+    lin.weight.grad = torch.ones(16, 32)
+    opt.step()
+    state = opt.state_dict()
+    moments = [v for st in state["state"].values() for v in st.values() if isinstance(v, torch.Tensor)]
+    assert moments and all(type(v) is torch.Tensor for v in moments)
+    buf = io.BytesIO()
+    torch.save(state, buf)
+    buf.seek(0)
+    back = torch.load(buf, weights_only=True)
+    assert torch.equal(back["state"][0]["exp_avg"], state["state"][0]["exp_avg"])
+    assert isinstance(lin.weight, MXFP8TrainingWeight) and isinstance(lin.weight, nn.Parameter)
+    q = pickle.loads(pickle.dumps(lin.weight))
+    assert isinstance(q, nn.Parameter) and isinstance(q, MXFP8TrainingWeight) and q.requires_grad
+    assert q.mx_config.scale_mode == "floor" and torch.equal(q.detach().as_subclass(torch.Tensor),
+                                                              lin.weight.detach().as_subclass(torch.Tensor))

@@ -11,7 +11,7 @@ import torch
 import torch.nn.functional as F
 
 from . import ops
-from .mx_tensor import (MXFP8Config, MXFP8TrainingWeight, _cast_activation, _cast_cols_padded,
+from .mx_tensor import (MXFP8Config, MXFP8TrainingWeight, _cast_activation, _cast_cache, _cast_cols_padded,
                         _cast_into_groups, _cast_rows_padded, _cast_weight, _grouped_2d3d_padded,
                         _pad_plan, _unwrap)
 from .ops import MX_SCALES_MFMA, MX_SCALES_ROWMAJOR, MXData
@@ -153,6 +153,7 @@ class _MXFeedForward(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dy):
+        _cast_cache.clear()  # the forward that shared x's cast with a sibling is over
         mode = ctx.cfg.scale_mode
         saved = list(ctx.saved_tensors)
         take = lambda: MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)

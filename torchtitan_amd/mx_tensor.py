@@ -53,20 +53,39 @@ class _ActivationCastCache:
 
     w1(x) and w3(x) of a SwiGLU block, or wq/wk/wv of attention, receive the same tensor object;
     the second and third linear reuse the codes instead of re-reading x.  The entry is keyed on
-    object identity and the tensor's version counter and holds only a weak reference.
+    object identity, the tensor's version counter and its address, and holds only a weak
+    reference to the activation.
+
+    What keeps a hit from being stale: an entry lives for one forward at most.  It is dropped at
+    the start of every backward of a converted linear, whenever the stream's graph-capture state
+    changes (an entry made by an eager warm-up is never reused under capture, so the cast is
+    always recorded into the graph, and an entry made under capture is never reused by eager
+    code), and by `clear_cast_cache()`.  Writes through this package's `out=` arguments bump the
+    destination's version counter.  A caller that overwrites an activation behind autograd's back
+    (`.data`, a foreign kernel) between two forwards without a backward in between must call
+    `clear_cast_cache()`.
     """
 
     def __init__(self):
         self._ref = None
         self._key = None
         self._value = None
+        self._capturing = False
+
+    def _sync_capture_state(self):
+        capturing = torch.cuda.is_available() and torch.cuda.is_current_stream_capturing()
+        if capturing != self._capturing:
+            self.clear()
+            self._capturing = capturing
 
     def get(self, x: torch.Tensor, mode: str):
+        self._sync_capture_state()
         if self._ref is not None and self._ref() is x and self._key == (x._version, mode, x.data_ptr()):
             return self._value
         return None
 
     def put(self, x: torch.Tensor, mode: str, value):
+        self._sync_capture_state()
         self._ref = weakref.ref(x)
         self._key = (x._version, mode, x.data_ptr())
         self._value = value
@@ -76,6 +95,11 @@ class _ActivationCastCache:
 
 
 _cast_cache = _ActivationCastCache()
+
+
+def clear_cast_cache() -> None:
+    """Forget the remembered activation cast (see `_ActivationCastCache`)."""
+    _cast_cache.clear()
 
 
 def _cast_activation(x2: torch.Tensor, src: torch.Tensor, mode: str, need_cols: bool):
@@ -188,6 +212,7 @@ class _MXLinear(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dy):
+        _cast_cache.clear()  # the forward whose sibling linears shared a cast is over
         mode = ctx.cfg.scale_mode
         need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         saved = list(ctx.saved_tensors)
@@ -449,9 +474,12 @@ class MXFP8TrainingWeight(torch.Tensor):
             out = func(*args, **kwargs)
         return _rewrap(out, cls, cfg, func)
 
-    # pickling: the plain tensor plus the config
+    # pickling: the plain tensor plus the config (and whether it was a Parameter)
     def __reduce_ex__(self, proto):
-        return (MXFP8TrainingWeight, (self.as_subclass(torch.Tensor), self.mx_config))
+        plain = self.as_subclass(torch.Tensor)
+        if getattr(self, "_is_param", False):
+            return (_rebuild_parameter, (plain.detach(), self.mx_config, self.requires_grad))
+        return (MXFP8TrainingWeight, (plain, self.mx_config))
 
     def __deepcopy__(self, memo):
         """An independent copy that is still a converted weight (and still a Parameter if this
@@ -469,11 +497,18 @@ class MXFP8TrainingWeight(torch.Tensor):
         return out
 
 
+def _rebuild_parameter(data: torch.Tensor, cfg: MXFP8Config, requires_grad: bool):
+    return torch.nn.Parameter(MXFP8TrainingWeight(data, cfg), requires_grad=requires_grad)
+
+
+# views, casts, detach and clone of a weight are still that weight, and so is the storage that
+# `Module.to_empty` gives a meta-device parameter (torch.empty_like); zeros_like and the other
+# factory functions (optimizer state) make plain tensors
 _KEEP_WRAPPED = {
     torch.Tensor.transpose, torch.Tensor.t, torch.Tensor.bfloat16, torch.Tensor.to,
     torch.Tensor.detach, torch.Tensor.requires_grad_, torch.Tensor.contiguous,
     torch.Tensor.view, torch.Tensor.reshape, torch.Tensor.float, torch.Tensor.half,
-    torch.transpose, torch.empty_like, torch.zeros_like, torch.Tensor.clone, torch.clone,
+    torch.transpose, torch.empty_like, torch.Tensor.clone, torch.clone,
     torch.Tensor.cuda, torch.Tensor.cpu, torch.Tensor.type,
 }
 

@@ -89,6 +89,14 @@ def _ptr(t: torch.Tensor) -> ctypes.c_void_p:
     return ctypes.c_void_p(t.data_ptr())
 
 
+def _wrote(out: torch.Tensor) -> torch.Tensor:
+    """A library write into a caller's tensor is an in-place op that autograd did not see: bump
+    the version counter so that whatever is keyed on it (saved-tensor checks, the activation cast
+    reuse of mx_tensor) notices the new contents."""
+    torch.autograd.graph.increment_version(out)
+    return out
+
+
 def _check_hp(x: torch.Tensor) -> torch.Tensor:
     if not x.is_cuda:
         raise _lib.MXLibraryError("the MXFP8 kernels run on the GPU only; got a CPU tensor")
@@ -269,6 +277,8 @@ def mx_dequant(d: MXData, out: torch.Tensor | None = None) -> torch.Tensor:
         raise ValueError(f"cols {cols} is not a multiple of {BLOCK}")
     if out is None:
         out = torch.empty((rows, cols), dtype=torch.bfloat16, device=codes.device)
+    else:
+        _wrote(out)
     scales = d.scales.contiguous()
     _call("mx_dequant", "dequant", codes.device, _ptr(codes), _ptr(scales), rows, cols, d.scale_order,
           _ptr(out), out.stride(0), _stream(codes))
@@ -503,7 +513,7 @@ def mx_gemm_nt(a: MXData, b: MXData, out: torch.Tensor | None = None) -> torch.T
         return _gemm_nt_op(a.codes, sa, b.codes, sb)
     if out.shape != (M, N) or out.dtype != torch.bfloat16 or out.stride(1) != 1:
         raise ValueError("out must be a bf16 [M, N] tensor with unit inner stride")
-    return _gemm_nt_into(a.codes, sa, b.codes, sb, out)
+    return _gemm_nt_into(a.codes, sa, b.codes, sb, _wrote(out))
 
 
 def mx_gemm_nt_pair(a: MXData, b: MXData, a2: MXData, b2: MXData) -> torch.Tensor:
@@ -603,7 +613,7 @@ def mx_grouped_gemm_2d3d(a: MXData, b: MXData, offs: torch.Tensor,
             return torch.ops.torchtitan_amd.mx_grouped_gemm_2d3d(a.codes, a.scales, a.scale_order,
                                                                  b.codes, b.scales, offs)
         return _grouped_2d3d_op(a.codes, a.scales, a.scale_order, b.codes, b.scales, offs)
-    return _grouped_2d3d_into(a.codes, a.scales, a.scale_order, b.codes, b.scales, offs, out)
+    return _grouped_2d3d_into(a.codes, a.scales, a.scale_order, b.codes, b.scales, offs, _wrote(out))
 
 
 def mx_grouped_gemm_2d3d_pair(a: MXData, b: MXData, a2: MXData, b2: MXData, offs: torch.Tensor,
@@ -623,6 +633,8 @@ def mx_grouped_gemm_2d3d_pair(a: MXData, b: MXData, a2: MXData, b2: MXData, offs
         raise ValueError("offs must be int32 with one entry per group")
     if out is None:
         out = torch.empty((T, N), dtype=torch.bfloat16, device=a.codes.device)
+    else:
+        _wrote(out)
     _call("mx_grouped_gemm_2d3d_pair", "grouped_gemm_2d3d_pair", out.device, _ptr(a.codes), _ptr(a.scales),
           _ptr(b.codes), _ptr(b.scales), _ptr(a2.codes), _ptr(a2.scales), _ptr(b2.codes), _ptr(b2.scales),
           _ptr(offs), _ptr(out), T, N, K, G, out.stride(0), _stream(out))
@@ -647,6 +659,8 @@ def mx_grouped_gemm_2d2d(at: MXData, bt: MXData, offs: torch.Tensor,
     G = offs.numel()
     if out is None:
         out = torch.empty((G, N, K), dtype=torch.bfloat16, device=at.codes.device)
+    else:
+        _wrote(out)
     _call("mx_grouped_gemm_2d2d", "grouped_gemm_2d2d", out.device, _ptr(at.codes), _ptr(at.scales), _ptr(bt.codes), _ptr(bt.scales), _ptr(offs), _ptr(out), T, N, K, G, at.scale_order, _stream(out))
     return out
 

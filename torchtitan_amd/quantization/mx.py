@@ -12,6 +12,7 @@ from __future__ import annotations
 
 import logging
 from dataclasses import dataclass, field
+from functools import partial
 from typing import Any, ClassVar, Literal
 
 import torch
@@ -22,23 +23,34 @@ from ..modules.linear import Linear
 from ..mx_tensor import MXFP8Config, MXFP8TrainingWeight, _cast_weight, wrap_parameter
 from . import QuantizationConverter
 from .module_utils import capture_module_attrs, inject_module_protocol, verify_module_protocol
+from .utils import module_filter_fn
 
 logger = logging.getLogger("torchtitan_amd")
 
 _RECIPES = {"mxfp8_rceil": "rceil", "mxfp8_floor": "floor"}
 
 
-def has_rocm_capability(major: int, minor: int) -> bool:
-    """True on an AMD GPU of at least gfx<major><minor>x (9, 5 -> gfx950 = MI350X / MI355X)."""
-    if not torch.cuda.is_available() or torch.version.hip is None:
-        return False
-    arch = torch.cuda.get_device_properties(0).gcnArchName.split(":")[0]
-    digits = arch.removeprefix("gfx")
+def _arch_has_capability(arch: str, major: int, minor: int) -> bool:
+    """Whether the architecture string `arch` ("gfx950", "gfx950:sramecc+:xnack-") names a GPU of
+    the family gfx<major><minor>x.  The family must match exactly: the kernels are written for
+    one instruction set, and a larger number (gfx11xx, gfx12xx) is a different one, not a newer
+    member of it."""
+    digits = arch.split(":")[0].removeprefix("gfx")
     try:
         got = (int(digits[:-2]), int(digits[-2], 16))
-    except ValueError:
+    except (ValueError, IndexError):
         return False
-    return got >= (major, minor)
+    return got == (major, minor)
+
+
+def has_rocm_capability(major: int, minor: int) -> bool:
+    """True when the current device is an AMD GPU of the family gfx<major><minor>x
+    (9, 5 -> gfx950 = MI350X / MI355X).  Stands where the reference asks
+    `has_cuda_capability(10, 0)` (torchtitan/tools/utils.py:28-33)."""
+    if not torch.cuda.is_available() or torch.version.hip is None:
+        return False
+    arch = torch.cuda.get_device_properties(torch.cuda.current_device()).gcnArchName
+    return _arch_has_capability(arch, major, minor)
 
 
 def _plain_state_dict_entries(module, state_dict, prefix, local_metadata):
@@ -64,6 +76,13 @@ class MXFP8Converter(QuantizationConverter):
         fqns: list[str] = field(default_factory=list)
         """Modules whose fully qualified name contains any of these strings are converted.
         The default (empty) converts nothing."""
+
+        filter_fqns: list[str] = field(default_factory=list)
+        """Modules whose fully qualified name contains any of these strings are left in high
+        precision even when `fqns` selects them (the exclusion list the reference's low-precision
+        converters carry, torchtitan/components/quantization/float8.py:51-56).  nn.Linear modules
+        with a weight dimension that is not a multiple of 16 are always skipped.
+        Example: fqns=["layers"], filter_fqns=["attention.wk", "attention.wv"]."""
 
         pad_token_groups_for_grouped_mm: bool = True
         """Pad token groups to multiples of 32 inside the grouped GEMM.  Set to false when the
@@ -102,10 +121,15 @@ class MXFP8Converter(QuantizationConverter):
         if model_compile_enabled:
             logger.warning("the MXFP8 path runs eager HIP kernels; torch.compile adds nothing to it")
         self.config = config
+        # which nn.Linear modules may be converted: dims % 16 and not excluded by name
+        # (built as in torchtitan/components/quantization/float8.py:176)
+        self.filter_fn = partial(module_filter_fn, filter_fqns=config.filter_fqns)
         self.enabled = True
         logger.info("MXFP8 training enabled")
 
     def _matches(self, fqn: str) -> bool:
+        if any(part in fqn for part in self.config.filter_fqns):
+            return False
         return any(target in fqn for target in self.config.fqns)
 
     def convert(self, model: nn.Module):
@@ -125,6 +149,10 @@ class MXFP8Converter(QuantizationConverter):
                 continue
             before = n_linear + n_grouped
             if isinstance(mod, nn.Linear):
+                if not self.filter_fn(mod, fqn):
+                    logger.warning("skipping %s: weight %s has a dimension that is not a multiple of 16",
+                                   fqn, tuple(mod.weight.shape))
+                    continue
                 if mod.in_features % 32:
                     logger.warning("skipping %s: in_features %d is not a multiple of 32", fqn, mod.in_features)
                     continue
