@@ -3,8 +3,10 @@
  *
  * Every entry point takes raw device pointers, sizes and a HIP stream (as void*), launches
  * asynchronously on that stream, allocates nothing, never synchronises, and returns an
- * mx_status_t (0 = ok).  No exceptions cross this boundary.  Calls are thread-safe as long
- * as concurrent calls use distinct output buffers.
+ * mx_status_t (0 = ok).  No exceptions cross this boundary.  Calls may come from several host
+ * threads and for several GPUs (each call works on the calling thread's current device): the
+ * library keeps no mutable state of its own beyond per-device set-up flags, which are atomic.
+ * Concurrent calls must use distinct output buffers.
  *
  * The reference has no native interface for this path: its converter hands the arithmetic
  * to an external Python library.  Each declaration cites the reference statement that the

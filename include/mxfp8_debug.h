@@ -1,8 +1,8 @@
 /*
- * Measurement hooks of libmxfp8_gfx950.so.  NOT part of the ABI in mxfp8.h: nothing in the
- * product path calls them, their meaning may change with the kernels, and they are process-wide
- * (not thread-safe).  They exist so that timing experiments can be run against the shipped
- * library instead of a special build.
+ * Test hooks of libmxfp8_gfx950.so.  NOT part of the ABI in mxfp8.h: nothing in the product path
+ * calls them, their meaning may change with the kernels, and they are process-wide (a test sets
+ * one, runs, and sets it back).  mx_debug_set_prof and the kernel instances it switches to exist
+ * only in a library built with -DMX_TIMING_BUILD; the product build leaves them out.
  */
 #ifndef MXFP8_DEBUG_H_
 #define MXFP8_DEBUG_H_
@@ -20,7 +20,7 @@ void mx_debug_force_kernel(int which);
  * (also lowers how many tiles one grouped launch covers); 0: one per CU (default). */
 void mx_debug_set_grid(int workgroups);
 
-/* Device buffer of 256 * 4 * 8 uint64 that the timing build of the 32x32x64 kernel fills with
+/* -DMX_TIMING_BUILD only.  Device buffer of 256 * 4 * 8 uint64 that the timing build of the 32x32x64 kernel fills with
  * per-wave cycle counts {copy wait, barriers, step body, epilogue, ...}; NULL switches the timing
  * build off (default). */
 void mx_debug_set_prof(void* device_buffer);

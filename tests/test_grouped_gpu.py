@@ -186,6 +186,26 @@ def test_aligned_group_forms_poison_the_output_when_a_group_end_is_not_a_multipl
     assert torch.isnan(dw).all()
 
 
+def test_row_major_wgrad_poisons_groups_that_break_the_32_token_rule(device):
+    """Row-major scales: a group may be any multiple of 32 tokens.  A group that starts or ends
+    inside a 32-token block would share scale blocks with its neighbour; its weight gradient
+    comes out as NaN, the groups that keep the rule are still right."""
+    rng = np.random.default_rng(8)
+    sizes, N, K = [64, 40, 56, 96], 160, 96   # ends 64, 104, 160, 256: groups 1 and 2 touch 104
+    T = sum(sizes)
+    x_bits, dy_bits = randn_bits(rng, (T, K)), randn_bits(rng, (T, N), std=1e-3)
+    x, dy = bf16_from_bits(x_bits, device), bf16_from_bits(dy_bits, device)
+    offs = _sizes_to_offs(sizes, device)
+    dw = ops.mx_grouped_gemm_2d2d(ops.to_mx_dim1(dy, "rceil", R), ops.to_mx_dim1(x, "rceil", R), offs)
+    assert torch.isnan(dw[1]).all() and torch.isnan(dw[2]).all()
+    lo = 0
+    for g, n in enumerate(sizes):
+        if g in (0, 3):
+            ref = mo.mx_matmul(np.ascontiguousarray(dy_bits[lo:lo + n].T), np.ascontiguousarray(x_bits[lo:lo + n].T), mo.RCEIL)
+            assert rel_l2(_f32(bits_of(dw[g])), _f32(ref)) <= TOL, g
+        lo += n
+
+
 def test_batched_weight_casts_match_per_matrix(device):
     rng = np.random.default_rng(11)
     w_bits = randn_bits(rng, (5, 96, 160), std=0.02, outliers=1e-3)

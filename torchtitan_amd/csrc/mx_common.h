@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "mxfp8.h"
 
 namespace mx {
@@ -93,6 +95,45 @@ __device__ __host__ __forceinline__ int64_t mfma_scale_offset(int64_t row, int64
 }
 __device__ __host__ __forceinline__ int64_t mfma_scale_bytes(int64_t rows, int64_t nblk) {
   return ((rows + 127) >> 7) * ((nblk + 1) >> 1) * 256;
+}
+
+// ---- per-device host state -------------------------------------------------------------------
+// A process may drive several GPUs, from several threads: whatever the host side remembers about
+// "the device" (its CU count, whether a kernel's dynamic-LDS limit has been raised there) is kept
+// per device ordinal in atomics.  Two threads that race on the first call both do the same
+// idempotent set-up.
+constexpr int kMaxDevices = 64;
+
+// Ordinal of the calling thread's current device, -1 if it cannot be asked or is out of range.
+inline int current_device() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return -1;
+  return dev;
+}
+
+// Compute units of the current device (0: unknown).
+inline int current_device_cus() {
+  static std::atomic<int> cus[kMaxDevices];
+  const int dev = current_device();
+  if (dev < 0) return 0;
+  int n = cus[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 0;
+    cus[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
+
+// Raises a kernel's dynamic-LDS limit once per device.  `done` is the kernel's own table
+// (a function-local static of the launcher, one per template instance).
+inline bool raise_lds_limit(const void* kernel, int bytes, std::atomic<bool> (&done)[kMaxDevices]) {
+  const int dev = current_device();
+  if (dev < 0) return false;
+  if (!done[dev].load(std::memory_order_acquire)) {
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return false;
+    done[dev].store(true, std::memory_order_release);
+  }
+  return true;
 }
 
 }  // namespace mx

@@ -31,14 +31,8 @@ template <int BM, int BN>
 static int launch_dense(const DenseArgs& p, hipStream_t st) {
   using Tile = GemmTile<BM, BN, false, false>;
   auto kern = gemm_nt_kernel<BM, BN>;
-  static bool configured = false;  // raising the dynamic-LDS limit is a per-function setting
-  if (!configured) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                            hipFuncAttributeMaxDynamicSharedMemorySize,
-                            Tile::kLdsBytes) != hipSuccess)
-      return MX_ERR_LAUNCH;
-    configured = true;
-  }
+  static std::atomic<bool> configured[kMaxDevices];  // a per-function, per-device setting
+  if (!raise_lds_limit(reinterpret_cast<const void*>(kern), Tile::kLdsBytes, configured)) return MX_ERR_LAUNCH;
   const int64_t nb = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
   const int64_t grid = (nb + 7) / 8 * 8;
   if (grid > 0x7FFFFFFF) return MX_ERR_UNSUPPORTED;
@@ -61,15 +55,18 @@ int launch_gemm_nt32_splitk(const uint8_t* a_codes, const uint8_t* a_scales, con
                             const uint8_t* b_scales, void* d, int64_t M, int64_t N, int64_t K,
                             int64_t ldd, int slices, void* workspace, hipStream_t st);
 }
+// Test hooks (include/mxfp8_debug.h), process-wide.
 // 0: pick by shape; 1 / 2: the 16x16x128 tile kernel with 256x256 / 128x128 tiles for every
 // shape; 3: the persistent kernel wherever it is legal (comparison runs and tests)
-static int force_kernel = 0;
+static std::atomic<int> force_kernel{0};
 extern "C" void mx_debug_force_kernel(int which) { force_kernel = which; }
 namespace mx { void set_debug_grid(int g); }
 extern "C" void mx_debug_set_grid(int g) { mx::set_debug_grid(g); }
+#ifdef MX_TIMING_BUILD
 namespace mx { void set_debug_prof(uint64_t* buf); }
-// device buffer of 256*4*4 uint64 receiving per-wave cycle counts; nullptr switches timing off
+// device buffer of 256*4*8 uint64 receiving per-wave cycle counts; nullptr switches timing off
 extern "C" void mx_debug_set_prof(void* buf) { mx::set_debug_prof((uint64_t*)buf); }
+#endif
 
 static int check_dense(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                        const uint8_t* b_scales, const void* d, int64_t M, int64_t N, int64_t K,
@@ -102,13 +99,8 @@ extern "C" int mx_gemm_nt(const uint8_t* a_codes, const uint8_t* a_scales,
   // Few 256x256 tiles leave most CUs of the persistent kernel idle when the contraction is not
   // split: up to 3/8 of the CUs' worth of tiles, four times as many 128x128 tiles finish sooner
   // (measured: 64 tiles 58 vs 71 us at K = 8192; 128 tiles 46 vs 43 us).
-  static int num_cus = 0;
-  if (num_cus == 0) {
-    int dev = 0, n = 0;
-    num_cus = (hipGetDevice(&dev) == hipSuccess &&
-               hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-                  ? n : 256;
-  }
+  int num_cus = current_device_cus();
+  if (num_cus == 0) num_cus = 256;
   const int64_t tiles256 = ((M + 255) / 256) * ((N + 255) / 256);
   if (force_kernel == 0 && tiles256 * 8 <= (int64_t)num_cus * 3) return launch_dense<128, 128>(p, st);
   if (force_kernel == 1 || !persistent_ok(d, N, K, ldd)) return launch_dense<256, 256>(p, st);

@@ -39,6 +39,7 @@ constexpr int kOperand32 = kT32 * kKB;           // 32 KB: 256 rows x 128 B
 constexpr int kCodes32 = 2 * kOperand32;         // A rows then B rows
 constexpr int kBlock32 = kCodes32 + 2048;        // + scales: 4 groups (A0, A1, B0, B1) x 2 steps x 256 B
 constexpr int kRing32 = 2 * kBlock32;            // 132 KB
+constexpr uint32_t kMaxTileRecords = 120;        // grouped modes: tile records a workgroup keeps in LDS
 
 // What a launch works on.  One kernel serves three problems that differ only in how a linear
 // tile number maps to operand rows, K range and output address:
@@ -262,7 +263,12 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   }
   if (n_my == 0) return;
   if (PAIR) n_my *= 2;  // from here on n_my counts segments: two per output tile
-  if (MODE != kDense && n_my > 120) return;  // more tiles than records: the host never launches this
+  if (MODE != kDense && n_my > kMaxTileRecords) {
+    // More tiles than records: the host splits launches so that this cannot happen.  Should it
+    // ever, the tiles that have a record are written as NaN rather than left as they were.
+    n_my = kMaxTileRecords;
+    poison = true;
+  }
 
   // Tile number -> operands.
   auto describe = [&](uint32_t t, uint32_t seg) -> Tile32 {
@@ -825,19 +831,20 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   }
 }
 
-static int debug_grid = 0;
-static uint64_t* debug_prof = nullptr;  // > 0: number of persistent workgroups (experiments only)
+// Test hook, process-wide: > 0 = number of persistent workgroups (also lowers how many tiles one
+// grouped launch covers, which is what the tests use it for); 0 = one per CU.
+static std::atomic<int> debug_grid{0};
+#ifdef MX_TIMING_BUILD
+static uint64_t* debug_prof = nullptr;  // device buffer for the per-wave cycle counts, or nullptr
+#else
+static constexpr uint64_t* debug_prof = nullptr;
+#endif
 
-// One persistent workgroup per CU, a multiple of the 8 XCDs (0: the device cannot be queried).
+// One persistent workgroup per CU of the current device, a multiple of the 8 XCDs (0: the device
+// cannot be queried).
 static int64_t persistent_grid() {
-  static int num_cus = 0;
-  if (num_cus == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-      return 0;
-    num_cus = n;
-  }
+  const int num_cus = current_device_cus();
+  if (num_cus == 0) return 0;
   int64_t grid = (num_cus / 8) * 8;
   if (grid < 8) grid = 8;
   if (debug_grid > 0) grid = (debug_grid + 7) / 8 * 8;
@@ -848,13 +855,8 @@ template <int MODE, bool PROF, bool PAIR = false>
 static int launch32(const Gemm32Args& p, int64_t nb, hipStream_t st) {
   auto kern = gemm_nt32_kernel<MODE, PROF, PAIR>;
   constexpr int lds = kRing32 + 4 * 7168;  // ring + one output patch per wave = all 160 KB
-  static bool configured = false;
-  if (!configured) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
-      return MX_ERR_LAUNCH;
-    configured = true;
-  }
+  static std::atomic<bool> configured[kMaxDevices];
+  if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds, configured)) return MX_ERR_LAUNCH;
   int64_t grid = persistent_grid();
   if (grid == 0) return MX_ERR_LAUNCH;
   const int64_t need = (nb + 7) / 8 * 8;  // nb: the tile count, or an upper bound of it
@@ -864,14 +866,18 @@ static int launch32(const Gemm32Args& p, int64_t nb, hipStream_t st) {
 }
 
 void set_debug_grid(int g) { debug_grid = g; }
+#ifdef MX_TIMING_BUILD
 void set_debug_prof(uint64_t* buf) { debug_prof = buf; }
+#endif
 
 int launch_gemm_nt32(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                      const uint8_t* b_scales, void* d, int64_t M, int64_t N, int64_t K,
                      int64_t ldd, hipStream_t st) {
   Gemm32Args p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, M, N, K, ldd, nullptr, 0, 0, 0, debug_prof};
   const int64_t nb = ((M + kT32 - 1) / kT32) * ((N + kT32 - 1) / kT32);
+#ifdef MX_TIMING_BUILD
   if (debug_prof) return launch32<kDense, true>(p, nb, st);
+#endif
   return launch32<kDense, false>(p, nb, st);
 }
 
@@ -962,7 +968,7 @@ int launch_gemm_nt32_splitk(const uint8_t* a_codes, const uint8_t* a_scales, con
 // (a_scales over the whole [T, K/32] matrix, b_scales one block per expert).  A workgroup keeps
 // a record per tile in LDS, at most kMaxRecords of them: larger problems are cut into several
 // launches over ranges of tile columns.
-constexpr int64_t kMaxRecords = 120;
+constexpr int64_t kMaxRecords = kMaxTileRecords;
 
 template <int MODE, bool PAIR = false>
 static int launch_grouped32(Gemm32Args p, int64_t tiles_per_column, int64_t tiles_n, hipStream_t st) {
@@ -980,8 +986,13 @@ static int launch_grouped32(Gemm32Args p, int64_t tiles_per_column, int64_t tile
     int rc;
     if constexpr (PAIR)
       rc = launch32<MODE, false, true>(p, nb, st);
-    else
+    else {
+#ifdef MX_TIMING_BUILD
       rc = p.prof ? launch32<MODE, true>(p, nb, st) : launch32<MODE, false>(p, nb, st);
+#else
+      rc = launch32<MODE, false>(p, nb, st);
+#endif
+    }
     if (rc != MX_OK) return rc;
   }
   return MX_OK;

@@ -82,20 +82,25 @@ __global__ __launch_bounds__(256, 1) void grouped_2d2d_kernel(G2d2dArgs p) {
   const int64_t tm = in % tiles_m, tn = in / tiles_m;
   const int64_t lo = g ? p.offs[g - 1] : 0, hi = p.offs[g];
   const int64_t nblk = p.T / 32;
+  if (((lo | hi) & 31) || hi < lo || lo < 0 || hi > p.T) {
+    // a group that does not start and end on a 32-token block would share scale blocks with its
+    // neighbour: the contract is broken, and the result must not pass for a gradient.  NaN.
+    const int64_t row0 = tm * BM, col0 = tn * BN;
+    const int64_t rows = p.N - row0 < BM ? p.N - row0 : BM, cols = p.K - col0 < BN ? p.K - col0 : BN;
+    uint16_t* out = p.d + g * p.N * p.K + row0 * p.K + col0;
+    for (int64_t r = threadIdx.x >> 6; r < rows; r += 4)
+      for (int64_t c = threadIdx.x & 63; c < cols; c += 64) out[r * p.K + c] = 0x7FC0;
+    return;
+  }
   Operand A{p.at_codes + tm * BM * p.T, p.T, p.N - tm * BM, p.at_scales + tm * BM * nblk, nblk};
   Operand B{p.bt_codes + tn * BN * p.T, p.T, p.K - tn * BN, p.bt_scales + tn * BN * nblk, nblk};
   Tile::run(smem, A, B, lo, hi, p.d + g * p.N * p.K + tm * BM * p.K + tn * BN, p.K);
 }
 
 template <class Kern, class Args>
-static int launch_tile_kernel(Kern kern, bool& configured, int lds_bytes, int64_t nb,
-                              const Args& p, hipStream_t st) {
-  if (!configured) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
-      return MX_ERR_LAUNCH;
-    configured = true;
-  }
+static int launch_tile_kernel(Kern kern, std::atomic<bool> (&configured)[kMaxDevices], int lds_bytes,
+                              int64_t nb, const Args& p, hipStream_t st) {
+  if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return MX_ERR_LAUNCH;
   const int64_t grid = (nb + 7) / 8 * 8;
   if (grid > 0x7FFFFFFF) return MX_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds_bytes, st, p);
@@ -104,7 +109,7 @@ static int launch_tile_kernel(Kern kern, bool& configured, int lds_bytes, int64_
 
 template <int BM, int BN>
 static int launch_2d3d(G2d3dArgs p, hipStream_t st) {
-  static bool configured = false;
+  static std::atomic<bool> configured[kMaxDevices];
   p.max_mtiles = (p.T + BM - 1) / BM + p.G + 1;
   const int64_t nb = p.max_mtiles * ((p.N + BN - 1) / BN);
   return launch_tile_kernel(grouped_2d3d_kernel<BM, BN>, configured,
@@ -113,7 +118,7 @@ static int launch_2d3d(G2d3dArgs p, hipStream_t st) {
 
 template <int BM, int BN>
 static int launch_2d2d(const G2d2dArgs& p, hipStream_t st) {
-  static bool configured = false;
+  static std::atomic<bool> configured[kMaxDevices];
   const int64_t nb = p.G * ((p.N + BM - 1) / BM) * ((p.K + BN - 1) / BN);
   return launch_tile_kernel(grouped_2d2d_kernel<BM, BN>, configured,
                             GemmTile<BM, BN, true, true>::kLdsBytes, nb, p, st);
