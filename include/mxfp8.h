@@ -6,7 +6,7 @@
  * mx_status_t (0 = ok).  No exceptions cross this boundary.  Calls may come from several host
  * threads and for several GPUs (each call works on the calling thread's current device): the
  * library keeps no mutable state of its own beyond per-device set-up flags, which are atomic.
- * Concurrent calls must use distinct output buffers.
+ * Concurrent calls must use distinct output buffers; mx_gemm_nt_static has its own rule (below).
  *
  * The reference has no native interface for this path: its converter hands the arithmetic
  * to an external Python library.  Each declaration cites the reference statement that the
@@ -31,7 +31,8 @@ typedef enum {
   MX_ERR_INVALID_ARG = 1,   /* null pointer, negative size, bad enum */
   MX_ERR_ALIGNMENT = 2,     /* a dimension is not a multiple of what the kernel needs */
   MX_ERR_LAUNCH = 3,        /* hipLaunchKernel reported an error */
-  MX_ERR_UNSUPPORTED = 4    /* shape outside what this build handles */
+  MX_ERR_UNSUPPORTED = 4,   /* shape outside what this build handles */
+  MX_ERR_SCRATCH_TOO_SMALL = 5 /* mx_gemm_nt_static: the split needs more than the built-in scratch */
 } mx_status_t;
 
 /* How the E8M0 scale is derived from the block's max |x| (amax = (1+m) 2^E):
@@ -232,6 +233,22 @@ int64_t mx_gemm_nt_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int mx_gemm_nt_ws(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                   const uint8_t* b_scales, void* d, int64_t M, int64_t N, int64_t K, int64_t ldd,
                   void* workspace, int64_t workspace_bytes, void* stream);
+
+/* mx_gemm_nt_ws for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The
+ * float32 partial sums of the split live in a device array built into the library
+ * (mx_gemm_nt_static_max_bytes() = 64 MiB, held on every GPU the library runs on until the process
+ * ends) instead of a caller's workspace; the call allocates nothing, on the host or the device.
+ * Runs the kernels mx_gemm_nt_ws runs with a workspace of mx_gemm_nt_workspace_bytes(M, N, K), so
+ * the results are bit-identical to that call's; shapes that are not split run what mx_gemm_nt
+ * runs.  A shape whose split needs more than the array holds returns MX_ERR_SCRATCH_TOO_SMALL and
+ * launches nothing.  All calls on one GPU share that GPU's array: calls that overlap in time on
+ * the same GPU (two streams, two threads) race on it.  Nothing in the array needs clearing between
+ * calls: every partial tile is written in full before the reduction reads it. */
+int64_t mx_gemm_nt_static_max_bytes(void);
+int mx_gemm_nt_static(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                      const uint8_t* b_scales, void* d, int64_t M, int64_t N, int64_t K,
+                      int64_t ldd, void* stream);
 
 /* D = deq(A) deq(B)^T + deq(A2) deq(B2)^T in one pass, both operand sets of the shapes of
  * mx_gemm_nt: every output tile accumulates the products of the first set and then of the second

@@ -44,6 +44,8 @@ SIGNATURES = {
     "mx_gemm_nt": (c_int, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "mx_gemm_nt_workspace_bytes": (_I, [_I, _I, _I]),
     "mx_gemm_nt_ws": (c_int, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _I, _P]),
+    "mx_gemm_nt_static_max_bytes": (_I, []),
+    "mx_gemm_nt_static": (c_int, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "mx_gemm_nt_pair": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "mx_grouped_gemm_2d3d_pair": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "mx_grouped_gemm_2d3d": (c_int, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, c_int, _P]),

@@ -1,4 +1,6 @@
 // Dense MXFP8 GEMM entry point: D[M,N] = deq(A)[M,K] * deq(B)[N,K]^T (bf16 out).
+#include <mutex>
+
 #include "mx_gemm_tile.h"
 
 namespace mx {
@@ -147,4 +149,44 @@ extern "C" int mx_gemm_nt_ws(const uint8_t* a_codes, const uint8_t* a_scales,
     return mx_gemm_nt(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd, stream);
   return launch_gemm_nt32_splitk(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd,
                                  (int)(need / (M * N * 4)), workspace, (hipStream_t)stream);
+}
+
+// ---- the split GEMM for callers that cannot allocate -------------------------------------------
+// The float32 partial tiles of the split along K live in a file-scope device array instead of a
+// caller-provided workspace.  Every GPU holds its own copy of the array at its own address until
+// the process ends; the address is looked up once per device and is what the kernels receive.
+constexpr int64_t kScratchBytes = 64ll << 20;
+static __device__ __align__(256) uint8_t scratch[kScratchBytes];
+
+static void* scratch_ptr[kMaxDevices];  // device address of `scratch` per GPU, nullptr: not looked up yet
+static std::mutex scratch_mutex;
+
+// Device address of this GPU's scratch array (nullptr: the lookup failed).
+static void* scratch_of_current_device() {
+  const int dev = current_device();
+  if (dev < 0) return nullptr;
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (!scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess) return nullptr;
+    scratch_ptr[dev] = ptr;
+  }
+  return scratch_ptr[dev];
+}
+
+extern "C" int64_t mx_gemm_nt_static_max_bytes(void) { return kScratchBytes; }
+
+extern "C" int mx_gemm_nt_static(const uint8_t* a_codes, const uint8_t* a_scales,
+                                 const uint8_t* b_codes, const uint8_t* b_scales, void* d,
+                                 int64_t M, int64_t N, int64_t K, int64_t ldd, void* stream) {
+  const int rc = check_dense(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd);
+  if (rc != MX_OK || M == 0 || N == 0) return rc;
+  const int64_t need = force_kernel == 0 ? mx_gemm_nt_workspace_bytes(M, N, K) : 0;
+  if (need == 0 || !persistent_ok(d, N, K, ldd))  // not a split shape: no scratch involved
+    return mx_gemm_nt(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd, stream);
+  if (need > kScratchBytes) return MX_ERR_SCRATCH_TOO_SMALL;
+  void* ws = scratch_of_current_device();
+  if (!ws) return MX_ERR_LAUNCH;
+  return launch_gemm_nt32_splitk(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd,
+                                 (int)(need / (M * N * 4)), ws, (hipStream_t)stream);
 }

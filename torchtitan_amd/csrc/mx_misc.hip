@@ -10,6 +10,8 @@ extern "C" const char* mx_status_string(int status) {
     case MX_ERR_ALIGNMENT: return "dimension or pointer not aligned to what the kernel needs";
     case MX_ERR_LAUNCH: return "kernel launch failed";
     case MX_ERR_UNSUPPORTED: return "shape not supported";
+    case MX_ERR_SCRATCH_TOO_SMALL:
+      return "the split of this shape needs more than the library's built-in scratch array holds";
     default: return "unknown status";
   }
 }
