@@ -54,6 +54,10 @@ def parse():
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run 4 elementwise passes over a 512 MiB tensor (reads 512 MiB, writes 512 MiB "
                          "each): the known-size kernel that scales FETCH_SIZE / WRITE_SIZE counter readings")
+    ap.add_argument("--clock-table", action="store_true",
+                    help="instead of the benchmark: the GEMM kernel at the benchmark shape on random data, on "
+                         "constant operands and on half of the CUs, and the vendor library's fp8 GEMM, 8 launches "
+                         "each in that order (for a rocprofv3 --pmc run: active cycles / time = shader clock)")
     return ap.parse_args()
 
 
@@ -182,6 +186,67 @@ def time_yardsticks(dev):
     sec = timed(lambda: dst.copy_(src), reps=10)
     out["device_copy_512MiB"] = {"GB/s": round(2 * src.numel() * 2 / sec / 1e9, 1),
                                  "frac_hbm": round(2 * src.numel() * 2 / sec / 1e9 / PEAK_HBM_GBPS, 3)}
+    return out
+
+
+def clock_table(dev, recipe_mode):
+    """Evidence for what bounds the dense GEMM: the same kernel, same shape (M 16384, N 14336,
+    K 4096), 8 launches per case, cases in a fixed order so that a counter run can tell them apart:
+      0 random BASELINE data (x ~ N(0,1), w ~ N(0,0.02))      4 the vendor library's tensor-scaled fp8 GEMM,
+      1 all-ones operands                                        random data, through torch._scaled_mm
+      2 all-zero operands
+      3 random data on half of the CUs (128 workgroups)
+    Prints one JSON line with the HIP-event time and TFLOP/s of every case.  Under
+    `rocprofv3 --pmc GRBM_GUI_ACTIVE SQ_VALU_MFMA_BUSY_CYCLES` the per-launch counters give the
+    shader clock (active cycles / 8 XCDs / duration) and the matrix-pipe utilisation of each."""
+    import torch
+
+    from torchtitan_amd import _lib, ops
+
+    lib = _lib.load()
+    flops = 2.0 * M * HIDDEN * DIM
+    L = ops.MX_SCALES_MFMA
+    g = torch.Generator(device=dev).manual_seed(0)
+    x = torch.randn((M, DIM), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    w = (torch.randn((HIDDEN, DIM), generator=g, device=dev, dtype=torch.float32) * 0.02).to(torch.bfloat16)
+    dst = torch.empty((M, HIDDEN), device=dev, dtype=torch.bfloat16)
+
+    def timed(fn, reps=8):
+        fn()
+        torch.cuda.synchronize()
+        time.sleep(0.5)  # let the chip settle between cases
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(reps):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        sec = s.elapsed_time(e) * 1e-3 / reps
+        return {"us_per_launch": round(sec * 1e6, 1), "TFLOP/s": round(flops / sec / 1e12, 1),
+                "frac_of_peak": round(flops / sec / 1e12 / PEAK_MXFP8_TFLOPS, 3)}
+
+    out = {"shape": [M, HIDDEN, DIM], "launches_per_case": 9}
+    xa, wa = ops.to_mx_dim0(x, recipe_mode, L), ops.to_mx_dim0(w, recipe_mode, L)
+    out["0_this_kernel_random_data"] = timed(lambda: ops.mx_gemm_nt(xa, wa, out=dst))
+    oa = ops.to_mx_dim0(torch.ones_like(x), recipe_mode, L)
+    ob = ops.to_mx_dim0(torch.ones_like(w), recipe_mode, L)
+    out["1_this_kernel_all_ones"] = timed(lambda: ops.mx_gemm_nt(oa, ob, out=dst))
+    za = ops.to_mx_dim0(torch.zeros_like(x), recipe_mode, L)
+    zb = ops.to_mx_dim0(torch.zeros_like(w), recipe_mode, L)
+    out["2_this_kernel_all_zeros"] = timed(lambda: ops.mx_gemm_nt(za, zb, out=dst))
+    lib.mx_debug_set_grid(128)
+    try:
+        out["3_this_kernel_random_data_128_of_256_CUs"] = timed(lambda: ops.mx_gemm_nt(xa, wa, out=dst))
+    finally:
+        lib.mx_debug_set_grid(0)
+    a8 = x.to(torch.float8_e4m3fn)
+    b8 = (w.float() * 64).to(torch.float8_e4m3fn)  # spread over the fp8 range like the block-scaled codes
+    one = torch.ones((), device=dev)
+    try:
+        out["4_vendor_fp8_tensorwise_gemm_random_data"] = timed(
+            lambda: torch._scaled_mm(a8, b8.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16))
+    except Exception as ex:
+        out["4_vendor_fp8_tensorwise_gemm_random_data"] = {"error": f"{type(ex).__name__}: {str(ex)[:120]}"}
     return out
 
 
@@ -770,6 +835,9 @@ def main():
     _lib.load()  # fail loudly if the HIP library is missing
     dev = torch.device("cuda:0")
     recipe_mode = {"mxfp8_rceil": "rceil", "mxfp8_floor": "floor"}[args.recipe]
+    if args.clock_table:
+        print(json.dumps(clock_table(dev, recipe_mode)))
+        return
     ffn, x, h, dy_h, dy_o = build_linears(dev, args.recipe)
     x.requires_grad_(True)
     h.requires_grad_(True)
