@@ -54,6 +54,10 @@ def parse():
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run 4 elementwise passes over a 512 MiB tensor (reads 512 MiB, writes 512 MiB "
                          "each): the known-size kernel that scales FETCH_SIZE / WRITE_SIZE counter readings")
+    ap.add_argument("--cast-table", action="store_true",
+                    help="instead of the benchmark: the HBM yardsticks (copy, read, write) and the three casts on "
+                         "X [16384, 4096] and dY [16384, 14336], 8 launches each in that order on rotating buffers "
+                         "(for rocprofv3 --pmc runs of the memory-path counters)")
     ap.add_argument("--clock-table", action="store_true",
                     help="instead of the benchmark: the GEMM kernel at the benchmark shape on random data, on "
                          "constant operands and on half of the CUs, and the vendor library's fp8 GEMM, 8 launches "
@@ -186,6 +190,62 @@ def time_yardsticks(dev):
     sec = timed(lambda: dst.copy_(src), reps=10)
     out["device_copy_512MiB"] = {"GB/s": round(2 * src.numel() * 2 / sec / 1e9, 1),
                                  "frac_hbm": round(2 * src.numel() * 2 / sec / 1e9 / PEAK_HBM_GBPS, 3)}
+    del src, dst
+    torch.cuda.empty_cache()
+    out.update(_stream_yardsticks(dev))
+    return out
+
+
+def _stream_yardsticks(dev, nbuf=3, mib=512):
+    """The library's plain streaming kernels (16 bytes per lane, nontemporal) on buffers rotated
+    through more memory than the last-level cache: GB/s of copy (bytes read + bytes written),
+    read and write.  The practical ceiling of anything that only moves bytes on this box."""
+    import ctypes
+
+    import torch
+
+    from torchtitan_amd import _lib
+
+    lib = _lib.load()
+    lib.mx_debug_stream.restype = ctypes.c_int
+    lib.mx_debug_stream.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
+    nbytes = mib << 20
+    bufs = [torch.randint(0, 255, (nbytes,), device=dev, dtype=torch.uint8) for _ in range(nbuf + 1)]
+    sink = torch.zeros(16, device=dev, dtype=torch.uint8)
+    st = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+    def run(kind, i):
+        src = bufs[i % nbuf]
+        dst = bufs[i % nbuf + 1] if kind != 1 else sink
+        rc = lib.mx_debug_stream(kind, ctypes.c_void_p(src.data_ptr()), ctypes.c_void_p(dst.data_ptr()), nbytes, st)
+        assert rc == 0, rc
+
+    out = {}
+    for name, kind, moved in (("stream_copy", 0, 2 * nbytes), ("stream_read", 1, nbytes), ("stream_write", 2, nbytes)):
+        for i in range(2):
+            run(kind, i)
+        torch.cuda.synchronize()
+        reps = 8
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for i in range(reps):
+            run(kind, i)
+        e.record()
+        torch.cuda.synchronize()
+        sec = s.elapsed_time(e) * 1e-3 / reps
+        out[name] = {"MiB": mib, "us": round(sec * 1e6, 1), "GB/s": round(moved / sec / 1e9, 1),
+                     "frac_hbm": round(moved / sec / 1e9 / PEAK_HBM_GBPS, 3)}
+    return out
+
+
+def cast_table(dev, recipe_mode):
+    """The HBM yardsticks and then the casts, in a fixed order (see --cast-table): one JSON line of
+    HIP-event times; under rocprofv3 --pmc the dispatches appear in the same order."""
+    out = {"order": ["stream_copy", "stream_read", "stream_write", "dim0:x", "dim1:x", "dim0_dim1:x", "dim0:dy",
+                     "dim1:dy", "dim0_dim1:dy", "dim0:w", "dim1:w", "dim0_dim1:w"],
+           "launches_per_kernel": "2 warm-up + 8 timed (casts: 2 + 3 x buffers)"}
+    out["yardsticks"] = _stream_yardsticks(dev)
+    out["casts"] = time_casts(dev, recipe_mode)
     return out
 
 
@@ -837,6 +897,9 @@ def main():
     recipe_mode = {"mxfp8_rceil": "rceil", "mxfp8_floor": "floor"}[args.recipe]
     if args.clock_table:
         print(json.dumps(clock_table(dev, recipe_mode)))
+        return
+    if args.cast_table:
+        print(json.dumps(cast_table(dev, recipe_mode)))
         return
     ffn, x, h, dy_h, dy_o = build_linears(dev, args.recipe)
     x.requires_grad_(True)

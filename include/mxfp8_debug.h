@@ -7,6 +7,8 @@
 #ifndef MXFP8_DEBUG_H_
 #define MXFP8_DEBUG_H_
 
+#include <stdint.h>
+
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -24,6 +26,12 @@ void mx_debug_set_grid(int workgroups);
  * per-wave cycle counts {copy wait, barriers, step body, epilogue, ...}; NULL switches the timing
  * build off (default). */
 void mx_debug_set_prof(void* device_buffer);
+
+/* HBM yardsticks for bench.py: the plainest streaming kernels (16 bytes per lane, nontemporal),
+ * kind 0 = copy `bytes` from src to dst, 1 = read `bytes` of src (dst: 16 bytes that are never
+ * written for ordinary data), 2 = write `bytes` to dst.  bytes % 16 == 0, 16-byte aligned.
+ * Returns an mx_status_t. */
+int mx_debug_stream(int kind, const void* src, void* dst, int64_t bytes, void* stream);
 
 #ifdef __cplusplus
 }

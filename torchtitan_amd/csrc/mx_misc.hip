@@ -15,3 +15,50 @@ extern "C" const char* mx_status_string(int status) {
     default: return "unknown status";
   }
 }
+
+// ---- HBM yardsticks (include/mxfp8_debug.h) --------------------------------------------------
+// The plainest streaming kernels there are, 16 bytes per lane, every lane of a wave next to its
+// neighbour, nontemporal like the casts' accesses: what this chip's memory system gives a kernel
+// that does nothing but move bytes.  bench.py times them next to the casts.
+namespace mx {
+typedef uint32_t y_u32x4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void stream_copy_kernel(const y_u32x4* __restrict__ src,
+                                                          y_u32x4* __restrict__ dst, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+}
+__global__ __launch_bounds__(256) void stream_read_kernel(const y_u32x4* __restrict__ src, int64_t n,
+                                                          y_u32x4* __restrict__ sink) {
+  const int64_t i = (int64_t)blockIdx.x * 1024 + threadIdx.x;
+  y_u32x4 acc = {0, 0, 0, 0};
+#pragma unroll
+  for (int k = 0; k < 4; ++k)
+    if (i + k * 256 < n) {
+      const y_u32x4 v = __builtin_nontemporal_load(src + i + k * 256);
+      acc.x ^= v.x; acc.y ^= v.y; acc.z ^= v.z; acc.w ^= v.w;
+    }
+  // never true for the patterns bench.py fills the buffer with: keeps the loads alive
+  if (acc.x == 0x12345678u && acc.y == 0x9ABCDEF1u && acc.z == 0x0F1E2D3Cu) *sink = acc;
+}
+__global__ __launch_bounds__(256) void stream_write_kernel(y_u32x4* __restrict__ dst, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) __builtin_nontemporal_store(y_u32x4{(uint32_t)i, 1u, 2u, 3u}, dst + i);
+}
+}  // namespace mx
+
+extern "C" int mx_debug_stream(int kind, const void* src, void* dst, int64_t bytes, void* stream) {
+  if (bytes <= 0 || bytes % 16 || kind < 0 || kind > 2) return MX_ERR_INVALID_ARG;
+  if ((kind != 2 && (!src || ((uintptr_t)src & 15))) || !dst || ((uintptr_t)dst & 15)) return MX_ERR_INVALID_ARG;
+  const int64_t n = bytes / 16;
+  hipStream_t st = (hipStream_t)stream;
+  if (kind == 0)
+    hipLaunchKernelGGL(mx::stream_copy_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+                       (const mx::y_u32x4*)src, (mx::y_u32x4*)dst, n);
+  else if (kind == 1)
+    hipLaunchKernelGGL(mx::stream_read_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, st,
+                       (const mx::y_u32x4*)src, n, (mx::y_u32x4*)dst);
+  else
+    hipLaunchKernelGGL(mx::stream_write_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+                       (mx::y_u32x4*)dst, n);
+  return hipGetLastError() == hipSuccess ? MX_OK : MX_ERR_LAUNCH;
+}
