@@ -31,16 +31,34 @@ METRIC = "MXFP8 linear TFLOP/s fwd+bwd at 8B FFN shape; to_mx cast GB/s"
 M, DIM, HIDDEN = 16384, 4096, 14336
 PEAK_MXFP8_TFLOPS = 5000.0  # MI355X dense fp8 / MXFP8 MFMA peak
 PEAK_HBM_GBPS = 8000.0
-# Bytes the GEMM kernel moves between L2 and the memory fabric per launch, mean over the step's
-# nine GEMMs: rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the same counter reads for a
-# known-size elementwise kernel (profiles/gemm_nt32_kernel_and_cast_tile_kernel__ffn_fwd_bwd_M16384__hbm_traffic_pmc.txt).  Counters cannot
-# be read from inside this process, so the figure is carried here and re-measured when the kernel
-# changes.
-# Share of the GPU's active cycles in which the matrix pipes are busy under the GEMM kernel:
-# rocprofv3's MfmaUtil (SQ_VALU_MFMA_BUSY_CYCLES / (GRBM_GUI_ACTIVE x SIMDs)), measured offline
-# on the same command (profiles/gemm_nt32_kernel__ffn_fwd_bwd_M16384__mfma_utilisation_pmc.txt).
-GEMM_MFMA_UTIL_ROCPROF = 0.725
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 1813553618
+# Counter-derived figures of the GEMM kernel (bytes moved between L2 and the memory fabric per
+# launch; share of active cycles with the matrix pipes busy) cannot be read from inside this
+# process.  They are taken from the committed rocprofv3 summary below, which records the SHA-256 of
+# the kernel source it was measured on; when the source has changed since, they are left out.
+GEMM_COUNTER_SUMMARY = ROOT / "profiles" / "gemm_nt32_kernel__ffn_fwd_bwd_M16384__roofline_inputs.txt"
+GEMM_KERNEL_SOURCE = ROOT / "torchtitan_amd" / "csrc" / "mx_gemm32.hip"
+
+
+def profiled_gemm_figures():
+    """{'traffic': bytes per launch or None, 'mfma_util': float or None, 'note': str} from the
+    committed counter summary, if it belongs to the kernel source in this tree."""
+    import hashlib
+
+    none = {"traffic": None, "mfma_util": None}
+    try:
+        fields = dict(line.split(":", 1) for line in GEMM_COUNTER_SUMMARY.read_text().splitlines()
+                      if ":" in line and not line.startswith((" ", "#")))
+        fields = {k.strip(): v.strip() for k, v in fields.items()}
+        have = hashlib.sha256(GEMM_KERNEL_SOURCE.read_bytes()).hexdigest()
+    except OSError as ex:
+        return {**none, "note": f"no counter summary ({ex.__class__.__name__})"}
+    if fields.get("kernel_source_sha256") != have:
+        return {**none, "note": f"{GEMM_COUNTER_SUMMARY.name} was measured on another version of "
+                                f"{GEMM_KERNEL_SOURCE.name} (commit {fields.get('measured_at_commit', '?')}): left out"}
+    return {"traffic": int(fields["traffic_bytes_per_launch"]), "mfma_util": float(fields["mfma_util_steady_state"]),
+            "note": f"rocprofv3 counters, offline, {GEMM_COUNTER_SUMMARY.name} (commit {fields.get('measured_at_commit', '?')}): "
+                    "traffic = FETCH_SIZE + WRITE_SIZE per launch between L2 and the memory fabric (operands and output "
+                    "once would be 488.5e6); mfma_util = matrix-pipe busy cycles / active cycles in steady state"}
 
 
 def parse():
@@ -106,8 +124,10 @@ def one_step(ffn, x, h, dy_h, dy_o):
         y.backward(dy)
 
 
-def time_casts(dev, recipe_mode):
-    """to_mx GB/s per direction on cold inputs (rotating buffers > last-level cache)."""
+def time_casts(dev, recipe_mode, also_floor=False):
+    """to_mx GB/s per direction on cold inputs (rotating buffers > last-level cache).  With
+    `also_floor`, X is also cast with FLOOR scales (the mode BASELINE configs[0] names; it adds a
+    clamp per element on the finite path), keys suffixed ":floor"."""
     import torch
 
     from torchtitan_amd import ops
@@ -134,6 +154,36 @@ def time_casts(dev, recipe_mode):
             out[f"{kind}:{name}"] = {"us": round(sec * 1e6, 1), "GB/s": round(el * bpe / sec / 1e9, 1),
                                      "frac_hbm": round(el * bpe / sec / 1e9 / PEAK_HBM_GBPS, 3)}
         del bufs
+    if also_floor and recipe_mode != "floor":
+        floor = time_casts_one(dev, "floor", "x_16384x4096", (M, DIM), 6)
+        out.update({f"{k}:floor": v for k, v in floor.items()})
+    return out
+
+
+def time_casts_one(dev, mode, name, shape, nbuf):
+    import torch
+
+    from torchtitan_amd import ops
+
+    out = {}
+    L = ops.MX_SCALES_MFMA
+    bufs = [torch.randn(shape, device=dev, dtype=torch.bfloat16) for _ in range(nbuf)]
+    el = shape[0] * shape[1]
+    for kind, fn, bpe in (("dim0", ops.to_mx_dim0, 3.03125), ("dim1", ops.to_mx_dim1, 3.03125),
+                          ("dim0_dim1", ops.to_mx_dim0_dim1, 4.0625)):
+        for b in bufs[:2]:
+            fn(b, mode, L)
+        torch.cuda.synchronize()
+        reps = 3 * nbuf
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for i in range(reps):
+            fn(bufs[i % nbuf], mode, L)
+        e.record()
+        torch.cuda.synchronize()
+        sec = s.elapsed_time(e) * 1e-3 / reps
+        out[f"{kind}:{name}"] = {"us": round(sec * 1e6, 1), "GB/s": round(el * bpe / sec / 1e9, 1),
+                                 "frac_hbm": round(el * bpe / sec / 1e9 / PEAK_HBM_GBPS, 3)}
     return out
 
 
@@ -829,9 +879,10 @@ def time_expert_block(dev, recipe_mode, counts):
 
 
 def cpu_baseline(recipe_mode_int, target_s=15.0):
-    """CPU oracle on a bounded sample of BASELINE config 1: the emulated MX linear forward
-    (to_mx of X and W along K, dequantize, fp32 matmul, bf16 round) plus the column-wise casts
-    the backward needs, at N=14336, K=4096 and as many rows M as fit about `target_s` seconds
+    """CPU oracle on a bounded sample of the benchmark workload (BASELINE configs[1], the w1
+    linear): the emulated MX linear forward (to_mx of X and W along K, dequantize, fp32 matmul,
+    bf16 round) plus the column-wise casts the backward needs, with X ~ N(0,1) and W ~ N(0,0.02)
+    as in the GPU run, at N=14336, K=4096 and as many rows M as fit about `target_s` seconds
     (calibrated on M=1024 first)."""
     import numpy as np
 
@@ -842,8 +893,12 @@ def cpu_baseline(recipe_mode_int, target_s=15.0):
     os.environ.setdefault("OMP_NUM_THREADS", str(cores))
     K, N = DIM, HIDDEN
 
+    rng = np.random.default_rng(0)
+    wb = mo.f32_to_bf16_bits(rng.standard_normal((N, K), dtype=np.float32) * np.float32(0.02))
+    x_all = mo.f32_to_bf16_bits(rng.standard_normal((M, K), dtype=np.float32))
+
     def run(Ms):
-        xb, wb = mo.make_cfg1_inputs(0, Ms, K, N)
+        xb = x_all[:Ms]
         t0 = time.perf_counter()
         xc, xs = co.cast_dim0(xb, recipe_mode_int)
         wc, ws = co.cast_dim0(wb, recipe_mode_int)
@@ -874,8 +929,9 @@ def cpu_baseline(recipe_mode_int, target_s=15.0):
         "unit": "TFLOP/s",
         "cores": cores,
         "kind": "port",
-        "sample": f"config 1 at M={Ms} of {M} rows (X[{Ms},{K}], W[{N},{K}], 0.1% x100 outliers): to_mx dim0 and "
-                  f"dim1 of X and W (C oracle, OpenMP) + dequantize + fp32 matmul (NumPy BLAS) + bf16 round; "
+        "sample": f"configs[1], the w1 linear, first {Ms} of {M} token rows (X[{Ms},{K}] ~ N(0,1), W[{N},{K}] ~ "
+                  f"N(0,0.02), bf16): to_mx dim0 and dim1 of X and W (C oracle, OpenMP, recipe "
+                  f"{'rceil' if recipe_mode_int else 'floor'}) + dequantize + fp32 matmul (NumPy BLAS) + bf16 round; "
                   f"casts {cast_bytes / c_s / 1e9:.2f} GB/s in {c_s:.2f} s, matmul part "
                   f"{flops / m_s / 1e12:.3f} TFLOP/s in {m_s:.2f} s; mean of {reps} run(s)",
         "checksum": int(y.astype(np.uint64).sum() % (1 << 32)),
@@ -932,6 +988,7 @@ def main():
     n_gemm, gemm_ms = per_kernel["gemm_nt"]
     achieved = gemm_flops / (gemm_ms * 1e-3) / 1e12
     cast_ms = sum(ms * n for k, (n, ms) in per_kernel.items() if k.startswith("cast")) / args.steps
+    counters = profiled_gemm_figures()
     line = {
         "metric": METRIC,
         "value": round(value, 1),
@@ -959,12 +1016,9 @@ def main():
             "peak": PEAK_MXFP8_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_MXFP8_TFLOPS, 4),
-            "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH,
-            "traffic_note": "bytes per launch between L2 and fabric (rocprofv3 FETCH_SIZE + WRITE_SIZE, offline); "
-                            "operands and output once would be 488.5e6",
-            "mfma_util_rocprof": GEMM_MFMA_UTIL_ROCPROF,
-            "mfma_util_note": "matrix-pipe busy cycles / active cycles (rocprofv3 MfmaUtil, offline); frac = this x "
-                              "shader clock under the kernel (about 1.75 GHz) / 2.4 GHz",
+            "traffic": counters["traffic"],
+            "mfma_util_rocprof": counters["mfma_util"],
+            "counters_note": counters["note"],
             "launches_timed": n_gemm,
             "avg_launch_ms": round(gemm_ms, 4),
         },
@@ -976,7 +1030,7 @@ def main():
         "kernels_ms": {k: {"launches": n, "avg_ms": round(ms, 4)} for k, (n, ms) in sorted(per_kernel.items())},
     }
     if not args.no_casts:
-        line["casts"] = time_casts(dev, recipe_mode)
+        line["casts"] = time_casts(dev, recipe_mode, also_floor=True)
         line["moe_grouped_gemms"] = time_moe_grouped(dev, recipe_mode)
         del ffn, x, h, dy_h, dy_o
         torch.cuda.empty_cache()

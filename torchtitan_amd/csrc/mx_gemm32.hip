@@ -777,6 +777,8 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     });
   };
 
+  uint64_t prof_t0 = 0;
+  if constexpr (PROF) prof_t0 = __builtin_readcyclecounter();
   // ---- prologue: fill the ring, fetch the first fragments
   loader_open_tile();
   issue_block();
@@ -827,6 +829,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       o[4] = prof_e_stage;
       o[5] = prof_e_wait;
       o[6] = prof_e_store;
+      o[7] = __builtin_readcyclecounter() - prof_t0;
     }
   }
 }
