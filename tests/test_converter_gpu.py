@@ -703,3 +703,40 @@ def test_decoder_block_with_all_seven_linears_converted(device):
     for (n, pa), (_, pb) in zip(blk.named_parameters(), ref.named_parameters()):
         if pa.ndim == 2:
             assert rel_l2(pa.grad.float().cpu().numpy(), pb.grad.float().cpu().numpy()) < 0.15, n
+
+
+def test_decoder_block_under_torch_compile_equals_eager(device):
+    """The block wrapped as the reference wraps its transformer blocks
+    (torchtitan/models/llama3/parallelize.py:271-284: ``torch.compile(block, fullgraph=True)``):
+    every converted linear enters the graph as one opaque operator, forward and backward run
+    without a graph break, and output and all gradients equal the eager run bit for bit.  The
+    eager side runs with the gate fusion off, i.e. the same sequence of kernels; the backend
+    replays the traced graph op by op, so no code generator for the glue ops is involved."""
+    import torch._dynamo
+
+    torch.manual_seed(17)
+    blk = _MiniDecoderBlock(256, 4, 2, 512).to(device).to(torch.bfloat16)
+    for m in blk.modules():
+        if isinstance(m, nn.Linear):
+            nn.init.normal_(m.weight, std=0.02)
+    _convert(blk, ["attention", "feed_forward"], fuse=False)
+    x = torch.randn(2, 128, 256, device=device, dtype=torch.bfloat16)
+    dy = torch.randn_like(x) * 1e-2
+
+    def run(fn):
+        for p in blk.parameters():
+            p.grad = None
+        xi = x.clone().requires_grad_(True)
+        y = fn(xi)
+        y.backward(dy)
+        return [y.detach().clone(), xi.grad.clone()] + [p.grad.clone() for p in blk.parameters()]
+
+    want = run(blk)
+    torch._dynamo.reset()
+    compiled_blk = torch.compile(blk, backend="aot_eager", fullgraph=True)
+    got = run(compiled_blk)
+    again = run(compiled_blk)  # the second call reuses the compiled graph
+    assert len(got) == len(want)
+    for g, a, w in zip(got, again, want):
+        assert torch.equal(g, w) and torch.equal(a, w)
+    torch._dynamo.reset()

@@ -83,6 +83,8 @@ class _MXSwiGLULinear(torch.autograd.Function):
 def swiglu_fusable(h1: torch.Tensor, h3: torch.Tensor, weight: torch.Tensor) -> bool:
     """The fused gate + cast needs bf16 row-contiguous inputs of one shape with 32-aligned token
     and hidden counts (what a converted SwiGLU block produces) and a converted weight."""
+    if torch.compiler.is_compiling():  # the fused block functions are eager-only
+        return False
     if not isinstance(weight, MXFP8TrainingWeight) or not weight.mx_config.fuse_swiglu_cast:
         return False
     if h1.dtype != torch.bfloat16 or h3.dtype != torch.bfloat16 or h1.shape != h3.shape:
@@ -191,6 +193,8 @@ class _MXFeedForward(torch.autograd.Function):
 def feed_forward_fusable(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, w3: torch.Tensor) -> bool:
     """The whole-block function needs all three weights converted with gate fusion on, a bf16
     GPU activation and 32-aligned token, model and hidden sizes."""
+    if torch.compiler.is_compiling():  # the fused block functions are eager-only
+        return False
     ws = (w1, w2, w3)
     if not all(isinstance(w, MXFP8TrainingWeight) and w.mx_config.fuse_swiglu_cast for w in ws):
         return False
@@ -286,6 +290,8 @@ def norm_fusable(x: torch.Tensor, norm_weight: torch.Tensor | None, *weights: to
     """RMSNorm can move into the cast when the converter was built with `fuse_rmsnorm_cast`, the
     norm has a bf16 weight, every linear behind it is converted with in_features % 32 == 0 and
     out_features % 32 == 0, and x is a bf16 GPU tensor with a multiple of 32 tokens."""
+    if torch.compiler.is_compiling():  # the fused block functions are eager-only
+        return False
     if norm_weight is None or norm_weight.dtype != torch.bfloat16 or not weights:
         return False
     if not all(isinstance(w, MXFP8TrainingWeight) and w.mx_config.fuse_rmsnorm_cast and w.dim() == 2 for w in weights):
@@ -418,6 +424,8 @@ def grouped_feed_forward_fusable(x: torch.Tensor, w1: torch.Tensor, w2: torch.Te
                                  w3: torch.Tensor) -> bool:
     """All three expert parameters converted with gate fusion on, a 2-D GPU activation, model
     and hidden sizes multiples of 32."""
+    if torch.compiler.is_compiling():  # the fused block functions are eager-only
+        return False
     ws = (w1, w2, w3)
     if not all(isinstance(w, MXFP8TrainingWeight) and w.mx_config.fuse_swiglu_cast and w.dim() == 3 for w in ws):
         return False

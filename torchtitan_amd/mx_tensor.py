@@ -463,6 +463,13 @@ class MXFP8TrainingWeight(torch.Tensor):
             w = args[1] if len(args) > 1 else kwargs["weight"]
             b = args[2] if len(args) > 2 else kwargs.get("bias")
             if isinstance(w, cls) and not isinstance(x, cls):
+                if torch.compiler.is_compiling():
+                    # a tracer cannot follow the eager path's library calls: the linear enters
+                    # the graph as one opaque operator (torchtitan_amd/compiled.py)
+                    from .compiled import mx_linear_traced
+
+                    with torch._C.DisableTorchFunctionSubclass():
+                        return mx_linear_traced(x, w, b, w.mx_config.scale_mode)
                 return mx_linear(x, _unwrap(w), _unwrap(b), w.mx_config)
         elif func in _GROUPED_FUNCS:
             a, b = args[0], args[1]

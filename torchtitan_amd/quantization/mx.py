@@ -119,7 +119,8 @@ class MXFP8Converter(QuantizationConverter):
         if config.recipe_name not in _RECIPES:
             raise ValueError(f"unknown recipe {config.recipe_name!r}; options: {sorted(_RECIPES)}")
         if model_compile_enabled:
-            logger.warning("the MXFP8 path runs eager HIP kernels; torch.compile adds nothing to it")
+            logger.info("under torch.compile a converted linear is one opaque operator per pass; cast sharing "
+                        "between sibling linears and the gate / norm fusions are features of the eager path")
         self.config = config
         # which nn.Linear modules may be converted: dims % 16 and not excluded by name
         # (built as in torchtitan/components/quantization/float8.py:176)
