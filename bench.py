@@ -80,6 +80,12 @@ def parse():
                     help="instead of the benchmark: the GEMM kernel at the benchmark shape on random data, on "
                          "constant operands and on half of the CUs, and the vendor library's fp8 GEMM, 8 launches "
                          "each in that order (for a rocprofv3 --pmc run: active cycles / time = shader clock)")
+    ap.add_argument("--gemm-ablation", action="store_true",
+                    help="instead of the benchmark: the dense GEMM at the benchmark shape and the three grouped "
+                         "GEMMs of the MoE config (equal groups and the skewed routing), timed with whatever build "
+                         "of the library MXFP8_LIBRARY names: run once with the product library and once each with "
+                         "variants built without the output stores / without the epilogue "
+                         "(python -m torchtitan_amd._build --define MX_ABL_STORE_ROWS=0 | MX_ABL_NO_EPILOGUE --out ...)")
     return ap.parse_args()
 
 
@@ -249,7 +255,9 @@ def time_yardsticks(dev):
 def _stream_yardsticks(dev, nbuf=3, mib=512):
     """The library's plain streaming kernels (16 bytes per lane, nontemporal) on buffers rotated
     through more memory than the last-level cache: GB/s of copy (bytes read + bytes written),
-    read and write.  The practical ceiling of anything that only moves bytes on this box."""
+    read, write, and 2 bytes read per byte written (the mix of a one-direction cast; a fused cast
+    writes as much as it reads, like the copy).  The practical ceiling of anything that only moves
+    bytes on this box."""
     import ctypes
 
     import torch
@@ -271,7 +279,8 @@ def _stream_yardsticks(dev, nbuf=3, mib=512):
         assert rc == 0, rc
 
     out = {}
-    for name, kind, moved in (("stream_copy", 0, 2 * nbytes), ("stream_read", 1, nbytes), ("stream_write", 2, nbytes)):
+    for name, kind, moved in (("stream_copy", 0, 2 * nbytes), ("stream_read", 1, nbytes), ("stream_write", 2, nbytes),
+                              ("stream_2to1", 3, nbytes + nbytes // 2)):
         for i in range(2):
             run(kind, i)
         torch.cuda.synchronize()
@@ -288,14 +297,93 @@ def _stream_yardsticks(dev, nbuf=3, mib=512):
     return out
 
 
+def _casts_against_streams(casts, yardsticks):
+    """Adds to every cast its rate as a share of the plain streaming kernel with the same read : write
+    mix, timed in the same run: 2 : 1 for one direction, 1 : 1 (the copy) for the fused cast."""
+    for key, row in casts.items():
+        ref = yardsticks.get("stream_copy" if key.startswith("dim0_dim1") else "stream_2to1")
+        if ref and ref.get("GB/s"):
+            row["frac_of_stream_same_mix"] = round(row["GB/s"] / ref["GB/s"], 3)
+
+
 def cast_table(dev, recipe_mode):
     """The HBM yardsticks and then the casts, in a fixed order (see --cast-table): one JSON line of
     HIP-event times; under rocprofv3 --pmc the dispatches appear in the same order."""
-    out = {"order": ["stream_copy", "stream_read", "stream_write", "dim0:x", "dim1:x", "dim0_dim1:x", "dim0:dy",
+    out = {"order": ["stream_copy", "stream_read", "stream_write", "stream_2to1", "dim0:x", "dim1:x", "dim0_dim1:x", "dim0:dy",
                      "dim1:dy", "dim0_dim1:dy", "dim0:w", "dim1:w", "dim0_dim1:w"],
            "launches_per_kernel": "2 warm-up + 8 timed (casts: 2 + 3 x buffers)"}
     out["yardsticks"] = _stream_yardsticks(dev)
     out["casts"] = time_casts(dev, recipe_mode)
+    _casts_against_streams(out["casts"], out["yardsticks"])
+    return out
+
+
+def gemm_ablation(dev, recipe_mode):
+    """Wall time of the GEMM kernel's launches under the library build in use (see --gemm-ablation):
+    with builds that leave out the output stores or the whole epilogue the differences say what the
+    stores, the epilogue's instructions and the K loop each cost.  Outputs of such builds are not
+    results; nothing here checks them."""
+    import torch
+
+    from torchtitan_amd import _lib, ops
+
+    L = ops.MX_SCALES_MFMA
+
+    def timed(fn, reps=8):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(5):
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            for _ in range(reps):
+                fn()
+            e.record()
+            torch.cuda.synchronize()
+            ts.append(s.elapsed_time(e) * 1e-3 / reps)
+        return sorted(ts)[2]
+
+    out = {"library": str(_lib.LIB_PATH)}
+    g = torch.Generator(device=dev).manual_seed(0)
+    x = torch.randn((M, DIM), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    w = (torch.randn((HIDDEN, DIM), generator=g, device=dev, dtype=torch.float32) * 0.02).to(torch.bfloat16)
+    xa, wa = ops.to_mx_dim0(x, recipe_mode, L), ops.to_mx_dim0(w, recipe_mode, L)
+    dst = torch.empty((M, HIDDEN), device=dev, dtype=torch.bfloat16)
+    sec = timed(lambda: ops.mx_gemm_nt(xa, wa, out=dst), reps=6)
+    out["dense_M16384_N14336_K4096"] = {"us": round(sec * 1e6, 1), "TFLOP/s": round(2.0 * M * HIDDEN * DIM / sec / 1e12, 1)}
+    del x, w, xa, wa, dst
+    E, dim, hid, tokens, topk = 128, 2048, 768, 16384, 8
+    routed = tokens * topk
+    flops = 2.0 * routed * dim * hid
+    for kind in ("equal_groups", "skewed_routing"):
+        if kind == "equal_groups":
+            counts = torch.full((E,), routed // E, dtype=torch.int32, device=dev)
+        else:
+            gg = torch.Generator(device=dev).manual_seed(3)
+            logits = torch.randn((tokens, E), generator=gg, device=dev) + 0.5 * torch.randn((1, E), generator=gg, device=dev)
+            gumbel = -torch.log(-torch.log(torch.rand((tokens, E), generator=gg, device=dev).clamp_min(1e-9)))
+            top = torch.topk(torch.softmax(logits + gumbel, dim=-1), topk, dim=-1).indices
+            counts = torch.bincount(top.flatten(), minlength=E).to(torch.int32)
+        max_len = -(-(routed + 128 * E) // 128) * 128
+        _, _, offs = ops.group_offsets_pad(counts, E, 1, max_len, 128)
+        xm = torch.randn((max_len, dim), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        wm = (torch.randn((E, hid, dim), generator=g, device=dev, dtype=torch.float32) * 0.02).to(torch.bfloat16)
+        dy = (torch.randn((max_len, hid), generator=g, device=dev, dtype=torch.float32) * 1e-3).to(torch.bfloat16)
+        xq0, xq1 = ops.to_mx_dim0_dim1(xm, recipe_mode, L)
+        dyq0, dyq1 = ops.to_mx_dim0_dim1(dy, recipe_mode, L)
+        wq0, wq1 = ops.to_mx_dim0_dim1_batched(wm, recipe_mode, L)
+        y = torch.empty((max_len, hid), device=dev, dtype=torch.bfloat16)
+        dx = torch.empty((max_len, dim), device=dev, dtype=torch.bfloat16)
+        dw = torch.empty((E, hid, dim), device=dev, dtype=torch.bfloat16)
+        row = {"padded_rows": int(offs[-1])}
+        for name, fn in (("fwd_2d3d", lambda: ops.mx_grouped_gemm_2d3d(xq0, wq0, offs, y)),
+                         ("dgrad_2d3d", lambda: ops.mx_grouped_gemm_2d3d(dyq0, wq1, offs, dx)),
+                         ("wgrad_2d2d", lambda: ops.mx_grouped_gemm_2d2d(dyq1, xq1, offs, dw))):
+            sec = timed(fn)
+            row[name] = {"us": round(sec * 1e6, 1), "TFLOP/s": round(flops / sec / 1e12, 1)}
+        out[kind] = row
+        del xm, wm, dy, xq0, xq1, dyq0, dyq1, wq0, wq1, y, dx, dw
     return out
 
 
@@ -954,6 +1042,9 @@ def main():
     if args.clock_table:
         print(json.dumps(clock_table(dev, recipe_mode)))
         return
+    if args.gemm_ablation:
+        print(json.dumps(gemm_ablation(dev, recipe_mode)))
+        return
     if args.cast_table:
         print(json.dumps(cast_table(dev, recipe_mode)))
         return
@@ -1043,6 +1134,7 @@ def main():
         line["policy_loss_logprobs"] = time_policy_loss(dev)
         torch.cuda.empty_cache()
         line["yardsticks"] = time_yardsticks(dev)
+        _casts_against_streams(line["casts"], line["yardsticks"])
         same = line["yardsticks"].get("this_gemm_kernel_on_constant_operands", {})
         if "frac_of_peak" in same:
             line["roofline"]["frac_on_constant_operands"] = same["frac_of_peak"]

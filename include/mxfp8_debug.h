@@ -29,7 +29,8 @@ void mx_debug_set_prof(void* device_buffer);
 
 /* HBM yardsticks for bench.py: the plainest streaming kernels (16 bytes per lane, nontemporal),
  * kind 0 = copy `bytes` from src to dst, 1 = read `bytes` of src (dst: 16 bytes that are never
- * written for ordinary data), 2 = write `bytes` to dst.  bytes % 16 == 0, 16-byte aligned.
+ * written for ordinary data), 2 = write `bytes` to dst, 3 = read `bytes` of src and write
+ * `bytes` / 2 to dst (the read : write mix of a one-direction cast).  bytes % 16 == 0, 16-byte aligned.
  * Returns an mx_status_t. */
 int mx_debug_stream(int kind, const void* src, void* dst, int64_t bytes, void* stream);
 

@@ -9,7 +9,11 @@ import ctypes
 from ctypes import c_int, c_int64, c_void_p, c_char_p
 from pathlib import Path
 
-LIB_PATH = Path(__file__).resolve().parent / "libmxfp8_gfx950.so"
+import os
+
+# MXFP8_LIBRARY names another build of the same library (a measurement variant made by
+# `python -m torchtitan_amd._build --define ... --out ...`); unset, the in-tree product library.
+LIB_PATH = Path(os.environ.get("MXFP8_LIBRARY") or Path(__file__).resolve().parent / "libmxfp8_gfx950.so").resolve()
 
 MX_SCALE_FLOOR = 0
 MX_SCALE_RCEIL = 1

@@ -23,8 +23,9 @@
 // of 32-element block b is taken from lane group b.  With the first operand = B rows and the
 // second = A rows, a lane ends up with D[row = l & 31][col = 8q + 4j + 0..3], q = 0..3.
 //
-// MX_ABL_NO_DMA / MX_ABL_NO_READ (never defined in the product build) drop the copies or the
-// fragment reads from the steady state, to time what is left; results are then meaningless.
+// MX_ABL_NO_DMA / MX_ABL_NO_READ / MX_ABL_STORE_ROWS (never defined in the product build) drop the
+// copies, the fragment reads or part of the output stores from the steady state, to time what is
+// left; results are then meaningless.
 #include "mx_gemm_tile.h"
 
 namespace mx {
@@ -770,6 +771,9 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
         }
         const v4i rq = pin(r[pc & 1][q]);
         const u32x4 w = {(uint32_t)rq.x, (uint32_t)rq.y, (uint32_t)rq.z, (uint32_t)rq.w};
+#ifdef MX_ABL_STORE_ROWS  // timing ablation: only sub-tile rows below this many are written
+        if constexpr (m < MX_ABL_STORE_ROWS)
+#endif
         __builtin_amdgcn_raw_buffer_store_b128(w, rd, v, (m * 32 + q * 8) * ldd_b, MX_STORE_AUX);
         __builtin_amdgcn_sched_barrier(0);
       });
@@ -814,7 +818,11 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
         prof_last = __builtin_readcyclecounter();
         prof_epi += prof_last - e0;
       } else {
+#ifndef MX_ABL_NO_EPILOGUE
         epilogue(t);
+#else
+        (void)t;  // timing ablation: the MFMAs are volatile assembly and stay
+#endif
       }
     }
   }

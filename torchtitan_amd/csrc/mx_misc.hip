@@ -40,6 +40,16 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const y_u32x4* __restr
   // never true for the patterns bench.py fills the buffer with: keeps the loads alive
   if (acc.x == 0x12345678u && acc.y == 0x9ABCDEF1u && acc.z == 0x0F1E2D3Cu) *sink = acc;
 }
+// a row-wise cast's traffic without the cast: 16 bytes read and 8 bytes written per lane
+typedef uint32_t y_u32x2 __attribute__((ext_vector_type(2)));
+__global__ __launch_bounds__(256) void stream_2to1_kernel(const y_u32x4* __restrict__ src,
+                                                          y_u32x2* __restrict__ dst, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) {
+    const y_u32x4 v = __builtin_nontemporal_load(src + i);
+    __builtin_nontemporal_store(y_u32x2{v.x ^ v.z, v.y ^ v.w}, dst + i);
+  }
+}
 __global__ __launch_bounds__(256) void stream_write_kernel(y_u32x4* __restrict__ dst, int64_t n) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i < n) __builtin_nontemporal_store(y_u32x4{(uint32_t)i, 1u, 2u, 3u}, dst + i);
@@ -47,7 +57,7 @@ __global__ __launch_bounds__(256) void stream_write_kernel(y_u32x4* __restrict__
 }  // namespace mx
 
 extern "C" int mx_debug_stream(int kind, const void* src, void* dst, int64_t bytes, void* stream) {
-  if (bytes <= 0 || bytes % 16 || kind < 0 || kind > 2) return MX_ERR_INVALID_ARG;
+  if (bytes <= 0 || bytes % 16 || kind < 0 || kind > 3) return MX_ERR_INVALID_ARG;
   if ((kind != 2 && (!src || ((uintptr_t)src & 15))) || !dst || ((uintptr_t)dst & 15)) return MX_ERR_INVALID_ARG;
   const int64_t n = bytes / 16;
   hipStream_t st = (hipStream_t)stream;
@@ -57,6 +67,9 @@ extern "C" int mx_debug_stream(int kind, const void* src, void* dst, int64_t byt
   else if (kind == 1)
     hipLaunchKernelGGL(mx::stream_read_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, st,
                        (const mx::y_u32x4*)src, n, (mx::y_u32x4*)dst);
+  else if (kind == 3)
+    hipLaunchKernelGGL(mx::stream_2to1_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+                       (const mx::y_u32x4*)src, (mx::y_u32x2*)dst, n);
   else
     hipLaunchKernelGGL(mx::stream_write_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
                        (mx::y_u32x4*)dst, n);
