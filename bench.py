@@ -365,8 +365,8 @@ def gemm_ablation(dev, recipe_mode):
             gumbel = -torch.log(-torch.log(torch.rand((tokens, E), generator=gg, device=dev).clamp_min(1e-9)))
             top = torch.topk(torch.softmax(logits + gumbel, dim=-1), topk, dim=-1).indices
             counts = torch.bincount(top.flatten(), minlength=E).to(torch.int32)
-        max_len = -(-(routed + 128 * E) // 128) * 128
-        _, _, offs = ops.group_offsets_pad(counts, E, 1, max_len, 128)
+        max_len = -(-(routed + 32 * E) // 128) * 128
+        _, _, offs = ops.group_offsets_pad(counts, E, 1, max_len, 32)
         xm = torch.randn((max_len, dim), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
         wm = (torch.randn((E, hid, dim), generator=g, device=dev, dtype=torch.float32) * 0.02).to(torch.bfloat16)
         dy = (torch.randn((max_len, hid), generator=g, device=dev, dtype=torch.float32) * 1e-3).to(torch.bfloat16)
@@ -819,8 +819,8 @@ def time_policy_loss(dev):
 def time_moe_grouped(dev, recipe_mode):
     """BASELINE configs[3] GEMMs (not the headline): 128 experts, hidden 2048, expert FFN 768,
     top-8 routing of 16384 tokens from softmax over seeded Gumbel-perturbed logits (uneven
-    groups), groups padded to multiples of 128 rows for the persistent kernel.  TFLOP/s counts
-    the unpadded routed rows only."""
+    groups), groups padded to multiples of 32 rows as the config says (the token axis to a
+    multiple of 128).  TFLOP/s counts the unpadded routed rows only."""
     import torch
 
     from torchtitan_amd import ops
@@ -832,8 +832,8 @@ def time_moe_grouped(dev, recipe_mode):
     top = torch.topk(torch.softmax(logits + gumbel, dim=-1), topk, dim=-1).indices
     counts = torch.bincount(top.flatten(), minlength=E).to(torch.int32)
     routed = tokens * topk
-    max_len = -(-(routed + 128 * E) // 128) * 128
-    _, m_sizes, offs = ops.group_offsets_pad(counts, E, 1, max_len, 128)
+    max_len = -(-(routed + 32 * E) // 128) * 128
+    _, m_sizes, offs = ops.group_offsets_pad(counts, E, 1, max_len, 32)
     L = ops.MX_SCALES_MFMA
     x = torch.randn((max_len, dim), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
     w = (torch.randn((E, hid, dim), generator=g, device=dev, dtype=torch.float32) * 0.02).to(torch.bfloat16)

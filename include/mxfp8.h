@@ -269,10 +269,11 @@ int mx_gemm_nt_pair(const uint8_t* a_codes, const uint8_t* a_scales, const uint8
  * zeros.  a_scale_order says how a_scales is laid out:
  *   MX_SCALES_ROWMAJOR  [T, K/32]; groups may end anywhere (tile kernel);
  *   MX_SCALES_MFMA      MFMA order over the whole [T, K/32] matrix; every group must end at a
- *                       multiple of 128 rows, T % 128 == 0, K % 128 == 0, N % 8 == 0,
- *                       G <= 638: the persistent 32x32x64 kernel (several times faster).  The
- *                       group ends live on the device, so they are checked there: a violation
- *                       fills D with NaN.
+ *                       multiple of 32 rows (the alignment of the reference's padded token
+ *                       groups, torchtitan/components/quantization/__init__.py:36),
+ *                       T % 32 == 0, K % 128 == 0, N % 8 == 0, G <= 510: the persistent
+ *                       32x32x64 kernel (several times faster).  The group ends live on the
+ *                       device, so they are checked there: a violation fills D with NaN.
  * Stands in for torch._grouped_mm(x, w^T, offs) in forward and dgrad
  * (torchtitan/models/common/moe/moe.py:59-76). */
 int mx_grouped_gemm_2d3d(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
@@ -296,7 +297,7 @@ int mx_grouped_gemm_2d3d_pair(const uint8_t* a_codes, const uint8_t* a_scales,
  * column-wise casts; scale_order says how both scale buffers are laid out:
  *   MX_SCALES_ROWMAJOR  [N, T/32] and [K, T/32]; every group size a multiple of 32
  *                       (torchtitan/models/common/moe/utils.py:47-52);
- *   MX_SCALES_MFMA      MFMA order; every group must end at a multiple of 128 tokens,
+ *   MX_SCALES_MFMA      MFMA order; every group must end at a multiple of 32 tokens,
  *                       T % 128 == 0, K % 8 == 0: the persistent kernel; checked on the
  *                       device, a violation fills D with NaN.
  * Empty groups give zeros.  d is [G,N,K] bf16 dense. */

@@ -77,18 +77,23 @@ def test_grouped_wgrad(device, sizes, N, K):
 
 
 FAST_CASES = [
-    # (group sizes, all multiples of 128; N; K) -- the persistent-kernel forms (MFMA-order scales)
+    # (group sizes, multiples of 32; N; K) -- the persistent-kernel forms (MFMA-order scales)
     ([128, 256, 384], 256, 128),
     ([0, 128, 0, 640, 0], 128, 256),
     ([512, 128, 0, 1024, 256], 768, 384),
     ([1280, 384], 264, 512),
+    # groups that start and end inside 128-row scale groups / 128-deep K blocks
+    ([96, 160, 32, 0, 416, 288], 256, 256),
+    ([32, 32, 32, 32, 32, 1056, 64], 384, 128),
+    ([352, 2880, 0, 64, 992], 256, 384),
+    ([224, 0, 0, 32, 608, 96, 320], 520, 256),
 ]
 
 
 @pytest.mark.parametrize("sizes,N,K", FAST_CASES)
 @pytest.mark.parametrize("tail_rows", [0, 128, 384])
 def test_grouped_forward_and_dgrad_aligned_groups(device, sizes, N, K, tail_rows):
-    """2D x 3D through the persistent kernel: groups end at multiples of 128, MFMA-order scales."""
+    """2D x 3D through the persistent kernel: groups end at multiples of 32, MFMA-order scales."""
     rng = np.random.default_rng(sum(sizes) + N + K + 7)
     T = sum(sizes) + tail_rows
     G = len(sizes)
@@ -116,9 +121,10 @@ def test_grouped_forward_and_dgrad_aligned_groups(device, sizes, N, K, tail_rows
 
 @pytest.mark.parametrize("sizes,N,K", FAST_CASES)
 def test_grouped_wgrad_aligned_groups(device, sizes, N, K):
-    """2D x 2D through the persistent kernel: token groups end at multiples of 128."""
+    """2D x 2D through the persistent kernel: token groups end at multiples of 32 (the token axis
+    itself is a multiple of 128 and runs past the last group)."""
     rng = np.random.default_rng(sum(sizes) * 5 + N + K)
-    T = sum(sizes) + 128
+    T = -(-(sum(sizes) + 128) // 128) * 128
     x_bits = randn_bits(rng, (T, K), outliers=1e-3)
     dy_bits = randn_bits(rng, (T, N), std=1e-3)
     offs = _sizes_to_offs(sizes, device)
@@ -172,9 +178,36 @@ def test_aligned_group_forms_split_into_several_launches(device):
         lib.mx_debug_set_grid(0)
 
 
-def test_aligned_group_forms_poison_the_output_when_a_group_end_is_not_a_multiple_of_128(device):
+def test_neighbouring_groups_do_not_leak_into_a_ragged_group(device):
+    """A group that ends inside a 128-row scale group / a 128-deep K block shares that block with
+    its neighbour in memory.  NaN everywhere in the neighbours must not reach its results."""
+    rng = np.random.default_rng(77)
+    sizes, N, K = [160, 96, 224, 32], 256, 256    # ends 160, 256, 480, 512
+    T = sum(sizes)
+    x_bits = randn_bits(rng, (T, K), outliers=1e-3)
+    dy_bits = randn_bits(rng, (T, N), std=1e-3)
+    w_bits = randn_bits(rng, (len(sizes), N, K), std=0.02)
+    lo, hi = 256, 480                               # group 2
+    x_nan, dy_nan = x_bits.copy(), dy_bits.copy()
+    x_nan[:lo] = 0x7FC0
+    x_nan[hi:] = 0x7FC0
+    dy_nan[:lo] = 0x7FC0
+    dy_nan[hi:] = 0x7FC0
+    offs = _sizes_to_offs(sizes, device)
+    x, dy, w = bf16_from_bits(x_nan, device), bf16_from_bits(dy_nan, device), bf16_from_bits(w_bits, device)
+    y = ops.mx_grouped_gemm_2d3d(ops.to_mx_dim0(x, "rceil", L), ops.to_mx_dim0_batched(w, "rceil", L), offs)
+    ref = mo.grouped_fwd(x_bits, w_bits, np.cumsum(sizes), mo.RCEIL)
+    assert rel_l2(_f32(bits_of(y)[lo:hi]), _f32(ref[lo:hi])) <= TOL
+    assert torch.isnan(y[:lo]).all() and torch.isnan(y[hi:]).all()
+    dw = ops.mx_grouped_gemm_2d2d(ops.to_mx_dim1(dy, "rceil", L), ops.to_mx_dim1(x, "rceil", L), offs)
+    refw = mo.grouped_wgrad(dy_bits, x_bits, np.cumsum(sizes), mo.RCEIL)
+    assert rel_l2(_f32(bits_of(dw)[2]), _f32(refw[2])) <= TOL
+    assert torch.isnan(dw[0]).all() and torch.isnan(dw[1]).all() and torch.isnan(dw[3]).all()
+
+
+def test_aligned_group_forms_poison_the_output_when_a_group_end_is_not_a_multiple_of_32(device):
     rng = np.random.default_rng(5)
-    sizes, N, K = [128, 160, 96], 128, 128
+    sizes, N, K = [128, 144, 112], 128, 128
     T = sum(sizes)
     x = bf16_from_bits(randn_bits(rng, (T, K)), device)
     w = bf16_from_bits(randn_bits(rng, (len(sizes), N, K), std=0.02), device)

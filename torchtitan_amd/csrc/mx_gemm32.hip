@@ -38,9 +38,13 @@ constexpr int kK32 = 64;                         // K per compute step
 constexpr int kKB = 128;                         // K per ring block (= one cache line per row)
 constexpr int kOperand32 = kT32 * kKB;           // 32 KB: 256 rows x 128 B
 constexpr int kCodes32 = 2 * kOperand32;         // A rows then B rows
-constexpr int kBlock32 = kCodes32 + 2048;        // + scales: 4 groups (A0, A1, B0, B1) x 2 steps x 256 B
-constexpr int kRing32 = 2 * kBlock32;            // 132 KB
-constexpr uint32_t kMaxTileRecords = 120;        // grouped modes: tile records a workgroup keeps in LDS
+constexpr int kBlock32 = kCodes32 + 3072;        // + scales: groups A0, A1, B0, B1, A2 (+ 512 unused) x 2 steps x 256 B
+constexpr int kRing32 = 2 * kBlock32;            // 134 KB
+constexpr int kPatch32 = 6656;                   // per wave: 4608 B output patch + 2 KB of records / tables
+constexpr int kPatchUsed = 4608;
+constexpr uint32_t kRecordsPerPatch = (kPatch32 - kPatchUsed) / 64;
+constexpr uint32_t kMaxTileRecords = 3 * kRecordsPerPatch;  // grouped modes: tile records a workgroup keeps in LDS
+static_assert(kRing32 + 4 * kPatch32 == 160 * 1024, "the kernel's LDS map fills the CU's 160 KB");
 
 // What a launch works on.  One kernel serves three problems that differ only in how a linear
 // tile number maps to operand rows, K range and output address:
@@ -82,6 +86,10 @@ struct Tile32 {
   bool empty;              // no K range (an empty group, rows behind the last group, or poison):
                            // one block of out-of-range reads, i.e. zeros, stands in for it
   bool poison;             // grouped modes: the group ends break the alignment contract
+  uint32_t rot;            // kGrouped2d3d: 32-row blocks between the tile's first row and the start of
+                           // its 128-row scale group (0..3): the A scale bytes are turned by as much
+  uint32_t head, tail;     // kGrouped2d2d: the K range starts `head` 32-deep blocks into its first
+                           // 128-deep block and ends `tail` of them into its last (0: at its end)
 };
 
 // Tile order: 8-tall column-major panels, so tiles that run together share A and B panels.
@@ -137,6 +145,7 @@ struct Frags32 {
   v8i a[4];
   v8i b[4];
   uint32_t sa, sb;
+  uint32_t sa_hi;  // kGrouped2d3d: the A scale dword of the next 128-row group (see rotate_scales)
 };
 
 template <int MODE, bool PROF, bool PAIR = false>
@@ -156,16 +165,16 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
 
   // ---- tile count.  kGrouped2d3d: group g has ceil(rows_g / 256) x tiles_n tiles; the first
   //      tile number of every group (G + 2 entries, the last group being the zero rows behind
-  //      offs[G-1]) is kept in the 2.5 KB that wave 0's output patch leaves unused.
+  //      offs[G-1]) is kept in the 2 KB that wave 0's output patch leaves unused.
   bool poison = false;
   bool dealt = false;  // kGrouped2d2d: tiles dealt by length (below) instead of in tile order
-  constexpr uint32_t kMaxDealt = 640;  // two uint16 per group in wave 0's 2.5 KB of spare patch LDS
+  constexpr uint32_t kMaxDealt = (kPatch32 - kPatchUsed) / 4;  // two uint16 per group in wave 0's spare patch LDS
   constexpr uint32_t kMinDealt = 32;   // fewer groups than that cannot be spread evenly over 8 XCDs
   uint32_t nb;
   // "any thread saw a bad group end", through a word of wave 1's spare patch bytes (the
   // kernel's whole 160 KB are dynamic LDS: a library reduction would ask for more)
   auto any_bad = [&](int bad) -> bool {
-    uint32_t* flag = reinterpret_cast<uint32_t*>(smem + kRing32 + 7168 + 4608);
+    uint32_t* flag = reinterpret_cast<uint32_t*>(smem + kRing32 + kPatch32 + kPatchUsed);
     if (tid == 0) *flag = 0;
     __syncthreads();
     if (bad) atomicOr(flag, 1u);
@@ -179,13 +188,13 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   } else if constexpr (MODE == kGrouped2d2d) {
     nb = G * (uint32_t)((p.M + kT32 - 1) / kT32) * tiles_n;
     // group lengths in K blocks, kept for the dealing below (up to kMaxDealt groups)
-    uint16_t* g_blocks = reinterpret_cast<uint16_t*>(smem + kRing32 + 4608);
+    uint16_t* g_blocks = reinterpret_cast<uint16_t*>(smem + kRing32 + kPatchUsed);
     int bad = 0;
     for (uint32_t g = tid; g < G; g += 256) {
       const int32_t hi = p.offs[g], lo = g ? p.offs[g - 1] : 0;
-      bad |= (hi & 127) | (hi < lo) | (hi > (int64_t)K) | (lo < 0);
+      bad |= (hi & 31) | (hi < lo) | (hi > (int64_t)K) | (lo < 0);
       if (G <= kMaxDealt && G >= kMinDealt) {
-        const int64_t len = hi > lo ? ((int64_t)hi - lo) >> 7 : 0;
+        const int64_t len = hi > lo ? (((int64_t)hi + 127) >> 7) - (lo >> 7) : 0;
         g_blocks[g] = (uint16_t)(len > 0xFFFF ? 0xFFFF : len);
       }
     }
@@ -207,11 +216,11 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       __syncthreads();
     }
   } else {
-    uint32_t* first = reinterpret_cast<uint32_t*>(smem + kRing32 + 4608);
+    uint32_t* first = reinterpret_cast<uint32_t*>(smem + kRing32 + kPatchUsed);
     int bad = 0;
     for (uint32_t g = tid; g <= G; g += 256) {
       const int64_t lo = g ? p.offs[g - 1] : 0, hi = g < G ? (int64_t)p.offs[g] : p.M;
-      bad |= (g < G && (hi & 127)) | (hi < lo) | (hi > p.M) | (lo < 0);
+      bad |= (g < G && (hi & 31)) | (hi < lo) | (hi > p.M) | (lo < 0);
       const int64_t rows = hi > lo ? hi - lo : 0;
       first[g + 1] = (uint32_t)((rows + kT32 - 1) / kT32) * tiles_n;
     }
@@ -277,6 +286,9 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     r.poison = poison;
     r.koff = 0;
     r.empty = false;
+    r.rot = 0;
+    r.head = 0;
+    r.tail = 0;
     const uint8_t* const a_codes = (PAIR && seg) ? p.a2_codes : p.a_codes;
     const uint8_t* const a_scales = (PAIR && seg) ? p.a2_scales : p.a_scales;
     const uint8_t* const b_codes = (PAIR && seg) ? p.b2_codes : p.b_codes;
@@ -295,7 +307,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       r.nblocks = poison ? 1 : K / kKB;
       r.empty = poison;
     } else if (MODE == kGrouped2d3d) {
-      const uint32_t* first = reinterpret_cast<const uint32_t*>(smem + kRing32 + 4608);
+      const uint32_t* first = reinterpret_cast<const uint32_t*>(smem + kRing32 + kPatchUsed);
       uint32_t g = 0, hi_g = G + 1;  // first[g] <= t < first[g + 1]
       while (hi_g - g > 1) {
         const uint32_t mid = (g + hi_g) >> 1;
@@ -310,6 +322,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       r.a = a_codes + row0 * K;
       r.b = b_codes + ((int64_t)gb * p.N + (int64_t)tn * kT32) * K;
       r.sa = a_scales + (row0 >> 7) * ks_n * 256;
+      r.rot = (uint32_t)(row0 >> 5) & 3;
       r.sb = b_scales + ((int64_t)gb * ((p.N + 127) >> 7) + tn * 2) * ks_n * 256;
       r.d = p.d + row0 * p.ldd + (int64_t)tn * kT32;
       r.rows_a = hi - row0;
@@ -339,7 +352,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       const uint32_t tiles_m = (uint32_t)((p.M + kT32 - 1) / kT32), per_g = tiles_m * tiles_n;
       uint32_t g = t / per_g, in_g = t - g * per_g;
       if (dealt) {  // t counts this workgroup's tiles: the i-th tile it was dealt
-        const uint16_t* g_sorted = reinterpret_cast<const uint16_t*>(smem + kRing32 + 4608) + kMaxDealt;
+        const uint16_t* g_sorted = reinterpret_cast<const uint16_t*>(smem + kRing32 + kPatchUsed) + kMaxDealt;
         const uint32_t q = wgs_per_xcd * t + snake(t, idx, wgs_per_xcd);  // place in the XCD's tile list
         const uint32_t j = q / per_g;
         in_g = q - j * per_g;
@@ -348,15 +361,21 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       tile_coords(in_g, tiles_m, tiles_n, tm, tn);
       tn += tn0;
       const int64_t lo = poison ? 0 : (g ? p.offs[g - 1] : 0), hi = poison ? 0 : p.offs[g];
-      r.a = a_codes + (int64_t)tm * kT32 * K + lo;
-      r.b = b_codes + (int64_t)tn * kT32 * K + lo;
-      r.sa = a_scales + ((int64_t)(tm * 2) * ks_n + (lo >> 6)) * 256;
-      r.sb = b_scales + ((int64_t)(tn * 2) * ks_n + (lo >> 6)) * 256;
+      // the K blocks keep to multiples of 128 (whole cache lines per operand row: a copy that
+      // straddles two lines costs the texture path twice); a range that starts or ends inside
+      // a block has the 32-deep blocks outside it masked (head, tail)
+      const int64_t lo128 = lo & ~(int64_t)127;
+      r.a = a_codes + (int64_t)tm * kT32 * K + lo128;
+      r.b = b_codes + (int64_t)tn * kT32 * K + lo128;
+      r.sa = a_scales + ((int64_t)(tm * 2) * ks_n + (lo128 >> 6)) * 256;
+      r.sb = b_scales + ((int64_t)(tn * 2) * ks_n + (lo128 >> 6)) * 256;
       r.d = p.d + ((int64_t)g * p.M + (int64_t)tm * kT32) * p.ldd + (int64_t)tn * kT32;
       r.rows_a = p.M - (int64_t)tm * kT32;
       r.rows_b = p.N - (int64_t)tn * kT32;
-      r.koff = (uint32_t)lo;
-      r.nblocks = (uint32_t)((hi - lo) >> 7);
+      r.koff = (uint32_t)lo128;
+      r.nblocks = hi > lo ? (uint32_t)(((hi + 127) >> 7) - (lo >> 7)) : 0;
+      r.head = (uint32_t)(lo >> 5) & 3;
+      r.tail = (uint32_t)(hi >> 5) & 3;
       if (r.nblocks == 0) {
         r.nblocks = 1;
         r.empty = true;
@@ -367,11 +386,11 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
 
   // Grouped modes: the map needs loads of the group ends and a search, far too slow for the
   // in-order instruction stream of the MFMA waves.  Every thread works out one of this
-  // workgroup's tiles up front and leaves a 64-byte record in the spare 2.5 KB behind the
-  // output patches of waves 1-3 (40 records each; the host splits launches so that a
+  // workgroup's tiles up front and leaves a 64-byte record in the spare 2 KB behind the
+  // output patches of waves 1-3 (32 records each; the host splits launches so that a
   // workgroup never has more than kMaxRecords tiles).
   auto record_offset = [&](uint32_t i) -> uint32_t {
-    return kRing32 + (1 + i / 40) * 7168 + 4608 + (i % 40) * 64;
+    return kRing32 + (1 + i / kRecordsPerPatch) * kPatch32 + kPatchUsed + (i % kRecordsPerPatch) * 64;
   };
   if constexpr (MODE != kDense) {
     for (uint32_t i = tid; i < n_my; i += 256) {
@@ -389,6 +408,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       w[2] = (int32_t)t.nblocks;
       w[3] = (int32_t)t.koff;
       w[4] = t.empty ? 1 : 0;
+      w[5] = (int32_t)(t.rot | (t.tail << 8) | (t.head << 16));
     }
     __syncthreads();
   }
@@ -421,6 +441,10 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       t.nblocks = (uint32_t)__builtin_amdgcn_readfirstlane(r3.x);
       t.koff = (uint32_t)__builtin_amdgcn_readfirstlane(r3.y);
       t.empty = __builtin_amdgcn_readfirstlane(r3.z) != 0;
+      const uint32_t rt = (uint32_t)__builtin_amdgcn_readfirstlane(r3.w);
+      t.rot = rt & 3;
+      t.tail = (rt >> 8) & 3;
+      t.head = (rt >> 16) & 3;
       t.poison = poison;
       return t;
     }
@@ -441,17 +465,47 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   const uint32_t fa0 = (wm * 128 + li) * kKB + ((lj ^ sw) << 4);
   const uint32_t fb_delta = kOperand32 + (wn - wm) * 128 * kKB;
   const uint32_t lane4 = lane * 4;
-  const uint32_t v_scale = (uint32_t)(lane >> 5) * ks_n * 256 + (lane & 31) * 16;  // scale copy
+  // scale copy: lanes 0-31 fetch one 128-row group's 512 bytes of a block, lanes 32-63 the next
+  // group's; wave 1 (kGrouped2d3d: a third group of A) has its upper lanes read nothing
+  const uint32_t v_scale = (MODE == kGrouped2d3d && wave == 1)
+                               ? (lane < 32 ? (uint32_t)lane * 16 : 0x80000000u)
+                               : (uint32_t)(lane >> 5) * ks_n * 256 + (lane & 31) * 16;
+  // scale groups of a ring block: A0, A1, B0, B1, A2 (512 bytes each, then 512 unused)
   const uint32_t fsa_s = kCodes32 + wm * 512, fsb_s = kCodes32 + 1024 + wn * 512;
+  const uint32_t fsa_hi_s = kCodes32 + (wm == 0 ? 512 : 2048);
 
   // ---- loader stream: fills ring block `ld_slot` with K block `ld_kb` of tile `ld_tile`
   uint32_t ld_tile = 0, ld_kb = 0, ld_nb = 1;
   int ld_slot = 0;
   __amdgpu_buffer_rsrc_t ra, rb, rs;  // codes of A, codes of B, scales this wave copies
+  // kGrouped2d3d: a group may start at any multiple of 32 rows, the scales come in 128-row groups
+  // of the whole matrix: a tile that starts `rot` 32-row blocks into a group fetches three groups
+  // and turns the bytes of every scale dword by `rot` (rotate_scales).  The rotation belongs to
+  // the tile whose block sits in a ring slot.
+  uint32_t ld_rot = 0, slot_rot0 = 0, slot_rot1 = 0;
+  // kGrouped2d2d: a K range may start and end at any multiple of 32.  Its first and last
+  // 128-deep blocks send the chunks outside the range out of range, so that zeros land in the
+  // ring instead of the neighbouring groups' codes and scales.
+  uint32_t ld_head = 0, ld_tail = 0;
+  uint32_t cur_v_even = v_even, cur_v_odd = v_even ^ 64, cur_v_scale = v_scale;
+  auto set_block_offsets = [&]() {
+    if constexpr (MODE == kGrouped2d2d) {
+      // 32-deep blocks [first, lim) of this 128-deep block are fetched
+      const uint32_t first = ld_kb == 0 ? ld_head : 0;
+      const uint32_t lim = (ld_tail != 0 && ld_kb + 1 == ld_nb) ? ld_tail : 4;
+      auto inside = [&](uint32_t blk) { return blk >= first && blk < lim; };
+      cur_v_even = inside(c_even >> 1) ? v_even : 0x80000000u;
+      cur_v_odd = inside((c_even ^ 4) >> 1) ? (v_even ^ 64) : 0x80000000u;
+      cur_v_scale = inside((uint32_t)(lane & 31) >> 3) ? v_scale : 0x80000000u;
+    }
+  };
   auto loader_open_tile = [&]() {
     if (ld_tile < n_my) {
       const Tile32 t = get_tile(ld_tile);
       ld_nb = t.nblocks;
+      ld_rot = t.rot;
+      ld_head = t.head;
+      ld_tail = t.tail;
       // (kGrouped2d2d: the range stops at the end of the operand rows, not of the K range;
       //  the K range is exact because nblocks is.)  A tile without a K range reads nothing:
       // its one block arrives as zeros, scales included.
@@ -461,17 +515,26 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       // wave 0 copies the scales of A's two 128-row groups, wave 2 those of B's (one copy per
       // block each: lanes 0-31 fetch group 0, lanes 32-63 group 1); a group beyond the operand
       // is cut off by the range and arrives as zeros
-      const int64_t rows = wave < 2 ? t.rows_a : t.rows_b;
+      // (kGrouped2d3d: rows counted from the start of the first scale group; wave 1 copies a
+      // third group of A when the tile's rows reach into it)
+      const int64_t rows = wave < 2 ? (t.rows_a > 0 ? t.rows_a + 32 * (int64_t)t.rot : 0) : t.rows_b;
       const uint8_t* sbase = wave < 2 ? t.sa : t.sb;
-      rs = make_rsrc(sbase, none ? 0
-                                 : rows > 128 ? (int64_t)ks_n * 256 + (int64_t)ld_nb * 512
-                                              : (rows > 0 ? (int64_t)ld_nb * 512 : 0));
+      if (MODE == kGrouped2d3d && wave == 1)
+        rs = make_rsrc(sbase + (int64_t)ks_n * 512, (none || rows <= 256) ? 0 : (int64_t)ld_nb * 512);
+      else
+        rs = make_rsrc(sbase, none ? 0
+                                   : rows > 128 ? (int64_t)ks_n * 256 + (int64_t)ld_nb * 512
+                                                : (rows > 0 ? (int64_t)ld_nb * 512 : 0));
     } else {  // past the last tile: every lane reads out of range (zeros, no traffic)
       ld_nb = 1;
+      ld_rot = 0;
+      ld_head = 0;
+      ld_tail = 0;
       ra = make_rsrc(p.a_codes, 0);
       rb = ra;
       rs = ra;
     }
+    set_block_offsets();
   };
   // The 17 copies of a block are issued one at a time, between MFMAs (see block_steps):
   // piece 0..15 = unit pairs (A unit, B unit alternating), 16 = scales, then advance.
@@ -481,7 +544,8 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     if constexpr (i < 16) {
       constexpr int q = i >> 1;
       const int unit = wave * 8 + q;
-      const uint32_t v = (q & 1) ? (v_even ^ 64) : v_even;
+      const uint32_t v = MODE == kGrouped2d2d ? ((q & 1) ? cur_v_odd : cur_v_even)
+                                              : ((q & 1) ? (v_even ^ 64) : v_even);
       const uint32_t so = (uint32_t)(unit * 8) * K + ld_kb * kKB;
       if constexpr ((i & 1) == 0)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void_t*)(uintptr_t)(sbase + unit * 1024), 16, v, so, 0, 0);
@@ -493,15 +557,25 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       // two groups land behind one another, which is the order the fragment reads expect
       if ((wave & 1) == 0)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(
-            rs, (lds_void_t*)(uintptr_t)(sbase + kCodes32 + wave * 512), 16, v_scale,
-            ld_kb * 512, 0, 0);
+            rs, (lds_void_t*)(uintptr_t)(sbase + kCodes32 + wave * 512), 16,
+            MODE == kGrouped2d2d ? cur_v_scale : v_scale, ld_kb * 512, 0, 0);
+      if constexpr (MODE == kGrouped2d3d) {
+        if (wave == 1)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(
+              rs, (lds_void_t*)(uintptr_t)(sbase + kCodes32 + 2048), 16, v_scale, ld_kb * 512, 0, 0);
+      }
     }
   };
   auto issue_advance = [&]() {
+    if constexpr (MODE == kGrouped2d3d) {
+      if (ld_slot) slot_rot1 = ld_rot; else slot_rot0 = ld_rot;
+    }
     if (++ld_kb == ld_nb) {
       ld_kb = 0;
       ++ld_tile;
       loader_open_tile();
+    } else {
+      set_block_offsets();
     }
     ld_slot ^= 1;
   };
@@ -539,6 +613,10 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     } else if constexpr (i == 16) {
       const uint32_t psa = sbase + fsa_s + h * 256 + lane4;
       asm volatile("ds_read_b32 %0, %1" : "=v"(f.sa) : "v"(psa));
+      if constexpr (MODE == kGrouped2d3d) {
+        const uint32_t psa_hi = sbase + fsa_hi_s + h * 256 + lane4;
+        asm volatile("ds_read_b32 %0, %1" : "=v"(f.sa_hi) : "v"(psa_hi));
+      }
     } else {
       const uint32_t psb = sbase + fsb_s + h * 256 + lane4;
       asm volatile("ds_read_b32 %0, %1" : "=v"(f.sb) : "v"(psb));
@@ -554,6 +632,16 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
 #pragma unroll
     for (int n = 0; n < 4; ++n) asm volatile("" : "+v"(f.b[n]));
     asm volatile("" : "+v"(f.sa), "+v"(f.sb));
+    if constexpr (MODE == kGrouped2d3d) asm volatile("" : "+v"(f.sa_hi));
+  };
+  // kGrouped2d3d, once per fragment set, after its reads have landed: byte m of the A scale dword
+  // becomes the scale of the tile's m-th 32-row block, which is byte (rot + m) of the eight bytes
+  // that two neighbouring 128-row groups hold for this lane
+  auto rotate_scales = [&](Frags32& f, int slot) {
+    if constexpr (MODE == kGrouped2d3d) {
+      const uint32_t rot = slot ? slot_rot1 : slot_rot0;
+      f.sa = __builtin_amdgcn_alignbyte(f.sa_hi, f.sa, rot);
+    }
   };
 
   // ---- compute stream
@@ -641,6 +729,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
 
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     pin_frags(f1);
+    rotate_scales(f1, c_slot);
     uint64_t t0 = 0, t1 = 0;
     if constexpr (PROF) {
       t0 = __builtin_readcyclecounter();
@@ -683,6 +772,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     // flight would lose the data)
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     pin_frags(f0);
+    rotate_scales(f0, c_slot);
     issue_advance();
   };
 
@@ -695,7 +785,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   // offsets per piece.  Requires N % 8 == 0 and ldd % 8 == 0 (checked on the host).
   // (LDS accesses as assembly, for the reason given at read_piece.)
   constexpr int kPatchPitch = 144;  // bytes per staged row: 128 + 16, keeps b128 accesses spread
-  const uint32_t patch = lds_base + kRing32 + wave * 7168;
+  const uint32_t patch = lds_base + kRing32 + wave * kPatch32;
   const uint32_t patch_w = patch + li * kPatchPitch + lj * 16;                 // + (n&1)*64 + h*32
   const uint32_t patch_r = patch + (lane >> 3) * kPatchPitch + (lane & 7) * 16;  // + pass*8 rows
   const uint32_t nan_mask = (MODE != kDense && poison) ? 0x7FC07FC0u : 0u;
@@ -793,6 +883,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   read_frags(f0, 0, std::integral_constant<int, 0>{});
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   pin_frags(f0);
+  rotate_scales(f0, 0);
   if constexpr (PROF) prof_last = __builtin_readcyclecounter();
 
   // ---- tiles; at the top of every tile f0 holds the fragments of its first half block (the
@@ -865,7 +956,7 @@ static int64_t persistent_grid() {
 template <int MODE, bool PROF, bool PAIR = false>
 static int launch32(const Gemm32Args& p, int64_t nb, hipStream_t st) {
   auto kern = gemm_nt32_kernel<MODE, PROF, PAIR>;
-  constexpr int lds = kRing32 + 4 * 7168;  // ring + one output patch per wave = all 160 KB
+  constexpr int lds = kRing32 + 4 * kPatch32;  // ring + one output patch per wave = all 160 KB
   static std::atomic<bool> configured[kMaxDevices];
   if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds, configured)) return MX_ERR_LAUNCH;
   int64_t grid = persistent_grid();

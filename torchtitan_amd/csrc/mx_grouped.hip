@@ -153,12 +153,12 @@ extern "C" int mx_grouped_gemm_2d3d_pair(const uint8_t* a_codes, const uint8_t* 
   if (!a_codes || !a_scales || !b_codes || !b_scales || !a2_codes || !a2_scales || !b2_codes ||
       !b2_scales || !offs || !d)
     return MX_ERR_INVALID_ARG;
-  if (K == 0 || K % 128 || N % 8 || ldd % 8 || T % 128) return MX_ERR_ALIGNMENT;
+  if (K == 0 || K % 128 || N % 8 || ldd % 8 || T % 32) return MX_ERR_ALIGNMENT;
   if (((uintptr_t)a_codes & 15) || ((uintptr_t)b_codes & 15) || ((uintptr_t)a2_codes & 15) ||
       ((uintptr_t)b2_codes & 15) || ((uintptr_t)a_scales & 3) || ((uintptr_t)b_scales & 3) ||
       ((uintptr_t)a2_scales & 3) || ((uintptr_t)b2_scales & 3) || ((uintptr_t)d & 15))
     return MX_ERR_ALIGNMENT;
-  if (256 * K > 0x7FFFFFFFll || G > 638 || ldd * 512 > 0x7FFFFFFFll) return MX_ERR_UNSUPPORTED;
+  if (256 * K > 0x7FFFFFFFll || G > 510 || ldd * 512 > 0x7FFFFFFFll) return MX_ERR_UNSUPPORTED;
   return launch_grouped32_2d3d_pair(a_codes, a_scales, b_codes, b_scales, a2_codes, a2_scales,
                                     b2_codes, b2_scales, offs, d, T, N, K, G, ldd,
                                     (hipStream_t)stream);
@@ -179,11 +179,11 @@ extern "C" int mx_grouped_gemm_2d3d(const uint8_t* a_codes, const uint8_t* a_sca
   if (256 * K > 0x7FFFFFFFll) return MX_ERR_UNSUPPORTED;
   hipStream_t st = (hipStream_t)stream;
   if (a_scale_order == MX_SCALES_MFMA) {
-    // group ends at multiples of 128 (checked on the device): the persistent 32x32x64 kernel
+    // group ends at multiples of 32 (checked on the device): the persistent 32x32x64 kernel
     if (K % 128 || N % 8 || ldd % 8 || ((uintptr_t)d & 15) || ((uintptr_t)a_scales & 3) ||
-        T % 128)
+        T % 32)
       return MX_ERR_ALIGNMENT;
-    if (G > 638 || ldd * 512 > 0x7FFFFFFFll) return MX_ERR_UNSUPPORTED;
+    if (G > 510 || ldd * 512 > 0x7FFFFFFFll) return MX_ERR_UNSUPPORTED;
     return launch_grouped32_2d3d(a_codes, a_scales, b_codes, b_scales, offs, d, T, N, K, G, ldd,
                                  st);
   }

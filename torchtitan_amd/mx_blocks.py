@@ -342,11 +342,11 @@ class _MXGroupedFeedForward(torch.autograd.Function):
         G, H, _ = w1.shape
         xb = _bf16(x)
         pad = cfg.pad_token_groups_for_grouped_mm
-        fast = D % 128 == 0 and H % 128 == 0 and G <= 638  # 128-row groups: persistent kernel
+        fast = D % 128 == 0 and H % 128 == 0 and G <= ops.FAST_MAX_GROUPS  # persistent kernel
         order = MX_SCALES_MFMA if fast else MX_SCALES_ROWMAJOR
         plan = perm = back = None
         if pad or fast:
-            plan = _pad_plan(offs, T, 128 if fast else ops.BLOCK)
+            plan = _pad_plan(offs, T, ops.BLOCK, ops.FAST_LENGTH_MULTIPLE if fast else 1)
             perm, offs_p, back = plan
         else:
             offs_p = offs
@@ -465,11 +465,11 @@ class _MXRoutedExperts(torch.autograd.Function):
         G, H, _ = w1.shape
         xb = _bf16(x).contiguous()
         scores = top_scores.float().contiguous()
-        fast = D % 128 == 0 and H % 128 == 0 and G <= 638
+        fast = D % 128 == 0 and H % 128 == 0 and G <= ops.FAST_MAX_GROUPS
         order = MX_SCALES_MFMA if fast else MX_SCALES_ROWMAJOR
         # aligned group layout and the maps between padded rows, tokens and (token, j) pairs
         offs_p, src_row, row_score, pos = ops.moe_route_plan(counts, tok_sorted, scores.view(-1), k,
-                                                             128 if fast else ops.BLOCK)
+                                                             ops.BLOCK, ops.FAST_LENGTH_MULTIPLE if fast else 1)
         pos = pos.view(T, k)
         need_dx = ctx.needs_input_grad[0]
         need_ds = ctx.needs_input_grad[1]

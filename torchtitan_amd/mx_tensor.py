@@ -288,16 +288,18 @@ def mx_linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, 
 
 
 # ----------------------------------------------------------------------------- grouped GEMM
-def _pad_plan(offs: torch.Tensor, T: int, align: int = 32):
+def _pad_plan(offs: torch.Tensor, T: int, align: int = 32, length_multiple: int = 1):
     """Device-side plan that moves rows of variable-size groups into `align`-aligned groups.
 
     Returns (gather indices into [x; 0-row] for the padded layout, padded inclusive offsets,
     for every original row its row in the padded layout or the index of an appended zero row).
-    No host synchronisation: the padded length is the static bound round_up(T + align G, align).
+    No host synchronisation: the padded length is the static bound round_up(T + align G, align),
+    rounded up further to `length_multiple` (a multiple of align) when one is given.
     """
     G = offs.numel()
     sizes = torch.diff(offs, prepend=offs.new_zeros(1))
-    max_len = -(-(T + align * G) // align) * align
+    step = max(align, length_multiple)
+    max_len = -(-(T + align * G) // step) * step
     perm, _, m_offsets = ops.group_offsets_pad(sizes, G, 1, max_len, align)
     back = torch.full((T + 1,), max_len, dtype=torch.int64, device=offs.device)
     back[perm] = torch.arange(max_len, device=offs.device)  # perm == -1 writes the spare slot T
@@ -341,15 +343,13 @@ class _MXGroupedMM(torch.autograd.Function):
         w = weight if weight.dtype == torch.bfloat16 else weight.to(torch.bfloat16)
         w = w.contiguous()
         plan = None
-        # Padding to 128-row groups (instead of the 32 the format needs) lets all three GEMMs
-        # run on the persistent kernel, which wants whole 128-row scale groups per expert.
-        # (also when the caller's groups are already 32-aligned: the move costs nothing extra
-        # inside the gathered cast and the persistent kernel is about twice as fast)
-        fast = K % 128 == 0 and N % 128 == 0 and G <= 638
+        # Groups are padded to the 32 rows the format needs; the persistent kernel takes them as
+        # they are (scales in MFMA order, the token axis rounded up to whole 128-deep blocks).
+        fast = K % 128 == 0 and N % 128 == 0 and G <= ops.FAST_MAX_GROUPS
         order = MX_SCALES_MFMA if fast else MX_SCALES_ROWMAJOR
         perm = back = None
         if cfg.pad_token_groups_for_grouped_mm or fast:
-            plan = _pad_plan(offs, T, 128 if fast else ops.BLOCK)
+            plan = _pad_plan(offs, T, ops.BLOCK, ops.FAST_LENGTH_MULTIPLE if fast else 1)
             perm, offs_p, back = plan
         else:
             offs_p = offs

@@ -188,11 +188,12 @@ def to_mx_rows_gathered(x: torch.Tensor, row_index: torch.Tensor, mode="floor",
 
 
 def moe_route_plan(counts: torch.Tensor, order: torch.Tensor, scores: torch.Tensor | None, top_k: int,
-                   alignment: int):
+                   alignment: int, length_multiple: int = 1):
     """(padded inclusive group ends int32 [E], token of every padded row int64 [max_len] (-1 =
     padding), score of every padded row float32 [max_len], padded row of every (token, choice)
     pair int64 [pairs]) for tokens-per-expert `counts` and the expert-sorted pair order; the
-    padded length is the static bound round_up(pairs + alignment * E, alignment)."""
+    padded length is the static bound round_up(pairs + alignment * E, alignment), rounded up
+    further to `length_multiple` (a multiple of the alignment) when one is given."""
     if not counts.is_cuda:
         raise _lib.MXLibraryError("moe_route_plan runs on the GPU only")
     dev = counts.device
@@ -205,7 +206,10 @@ def moe_route_plan(counts: torch.Tensor, order: torch.Tensor, scores: torch.Tens
         if scores.dtype != torch.float32 or scores.numel() != R or scores.device != dev:
             raise TypeError("scores must be float32 with one entry per pair")
         scores = scores.contiguous()
-    max_len = -(-(R + alignment * E) // alignment) * alignment
+    step = max(alignment, length_multiple)
+    if step % alignment:
+        raise ValueError("length_multiple must be a multiple of the alignment")
+    max_len = -(-(R + alignment * E) // step) * step
     offs = torch.empty(E, dtype=torch.int32, device=dev)
     src_row = torch.empty(max_len, dtype=torch.int64, device=dev)
     row_score = torch.empty(max_len, dtype=torch.float32, device=dev)
@@ -590,6 +594,10 @@ def to_mx_dim0_dim1_batched(w: torch.Tensor, mode="floor", order: int = MX_SCALE
 
 
 # --------------------------------------------------------------------------- grouped GEMMs
+FAST_MAX_GROUPS = 510   # groups the persistent kernel keeps a table of in LDS
+FAST_LENGTH_MULTIPLE = 128  # its operands' token axis: whole 128-deep K blocks / 128-row scale groups
+
+
 def mx_grouped_gemm_2d3d(a: MXData, b: MXData, offs: torch.Tensor,
                          out: torch.Tensor | None = None) -> torch.Tensor:
     """out[rows of group g] = deq(a[rows of g]) @ deq(b[g])^T; rows past offs[-1] are zero.
@@ -597,7 +605,7 @@ def mx_grouped_gemm_2d3d(a: MXData, b: MXData, offs: torch.Tensor,
     a: codes [T, K]; b: codes [G, N, K] with MFMA-order scales (G per-matrix blocks); offs:
     int32 [G] inclusive cumulative group sizes on the device.  With row-major scales for a the
     groups may end anywhere; with MFMA-order scales for a every group must end at a multiple
-    of 128 rows (checked on the device: a violation fills the output with NaN) and the
+    of 32 rows (checked on the device: a violation fills the output with NaN) and the
     persistent 32x32x64 kernel runs.
     """
     T, K = a.codes.shape
@@ -619,14 +627,14 @@ def mx_grouped_gemm_2d3d(a: MXData, b: MXData, offs: torch.Tensor,
 def mx_grouped_gemm_2d3d_pair(a: MXData, b: MXData, a2: MXData, b2: MXData, offs: torch.Tensor,
                               out: torch.Tensor | None = None) -> torch.Tensor:
     """out[rows of g] = deq(a[rows of g]) @ deq(b[g])^T + deq(a2[rows of g]) @ deq(b2[g])^T, both
-    sets with MFMA-order scales and 128-aligned groups (the persistent kernel); other layouts:
+    sets with MFMA-order scales and 32-aligned groups (the persistent kernel); other layouts:
     two grouped GEMMs and a bf16 add."""
     T, K = a.codes.shape
     G, N, _ = b.codes.shape
     if a2.codes.shape != a.codes.shape or b2.codes.shape != b.codes.shape:
         raise ValueError("both operand sets must have the same shapes")
     fast = all(d.scale_order == MX_SCALES_MFMA for d in (a, b, a2, b2))
-    if not fast or K % 128 or N % 8 or T % 128 or G > 638:
+    if not fast or K % 128 or N % 8 or T % 32 or G > FAST_MAX_GROUPS:
         both = mx_grouped_gemm_2d3d(a, b, offs) + mx_grouped_gemm_2d3d(a2, b2, offs)
         return both if out is None else out.copy_(both)
     if offs.dtype != torch.int32 or offs.numel() != G:
@@ -646,9 +654,9 @@ def mx_grouped_gemm_2d2d(at: MXData, bt: MXData, offs: torch.Tensor,
     """out[g] = deq(at[:, tokens of g]) @ deq(bt[:, tokens of g])^T  ->  [G, N, K] bf16.
 
     at: codes [N, T], bt: codes [K, T] (column-wise casts), scales of both in the same order.
-    Row-major: groups may be any multiple of 32.  MFMA order: every group must end at a
-    multiple of 128 tokens (checked on the device: a violation fills the output with NaN) and
-    the persistent 32x32x64 kernel runs.
+    Groups may be any multiple of 32 tokens (checked on the device: a violation gives NaN).
+    MFMA order: T a multiple of 128 (the token axis may run past the last group) and the
+    persistent 32x32x64 kernel runs.
     """
     N, T = at.codes.shape
     K, Tb = bt.codes.shape
