@@ -431,8 +431,8 @@ def test_feed_forward_fused_with_frozen_parts(device):
 def test_grouped_experts_module(device, pad, align, dim, hidden):
     """torch._grouped_mm on converted 3-D weights, forward and backward, vs per-expert oracle.
 
-    With padding on and both dims multiples of 128 the wrapper pads groups to 128 rows and the
-    persistent kernels run; otherwise the general ones.  The results must not depend on it."""
+    With both dims multiples of 128 the wrapper pads groups to 32 rows (the token axis to 128) and
+    the persistent kernels run; otherwise the general ones.  The results must not depend on it."""
     rng = np.random.default_rng(17 + align + dim)
     E = 4
     counts = np.array([40, 0, 200, 16]) if pad else np.array([64, 0, 96, 32])
