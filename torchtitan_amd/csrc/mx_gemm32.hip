@@ -141,6 +141,15 @@ __device__ __forceinline__ void mfma_asm(v16f& c, const v8i& b, const v8i& a, ui
         : "v"(b), "v"(a), "v"(sb), "v"(sa), "n"(N & 1), "n"(M & 1), "n"(N >> 1), "n"(M >> 1));
 }
 
+// One accumulator register into a VGPR, where the caller says (as assembly: the compiler's own
+// copies out of the accumulator file are all placed at the top of the epilogue).
+template <int E>
+__device__ __forceinline__ float acc_read(const v16f& c) {
+  float x;
+  asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(x) : "a"(c[E]));
+  return x;
+}
+
 struct Frags32 {
   v8i a[4];
   v8i b[4];
@@ -786,10 +795,16 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   // (LDS accesses as assembly, for the reason given at read_piece.)
   constexpr int kPatchPitch = 144;  // bytes per staged row: 128 + 16, keeps b128 accesses spread
   const uint32_t patch = lds_base + kRing32 + wave * kPatch32;
-  const uint32_t patch_w = patch + li * kPatchPitch + lj * 16;                 // + (n&1)*64 + h*32
-  const uint32_t patch_r = patch + (lane >> 3) * kPatchPitch + (lane & 7) * 16;  // + pass*8 rows
   const uint32_t nan_mask = (MODE != kDense && poison) ? 0x7FC07FC0u : 0u;
   auto epilogue = [&](const Tile32& t) {
+    // The epilogue's per-lane addresses are worked out here, from a lane number the compiler
+    // cannot see through, every time: kept across the K loop instead they push its register
+    // file over the edge, and a spilled register's reload waits for every copy and store in
+    // flight (s_waitcnt vmcnt(0)) at exactly the two places where those should keep running.
+    uint32_t lane_e = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    asm volatile("" : "+v"(lane_e));
+    const uint32_t patch_w = patch + (lane_e & 31) * kPatchPitch + (lane_e >> 5) * 16;   // + (n&1)*64 + h*32
+    const uint32_t patch_r = patch + (lane_e >> 3) * kPatchPitch + (lane_e & 7) * 16;  // + pass*8 rows
     const int64_t rows_valid = t.rows_a;
     const uint32_t cols_valid = (uint32_t)(t.rows_b < kT32 ? t.rows_b : kT32);
     if constexpr (MODE == kSplitK) {
@@ -815,8 +830,8 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     const uint32_t ldd_b = (uint32_t)p.ldd * 2;
     const __amdgpu_buffer_rsrc_t rd = make_rsrc(t.d, rows_valid * ldd_b);
     // lane's place in a stored piece: row (lane >> 3) + 8*pass, columns (lane & 7)*8 .. +7
-    const uint32_t colp = wn * 128 + (lane & 7) * 8;
-    const uint32_t vrow = (wm * 128 + (lane >> 3)) * ldd_b + colp * 2;
+    const uint32_t colp = wn * 128 + (lane_e & 7) * 8;
+    const uint32_t vrow = (wm * 128 + (lane_e >> 3)) * ldd_b + colp * 2;
     // Pieces p = 0..7: 32 rows (sub-tile row m = p/2) x 64 columns (sub-tiles n = 2(p%2), +1).
     // A wave's LDS instructions execute in order, so a piece's reads may follow its writes
     // without a wait, and the next piece's writes may follow those reads: the only waits are
@@ -824,9 +839,14 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     auto stage_part = [&](auto p_, auto k_) {  // 32 rows x 16 columns: accumulators -> bf16 -> patch
       constexpr int m = decltype(p_)::value >> 1, np = decltype(p_)::value & 1;
       constexpr int n = 2 * np + (decltype(k_)::value >> 1), h = decltype(k_)::value & 1;
-      const v16f a = acc[m][n];
-      uint32_t x0 = pack_bf16(a[8 * h + 0], a[8 * h + 1]), y0 = pack_bf16(a[8 * h + 2], a[8 * h + 3]);
-      uint32_t x1 = pack_bf16(a[8 * h + 4], a[8 * h + 5]), y1 = pack_bf16(a[8 * h + 6], a[8 * h + 7]);
+      // the eight accumulator registers of this part, read here and now (left to the compiler, the
+      // reads of the whole tile are gathered at the top of the epilogue: 180 registers at once)
+      const v16f& c = acc[m][n];
+      const float a[8] = {acc_read<8 * h + 0>(c), acc_read<8 * h + 1>(c), acc_read<8 * h + 2>(c),
+                          acc_read<8 * h + 3>(c), acc_read<8 * h + 4>(c), acc_read<8 * h + 5>(c),
+                          acc_read<8 * h + 6>(c), acc_read<8 * h + 7>(c)};
+      uint32_t x0 = pack_bf16(a[0], a[1]), y0 = pack_bf16(a[2], a[3]);
+      uint32_t x1 = pack_bf16(a[4], a[5]), y1 = pack_bf16(a[6], a[7]);
       if constexpr (MODE != kDense) {  // a broken group contract must not pass unnoticed: NaN
         x0 |= nan_mask;
         y0 |= nan_mask;
@@ -837,6 +857,9 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       const u32x2 sy = __builtin_amdgcn_permlane32_swap(y0, y1, false, false);
       const v4i w = {(int)sx.x, (int)sy.x, (int)sx.y, (int)sy.y};
       lds_write_b128_hidden<(n & 1) * 64 + h * 32>(patch_w, w);
+      // keep a part's reads, conversion and write together: left free, the scheduler reads many
+      // accumulator blocks ahead and the epilogue spreads over registers the K loop's constants sit in
+      __builtin_amdgcn_sched_barrier(0);
     };
     v4i r[2][4];
     static_for<0, 4>([&](auto k_) { stage_part(std::integral_constant<int, 0>{}, k_); });
