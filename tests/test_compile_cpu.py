@@ -1,4 +1,5 @@
-"""CPU: a converted linear traces under ``torch.compile(fullgraph=True)`` as opaque operators.
+"""CPU: converted linears and grouped experts trace under ``torch.compile(fullgraph=True)`` as
+opaque operators.
 
 The reference compiles each transformer block as a whole graph
 (torchtitan/models/llama3/parallelize.py:271-284); here the tracing half of that is checked
@@ -10,9 +11,9 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from torchtitan_amd import compiled  # registers torchtitan_amd::mx_linear_fwd / _bwd
+from torchtitan_amd import compiled  # registers the torchtitan_amd:: traced operators
 from torchtitan_amd import ops
-from torchtitan_amd.modules import FeedForward, Linear
+from torchtitan_amd.modules import FeedForward, GroupedExperts, Linear
 from torchtitan_amd.mx_tensor import MXFP8Config, MXFP8TrainingWeight, wrap_parameter
 
 
@@ -89,7 +90,66 @@ def test_fake_kernels_reject_unaligned_shapes_and_give_backward_shapes():
             torch.ops.torchtitan_amd.mx_linear_fwd(torch.empty(40, 64), w, 1)
 
 
+_GFWD = (torch.ops.torchtitan_amd.mx_grouped_mm_fwd, torch.ops.torchtitan_amd.mx_grouped_mm_fwd.default)
+_PLAN = (torch.ops.torchtitan_amd.group_offsets_pad, torch.ops.torchtitan_amd.group_offsets_pad.default)
+
+
+def _experts(pad, dim=128, hidden=256, n=4):
+    ex = GroupedExperts(dim=dim, hidden_dim=hidden, num_experts=n, use_grouped_mm=True)
+    for name in ("w1", "w2", "w3"):
+        setattr(ex, name, wrap_parameter(getattr(ex, name), MXFP8Config("rceil", pad_token_groups_for_grouped_mm=pad)))
+    return ex
+
+
+@pytest.mark.parametrize("pad", [True, False])
+def test_grouped_experts_trace_as_three_grouped_operators(pad):
+    """The tracer does not offer ``torch._grouped_mm`` to a tensor subclass (underscore names are
+    not among the overridable functions), so the expert block calls the package's
+    ``grouped_mm``: three MXFP8 operators in one graph and no bf16 ``_grouped_mm`` left.
+    Experts that pad their groups themselves need no padding wrapper around them; the others
+    keep the wrapper, whose index fill is a graph node too."""
+    gm = _trace(_experts(pad), torch.randn(96, 128), torch.tensor([10, 40, 30, 16]))
+    t = _targets(gm)
+    assert sum(x in _GFWD for x in t) == 3
+    assert torch._grouped_mm not in t
+    assert sum(x in _PLAN for x in t) == (0 if pad else 1)
+    node = next(n for n in gm.graph.nodes if n.target in _GFWD)
+    assert node.args[3] == ops.SCALE_MODES["rceil"] and node.args[4] is pad
+
+
+@pytest.mark.parametrize("T,K,N,G,pad", [(96, 128, 256, 4, True), (96, 128, 256, 4, False),
+                                         (100, 96, 160, 3, True), (96, 96, 160, 3, False)])
+def test_grouped_fake_kernels_give_the_static_shapes(T, K, N, G, pad):
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    fast = K % 128 == 0 and N % 128 == 0
+    padded = pad or fast
+    step = 128 if fast else 32
+    Tp = -(-(T + 32 * G) // step) * step if padded else T
+    with FakeTensorMode():
+        x, w, offs = torch.empty(T, K), torch.empty(G, N, K), torch.empty(G, dtype=torch.int32)
+        y, offs_p, perm, back, xc, xs, wc, ws = torch.ops.torchtitan_amd.mx_grouped_mm_fwd(x, w, offs, 1, pad)
+        assert y.shape == (T, N) and y.dtype == torch.bfloat16 and offs_p.shape == (G,)
+        assert perm.shape == ((Tp,) if padded else (0,)) and back.shape == ((T,) if padded else (0,))
+        assert xc.shape == (K, Tp) and wc.shape == (G, K, N)
+        assert xs.shape == ((ops.mfma_scale_bytes(K, Tp // 32),) if fast else (K, Tp // 32))
+        assert ws.numel() == G * ops.mfma_scale_bytes(K, N // 32)
+        dx, dw = torch.ops.torchtitan_amd.mx_grouped_mm_bwd(torch.empty(T, N), offs_p, perm, back, xc, xs, wc, ws,
+                                                            1, True, True)
+        assert dx.shape == (T, K) and dw.shape == (G, N, K)
+        dx, dw = torch.ops.torchtitan_amd.mx_grouped_mm_bwd(torch.empty(T, N), offs_p, perm, back, xc, xs, wc, ws,
+                                                            1, True, False)
+        assert dx.shape == (T, K) and dw.numel() == 0
+        with pytest.raises(Exception):
+            torch.ops.torchtitan_amd.mx_grouped_mm_fwd(torch.empty(T, 40), torch.empty(G, N, 40), offs, 1, pad)
+
+
 def test_operators_have_no_cpu_kernel():
     """No fallback: off the GPU the operators fail instead of computing something else."""
     with pytest.raises(Exception):
         torch.ops.torchtitan_amd.mx_linear_fwd(torch.randn(32, 64), torch.randn(32, 64), 1)
+    with pytest.raises(Exception):
+        torch.ops.torchtitan_amd.mx_grouped_mm_fwd(torch.randn(32, 64), torch.randn(2, 32, 64),
+                                                   torch.tensor([16, 32], dtype=torch.int32), 1, True)
+    with pytest.raises(Exception):
+        torch.ops.torchtitan_amd.group_offsets_pad(torch.tensor([3, 5]), 2, 1, 64, 32)

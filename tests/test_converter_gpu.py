@@ -740,3 +740,82 @@ def test_decoder_block_under_torch_compile_equals_eager(device):
     for g, a, w in zip(got, again, want):
         assert torch.equal(g, w) and torch.equal(a, w)
     torch._dynamo.reset()
+
+
+@pytest.mark.parametrize("pad,align", [(True, 8), (False, 32)])
+@pytest.mark.parametrize("dim,hidden", [(128, 256), (96, 160)])
+def test_grouped_experts_under_torch_compile_equal_eager(device, pad, align, dim, hidden):
+    """The expert block compiled as one graph (the reference compiles MoE blocks as well): each
+    converted grouped GEMM is one opaque operator that holds the padding plan, the casts and the
+    grouped kernels of the eager path, so output and all gradients equal the eager run bit for
+    bit (gate fusion off on the eager side: the same unfused sequence).  With experts that pad
+    their own groups the compiled block leaves the outer padding wrapper out; rows of real
+    tokens do not depend on where padding rows sit."""
+    import torch._dynamo
+
+    torch.manual_seed(23)
+    moe_mod.set_token_group_alignment_size_m(align)
+    try:
+        ex = GroupedExperts(dim=dim, hidden_dim=hidden, num_experts=6, use_grouped_mm=True).to(device).to(torch.bfloat16)
+        ex.init_weights(init_std=0.05)
+        holder = nn.Module()
+        holder.experts = ex
+        _convert(holder, ["experts"], pad=pad, fuse=False)
+        counts = torch.tensor([5, 0, 33, 64, 1, 41], device=device)
+        x = torch.randn(int(counts.sum()), dim, device=device, dtype=torch.bfloat16)
+        dy = torch.randn_like(x) * 1e-2
+
+        def run(fn):
+            for p in ex.parameters():
+                p.grad = None
+            xi = x.clone().requires_grad_(True)
+            y = fn(xi, counts)
+            y.backward(dy)
+            return [y.detach().clone(), xi.grad.clone()] + [p.grad.clone() for p in ex.parameters()]
+
+        want = run(ex)
+        torch._dynamo.reset()
+        compiled_ex = torch.compile(ex, backend="aot_eager", fullgraph=True)
+        got = run(compiled_ex)
+        again = run(compiled_ex)
+        for g, a, w in zip(got, again, want):
+            assert torch.equal(g, w) and torch.equal(a, w)
+    finally:
+        moe_mod.set_token_group_alignment_size_m(8)
+        torch._dynamo.reset()
+
+
+def test_moe_layer_under_torch_compile_equals_eager(device):
+    """Router, reordering, converted experts, shared experts and the combine as one compiled
+    graph without a break; bit-identical to the eager layer built from the same unfused ops."""
+    import torch._dynamo
+
+    torch.manual_seed(29)
+    cfg = MoE.Config(num_experts=8, num_shared_experts=1, top_k=2, hidden_dim=128,
+                     score_before_experts=True, score_func="softmax", route_norm=True)
+    moe = MoE(cfg, dim=256).to(device).to(torch.bfloat16)
+    moe.init_weights(init_std=0.05, buffer_device=device)
+    holder = nn.Module()
+    holder.moe = moe
+    _convert(holder, ["experts"], fuse=False)
+    x = torch.randn(2, 96, 256, device=device, dtype=torch.bfloat16)
+    dy = torch.randn_like(x)
+
+    def run(fn):
+        for p in moe.parameters():
+            p.grad = None
+        xi = x.clone().requires_grad_(True)
+        y = fn(xi)
+        y.backward(dy)
+        return [y.detach().clone(), xi.grad.clone()] + [p.grad.clone() for p in moe.parameters()]
+
+    try:
+        want = run(moe)
+        torch._dynamo.reset()
+        compiled_moe = torch.compile(moe, backend="aot_eager", fullgraph=True)
+        got = run(compiled_moe)
+        assert len(got) == len(want)
+        for g, w in zip(got, want):
+            assert torch.equal(g, w)
+    finally:
+        torch._dynamo.reset()

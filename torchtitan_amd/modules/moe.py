@@ -17,7 +17,9 @@ from torch import nn
 
 from dataclasses import dataclass
 
-from ..mx_blocks import grouped_feed_forward_fusable, mx_grouped_feed_forward, mx_routed_experts
+from ..mx_blocks import (grouped_experts_align_themselves, grouped_feed_forward_fusable,
+                         mx_grouped_feed_forward, mx_routed_experts)
+from ..mx_tensor import grouped_mm
 from ..protocols import Module
 from .feed_forward import FeedForward
 from .linear import Linear
@@ -62,6 +64,11 @@ def generate_permute_indices(tokens_per_expert_group: torch.Tensor, experts_per_
                              num_ranks: int, max_len: int, alignment: int, use_cpu: bool = False):
     """(permuted_indices, m_sizes int32, m_offsets int32): expert-grouped, alignment-padded order."""
     if not use_cpu:
+        if torch.compiler.is_compiling():  # the same launch as a graph node
+            from .. import compiled
+
+            return torch.ops.torchtitan_amd.group_offsets_pad(tokens_per_expert_group, experts_per_rank,
+                                                              num_ranks, max_len, alignment)
         # product path: one HIP launch, no host round trip; raises on CPU tensors
         from .. import ops
 
@@ -122,9 +129,11 @@ def _run_experts_grouped_mm(w1, w2, w3, x, num_tokens_per_expert):
     if grouped_feed_forward_fusable(x, w1, w2, w3):  # converted experts: one fused function
         return mx_grouped_feed_forward(x, w1, w2, w3, offsets).type_as(x)
     xb = x.bfloat16()
-    h = F.silu(torch._grouped_mm(xb, w1.bfloat16().transpose(-2, -1), offs=offsets))
-    h = h * torch._grouped_mm(xb, w3.bfloat16().transpose(-2, -1), offs=offsets)
-    return torch._grouped_mm(h, w2.bfloat16().transpose(-2, -1), offs=offsets).type_as(x)
+    # grouped_mm is torch._grouped_mm, spelled so that converted weights keep their MXFP8 path
+    # inside a compiled graph as well
+    h = F.silu(grouped_mm(xb, w1.bfloat16().transpose(-2, -1), offsets))
+    h = h * grouped_mm(xb, w3.bfloat16().transpose(-2, -1), offsets)
+    return grouped_mm(h, w2.bfloat16().transpose(-2, -1), offsets).type_as(x)
 
 
 class GroupedExperts(Module):
@@ -141,9 +150,11 @@ class GroupedExperts(Module):
     def forward(self, x: torch.Tensor, num_tokens_per_expert: torch.Tensor) -> torch.Tensor:
         if self.use_grouped_mm:
             run = indices_padding_wrapper(_run_experts_grouped_mm)
-            if (num_tokens_per_expert.shape[0] == self.w1.shape[0]
-                    and grouped_feed_forward_fusable(x, self.w1, self.w2, self.w3)
-                    and self.w2.mx_config.pad_token_groups_for_grouped_mm):
+            if num_tokens_per_expert.shape[0] == self.w1.shape[0] and (
+                    (grouped_feed_forward_fusable(x, self.w1, self.w2, self.w3)
+                     and self.w2.mx_config.pad_token_groups_for_grouped_mm)
+                    or (torch.compiler.is_compiling()
+                        and grouped_experts_align_themselves(self.w1, self.w2, self.w3))):
                 # tokens already in expert order and the converted block aligns the groups itself
                 run = _run_experts_grouped_mm
         else:

@@ -420,6 +420,13 @@ class _MXGroupedFeedForward(torch.autograd.Function):
         return dx, dw1, dw2, dw3, None, None
 
 
+def grouped_experts_align_themselves(w1: torch.Tensor, w2: torch.Tensor, w3: torch.Tensor) -> bool:
+    """All three expert parameters converted with token-group padding on: their grouped GEMMs
+    take groups of any size, so nothing has to pad the groups around them."""
+    return all(isinstance(w, MXFP8TrainingWeight) and w.dim() == 3
+               and w.mx_config.pad_token_groups_for_grouped_mm for w in (w1, w2, w3))
+
+
 def grouped_feed_forward_fusable(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
                                  w3: torch.Tensor) -> bool:
     """All three expert parameters converted with gate fusion on, a 2-D GPU activation, model

@@ -425,6 +425,22 @@ def mx_grouped_mm(x: torch.Tensor, w_t: torch.Tensor, offs: torch.Tensor, cfg: M
     return _MXGroupedMM.apply(x, weight, offs.to(torch.int32), cfg)
 
 
+def grouped_mm(x: torch.Tensor, w_t: torch.Tensor, offs: torch.Tensor):
+    """``torch._grouped_mm(x, w_t, offs=offs)`` that reaches a converted weight in a traced graph
+    too.  Eagerly the weight's ``__torch_function__`` sees ``torch._grouped_mm``; Dynamo offers it
+    only the functions ``torch.overrides.get_overridable_functions()`` lists, which leaves out
+    underscore names, so a traced ``torch._grouped_mm`` on a converted weight would run in bf16
+    without a word.  Code that may be compiled calls this instead."""
+    if (torch.compiler.is_compiling() and isinstance(w_t, MXFP8TrainingWeight)
+            and not isinstance(x, MXFP8TrainingWeight)):
+        from .compiled import mx_grouped_mm_traced
+
+        cfg = w_t.mx_config
+        with torch._C.DisableTorchFunctionSubclass():
+            return mx_grouped_mm_traced(x, w_t, offs, cfg.scale_mode, cfg.pad_token_groups_for_grouped_mm)
+    return torch._grouped_mm(x, w_t, offs=offs)
+
+
 # ----------------------------------------------------------------------------- the wrapper
 _LINEAR_FUNCS = {F.linear}
 _GROUPED_FUNCS = {torch._grouped_mm}
@@ -475,6 +491,12 @@ class MXFP8TrainingWeight(torch.Tensor):
             a, b = args[0], args[1]
             offs = kwargs.get("offs", args[2] if len(args) > 2 else None)
             if isinstance(b, cls) and not isinstance(a, cls):
+                if torch.compiler.is_compiling():  # as for the linear: one opaque operator
+                    from .compiled import mx_grouped_mm_traced
+
+                    with torch._C.DisableTorchFunctionSubclass():
+                        return mx_grouped_mm_traced(a, b, offs, b.mx_config.scale_mode,
+                                                    b.mx_config.pad_token_groups_for_grouped_mm)
                 return mx_grouped_mm(a, _unwrap(b), offs, b.mx_config)
         cfg = next((a.mx_config for a in _flatten(args) if isinstance(a, cls)), None)
         with torch._C.DisableTorchFunctionSubclass():
