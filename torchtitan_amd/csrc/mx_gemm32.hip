@@ -28,6 +28,12 @@
 // left; results are then meaningless.
 #include "mx_gemm_tile.h"
 
+// 1: the K loop runs on v_mfma_scale_f32_16x16x128_f8f6f4 (one MFMA per 16x16 sub-tile and
+// 128-deep block); 0: on v_mfma_scale_f32_32x32x64_f8f6f4 (two per 32x32 sub-tile and block).
+#ifndef MX_MFMA16
+#define MX_MFMA16 1
+#endif
+
 namespace mx {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
@@ -141,10 +147,27 @@ __device__ __forceinline__ void mfma_asm(v16f& c, const v8i& b, const v8i& a, ui
         : "v"(b), "v"(a), "v"(sb), "v"(sa), "n"(N & 1), "n"(M & 1), "n"(N >> 1), "n"(M >> 1));
 }
 
+// The same for v_mfma_scale_f32_16x16x128_f8f6f4 (MX_MFMA16): NB / MB = scale byte of the first /
+// second operand's dword.
+template <int NB, int MB, bool FIRST>
+__device__ __forceinline__ void mfma16_asm(v4f& c, const v8i& b, const v8i& a, uint32_t sb,
+                                           uint32_t sa) {
+  if constexpr (FIRST)
+    asm volatile(
+        "v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, 0, %3, %4 op_sel:[%5,%6,0] op_sel_hi:[%7,%8,0]"
+        : "=a"(c)
+        : "v"(b), "v"(a), "v"(sb), "v"(sa), "n"(NB & 1), "n"(MB & 1), "n"(NB >> 1), "n"(MB >> 1));
+  else
+    asm volatile(
+        "v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[%5,%6,0] op_sel_hi:[%7,%8,0]"
+        : "+a"(c)
+        : "v"(b), "v"(a), "v"(sb), "v"(sa), "n"(NB & 1), "n"(MB & 1), "n"(NB >> 1), "n"(MB >> 1));
+}
+
 // One accumulator register into a VGPR, where the caller says (as assembly: the compiler's own
 // copies out of the accumulator file are all placed at the top of the epilogue).
-template <int E>
-__device__ __forceinline__ float acc_read(const v16f& c) {
+template <int E, class V>
+__device__ __forceinline__ float acc_read(const V& c) {
   float x;
   asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(x) : "a"(c[E]));
   return x;
@@ -157,6 +180,17 @@ struct Frags32 {
   uint32_t sa_hi;  // kGrouped2d3d: the A scale dword of the next 128-row group (see rotate_scales)
 };
 
+// MX_MFMA16: fragment sets of four 16-row sub-tiles each, whole 128-deep blocks (a[h][t] =
+// sub-tile 4h + t of the wave's 128 rows of A, b[h][t] likewise for B), the scale dwords of the
+// block being computed (one for the even and one for the odd sub-tiles) and those of the next.
+struct Frags16 {
+  v8i a[2][4];
+  v8i b[2][4];
+  uint32_t sa[2], sb[2];
+  uint32_t san[2], sbn[2];
+  uint32_t sa_hi[2];  // kGrouped2d3d: as san, of the next 128-row group (see next_scales)
+};
+
 template <int MODE, bool PROF, bool PAIR = false>
 __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
@@ -164,7 +198,11 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
+#if MX_MFMA16
+  const int li = lane & 15, lj = lane >> 4;
+#else
   const int li = lane & 31, lj = lane >> 5;
+#endif
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void_t*)smem;  // LDS byte address of the ring
   const uint32_t K = (uint32_t)p.K;  // bytes per operand row; a multiple of 128 for this kernel
   const uint32_t ks_n = K / kK32;    // 64-deep steps per 128-row scale group
@@ -462,7 +500,12 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   // ---- per-lane constants
   // global -> LDS: a load unit is 8 rows x 128 B; lane l fetches row l/8 and the logical 16-byte
   // chunk that belongs at physical chunk l%8 of that row: c = (l%8) ^ ((row >> 1) & 7)
+#if MX_MFMA16
+  // (16-row sub-tiles: c = (l%8) ^ ((row & 2) | ((row & 8) >> 1)), see the fragment reads)
+  const uint32_t c_even = (lane & 7) ^ ((lane >> 3) & 2);
+#else
   const uint32_t c_even = (lane & 7) ^ (lane >> 4);  // even units; odd units flip bit 2
+#endif
   const uint32_t v_even = (uint32_t)(lane >> 3) * K + c_even * 16;
   // (odd units: v_even ^ 64 -- K is a multiple of 128, so bit 6 belongs to the chunk alone)
   // LDS -> VGPR: for K half h of a block, lane (li, lj) reads chunks 4h+lj and 4h+2+lj of row li
@@ -470,16 +513,29 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   // address ^ 32 and h flips address bit 6.  Only the A address is kept per lane; B's differs by
   // a wave-uniform amount, as do the scale addresses (group g = A0, A1, B0, B1, K half h at
   // kCodes32 + (g*2 + h) * 256).
+#if MX_MFMA16
+  // MX_MFMA16: lane (li = l & 15, lj = l >> 4) of a 16-row sub-tile reads chunks lj and lj + 4 of
+  // row li (K bytes [16 lj, +16) and [64 + 16 lj, +16)); physical chunk = logical ^ sw with
+  // sw = (row & 2) | ((row & 8) >> 1), which spreads the 16 lanes of every b128 pass (lanes
+  // {0-3, 12-15, 20-23, 24-27} and {4-11, 16-19, 28-31} of a half-wave) over all bank groups;
+  // the second chunk is address ^ 64.  Scales: sub-tile m needs row 16m + li, 32-deep block lj,
+  // i.e. 64-deep step lj >> 1, lane 32 (lj & 1) + 16 (m & 1) + li of the 128-row group, byte
+  // m >> 1: one dword for the even sub-tiles, the one 64 bytes on for the odd ones.
+  const uint32_t sw = (li & 2) | ((li & 8) >> 1);
+  const uint32_t lane4 = (uint32_t)(lj >> 1) * 256 + (uint32_t)((lj & 1) * 32 + li) * 4;
+#else
   const uint32_t sw = (li >> 1) & 7;
+  const uint32_t lane4 = lane * 4;
+#endif
   const uint32_t fa0 = (wm * 128 + li) * kKB + ((lj ^ sw) << 4);
   const uint32_t fb_delta = kOperand32 + (wn - wm) * 128 * kKB;
-  const uint32_t lane4 = lane * 4;
   // scale copy: lanes 0-31 fetch one 128-row group's 512 bytes of a block, lanes 32-63 the next
   // group's; wave 1 (kGrouped2d3d: a third group of A) has its upper lanes read nothing
   const uint32_t v_scale = (MODE == kGrouped2d3d && wave == 1)
                                ? (lane < 32 ? (uint32_t)lane * 16 : 0x80000000u)
                                : (uint32_t)(lane >> 5) * ks_n * 256 + (lane & 31) * 16;
   // scale groups of a ring block: A0, A1, B0, B1, A2 (512 bytes each, then 512 unused)
+  const uint32_t scale_dst = kCodes32 + ((MODE == kGrouped2d3d && wave == 1) ? 2048u : (uint32_t)(wave >> 1) * 1024u);
   const uint32_t fsa_s = kCodes32 + wm * 512, fsb_s = kCodes32 + 1024 + wn * 512;
   const uint32_t fsa_hi_s = kCodes32 + (wm == 0 ? 512 : 2048);
 
@@ -562,17 +618,14 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
         __builtin_amdgcn_raw_ptr_buffer_load_lds(
             rb, (lds_void_t*)(uintptr_t)(sbase + kOperand32 + unit * 1024), 16, v, so, 0, 0);
     } else {
-      // scales (waves 0 and 2 only): a group's two 64-deep steps are 512 contiguous bytes, the
-      // two groups land behind one another, which is the order the fragment reads expect
-      if ((wave & 1) == 0)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(
-            rs, (lds_void_t*)(uintptr_t)(sbase + kCodes32 + wave * 512), 16,
-            MODE == kGrouped2d2d ? cur_v_scale : v_scale, ld_kb * 512, 0, 0);
-      if constexpr (MODE == kGrouped2d3d) {
-        if (wave == 1)
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(
-              rs, (lds_void_t*)(uintptr_t)(sbase + kCodes32 + 2048), 16, v_scale, ld_kb * 512, 0, 0);
-      }
+      // scales: a group's two 64-deep steps are 512 contiguous bytes, the two groups land behind
+      // one another, which is the order the fragment reads expect.  Waves 0 and 2 copy A's and
+      // B's; waves 1 and 3 copy the same bytes to the same place once more (kGrouped2d3d: wave 1
+      // the third group of A instead): every wave then runs the same instructions, where a
+      // branch around the copy costs the two waves that take it more than the copy itself
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rs, (lds_void_t*)(uintptr_t)(sbase + scale_dst), 16,
+          MODE == kGrouped2d2d ? cur_v_scale : v_scale, ld_kb * 512, 0, 0);
     }
   };
   auto issue_advance = [&]() {
@@ -604,6 +657,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(off));
     return v;
   };
+#if !MX_MFMA16
   // piece 0..7: A sub-tile m = piece/2, low/high 16 bytes; 8..15: same for B; 16,17: scales
   auto read_piece = [&](Frags32& f, uint32_t sbase, auto half_, auto i_) {
     constexpr int h = decltype(half_)::value;
@@ -785,6 +839,227 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     issue_advance();
   };
 
+#else
+  // ---- MX_MFMA16: fragment sets, scale dwords
+  // one b128 read of a fragment set: i = 2t + (0: K bytes [16 lj, +16), 1: [64 + 16 lj, +16)) of
+  // sub-tile 4h + t
+  auto read_set_piece = [&](v8i (&set)[4], uint32_t sbase, uint32_t delta, auto h_, auto i_) {
+    constexpr int h = decltype(h_)::value, i = decltype(i_)::value;
+    constexpr int t = i >> 1;
+    constexpr bool hi = i & 1;
+    const uint32_t base = (fa0 ^ (hi ? 64u : 0u)) + delta;
+    const v4i v = lds_b128(sbase + base, std::integral_constant<int, (4 * h + t) * 2048>{});
+    v8i& dst = set[t];
+    if constexpr (hi) {
+      dst[4] = v.x; dst[5] = v.y; dst[6] = v.z; dst[7] = v.w;
+    } else {
+      dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
+    }
+  };
+  // the scale dwords of a block, into the "next" registers: piece 0, 1 = A even / odd
+  // sub-tiles, 2, 3 = B, 4, 5 = A of the next 128-row group (kGrouped2d3d)
+  constexpr int kScalePieces = MODE == kGrouped2d3d ? 6 : 4;
+  auto read_scale_piece = [&](Frags16& f, uint32_t sbase, auto i_) {
+    constexpr int i = decltype(i_)::value;
+    constexpr int e = i & 1;
+    if constexpr (i < 2) {
+      const uint32_t ps = sbase + fsa_s + lane4 + e * 64;
+      asm volatile("ds_read_b32 %0, %1" : "=v"(f.san[e]) : "v"(ps));
+    } else if constexpr (i < 4) {
+      const uint32_t ps = sbase + fsb_s + lane4 + e * 64;
+      asm volatile("ds_read_b32 %0, %1" : "=v"(f.sbn[e]) : "v"(ps));
+    } else {
+      const uint32_t ps = sbase + fsa_hi_s + lane4 + e * 64;
+      asm volatile("ds_read_b32 %0, %1" : "=v"(f.sa_hi[e]) : "v"(ps));
+    }
+  };
+  auto pin_set = [&](v8i (&set)[4]) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) asm volatile("" : "+v"(set[t]));
+  };
+  // The next block's scales become the current ones, once their reads have landed.
+  // kGrouped2d3d: byte k of an A scale dword becomes the scale of the tile's k-th 32-row block,
+  // which is byte (rot + k) of the eight bytes that two neighbouring 128-row groups hold for
+  // this lane
+  auto next_scales = [&](Frags16& f, int slot) {
+    asm volatile("" : "+v"(f.san[0]), "+v"(f.san[1]), "+v"(f.sbn[0]), "+v"(f.sbn[1]));
+    if constexpr (MODE == kGrouped2d3d) {
+      asm volatile("" : "+v"(f.sa_hi[0]), "+v"(f.sa_hi[1]));
+      const uint32_t rot = slot ? slot_rot1 : slot_rot0;
+      f.sa[0] = __builtin_amdgcn_alignbyte(f.sa_hi[0], f.san[0], rot);
+      f.sa[1] = __builtin_amdgcn_alignbyte(f.sa_hi[1], f.san[1], rot);
+    } else {
+      f.sa[0] = f.san[0];
+      f.sa[1] = f.san[1];
+    }
+    f.sb[0] = f.sbn[0];
+    f.sb[1] = f.sbn[1];
+  };
+  // ---- compute stream
+  v4f acc[8][8];
+  int c_slot = 0;  // ring block holding the K block being computed
+  uint64_t prof_vm = 0, prof_bar = 0, prof_body = 0, prof_last = 0, prof_epi = 0;
+  uint64_t prof_e_stage = 0, prof_e_wait = 0, prof_e_store = 0;
+
+// Output stores carry the nontemporal policy bit: written once, never re-read by this kernel,
+// and without it the output lines displace operand panels in L2 and the copies of the next
+// tile's first blocks queue behind the draining stores.
+#ifndef MX_STORE_AUX
+#define MX_STORE_AUX 2
+#endif
+#ifndef MX_RELEASE16
+#define MX_RELEASE16 12
+#endif
+  // A K block is 64 MFMAs, one per 16x16 sub-tile, in four quarters of 16 (512 MFMA cycles each)
+  // over the fragment sets a[0], a[1] (rows 0-63, 64-127 of the wave) and b[0], b[1], in an
+  // order that needs every set for two quarters in a row (slots 0-63 = the block's MFMAs):
+  //   quarter 0: a[0] x b[0], a[0]'s sub-tiles one after the other.  Read meanwhile, from this
+  //              block: the last sub-tile of a[0] (slots 0, 1; used from slot 12) and b[1]
+  //              (2-9).  Once every wave has done so (barrier in front of slot kRelease) the
+  //              ring block is free and the copies of block b+2 start, one every third slot
+  //              (the copy unit takes about 20 cycles per copy for each of the four waves)
+  //   quarter 1: a[1] x b[0]
+  //   quarter 2: a[1] x b[1].  Block b+1 must have landed (wait, barrier); its b[0] and scales
+  //              are read
+  //   quarter 3: a[0] x b[1], a[0]'s sub-tiles one after the other.  a[1] takes block b+1's data,
+  //              and so does a sub-tile of a[0] as soon as an MFMA of the next sub-tile has been
+  //              issued (slots 52/53, 56/57, 60/61)
+  // A register is read from LDS between the last MFMA that uses its old contents and its first
+  // use; LDS reads return in order, so "the reads issued up to some point have landed" is
+  // s_waitcnt lgkmcnt(number of reads issued since).  An MFMA occupies the matrix pipe for 32
+  // cycles and the wave's issue for about half of that: what is issued behind it has to fit
+  // the other half, so copies and reads are spread over the slots as evenly as the rules above
+  // allow.
+  constexpr int kRelease = MX_RELEASE16;          // slot in front of which the ring block is released
+  constexpr int kFirstCopy = kRelease + 1;        // copy j goes behind the MFMA of slot kFirstCopy + 3j
+  constexpr int kCopiesA = (32 - kFirstCopy + 2) / 3;  // copies issued in quarters 0 and 1
+  static_assert(kRelease >= 12 && kFirstCopy + 3 * 16 < 64, "seventeen copies, three slots apart");
+  auto copy_at = [&](auto slot_) {  // slot 0..63 of the block
+#ifndef MX_ABL_NO_DMA
+    constexpr int sl = decltype(slot_)::value;
+    if constexpr (sl >= kFirstCopy && (sl - kFirstCopy) % 3 == 0 && (sl - kFirstCopy) / 3 < 17)
+      issue_piece(std::integral_constant<int, (sl - kFirstCopy) / 3>{});
+#endif
+  };
+  // quarter: 16 MFMAs of a[ah] x b[bh]; AMAJOR: a's sub-tiles one after the other (else b's);
+  // side(slot, false) runs in front of a slot's MFMA, side(slot, true) behind it
+  auto quarter = [&](Frags16& f, auto first_, auto ah_, auto bh_, auto amajor_, auto&& side) {
+    constexpr bool kFirst = decltype(first_)::value;
+    constexpr int ah = decltype(ah_)::value, bh = decltype(bh_)::value;
+    constexpr bool kAMajor = decltype(amajor_)::value;
+    static_for<0, 16>([&](auto i_) {
+      constexpr int i = decltype(i_)::value;
+      constexpr int tm = kAMajor ? i >> 2 : i & 3, tn = kAMajor ? i & 3 : i >> 2;
+      constexpr int m = 4 * ah + tm, n = 4 * bh + tn;
+      side(i_, std::false_type{});
+      mfma16_asm<(n >> 1), (m >> 1), kFirst>(acc[m][n], f.b[bh][tn], f.a[ah][tm], f.sb[n & 1], f.sa[m & 1]);
+      side(i_, std::true_type{});
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+  auto landed = [&](auto n_, v8i& frag) {  // all LDS reads but the n youngest have landed
+    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(decltype(n_)::value) : "memory");
+    asm volatile("" : "+v"(frag));
+  };
+  auto block_steps = [&](Frags16& f, auto first_) {
+    using H0 = std::integral_constant<int, 0>;
+    using H1 = std::integral_constant<int, 1>;
+    const uint32_t s_cur = lds_base + c_slot * kBlock32, s_nxt = lds_base + (c_slot ^ 1) * kBlock32;
+    // quarter 0.  In flight on entry, oldest first: the last two reads of a[1], a[0][1], the
+    // other last two reads of a[1], a[0][2] (see quarter 3)
+    quarter(f, first_, H0{}, H0{}, std::true_type{}, [&](auto i_, auto after_) {
+      constexpr int i = decltype(i_)::value;
+      if constexpr (!decltype(after_)::value) {
+        if constexpr (i == 4) landed(std::integral_constant<int, 4 + 4>{}, f.a[0][1]);
+        if constexpr (i == 8) landed(std::integral_constant<int, 8>{}, f.a[0][2]);
+        if constexpr (i == kRelease) {
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave's reads of the block are done
+          asm volatile("" : "+v"(f.a[0][3]));
+          uint64_t t0 = 0;
+          if constexpr (PROF) t0 = __builtin_readcyclecounter();
+          __builtin_amdgcn_s_barrier();
+          if constexpr (PROF) {
+            const uint64_t t1 = __builtin_readcyclecounter();
+            prof_bar += t1 - t0;
+            prof_last += t1 - t0;  // keep the barrier out of the body figure
+          }
+        }
+      } else {
+#ifndef MX_ABL_NO_READ
+        if constexpr (i < 2) read_set_piece(f.a[0], s_cur, 0u, H0{}, std::integral_constant<int, 6 + i>{});
+        else if constexpr (i < 10) read_set_piece(f.b[1], s_cur, fb_delta, H1{}, std::integral_constant<int, i - 2>{});
+#endif
+        copy_at(i_);
+      }
+    });
+    pin_set(f.a[1]);
+    pin_set(f.b[1]);
+    // quarter 1
+    quarter(f, first_, H1{}, H0{}, std::false_type{}, [&](auto i_, auto after_) {
+      if constexpr (decltype(after_)::value) copy_at(std::integral_constant<int, 16 + decltype(i_)::value>{});
+    });
+    uint64_t t0 = 0, t1 = 0;
+    if constexpr (PROF) {
+      t0 = __builtin_readcyclecounter();
+      prof_body += t0 - prof_last;
+    }
+    // block b+1 (and any output stores): everything but the copies issued so far in this block
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kCopiesA) : "memory");
+    if constexpr (PROF) {
+      t1 = __builtin_readcyclecounter();
+      prof_vm += t1 - t0;
+    }
+    __builtin_amdgcn_s_barrier();
+    if constexpr (PROF) {
+      prof_last = __builtin_readcyclecounter();
+      prof_bar += prof_last - t1;
+    }
+    // quarter 2: b[0] of block b+1 and its first three scale dwords, in the slots without a copy
+    quarter(f, first_, H1{}, H1{}, std::false_type{}, [&](auto i_, auto after_) {
+      constexpr int i = decltype(i_)::value, sl = 32 + i;
+      if constexpr (decltype(after_)::value) {
+        copy_at(std::integral_constant<int, sl>{});
+#ifndef MX_ABL_NO_READ
+        constexpr bool has_copy = sl >= kFirstCopy && (sl - kFirstCopy) % 3 == 0;
+        // free slots of the quarter before this one
+        constexpr int before = i - (sl - kFirstCopy + 2) / 3 + (32 - kFirstCopy + 2) / 3;
+        if constexpr (!has_copy) {
+          if constexpr (before < 8) read_set_piece(f.b[0], s_nxt, fb_delta, H0{}, std::integral_constant<int, before>{});
+          else if constexpr (before < 11) read_scale_piece(f, s_nxt, std::integral_constant<int, before - 8>{});
+        }
+#endif
+      }
+    });
+    // quarter 3, reads by slot: a[1] 0 (+ the fourth scale dword), 1, 2, 3 (+ the two dwords of
+    // the next scale group, kGrouped2d3d), a[0][0], a[1] 4, 5, a[0][1], a[1] 6, 7, a[0][2]
+    quarter(f, first_, H0{}, H1{}, std::true_type{}, [&](auto i_, auto after_) {
+      constexpr int i = decltype(i_)::value;
+      if constexpr (decltype(after_)::value) {
+        copy_at(std::integral_constant<int, 48 + i>{});
+#ifndef MX_ABL_NO_READ
+        if constexpr (i < 4) {
+          read_set_piece(f.a[1], s_nxt, 0u, H1{}, i_);
+          if constexpr (i == 0) read_scale_piece(f, s_nxt, std::integral_constant<int, 3>{});
+          if constexpr (kScalePieces == 6 && i >= 2) read_scale_piece(f, s_nxt, std::integral_constant<int, i + 2>{});
+        } else if constexpr (i < 14) {
+          constexpr int k = i - 4;  // 0, 1: a[0][0]; 2, 3: a[1] 4, 5; 4, 5: a[0][1]; 6, 7: a[1] 6, 7; 8, 9: a[0][2]
+          if constexpr ((k & 3) < 2) read_set_piece(f.a[0], s_nxt, 0u, H0{}, std::integral_constant<int, 2 * (k >> 2) + (k & 1)>{});
+          else read_set_piece(f.a[1], s_nxt, 0u, H1{}, std::integral_constant<int, 4 + 2 * (k >> 2) + (k & 1)>{});
+        }
+#endif
+      }
+    });
+    c_slot ^= 1;
+    // the next block's first MFMAs need its b[0], its scales and the first sub-tile of its
+    // a[0]: everything but the eight reads issued since
+    asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
+    pin_set(f.b[0]);
+    asm volatile("" : "+v"(f.a[0][0]));
+    next_scales(f, c_slot);
+    issue_advance();
+  };
+
+#endif  // MX_MFMA16
   // Output: a lane holds, per 32x32 sub-tile, row li and columns 8q + 4lj + 0..3.  The two
   // lanes of a row (lj = 0, 1) trade halves with v_permlane32_swap so that each owns 8
   // consecutive bf16; a 32-row x 64-column piece is then turned around in this wave's private
@@ -803,7 +1078,12 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     // flight (s_waitcnt vmcnt(0)) at exactly the two places where those should keep running.
     uint32_t lane_e = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
     asm volatile("" : "+v"(lane_e));
+#if MX_MFMA16
+    // + (m & 1) * 16 rows + (second sub-tile pair of the piece) * 64
+    const uint32_t patch_w = patch + (lane_e & 15) * kPatchPitch + ((lane_e >> 4) & 1) * 32 + (lane_e >> 5) * 16;
+#else
     const uint32_t patch_w = patch + (lane_e & 31) * kPatchPitch + (lane_e >> 5) * 16;   // + (n&1)*64 + h*32
+#endif
     const uint32_t patch_r = patch + (lane_e >> 3) * kPatchPitch + (lane_e & 7) * 16;  // + pass*8 rows
     const int64_t rows_valid = t.rows_a;
     const uint32_t cols_valid = (uint32_t)(t.rows_b < kT32 ? t.rows_b : kT32);
@@ -813,6 +1093,18 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       const uint32_t ld_b = (uint32_t)p.ldd * 4;
       const __amdgpu_buffer_rsrc_t rp = make_rsrc(t.d, rows_valid * ld_b);
       const uint32_t row_b = (wm * 128 + li) * ld_b;
+#if MX_MFMA16
+      // (a lane holds row 16m + li, columns 16n + 4lj + 0..3 of sub-tile (m, n))
+      static_for<0, 64>([&](auto i_) {
+        constexpr int m = decltype(i_)::value >> 3, n = decltype(i_)::value & 7;
+        const uint32_t col = wn * 128 + n * 16 + 4 * lj;
+        const uint32_t v = col < cols_valid ? row_b + col * 4 : 0x80000000u;
+        const u32x4 w = {__float_as_uint(acc_read<0>(acc[m][n])), __float_as_uint(acc_read<1>(acc[m][n])),
+                         __float_as_uint(acc_read<2>(acc[m][n])), __float_as_uint(acc_read<3>(acc[m][n]))};
+        __builtin_amdgcn_raw_buffer_store_b128(w, rp, v, m * 16 * ld_b, MX_STORE_AUX);
+      });
+      return;
+#else
       static_for<0, 16>([&](auto i_) {
         constexpr int m = decltype(i_)::value >> 2, n = decltype(i_)::value & 3;
         const v16f a = acc[m][n];
@@ -826,6 +1118,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
         });
       });
       return;
+#endif
     }
     const uint32_t ldd_b = (uint32_t)p.ldd * 2;
     const __amdgpu_buffer_rsrc_t rd = make_rsrc(t.d, rows_valid * ldd_b);
@@ -836,6 +1129,34 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     // A wave's LDS instructions execute in order, so a piece's reads may follow its writes
     // without a wait, and the next piece's writes may follow those reads: the only waits are
     // for the read data, with the next piece's conversion and writes already under way.
+#if MX_MFMA16
+    // MX_MFMA16: a lane holds row 16m + li, columns 16n + 4lj + 0..3 of sub-tile (m, n).  Part k of
+    // piece p covers 16 rows x 32 columns: sub-tiles (m, n) and (m, n + 1), m = 2(p / 2) + k / 2,
+    // n = 4(p % 2) + 2(k % 2).  v_permlane16_swap trades the halves of two neighbouring lane
+    // groups: the even groups end up with 8 consecutive columns of sub-tile n, the odd ones with
+    // 8 of sub-tile n + 1.
+    auto stage_part = [&](auto p_, auto k_) {
+      constexpr int mp = decltype(p_)::value >> 1, np = decltype(p_)::value & 1, k = decltype(k_)::value;
+      constexpr int m = 2 * mp + (k >> 1), n = 4 * np + 2 * (k & 1);
+      const v4f& c0 = acc[m][n];
+      const v4f& c1 = acc[m][n + 1];
+      const float a[8] = {acc_read<0>(c0), acc_read<1>(c0), acc_read<2>(c0), acc_read<3>(c0),
+                          acc_read<0>(c1), acc_read<1>(c1), acc_read<2>(c1), acc_read<3>(c1)};
+      uint32_t x0 = pack_bf16(a[0], a[1]), y0 = pack_bf16(a[2], a[3]);
+      uint32_t x1 = pack_bf16(a[4], a[5]), y1 = pack_bf16(a[6], a[7]);
+      if constexpr (MODE != kDense) {  // a broken group contract must not pass unnoticed: NaN
+        x0 |= nan_mask;
+        y0 |= nan_mask;
+        x1 |= nan_mask;
+        y1 |= nan_mask;
+      }
+      const u32x2 sx = __builtin_amdgcn_permlane16_swap(x0, x1, false, false);
+      const u32x2 sy = __builtin_amdgcn_permlane16_swap(y0, y1, false, false);
+      const v4i w = {(int)sx.x, (int)sy.x, (int)sx.y, (int)sy.y};
+      lds_write_b128_hidden<(m & 1) * 16 * kPatchPitch + (k & 1) * 64>(patch_w, w);
+      __builtin_amdgcn_sched_barrier(0);
+    };
+#else
     auto stage_part = [&](auto p_, auto k_) {  // 32 rows x 16 columns: accumulators -> bf16 -> patch
       constexpr int m = decltype(p_)::value >> 1, np = decltype(p_)::value & 1;
       constexpr int n = 2 * np + (decltype(k_)::value >> 1), h = decltype(k_)::value & 1;
@@ -861,6 +1182,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       // accumulator blocks ahead and the epilogue spreads over registers the K loop's constants sit in
       __builtin_amdgcn_sched_barrier(0);
     };
+#endif
     v4i r[2][4];
     static_for<0, 4>([&](auto k_) { stage_part(std::integral_constant<int, 0>{}, k_); });
     static_for<0, 8>([&](auto p_) {
@@ -902,11 +1224,28 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __builtin_amdgcn_s_barrier();
   issue_block();  // block 1: in flight when the first step starts
+#if MX_MFMA16
+  Frags16 f;
+  {
+    using Z = std::integral_constant<int, 0>;
+    using O = std::integral_constant<int, 1>;
+    static_for<0, 8>([&](auto i_) { read_set_piece(f.a[0], lds_base, 0u, Z{}, i_); });
+    static_for<0, 8>([&](auto i_) { read_set_piece(f.a[1], lds_base, 0u, O{}, i_); });
+    static_for<0, 8>([&](auto i_) { read_set_piece(f.b[0], lds_base, fb_delta, Z{}, i_); });
+    static_for<0, kScalePieces>([&](auto i_) { read_scale_piece(f, lds_base, i_); });
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    pin_set(f.a[0]);
+    pin_set(f.a[1]);
+    pin_set(f.b[0]);
+    next_scales(f, 0);
+  }
+#else
   Frags32 f0, f1;
   read_frags(f0, 0, std::integral_constant<int, 0>{});
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   pin_frags(f0);
   rotate_scales(f0, 0);
+#endif
   if constexpr (PROF) prof_last = __builtin_readcyclecounter();
 
   // ---- tiles; at the top of every tile f0 holds the fragments of its first half block (the
@@ -918,6 +1257,22 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       // PAIR: the loader walks both segments of the tile one after the other (same K for both);
       // for the compute stream they are one run of blocks
       const uint32_t nblocks = PAIR ? 2 * t.nblocks : t.nblocks;
+#if MX_MFMA16
+      block_steps(f, std::true_type{});
+      // two blocks per trip: a taken branch stalls the lone wave of a SIMD for longer than the
+      // 32 cycles its last MFMA covers, and the trip's end has two of them
+      uint32_t i = 1;
+      for (; i + 2 <= nblocks; i += 2) {
+        block_steps(f, std::false_type{});
+        block_steps(f, std::false_type{});
+      }
+      if (i < nblocks) block_steps(f, std::false_type{});
+      // the next tile's first fragments, read in the last quarter, become ordinary values
+      // before anything else runs
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      pin_set(f.a[0]);
+      pin_set(f.a[1]);
+#else
       block_steps(f0, f1, std::true_type{});
       for (uint32_t i = 1; i < nblocks; ++i) block_steps(f0, f1, std::false_type{});
       // the next tile's first fragments were read in the last step: make them ordinary
@@ -925,6 +1280,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       // its read was still in flight would lose the data)
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       pin_frags(f0);
+#endif
       if constexpr (PROF) {
         const uint64_t e0 = __builtin_readcyclecounter();
         prof_body += e0 - prof_last;
