@@ -80,6 +80,9 @@ def parse():
                     help="instead of the benchmark: the GEMM kernel at the benchmark shape on random data, on "
                          "constant operands and on half of the CUs, and the vendor library's fp8 GEMM, 8 launches "
                          "each in that order (for a rocprofv3 --pmc run: active cycles / time = shader clock)")
+    ap.add_argument("--mfma-ceiling", action="store_true",
+                    help="only time the MFMA-only yardstick (both MFMA shapes, three kinds of operand bits) and "
+                         "print its JSON line: what the power limit leaves of the matrix peak")
     ap.add_argument("--gemm-ablation", action="store_true",
                     help="instead of the benchmark: the dense GEMM at the benchmark shape and the three grouped "
                          "GEMMs of the MoE config (equal groups and the skewed routing), timed with whatever build "
@@ -384,6 +387,59 @@ def gemm_ablation(dev, recipe_mode):
             row[name] = {"us": round(sec * 1e6, 1), "TFLOP/s": round(flops / sec / 1e12, 1)}
         out[kind] = row
         del xm, wm, dy, xq0, xq1, dyq0, dyq1, wq0, wq1, y, dx, dw
+    return out
+
+
+def mfma_ceiling(dev, recipe_mode):
+    """What the power limit leaves of the matrix peak: the library's MFMA-only yardstick (operands
+    in registers, no LDS or memory traffic in the loop, one wave per SIMD on every CU) for both
+    shapes of the scaled fp8 MFMA, on three kinds of operand bits -- e4m3 codes of the benchmark's
+    activations and weights (cast with the recipe), uniformly random bytes, and one constant byte.
+    Every case runs for about a second and the rate of its second half is reported, so that the
+    clock has settled.  No GEMM can beat the figure of its operand kind."""
+    import ctypes
+
+    import torch
+
+    from torchtitan_amd import _lib, ops
+
+    lib = _lib.load()
+    lib.mx_debug_mfma_only.restype = ctypes.c_int
+    lib.mx_debug_mfma_only.argtypes = [ctypes.c_void_p if i in (1, 2, 5) else ctypes.c_int for i in range(6)]
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    nbytes = 16 * 256 * 32
+    g = torch.Generator(device=dev).manual_seed(0)
+    x = torch.randn((nbytes // 2 // DIM, DIM), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    w = (torch.randn((nbytes // 2 // DIM, DIM), generator=g, device=dev, dtype=torch.float32) * 0.02).to(torch.bfloat16)
+    cast = torch.cat((ops.to_mx_dim0(x, recipe_mode).codes.flatten(), ops.to_mx_dim0(w, recipe_mode).codes.flatten()))
+    rnd = torch.randint(0, 256, (nbytes,), generator=g, device=dev, dtype=torch.uint8)
+    rnd = torch.where((rnd & 0x7F) == 0x7F, rnd ^ 1, rnd)  # no NaN codes
+    operands = {"cast_of_benchmark_data": cast, "uniform_random_bytes": rnd,
+                "constant_byte_0x38": torch.full((nbytes,), 0x38, device=dev, dtype=torch.uint8)}
+    sink = torch.empty(cus * 256, device=dev, dtype=torch.float32)
+    st = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    out = {"workgroups": cus, "waves_per_simd": 1}
+    for shape, iters in ((32, 2400), (16, 1200)):
+        flop = iters * 16 * 2.0 * 32 * 32 * 64 * 4 * cus * (1 if shape == 32 else 2)
+        for name, buf in operands.items():
+            assert buf.numel() == nbytes and buf.data_ptr() % 32 == 0
+
+            def launch(n):
+                for _ in range(n):
+                    rc = lib.mx_debug_mfma_only(shape, ctypes.c_void_p(buf.data_ptr()), ctypes.c_void_p(sink.data_ptr()),
+                                                cus, iters, st)
+                    assert rc == 0, rc
+
+            launch(500)
+            torch.cuda.synchronize()
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            launch(500)
+            e.record()
+            torch.cuda.synchronize()
+            sec = s.elapsed_time(e) * 1e-3 / 500
+            out[f"mfma_{shape}_{name}"] = {"us_per_launch": round(sec * 1e6, 1), "TFLOP/s": round(flop / sec / 1e12, 1),
+                                           "frac_of_peak": round(flop / sec / 1e12 / PEAK_MXFP8_TFLOPS, 3)}
     return out
 
 
@@ -1042,6 +1098,9 @@ def main():
     if args.clock_table:
         print(json.dumps(clock_table(dev, recipe_mode)))
         return
+    if args.mfma_ceiling:
+        print(json.dumps(mfma_ceiling(dev, recipe_mode)))
+        return
     if args.gemm_ablation:
         print(json.dumps(gemm_ablation(dev, recipe_mode)))
         return
@@ -1101,7 +1160,7 @@ def main():
             "casts_per_step": 8,
         },
         "roofline": {
-            "kernel": "gemm_nt32_kernel (persistent 256x256 tiles, v_mfma_scale_f32_32x32x64_f8f6f4)",
+            "kernel": "gemm_nt32_kernel (persistent 256x256 tiles, v_mfma_scale_f32_16x16x128_f8f6f4)",
             "bound": "mfma",
             "achieved": round(achieved, 1),
             "peak": PEAK_MXFP8_TFLOPS,

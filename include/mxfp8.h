@@ -47,7 +47,8 @@ typedef enum { MX_SCALE_FLOOR = 0, MX_SCALE_RCEIL = 1 } mx_scale_mode_t;
  *   MFMA      [ceil(rows/128), ceil(nblk/2), 64, 4]: for row group rt, 64-deep K step ks,
  *             lane l, byte t the entry is scale[rt*128 + t*32 + (l & 31)][ks*2 + (l >> 5)]
  *             (zero beyond the matrix) -- one dword per lane feeds four 32-row sub-tiles of
- *             v_mfma_scale_f32_32x32x64_f8f6f4; the order mx_gemm_nt reads.
+ *             v_mfma_scale_f32_32x32x64_f8f6f4, or four 16-row sub-tiles 32 rows apart of
+ *             v_mfma_scale_f32_16x16x128_f8f6f4; the order mx_gemm_nt reads.
  */
 typedef enum { MX_SCALES_ROWMAJOR = 0, MX_SCALES_MFMA = 1 } mx_scale_order_t;
 
@@ -272,7 +273,7 @@ int mx_gemm_nt_pair(const uint8_t* a_codes, const uint8_t* a_scales, const uint8
  *                       multiple of 32 rows (the alignment of the reference's padded token
  *                       groups, torchtitan/components/quantization/__init__.py:36),
  *                       T % 32 == 0, K % 128 == 0, N % 8 == 0, G <= 510: the persistent
- *                       32x32x64 kernel (several times faster).  The group ends live on the
+ *                       persistent kernel (several times faster).  The group ends live on the
  *                       device, so they are checked there: a violation fills D with NaN.
  * Stands in for torch._grouped_mm(x, w^T, offs) in forward and dgrad
  * (torchtitan/models/common/moe/moe.py:59-76). */

@@ -13,16 +13,16 @@
 extern "C" {
 #endif
 
-/* 0: pick the dense GEMM kernel by shape (default); 1 / 2: the 16x16x128 tile kernel with
- * 256x256 / 128x128 tiles for every shape; 3: the persistent 32x32x64 kernel for every shape it
- * can take, however few tiles there are. */
+/* 0: pick the dense GEMM kernel by shape (default); 1 / 2: the one-tile-per-workgroup kernel with
+ * 256x256 / 128x128 tiles for every shape; 3: the persistent kernel for every shape it can take,
+ * however few tiles there are. */
 void mx_debug_force_kernel(int which);
 
-/* > 0: number of persistent workgroups of the 32x32x64 kernel, rounded up to a multiple of 8
+/* > 0: number of persistent workgroups of the persistent kernel, rounded up to a multiple of 8
  * (also lowers how many tiles one grouped launch covers); 0: one per CU (default). */
 void mx_debug_set_grid(int workgroups);
 
-/* -DMX_TIMING_BUILD only.  Device buffer of 256 * 4 * 8 uint64 that the timing build of the 32x32x64 kernel fills with
+/* -DMX_TIMING_BUILD only.  Device buffer of 256 * 4 * 8 uint64 that the timing build of the persistent kernel fills with
  * per-wave cycle counts {copy wait, barriers, step body, epilogue, ...}; NULL switches the timing
  * build off (default). */
 void mx_debug_set_prof(void* device_buffer);
@@ -33,6 +33,13 @@ void mx_debug_set_prof(void* device_buffer);
  * `bytes` / 2 to dst (the read : write mix of a one-direction cast).  bytes % 16 == 0, 16-byte aligned.
  * Returns an mx_status_t. */
 int mx_debug_stream(int kind, const void* src, void* dst, int64_t bytes, void* stream);
+
+/* Matrix-pipe yardstick for bench.py: `workgroups` x 4 waves run `iters` rounds of independent
+ * scaled fp8 MFMAs on operands that stay in registers (shape 32: 16 x v_mfma_scale_f32_32x32x64
+ * per round, shape 16: 64 x v_mfma_scale_f32_16x16x128; 2 * 32 * 32 * 64 * 16 flop per wave and
+ * round either way), no LDS or memory traffic in the loop.  `operands`: 16 * 256 * 32 bytes of e4m3
+ * codes (32-byte aligned), `out`: workgroups * 256 floats.  Returns an mx_status_t. */
+int mx_debug_mfma_only(int shape, const void* operands, void* out, int workgroups, int iters, void* stream);
 
 #ifdef __cplusplus
 }

@@ -30,7 +30,7 @@ def _f32(bits):
                                    (4096, 4352, 128), (6144, 6400, 256)])
 @pytest.mark.parametrize("force", [0, 3])
 def test_gemm_matches_oracle(device, M, N, K, force):
-    """force 0: the kernel the library picks for the shape; 3: the persistent 32x32x64 kernel
+    """force 0: the kernel the library picks for the shape; 3: the persistent kernel (mx_gemm32.hip)
     wherever it can run (small shapes would otherwise go to the tile kernel)."""
     from torchtitan_amd import _lib
 

@@ -87,7 +87,8 @@ __device__ __forceinline__ uint32_t nan_block_codes2(uint32_t w) {
 // Byte offset of scale (row, blk) in MX_SCALES_MFMA order; ks_n = ceil(nblk / 2).
 // Groups of 128 rows x 2 blocks (one 64-deep K step) are 256 contiguous bytes: for lane l and
 // byte t the entry is row = 32 t + (l & 31), block = l >> 5 -- one dword per lane carries the
-// scales that a 32x32x64 MFMA lane needs for four 32-row sub-tiles.
+// scales that a 32x32x64 MFMA lane needs for four 32-row sub-tiles (a 16x16x128 MFMA lane: for
+// four 16-row sub-tiles 32 rows apart).
 __device__ __host__ __forceinline__ int64_t mfma_scale_offset(int64_t row, int64_t blk,
                                                               int64_t ks_n) {
   return (((row >> 7) * ks_n + (blk >> 1)) << 8) + ((((blk & 1) << 5) + (row & 31)) << 2) +

@@ -84,7 +84,7 @@ static int check_dense(const uint8_t* a_codes, const uint8_t* a_scales, const ui
   return MX_OK;
 }
 
-// What the persistent 32x32x64 kernel needs beyond the general checks.
+// What the persistent kernel (mx_gemm32.hip) needs beyond the general checks.
 static bool persistent_ok(const void* d, int64_t N, int64_t K, int64_t ldd) {
   return !(K % 128 || (uint64_t)K * 256 > 0x7FFFFFFFull || N % 8 || ldd % 8 || ((uintptr_t)d & 15) ||
            (uint64_t)ldd * 512 > 0x7FFFFFFFull);

@@ -1,5 +1,6 @@
-// MXFP8 GEMM for large shapes, dense and grouped: persistent 256x256 tiles on
-// v_mfma_scale_f32_32x32x64_f8f6f4.
+// MXFP8 GEMM for large shapes, dense and grouped: persistent 256x256 tiles on the scaled fp8
+// MFMA (v_mfma_scale_f32_16x16x128_f8f6f4; -DMX_MFMA16=0 builds the v_mfma_scale_f32_32x32x64_f8f6f4
+// form of the K loop instead).
 //
 //   D[M,N] (bf16) = deq(A)[M,K] * deq(B)[N,K]^T, fp32 accumulate.
 //
@@ -10,26 +11,39 @@
 //
 // Global -> LDS moves whole 128-byte rows (buffer_load_dwordx4 ... lds, 8 rows per instruction:
 // full cache lines, which the texture path delivers about twice as fast as 64-byte pieces), so
-// the ring holds two 128-deep blocks of 64 KB codes + 2 KB scales.  Compute runs in 64-deep
-// steps (two per block): 16 MFMAs per wave per step (1024 MFMA cycles), fragments LDS -> VGPR
-// double-buffered in registers and read one step ahead, conflict-free under the b128 pass
-// grouping.  Two barriers per block: one in the middle of the first step releases the ring
-// block whose last fragments have just been read (its refill starts there, spread over 22
-// MFMA slots because the copy path is the scarce resource), one before the second step makes
-// sure the next block has landed.
+// the ring holds two 128-deep blocks of 64 KB codes + 2 KB scales.  Two barriers per block: one
+// releases the ring block whose last fragments have just been read (its refill starts there,
+// spread thinly because the copy path is the scarce resource), one makes sure the next block
+// has landed.
 //
-// Operand layout of the 32x32x64 f8 MFMA (measured): lane (i = l & 31, j = l >> 5) holds row i,
-// K bytes [16j, 16j+16) in registers 0-3 and [32+16j, 32+16j+16) in registers 4-7; the scale
-// of 32-element block b is taken from lane group b.  With the first operand = B rows and the
-// second = A rows, a lane ends up with D[row = l & 31][col = 8q + 4j + 0..3], q = 0..3.
+// Which MFMA.  Both forms do 2048 flop per cycle and SIMD and read the same operand bytes per
+// flop; the 16x16x128 one reads and writes a quarter of the accumulator registers per
+// instruction.  Under the chip's power limit that is worth 9 % of sustained rate on the same
+// operand bits with nothing else running, and 6-10 % of shader clock inside this kernel, against
+// 2-3 % more cycles (64 MFMA slots of 32 cycles per block leave less room behind each MFMA for
+// the block's LDS reads and copies than 32 slots of 64 cycles).
+//   16x16x128 (default): a block is 64 MFMAs, one per 16x16 sub-tile, in four quarters over
+//     four fragment sets (two 64-row halves of A, two of B) that are refilled in place as soon
+//     as their last MFMA has been issued; see block_steps for the slot plan.  Operand layout
+//     (measured): lane (i = l & 15, j = l >> 4) holds row i, K bytes [16j, 16j+16) in registers
+//     0-3 and [64+16j, 64+16j+16) in registers 4-7; the scale of 32-element block b is taken
+//     from lane group b.  With the first operand = B rows and the second = A rows, a lane ends
+//     up with D[row = l & 15][col = 4j + 0..3].
+//   32x32x64: compute runs in 64-deep steps (two per block), 16 MFMAs per wave per step,
+//     fragments LDS -> VGPR double-buffered in registers and read one step ahead.  Operand
+//     layout (measured): lane (i = l & 31, j = l >> 5) holds row i, K bytes [16j, 16j+16) in
+//     registers 0-3 and [32+16j, 32+16j+16) in registers 4-7; scales as above; a lane ends up
+//     with D[row = l & 31][col = 8q + 4j + 0..3], q = 0..3.
+// Fragment reads are conflict-free under the b128 pass grouping in both forms.
 //
-// MX_ABL_NO_DMA / MX_ABL_NO_READ / MX_ABL_STORE_ROWS (never defined in the product build) drop the
-// copies, the fragment reads or part of the output stores from the steady state, to time what is
-// left; results are then meaningless.
+// MX_ABL_NO_DMA / MX_ABL_NO_READ / MX_ABL_STORE_ROWS / MX_ABL_NO_EPILOGUE (never defined in the
+// product build) drop the copies, the fragment reads, part of the output stores or the whole
+// epilogue from the steady state, to time what is left; results are then meaningless.
 #include "mx_gemm_tile.h"
 
 // 1: the K loop runs on v_mfma_scale_f32_16x16x128_f8f6f4 (one MFMA per 16x16 sub-tile and
-// 128-deep block); 0: on v_mfma_scale_f32_32x32x64_f8f6f4 (two per 32x32 sub-tile and block).
+// 128-deep block); 0: on v_mfma_scale_f32_32x32x64_f8f6f4 (two per 32x32 sub-tile and block):
+// kept as the reference point of the measurements that compare the two.
 #ifndef MX_MFMA16
 #define MX_MFMA16 1
 #endif

@@ -179,7 +179,7 @@ extern "C" int mx_grouped_gemm_2d3d(const uint8_t* a_codes, const uint8_t* a_sca
   if (256 * K > 0x7FFFFFFFll) return MX_ERR_UNSUPPORTED;
   hipStream_t st = (hipStream_t)stream;
   if (a_scale_order == MX_SCALES_MFMA) {
-    // group ends at multiples of 32 (checked on the device): the persistent 32x32x64 kernel
+    // group ends at multiples of 32 (checked on the device): the persistent kernel (mx_gemm32.hip)
     if (K % 128 || N % 8 || ldd % 8 || ((uintptr_t)d & 15) || ((uintptr_t)a_scales & 3) ||
         T % 32)
       return MX_ERR_ALIGNMENT;

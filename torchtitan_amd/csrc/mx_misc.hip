@@ -54,7 +54,87 @@ __global__ __launch_bounds__(256) void stream_write_kernel(y_u32x4* __restrict__
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i < n) __builtin_nontemporal_store(y_u32x4{(uint32_t)i, 1u, 2u, 3u}, dst + i);
 }
+// Matrix-pipe yardstick: nothing but independent scaled fp8 MFMAs on operands held in registers
+// (no LDS, no memory traffic after the first loads), one wave per SIMD.  What a launch of it
+// sustains is what the power limit leaves of the matrix peak for the given operand bits.
+typedef int y_v8i __attribute__((ext_vector_type(8)));
+typedef float y_v16f __attribute__((ext_vector_type(16)));
+typedef float y_v4f __attribute__((ext_vector_type(4)));
+
+template <int SHAPE>
+__global__ __launch_bounds__(256) void mfma_only_kernel(const y_v8i* __restrict__ src, float* __restrict__ dst,
+                                                        int iters) {
+  const int lane = threadIdx.x;
+  constexpr int kF = SHAPE == 32 ? 4 : 8;  // fragments per operand: 16 or 64 accumulator tiles, 256 registers
+  y_v8i a[kF], b[kF];
+#pragma unroll
+  for (int i = 0; i < kF; ++i) {
+    a[i] = src[i * 256 + lane];
+    b[i] = src[(kF + i) * 256 + lane];
+  }
+  const int sc = 0x7f7f7f7f;  // E8M0 127 = 1.0 in every scale byte
+  float s = 0.f;
+  if constexpr (SHAPE == 32) {
+    y_v16f acc[kF][kF];
+#pragma unroll
+    for (int i = 0; i < kF; ++i)
+#pragma unroll
+      for (int j = 0; j < kF; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+      for (int i = 0; i < kF; ++i)
+#pragma unroll
+        for (int j = 0; j < kF; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[i], b[j], acc[i][j], 0, 0, 0, sc, 0, sc);
+    }
+#pragma unroll
+    for (int i = 0; i < kF; ++i)
+#pragma unroll
+      for (int j = 0; j < kF; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s += acc[i][j][e];
+  } else {
+    y_v4f acc[kF][kF];
+#pragma unroll
+    for (int i = 0; i < kF; ++i)
+#pragma unroll
+      for (int j = 0; j < kF; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+      for (int i = 0; i < kF; ++i)
+#pragma unroll
+        for (int j = 0; j < kF; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a[i], b[j], acc[i][j], 0, 0, 0, sc, 0, sc);
+    }
+#pragma unroll
+    for (int i = 0; i < kF; ++i)
+#pragma unroll
+      for (int j = 0; j < kF; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) s += acc[i][j][e];
+  }
+  dst[blockIdx.x * 256 + lane] = s;
+}
 }  // namespace mx
+
+extern "C" int mx_debug_mfma_only(int shape, const void* operands, void* out, int workgroups, int iters,
+                                  void* stream) {
+  if ((shape != 16 && shape != 32) || !operands || !out || workgroups <= 0 || iters <= 0 ||
+      ((uintptr_t)operands & 31))
+    return MX_ERR_INVALID_ARG;
+  hipStream_t st = (hipStream_t)stream;
+  if (shape == 32)
+    hipLaunchKernelGGL(mx::mfma_only_kernel<32>, dim3((unsigned)workgroups), dim3(256), 0, st,
+                       (const mx::y_v8i*)operands, (float*)out, iters);
+  else
+    hipLaunchKernelGGL(mx::mfma_only_kernel<16>, dim3((unsigned)workgroups), dim3(256), 0, st,
+                       (const mx::y_v8i*)operands, (float*)out, iters);
+  return hipGetLastError() == hipSuccess ? MX_OK : MX_ERR_LAUNCH;
+}
 
 extern "C" int mx_debug_stream(int kind, const void* src, void* dst, int64_t bytes, void* stream) {
   if (bytes <= 0 || bytes % 16 || kind < 0 || kind > 3) return MX_ERR_INVALID_ARG;

@@ -606,7 +606,7 @@ def mx_grouped_gemm_2d3d(a: MXData, b: MXData, offs: torch.Tensor,
     int32 [G] inclusive cumulative group sizes on the device.  With row-major scales for a the
     groups may end anywhere; with MFMA-order scales for a every group must end at a multiple
     of 32 rows (checked on the device: a violation fills the output with NaN) and the
-    persistent 32x32x64 kernel runs.
+    persistent kernel (csrc/mx_gemm32.hip) runs.
     """
     T, K = a.codes.shape
     G, N, Kb = b.codes.shape
@@ -656,7 +656,7 @@ def mx_grouped_gemm_2d2d(at: MXData, bt: MXData, offs: torch.Tensor,
     at: codes [N, T], bt: codes [K, T] (column-wise casts), scales of both in the same order.
     Groups may be any multiple of 32 tokens (checked on the device: a violation gives NaN).
     MFMA order: T a multiple of 128 (the token axis may run past the last group) and the
-    persistent 32x32x64 kernel runs.
+    persistent kernel (csrc/mx_gemm32.hip) runs.
     """
     N, T = at.codes.shape
     K, Tb = bt.codes.shape
