@@ -103,3 +103,24 @@ def test_new_entry_points_validate_arguments_before_any_launch():
     # shapes that are never split need no device to say so
     assert lib.mx_gemm_nt_workspace_bytes(64, 64, 4096) == 0
     assert lib.mx_gemm_nt_workspace_bytes(4096, 4096, 0) == 0
+
+
+def test_library_exports_the_test_hooks_of_the_debug_header():
+    """include/mxfp8_debug.h: every hook is exported, except the one that exists in timing builds
+    only; the yardsticks check their arguments before any launch."""
+    debug = HEADER.with_name("mxfp8_debug.h")
+    text = re.sub(r"/\*.*?\*/", "", debug.read_text(), flags=re.S)
+    names = set(re.findall(r"\b(mx_debug_[a-z0-9_]+)\s*\(", text))
+    assert {"mx_debug_force_kernel", "mx_debug_set_grid", "mx_debug_stream", "mx_debug_mfma_only"} <= names
+    lib = ctypes.CDLL(str(_lib.LIB_PATH))
+    for name in names - {"mx_debug_set_prof"}:
+        assert hasattr(lib, name), name
+    assert not hasattr(lib, "mx_debug_set_prof"), "the product build carries no timing instances"
+    lib.mx_debug_mfma_only.restype = ctypes.c_int
+    lib.mx_debug_mfma_only.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
+                                       ctypes.c_void_p]
+    assert lib.mx_debug_mfma_only(8, None, None, 1, 1, None) == 1      # no such MFMA shape
+    assert lib.mx_debug_mfma_only(16, None, None, 256, 10, None) == 1  # null operands
+    lib.mx_debug_stream.restype = ctypes.c_int
+    lib.mx_debug_stream.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
+    assert lib.mx_debug_stream(0, None, None, 24, None) == 1           # not a multiple of 16 bytes
