@@ -390,7 +390,7 @@ def gemm_ablation(dev, recipe_mode):
     return out
 
 
-def mfma_ceiling(dev, recipe_mode):
+def mfma_ceiling(dev, recipe_mode, launches=500, kinds=None, shapes=(32, 16)):
     """What the power limit leaves of the matrix peak: the library's MFMA-only yardstick (operands
     in registers, no LDS or memory traffic in the loop, one wave per SIMD on every CU) for both
     shapes of the scaled fp8 MFMA, on three kinds of operand bits -- e4m3 codes of the benchmark's
@@ -419,9 +419,12 @@ def mfma_ceiling(dev, recipe_mode):
     sink = torch.empty(cus * 256, device=dev, dtype=torch.float32)
     st = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
     out = {"workgroups": cus, "waves_per_simd": 1}
-    for shape, iters in ((32, 2400), (16, 1200)):
+    for shape in shapes:
+        iters = 2400 if shape == 32 else 1200
         flop = iters * 16 * 2.0 * 32 * 32 * 64 * 4 * cus * (1 if shape == 32 else 2)
         for name, buf in operands.items():
+            if kinds is not None and name not in kinds:
+                continue
             assert buf.numel() == nbytes and buf.data_ptr() % 32 == 0
 
             def launch(n):
@@ -430,14 +433,14 @@ def mfma_ceiling(dev, recipe_mode):
                                                 cus, iters, st)
                     assert rc == 0, rc
 
-            launch(500)
+            launch(launches)
             torch.cuda.synchronize()
             s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             s.record()
-            launch(500)
+            launch(launches)
             e.record()
             torch.cuda.synchronize()
-            sec = s.elapsed_time(e) * 1e-3 / 500
+            sec = s.elapsed_time(e) * 1e-3 / launches
             out[f"mfma_{shape}_{name}"] = {"us_per_launch": round(sec * 1e6, 1), "TFLOP/s": round(flop / sec / 1e12, 1),
                                            "frac_of_peak": round(flop / sec / 1e12 / PEAK_MXFP8_TFLOPS, 3)}
     return out
@@ -1199,6 +1202,13 @@ def main():
             line["roofline"]["frac_on_constant_operands"] = same["frac_of_peak"]
             line["roofline"]["power_note"] = ("the same kernel and shape on all-ones operands, timed in this run: the "
                                               "gap to `frac` is the shader clock the power limit grants under random data")
+        # what an MFMA-only loop sustains on the benchmark's operand bits under the power limit
+        # (half a second per case): the ceiling of `roofline.frac` on this box
+        ceiling = mfma_ceiling(dev, recipe_mode, launches=250, kinds=("cast_of_benchmark_data",), shapes=(16,))
+        line["yardsticks"]["mfma_only_16x16x128_on_benchmark_operands"] = ceiling["mfma_16_cast_of_benchmark_data"]
+        top = ceiling["mfma_16_cast_of_benchmark_data"]["frac_of_peak"]
+        line["roofline"]["mfma_only_ceiling_frac"] = top
+        line["roofline"]["frac_of_mfma_only_ceiling"] = round(line["roofline"]["frac"] / top, 3) if top else None
         torch.cuda.empty_cache()
         line["llama3_8b_decoder_block"] = time_decoder_block(dev, args.recipe)
     if not args.no_cpu_baseline:
