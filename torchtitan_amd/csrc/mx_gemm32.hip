@@ -38,7 +38,9 @@
 //
 // MX_ABL_NO_DMA / MX_ABL_NO_READ / MX_ABL_STORE_ROWS / MX_ABL_NO_EPILOGUE (never defined in the
 // product build) drop the copies, the fragment reads, part of the output stores or the whole
-// epilogue from the steady state, to time what is left; results are then meaningless.
+// epilogue from the steady state, to time what is left; MX_ABL_SAME_PANEL makes all dense tiles
+// read the same twelve operand panels (nothing comes from beyond the L2).  Results are then
+// meaningless.
 #include "mx_gemm_tile.h"
 
 // 1: the K loop runs on v_mfma_scale_f32_16x16x128_f8f6f4 (one MFMA per 16x16 sub-tile and
@@ -358,8 +360,13 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     if (MODE == kDense || (MODE == kGrouped2d3d && poison)) {
       tile_coords(t, (uint32_t)((p.M + kT32 - 1) / kT32), tiles_n, tm, tn);
       tn += tn0;
+#ifdef MX_ABL_SAME_PANEL  // timing ablation: every 8 x 4 round reads the same twelve operand panels
+      r.a = a_codes + (int64_t)(tm & 7) * kT32 * K;
+      r.b = b_codes + (int64_t)(tn & 3) * kT32 * K;
+#else
       r.a = a_codes + (int64_t)tm * kT32 * K;
       r.b = b_codes + (int64_t)tn * kT32 * K;
+#endif
       r.sa = a_scales + (int64_t)(tm * 2) * ks_n * 256;
       r.sb = b_scales + (int64_t)(tn * 2) * ks_n * 256;
       r.d = p.d + (int64_t)tm * kT32 * p.ldd + (int64_t)tn * kT32;
