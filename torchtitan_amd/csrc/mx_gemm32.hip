@@ -290,14 +290,14 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     poison = any_bad(bad);
     if (tid < 64) {  // inclusive prefix sum of first[1 .. G+1] by wave 0, 10 entries per lane
       uint32_t sum = 0;
-      for (uint32_t g = 1 + tid * 10; g < 11 + tid * 10 && g <= G + 1; ++g) sum += first[g];
+      for (uint32_t g = 1 + (uint32_t)tid * 10; g < 11 + (uint32_t)tid * 10 && g <= G + 1; ++g) sum += first[g];
       uint32_t incl = sum;
       for (int d = 1; d < 64; d <<= 1) {
         const uint32_t o = __shfl_up(incl, d);
         if (tid >= d) incl += o;
       }
       uint32_t run = incl - sum;
-      for (uint32_t g = 1 + tid * 10; g < 11 + tid * 10 && g <= G + 1; ++g) {
+      for (uint32_t g = 1 + (uint32_t)tid * 10; g < 11 + (uint32_t)tid * 10 && g <= G + 1; ++g) {
         run += first[g];
         first[g] = run;
       }
