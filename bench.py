@@ -147,6 +147,9 @@ def time_casts(dev, recipe_mode, also_floor=False):
                               ("w_14336x4096", (HIDDEN, DIM), 6)):
         bufs = [torch.randn(shape, device=dev, dtype=torch.bfloat16) for _ in range(nbuf)]
         el = shape[0] * shape[1]
+        # the plain stream kernels over exactly this tensor's bytes, same rotation of buffers: a
+        # launch's fixed cost weighs three times as much on 134 MB as on the 512 MiB yardsticks
+        same_size = _streams_of_size(dev, bufs)
         for kind, fn, bpe in (("dim0", ops.to_mx_dim0, 3.03125), ("dim1", ops.to_mx_dim1, 3.03125),
                               ("dim0_dim1", ops.to_mx_dim0_dim1, 4.0625)):
             for b in bufs[:2]:
@@ -162,10 +165,49 @@ def time_casts(dev, recipe_mode, also_floor=False):
             sec = s.elapsed_time(e) * 1e-3 / reps
             out[f"{kind}:{name}"] = {"us": round(sec * 1e6, 1), "GB/s": round(el * bpe / sec / 1e9, 1),
                                      "frac_hbm": round(el * bpe / sec / 1e9 / PEAK_HBM_GBPS, 3)}
+            ref = same_size["stream_copy" if kind == "dim0_dim1" else "stream_2to1"]
+            out[f"{kind}:{name}"]["same_size_stream_us"] = ref["us"]
+            out[f"{kind}:{name}"]["frac_of_same_size_stream"] = round(el * bpe / sec / 1e9 / ref["GB/s"], 3)
         del bufs
     if also_floor and recipe_mode != "floor":
         floor = time_casts_one(dev, "floor", "x_16384x4096", (M, DIM), 6)
         out.update({f"{k}:floor": v for k, v in floor.items()})
+    return out
+
+
+def _streams_of_size(dev, bufs):
+    """GB/s of the library's copy (1 : 1) and 2 : 1 stream kernels over the bytes of one of `bufs`,
+    reading the buffers in turn like the casts do; destinations rotate too."""
+    import ctypes
+
+    import torch
+
+    from torchtitan_amd import _lib
+
+    lib = _lib.load()
+    lib.mx_debug_stream.restype = ctypes.c_int
+    lib.mx_debug_stream.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
+    nbytes = bufs[0].numel() * bufs[0].element_size()
+    dsts = [torch.empty(nbytes, device=dev, dtype=torch.uint8) for _ in range(min(len(bufs), 3))]
+    st = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    out = {}
+    for name, kind, moved in (("stream_copy", 0, 2 * nbytes), ("stream_2to1", 3, nbytes + nbytes // 2)):
+        def run(i):
+            rc = lib.mx_debug_stream(kind, ctypes.c_void_p(bufs[i % len(bufs)].data_ptr()),
+                                     ctypes.c_void_p(dsts[i % len(dsts)].data_ptr()), nbytes, st)
+            assert rc == 0, rc
+        for i in range(2):
+            run(i)
+        torch.cuda.synchronize()
+        reps = 3 * len(bufs)
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for i in range(reps):
+            run(i)
+        e.record()
+        torch.cuda.synchronize()
+        sec = s.elapsed_time(e) * 1e-3 / reps
+        out[name] = {"us": round(sec * 1e6, 1), "GB/s": round(moved / sec / 1e9, 1)}
     return out
 
 
@@ -302,7 +344,9 @@ def _stream_yardsticks(dev, nbuf=3, mib=512):
 
 def _casts_against_streams(casts, yardsticks):
     """Adds to every cast its rate as a share of the plain streaming kernel with the same read : write
-    mix, timed in the same run: 2 : 1 for one direction, 1 : 1 (the copy) for the fused cast."""
+    mix, timed in the same run: 2 : 1 for one direction, 1 : 1 (the copy) for the fused cast.
+    (`frac_of_stream_same_mix`: against the 512 MiB yardsticks; time_casts adds
+    `frac_of_same_size_stream`, against the same kernels over exactly the cast's input bytes.)"""
     for key, row in casts.items():
         ref = yardsticks.get("stream_copy" if key.startswith("dim0_dim1") else "stream_2to1")
         if ref and ref.get("GB/s"):
@@ -312,9 +356,10 @@ def _casts_against_streams(casts, yardsticks):
 def cast_table(dev, recipe_mode):
     """The HBM yardsticks and then the casts, in a fixed order (see --cast-table): one JSON line of
     HIP-event times; under rocprofv3 --pmc the dispatches appear in the same order."""
-    out = {"order": ["stream_copy", "stream_read", "stream_write", "stream_2to1", "dim0:x", "dim1:x", "dim0_dim1:x", "dim0:dy",
-                     "dim1:dy", "dim0_dim1:dy", "dim0:w", "dim1:w", "dim0_dim1:w"],
-           "launches_per_kernel": "2 warm-up + 8 timed (casts: 2 + 3 x buffers)"}
+    per_tensor = lambda t: [f"stream_copy_of_size:{t}", f"stream_2to1_of_size:{t}", f"dim0:{t}", f"dim1:{t}", f"dim0_dim1:{t}"]
+    out = {"order": ["stream_copy", "stream_read", "stream_write", "stream_2to1"] + per_tensor("x") + per_tensor("dy") + per_tensor("w"),
+           "launches_per_kernel": "2 warm-up + 8 timed (casts and the streams of a tensor's size: 2 + 3 x buffers, "
+                                  "x and w 6 buffers, dy 3)"}
     out["yardsticks"] = _stream_yardsticks(dev)
     out["casts"] = time_casts(dev, recipe_mode)
     _casts_against_streams(out["casts"], out["yardsticks"])
