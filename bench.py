@@ -5,7 +5,8 @@ Workload (BASELINE.json configs[1]): dense MXFP8 linear forward + dgrad + wgrad 
 Llama-3-8B FFN shapes, M = 16384 tokens; w1 and w3 are [14336, 4096], w2 is [4096, 14336];
 activations N(0,1), weights N(0,0.02), upstream grads N(0,1e-3), all bf16, seeded, resident in
 HBM before the timed region.  One step = the three linears, each through the converted module
-(product path): 2 fused casts + GEMM in forward, 1 fused cast + 2 GEMMs in backward.
+(product path): 2 fused casts + GEMM in forward, 1 fused cast + 2 GEMMs in backward; the step runs
+the three forwards and then the three backwards, as a block does, so w1 and w3 share the cast of x.
 
 Prints ONE JSON line.  `value` counts only GEMM flops (2 M N K each) over the whole step time,
 casts included in the time.  `roofline` is for the dominant kernel (the persistent 256x256-tile
@@ -127,9 +128,13 @@ def one_step(ffn, x, h, dy_h, dy_o):
     mx_tensor.clear_cast_cache()  # a new step has new activations: nothing carries over
     x.grad = None
     h.grad = None
+    # the order of a real block: all forwards, then the backwards in reverse (w1 and w3 read the
+    # same x, whose cast the second one reuses)
+    outs = []
     for lin, inp, dy in ((ffn.w1, x, dy_h), (ffn.w3, x, dy_h), (ffn.w2, h, dy_o)):
         lin.weight.grad = None
-        y = lin(inp)
+        outs.append((lin(inp), dy))
+    for y, dy in reversed(outs):
         y.backward(dy)
 
 

@@ -243,7 +243,11 @@ int mx_gemm_nt_ws(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t
  * Runs the kernels mx_gemm_nt_ws runs with a workspace of mx_gemm_nt_workspace_bytes(M, N, K), so
  * the results are bit-identical to that call's; shapes that are not split run what mx_gemm_nt
  * runs.  A shape whose split needs more than the array holds returns MX_ERR_SCRATCH_TOO_SMALL and
- * launches nothing.  All calls on one GPU share that GPU's array: calls that overlap in time on
+ * launches nothing (to know beforehand: mx_gemm_nt_workspace_bytes(M, N, K) against
+ * mx_gemm_nt_static_max_bytes(); such a shape runs through mx_gemm_nt unsplit, or through
+ * mx_gemm_nt_ws with memory of the caller's).  The first call on a GPU looks up that GPU's copy
+ * of the array and raises the kernel's LDS limit, neither of which belongs into a graph capture:
+ * make one call per GPU (any shape) before capturing.  All calls on one GPU share that GPU's array: calls that overlap in time on
  * the same GPU (two streams, two threads) race on it.  Nothing in the array needs clearing between
  * calls: every partial tile is written in full before the reduction reads it. */
 int64_t mx_gemm_nt_static_max_bytes(void);

@@ -52,18 +52,26 @@ def test_static_scratch_gemm_equals_the_workspace_form(device):
 
 def test_static_scratch_gemm_rejects_what_does_not_fit(device):
     lib = _lib.load()
+    # hooks another test may have left set must not decide whether anything is launched
+    lib.mx_debug_force_kernel(0)
+    lib.mx_debug_set_grid(0)
     # 289 output tiles: two rounds of tiles unsplit, so the split runs several rounds of slices and
     # needs more than one slice-tile per CU (the 64 MiB hold exactly one 256x256 float32 tile per CU)
     M, N, K = 4352, 4352, 147456
     with torch.cuda.device(device):
         need = int(lib.mx_gemm_nt_workspace_bytes(M, N, K))
     assert need > 64 << 20
-    # the shape check comes before anything is read: small dummy operands are enough
-    dummy = torch.zeros(1024, dtype=torch.uint8, device=device)
-    out = torch.zeros(8, dtype=torch.bfloat16, device=device)
-    with torch.cuda.device(device):
-        st = lib.mx_gemm_nt_static(ops._ptr(dummy), ops._ptr(dummy), ops._ptr(dummy), ops._ptr(dummy), ops._ptr(out),
-                                   M, N, K, N, ops._stream(out))
-    assert st == 5 and b"scratch" in lib.mx_status_string(st)
+    # operands and output of the real size (zeros): were the call ever to launch, it would stay in
+    # bounds and the status check below would be what fails
+    codes = torch.zeros((M, K), dtype=torch.uint8, device=device)
+    scales = torch.zeros(int(lib.mx_scales_mfma_bytes(M, K // 32)), dtype=torch.uint8, device=device)
+    out = torch.full((M, N), 7.0, dtype=torch.bfloat16, device=device)
+    for hook in (0, 3, 1):  # the size check does not depend on the kernel-selection hook
+        lib.mx_debug_force_kernel(hook)
+        with torch.cuda.device(device):
+            st = lib.mx_gemm_nt_static(ops._ptr(codes), ops._ptr(scales), ops._ptr(codes), ops._ptr(scales),
+                                       ops._ptr(out), M, N, K, N, ops._stream(out))
+        lib.mx_debug_force_kernel(0)
+        assert st == 5 and b"scratch" in lib.mx_status_string(st)
     torch.cuda.synchronize(device)
-    assert bool((out == 0).all())
+    assert bool((out == 7.0).all()), "nothing was launched"

@@ -181,10 +181,11 @@ extern "C" int mx_gemm_nt_static(const uint8_t* a_codes, const uint8_t* a_scales
                                  int64_t M, int64_t N, int64_t K, int64_t ldd, void* stream) {
   const int rc = check_dense(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd);
   if (rc != MX_OK || M == 0 || N == 0) return rc;
-  const int64_t need = force_kernel == 0 ? mx_gemm_nt_workspace_bytes(M, N, K) : 0;
-  if (need == 0 || !persistent_ok(d, N, K, ldd))  // not a split shape: no scratch involved
+  // the size check stands on the shape alone, whatever the test hooks say
+  const int64_t need = mx_gemm_nt_workspace_bytes(M, N, K);
+  if (need > kScratchBytes && persistent_ok(d, N, K, ldd)) return MX_ERR_SCRATCH_TOO_SMALL;
+  if (need == 0 || force_kernel != 0 || !persistent_ok(d, N, K, ldd))  // not split: no scratch involved
     return mx_gemm_nt(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd, stream);
-  if (need > kScratchBytes) return MX_ERR_SCRATCH_TOO_SMALL;
   void* ws = scratch_of_current_device();
   if (!ws) return MX_ERR_LAUNCH;
   return launch_gemm_nt32_splitk(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd,

@@ -71,7 +71,7 @@ static_assert(kRing32 + 4 * kPatch32 == 160 * 1024, "the kernel's LDS map fills 
 // What a launch works on.  One kernel serves three problems that differ only in how a linear
 // tile number maps to operand rows, K range and output address:
 //   kDense        D[M,N] = A[M,K] B[N,K]^T
-//   kGrouped2d3d  rows of A in groups (inclusive ends offs[g], all multiples of 128), group g
+//   kGrouped2d3d  rows of A in groups (inclusive ends offs[g], all multiples of 32), group g
 //                 against B[g][N,K]; rows from offs[G-1] to M are written as zeros
 //   kGrouped2d2d  D[g][M,N] = A[M, lo_g:hi_g] B[N, lo_g:hi_g]^T, K = row length of A and B
 //   kSplitK       as kGrouped2d2d with G equal slices of the K blocks worked out in the kernel
@@ -1466,7 +1466,7 @@ int launch_gemm_nt32_splitk(const uint8_t* a_codes, const uint8_t* a_scales, con
   return hipGetLastError() == hipSuccess ? MX_OK : MX_ERR_LAUNCH;
 }
 
-// Grouped forms with every group end a multiple of 128 and all scales in MFMA order
+// Grouped forms with every group end a multiple of 32 and all scales in MFMA order
 // (a_scales over the whole [T, K/32] matrix, b_scales one block per expert).  A workgroup keeps
 // a record per tile in LDS, at most kMaxRecords of them: larger problems are cut into several
 // launches over ranges of tile columns.
