@@ -38,7 +38,9 @@ int mx_debug_stream(int kind, const void* src, void* dst, int64_t bytes, void* s
  * scaled fp8 MFMAs on operands that stay in registers (shape 32: 16 x v_mfma_scale_f32_32x32x64
  * per round, shape 16: 64 x v_mfma_scale_f32_16x16x128; 2 * 32 * 32 * 64 * 16 flop per wave and
  * round either way), no LDS or memory traffic in the loop.  `operands`: 16 * 256 * 32 bytes of e4m3
- * codes (32-byte aligned), `out`: workgroups * 256 floats.  Returns an mx_status_t. */
+ * codes (32-byte aligned), `out`: workgroups * 256 floats.  Shapes 1601 / 1604 / 1608 run the
+ * 16x16x128 form in a fixed order in which 1 / 4 / 8 MFMAs in a row share an operand fragment
+ * (1604 is the order of the GEMM kernel's K loop).  Returns an mx_status_t. */
 int mx_debug_mfma_only(int shape, const void* operands, void* out, int workgroups, int iters, void* stream);
 
 #ifdef __cplusplus

@@ -1,6 +1,5 @@
 // MXFP8 GEMM for large shapes, dense and grouped: persistent 256x256 tiles on the scaled fp8
-// MFMA (v_mfma_scale_f32_16x16x128_f8f6f4; -DMX_MFMA16=0 builds the v_mfma_scale_f32_32x32x64_f8f6f4
-// form of the K loop instead).
+// MFMA v_mfma_scale_f32_16x16x128_f8f6f4.
 //
 //   D[M,N] (bf16) = deq(A)[M,K] * deq(B)[N,K]^T, fp32 accumulate.
 //
@@ -16,43 +15,32 @@
 // spread thinly because the copy path is the scarce resource), one makes sure the next block
 // has landed.
 //
-// Which MFMA.  Both forms do 2048 flop per cycle and SIMD and read the same operand bytes per
-// flop; the 16x16x128 one reads and writes a quarter of the accumulator registers per
-// instruction.  Under the chip's power limit that is worth 9 % of sustained rate on the same
-// operand bits with nothing else running, and 6-10 % of shader clock inside this kernel, against
-// 2-3 % more cycles (64 MFMA slots of 32 cycles per block leave less room behind each MFMA for
-// the block's LDS reads and copies than 32 slots of 64 cycles).
-//   16x16x128 (default): a block is 64 MFMAs, one per 16x16 sub-tile, in four quarters over
-//     four fragment sets (two 64-row halves of A, two of B) that are refilled in place as soon
-//     as their last MFMA has been issued; see block_steps for the slot plan.  Operand layout
-//     (measured): lane (i = l & 15, j = l >> 4) holds row i, K bytes [16j, 16j+16) in registers
-//     0-3 and [64+16j, 64+16j+16) in registers 4-7; the scale of 32-element block b is taken
-//     from lane group b.  With the first operand = B rows and the second = A rows, a lane ends
-//     up with D[row = l & 15][col = 4j + 0..3].
-//   32x32x64: compute runs in 64-deep steps (two per block), 16 MFMAs per wave per step,
-//     fragments LDS -> VGPR double-buffered in registers and read one step ahead.  Operand
-//     layout (measured): lane (i = l & 31, j = l >> 5) holds row i, K bytes [16j, 16j+16) in
-//     registers 0-3 and [32+16j, 32+16j+16) in registers 4-7; scales as above; a lane ends up
-//     with D[row = l & 31][col = 8q + 4j + 0..3], q = 0..3.
-// Fragment reads are conflict-free under the b128 pass grouping in both forms.
+// Which MFMA.  The 16x16x128 and the 32x32x64 form both do 2048 flop per cycle and SIMD and read
+// the same operand bytes per flop; the 16x16x128 one reads and writes a quarter of the
+// accumulator registers per instruction.  Under the chip's power limit that is worth 9 % of
+// sustained rate on the same operand bits with nothing else running, and was worth 6-10 % of
+// shader clock inside this kernel against 2-3 % more cycles when the K loop moved to it (64 MFMA
+// slots of 32 cycles per block leave less room behind each MFMA for the block's LDS reads and
+// copies than 32 slots of 64 cycles).
+//   A block is 64 MFMAs, one per 16x16 sub-tile, in four quarters over four fragment sets (two
+//   64-row halves of A, two of B) that are refilled in place as soon as their last MFMA has been
+//   issued; see block_steps for the slot plan.  Operand layout (measured): lane (i = l & 15,
+//   j = l >> 4) holds row i, K bytes [16j, 16j+16) in registers 0-3 and [64+16j, 64+16j+16) in
+//   registers 4-7; the scale of 32-element block b is taken from lane group b.  With the first
+//   operand = B rows and the second = A rows, a lane ends up with D[row = l & 15][col = 4j + 0..3].
+// Fragment reads are conflict-free under the b128 pass grouping.
 //
 // MX_ABL_NO_DMA / MX_ABL_NO_READ / MX_ABL_STORE_ROWS / MX_ABL_NO_EPILOGUE (never defined in the
 // product build) drop the copies, the fragment reads, part of the output stores or the whole
 // epilogue from the steady state, to time what is left; MX_ABL_SAME_PANEL makes all dense tiles
-// read the same twelve operand panels (nothing comes from beyond the L2).  Results are then
-// meaningless.
+// read the same twelve operand panels (MX_ABL_SAME_A / MX_ABL_SAME_B: the same A / B panels only), so
+// that every read beyond the L2 finds its line in the memory-side cache; MX_ABL_ROW_PAD=n reads the
+// rows of a tile n bytes further apart than they lie (what a padded row pitch would do to the
+// spread of a block's lines over the cache channels).  Results are then meaningless.
 #include "mx_gemm_tile.h"
-
-// 1: the K loop runs on v_mfma_scale_f32_16x16x128_f8f6f4 (one MFMA per 16x16 sub-tile and
-// 128-deep block); 0: on v_mfma_scale_f32_32x32x64_f8f6f4 (two per 32x32 sub-tile and block):
-// kept as the reference point of the measurements that compare the two.
-#ifndef MX_MFMA16
-#define MX_MFMA16 1
-#endif
 
 namespace mx {
 
-typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr int kT32 = 256;                        // tile edge (M and N)
@@ -128,7 +116,7 @@ __device__ __forceinline__ void tile_coords(uint32_t t, uint32_t tiles_m, uint32
   tm = first_m + (in - tn * gsz);
 }
 
-// LDS accesses the compiler must not see (see read_piece in the kernel)
+// LDS accesses the compiler must not see (see the fragment reads in the kernel)
 template <int OFF>
 __device__ __forceinline__ void lds_write_b128_hidden(uint32_t addr, v4i v) {
   asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(addr), "v"(v), "n"(OFF) : "memory");
@@ -145,26 +133,9 @@ __device__ __forceinline__ v4i pin(v4i v) {
 }
 
 // One scaled MFMA, C = 0 (FIRST) or accumulate.  Written as assembly: left as builtins, the
-// compiler gathers all 32 MFMAs of a tile's first block behind the block's copies, reads and
-// barriers instead of leaving them interleaved.  op_sel / op_sel_hi pick the scale byte of
-// the lane's scale dword: N for the first operand, M for the second.
-template <int N, int M, bool FIRST>
-__device__ __forceinline__ void mfma_asm(v16f& c, const v8i& b, const v8i& a, uint32_t sb,
-                                         uint32_t sa) {
-  if constexpr (FIRST)
-    asm volatile(
-        "v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, 0, %3, %4 op_sel:[%5,%6,0] op_sel_hi:[%7,%8,0]"
-        : "=a"(c)
-        : "v"(b), "v"(a), "v"(sb), "v"(sa), "n"(N & 1), "n"(M & 1), "n"(N >> 1), "n"(M >> 1));
-  else
-    asm volatile(
-        "v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[%5,%6,0] op_sel_hi:[%7,%8,0]"
-        : "+a"(c)
-        : "v"(b), "v"(a), "v"(sb), "v"(sa), "n"(N & 1), "n"(M & 1), "n"(N >> 1), "n"(M >> 1));
-}
-
-// The same for v_mfma_scale_f32_16x16x128_f8f6f4 (MX_MFMA16): NB / MB = scale byte of the first /
-// second operand's dword.
+// compiler gathers all MFMAs of a tile's first block behind the block's copies, reads and
+// barriers instead of leaving them interleaved.  op_sel / op_sel_hi pick the scale byte of the
+// lane's scale dword: NB for the first operand, MB for the second.
 template <int NB, int MB, bool FIRST>
 __device__ __forceinline__ void mfma16_asm(v4f& c, const v8i& b, const v8i& a, uint32_t sb,
                                            uint32_t sa) {
@@ -189,14 +160,7 @@ __device__ __forceinline__ float acc_read(const V& c) {
   return x;
 }
 
-struct Frags32 {
-  v8i a[4];
-  v8i b[4];
-  uint32_t sa, sb;
-  uint32_t sa_hi;  // kGrouped2d3d: the A scale dword of the next 128-row group (see rotate_scales)
-};
-
-// MX_MFMA16: fragment sets of four 16-row sub-tiles each, whole 128-deep blocks (a[h][t] =
+// Fragment sets of four 16-row sub-tiles each, whole 128-deep blocks (a[h][t] =
 // sub-tile 4h + t of the wave's 128 rows of A, b[h][t] likewise for B), the scale dwords of the
 // block being computed (one for the even and one for the odd sub-tiles) and those of the next.
 struct Frags16 {
@@ -214,11 +178,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
-#if MX_MFMA16
   const int li = lane & 15, lj = lane >> 4;
-#else
-  const int li = lane & 31, lj = lane >> 5;
-#endif
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void_t*)smem;  // LDS byte address of the ring
   const uint32_t K = (uint32_t)p.K;  // bytes per operand row; a multiple of 128 for this kernel
   const uint32_t ks_n = K / kK32;    // 64-deep steps per 128-row scale group
@@ -360,8 +320,14 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     if (MODE == kDense || (MODE == kGrouped2d3d && poison)) {
       tile_coords(t, (uint32_t)((p.M + kT32 - 1) / kT32), tiles_n, tm, tn);
       tn += tn0;
-#ifdef MX_ABL_SAME_PANEL  // timing ablation: every 8 x 4 round reads the same twelve operand panels
+#if defined(MX_ABL_SAME_PANEL)  // timing ablation: every 8 x 4 round reads the same twelve operand panels
       r.a = a_codes + (int64_t)(tm & 7) * kT32 * K;
+      r.b = b_codes + (int64_t)(tn & 3) * kT32 * K;
+#elif defined(MX_ABL_SAME_A)  // ... the same eight A panels only
+      r.a = a_codes + (int64_t)(tm & 7) * kT32 * K;
+      r.b = b_codes + (int64_t)tn * kT32 * K;
+#elif defined(MX_ABL_SAME_B)  // ... the same four B panels only
+      r.a = a_codes + (int64_t)tm * kT32 * K;
       r.b = b_codes + (int64_t)(tn & 3) * kT32 * K;
 #else
       r.a = a_codes + (int64_t)tm * kT32 * K;
@@ -481,7 +447,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     __syncthreads();
   }
   // this workgroup's i-th tile (records are read so that the compiler's wait-count model
-  // does not see an LDS read, see read_piece; every lane reads the same 64 bytes)
+  // does not see an LDS read, see the fragment reads; every lane reads the same 64 bytes)
   auto get_tile = [&](uint32_t i) -> Tile32 {
     if constexpr (MODE == kDense) {
       return describe(t_lo + (PAIR ? i >> 1 : i) * wgs_per_xcd, PAIR ? i & 1 : 0);
@@ -520,22 +486,16 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
 
   // ---- per-lane constants
   // global -> LDS: a load unit is 8 rows x 128 B; lane l fetches row l/8 and the logical 16-byte
-  // chunk that belongs at physical chunk l%8 of that row: c = (l%8) ^ ((row >> 1) & 7)
-#if MX_MFMA16
-  // (16-row sub-tiles: c = (l%8) ^ ((row & 2) | ((row & 8) >> 1)), see the fragment reads)
+  // chunk that belongs at physical chunk l%8 of that row:
+  // c = (l%8) ^ ((row & 2) | ((row & 8) >> 1)), see the fragment reads
   const uint32_t c_even = (lane & 7) ^ ((lane >> 3) & 2);
-#else
-  const uint32_t c_even = (lane & 7) ^ (lane >> 4);  // even units; odd units flip bit 2
+#ifndef MX_ABL_ROW_PAD  // timing ablation: the rows of a tile are read this many bytes further apart than they lie
+#define MX_ABL_ROW_PAD 0
 #endif
-  const uint32_t v_even = (uint32_t)(lane >> 3) * K + c_even * 16;
+  const uint32_t Kp = K + MX_ABL_ROW_PAD;
+  const uint32_t v_even = (uint32_t)(lane >> 3) * Kp + c_even * 16;
   // (odd units: v_even ^ 64 -- K is a multiple of 128, so bit 6 belongs to the chunk alone)
-  // LDS -> VGPR: for K half h of a block, lane (li, lj) reads chunks 4h+lj and 4h+2+lj of row li
-  // of each 32-row sub-tile; physical chunk = logical ^ ((row >> 1) & 7), so the second chunk is
-  // address ^ 32 and h flips address bit 6.  Only the A address is kept per lane; B's differs by
-  // a wave-uniform amount, as do the scale addresses (group g = A0, A1, B0, B1, K half h at
-  // kCodes32 + (g*2 + h) * 256).
-#if MX_MFMA16
-  // MX_MFMA16: lane (li = l & 15, lj = l >> 4) of a 16-row sub-tile reads chunks lj and lj + 4 of
+  // LDS -> VGPR: lane (li = l & 15, lj = l >> 4) of a 16-row sub-tile reads chunks lj and lj + 4 of
   // row li (K bytes [16 lj, +16) and [64 + 16 lj, +16)); physical chunk = logical ^ sw with
   // sw = (row & 2) | ((row & 8) >> 1), which spreads the 16 lanes of every b128 pass (lanes
   // {0-3, 12-15, 20-23, 24-27} and {4-11, 16-19, 28-31} of a half-wave) over all bank groups;
@@ -544,10 +504,6 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   // m >> 1: one dword for the even sub-tiles, the one 64 bytes on for the odd ones.
   const uint32_t sw = (li & 2) | ((li & 8) >> 1);
   const uint32_t lane4 = (uint32_t)(lj >> 1) * 256 + (uint32_t)((lj & 1) * 32 + li) * 4;
-#else
-  const uint32_t sw = (li >> 1) & 7;
-  const uint32_t lane4 = lane * 4;
-#endif
   const uint32_t fa0 = (wm * 128 + li) * kKB + ((lj ^ sw) << 4);
   const uint32_t fb_delta = kOperand32 + (wn - wm) * 128 * kKB;
   // scale copy: lanes 0-31 fetch one 128-row group's 512 bytes of a block, lanes 32-63 the next
@@ -566,7 +522,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   __amdgpu_buffer_rsrc_t ra, rb, rs;  // codes of A, codes of B, scales this wave copies
   // kGrouped2d3d: a group may start at any multiple of 32 rows, the scales come in 128-row groups
   // of the whole matrix: a tile that starts `rot` 32-row blocks into a group fetches three groups
-  // and turns the bytes of every scale dword by `rot` (rotate_scales).  The rotation belongs to
+  // and turns the bytes of every scale dword by `rot` (next_scales).  The rotation belongs to
   // the tile whose block sits in a ring slot.
   uint32_t ld_rot = 0, slot_rot0 = 0, slot_rot1 = 0;
   // kGrouped2d2d: a K range may start and end at any multiple of 32.  Its first and last
@@ -632,7 +588,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       const int unit = wave * 8 + q;
       const uint32_t v = MODE == kGrouped2d2d ? ((q & 1) ? cur_v_odd : cur_v_even)
                                               : ((q & 1) ? (v_even ^ 64) : v_even);
-      const uint32_t so = (uint32_t)(unit * 8) * K + ld_kb * kKB;
+      const uint32_t so = (uint32_t)(unit * 8) * Kp + ld_kb * kKB;
       if constexpr ((i & 1) == 0)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void_t*)(uintptr_t)(sbase + unit * 1024), 16, v, so, 0, 0);
       else
@@ -670,198 +626,15 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   // Fragment reads are issued as inline assembly: the compiler cannot tell which ring block a
   // ds_read touches, so for reads it can see it waits until every global->LDS copy in flight
   // has landed (vmcnt(0)) and the prefetch distance collapses.  The reads are therefore
-  // invisible to its wait-count tracking; `pin_frags` (after the explicit lgkmcnt(0) at the top
-  // of the next step) is what the MFMAs depend on.
+  // invisible to its wait-count tracking; `pin_set` / `landed` (after an explicit lgkmcnt wait)
+  // are what the MFMAs depend on.
   auto lds_b128 = [&](uint32_t addr, auto off_) -> v4i {
     constexpr int off = decltype(off_)::value;
     v4i v;
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(off));
     return v;
   };
-#if !MX_MFMA16
-  // piece 0..7: A sub-tile m = piece/2, low/high 16 bytes; 8..15: same for B; 16,17: scales
-  auto read_piece = [&](Frags32& f, uint32_t sbase, auto half_, auto i_) {
-    constexpr int h = decltype(half_)::value;
-    constexpr int i = decltype(i_)::value;
-    if constexpr (i < 16) {
-      constexpr int t = (i & 7) >> 1;       // sub-tile
-      constexpr bool hi = i & 1;
-      const uint32_t base = (fa0 ^ (h * 64 + (hi ? 32 : 0))) + (i < 8 ? 0u : fb_delta);
-      const v4i v = lds_b128(sbase + base, std::integral_constant<int, t * 4096>{});
-      v8i& dst = i < 8 ? f.a[t] : f.b[t];
-      if constexpr (hi) {
-        dst[4] = v.x; dst[5] = v.y; dst[6] = v.z; dst[7] = v.w;
-      } else {
-        dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
-      }
-    } else if constexpr (i == 16) {
-      const uint32_t psa = sbase + fsa_s + h * 256 + lane4;
-      asm volatile("ds_read_b32 %0, %1" : "=v"(f.sa) : "v"(psa));
-      if constexpr (MODE == kGrouped2d3d) {
-        const uint32_t psa_hi = sbase + fsa_hi_s + h * 256 + lane4;
-        asm volatile("ds_read_b32 %0, %1" : "=v"(f.sa_hi) : "v"(psa_hi));
-      }
-    } else {
-      const uint32_t psb = sbase + fsb_s + h * 256 + lane4;
-      asm volatile("ds_read_b32 %0, %1" : "=v"(f.sb) : "v"(psb));
-    }
-  };
-  auto read_frags = [&](Frags32& f, int slot, auto half_) {
-    const uint32_t sbase = lds_base + slot * kBlock32;
-    static_for<0, 18>([&](auto i_) { read_piece(f, sbase, half_, i_); });
-  };
-  auto pin_frags = [&](Frags32& f) {
-#pragma unroll
-    for (int m = 0; m < 4; ++m) asm volatile("" : "+v"(f.a[m]));
-#pragma unroll
-    for (int n = 0; n < 4; ++n) asm volatile("" : "+v"(f.b[n]));
-    asm volatile("" : "+v"(f.sa), "+v"(f.sb));
-    if constexpr (MODE == kGrouped2d3d) asm volatile("" : "+v"(f.sa_hi));
-  };
-  // kGrouped2d3d, once per fragment set, after its reads have landed: byte m of the A scale dword
-  // becomes the scale of the tile's m-th 32-row block, which is byte (rot + m) of the eight bytes
-  // that two neighbouring 128-row groups hold for this lane
-  auto rotate_scales = [&](Frags32& f, int slot) {
-    if constexpr (MODE == kGrouped2d3d) {
-      const uint32_t rot = slot ? slot_rot1 : slot_rot0;
-      f.sa = __builtin_amdgcn_alignbyte(f.sa_hi, f.sa, rot);
-    }
-  };
-
-  // ---- compute stream
-  v16f acc[4][4];
-  int c_slot = 0;  // ring block holding the K block being computed
-  uint64_t prof_vm = 0, prof_bar = 0, prof_body = 0, prof_last = 0, prof_epi = 0;
-  uint64_t prof_e_stage = 0, prof_e_wait = 0, prof_e_store = 0;
-
-  auto mfma_one = [&](const Frags32& f, auto first_, auto i_) {
-    constexpr bool kFirst = decltype(first_)::value;  // first step of a tile starts from zero
-    constexpr int n = decltype(i_)::value >> 2, m = decltype(i_)::value & 3;
-    mfma_asm<n, m, kFirst>(acc[m][n], f.b[n], f.a[m], f.sb, f.sa);
-  };
-
-  // A K block is two steps of 16 MFMAs.  Entering step A of block b, f0 holds the fragments of
-  // its first K half, ring block c_slot holds block b and c_slot^1 holds block b+1 (all of its
-  // copies issued, still landing).
-  //   step A: MFMAs on f0; the second half is read into f1 in slots 0-8.  Once every wave has
-  //           done so (barrier before slot kMidA) ring block c_slot is free, and the copies of
-  //           block b+2 into it start: kCopiesA of them in the rest of the step.
-  //   step B: block b+1 must have landed (all but the kCopiesA youngest copies: wait,
-  //           barrier); MFMAs on f1; the remaining copies of block b+2, three every four
-  //           slots; the first half of block b+1 is read into f0 in slots 0-8.
-  // The copy unit serves all four waves at about 20 cycles per copy, so four waves issuing
-  // one copy per 64-cycle slot keep it saturated and the MFMAs start to wait behind them:
-  // spreading the block's 17 copies over 22 slots instead of 16 is what the second barrier
-  // buys.  A wave issues in order and an MFMA occupies the matrix pipe for 64 cycles, so every
-  // other instruction is placed in the shadow of an MFMA; the sequence is pinned with
-  // scheduling fences.  (Waits are written as assembly: the compiler rewrites the immediates
-  // of s_waitcnt builtins from its own, here too pessimistic, model of what is outstanding.)
-#ifndef MX_READ_SLOTS_A
-#define MX_READ_SLOTS_A 9
-#endif
-#ifndef MX_READ_SLOTS_B
-#define MX_READ_SLOTS_B 9
-#endif
-  // the 18 fragment reads of a step are spread evenly over its first kReadSlots MFMA slots
-  constexpr int kReadSlotsA = MX_READ_SLOTS_A, kReadSlotsB = MX_READ_SLOTS_B;
-// Output stores carry the nontemporal policy bit: written once, never re-read by this kernel,
-// and without it the output lines displace operand panels in L2 and the copies of the next
-// tile's first blocks queue behind the draining stores.
-#ifndef MX_STORE_AUX
-#define MX_STORE_AUX 2
-#endif
-#ifndef MX_MID_A
-#define MX_MID_A 10
-#endif
-#ifndef MX_B_SKIP
-#define MX_B_SKIP 4
-#endif
-  constexpr int kMidA = MX_MID_A;  // slot of step A in front of which the ring block is released
-  constexpr int kSkipB = MX_B_SKIP;  // step B leaves every kSkipB-th slot without a copy (0: none)
-  constexpr int kCopiesA = 16 - kMidA;
-  auto block_steps = [&](Frags32& f0, Frags32& f1, auto first_) {
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    pin_frags(f0);
-    {
-      const uint32_t sbase = lds_base + c_slot * kBlock32;
-      static_for<0, 16>([&](auto i_) {
-        constexpr int i = decltype(i_)::value;
-        if constexpr (i == kMidA) {
-          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave's reads of the block are done
-          uint64_t t0 = 0;
-          if constexpr (PROF) t0 = __builtin_readcyclecounter();
-          __builtin_amdgcn_s_barrier();
-          if constexpr (PROF) {
-            const uint64_t t1 = __builtin_readcyclecounter();
-            prof_bar += t1 - t0;
-            prof_last += t1 - t0;  // keep the barrier out of the body figure
-          }
-        }
-        mfma_one(f0, first_, i_);
-#ifndef MX_ABL_NO_READ
-        if constexpr (i < kReadSlotsA) {
-          constexpr int r0 = i * 18 / kReadSlotsA, r1 = (i + 1) * 18 / kReadSlotsA;
-          static_for<r0, r1>([&](auto r_) { read_piece(f1, sbase, std::integral_constant<int, 1>{}, r_); });
-        }
-#endif
-#ifndef MX_ABL_NO_DMA
-        if constexpr (i >= kMidA) issue_piece(std::integral_constant<int, i - kMidA>{});
-#endif
-        __builtin_amdgcn_sched_barrier(0);
-      });
-    }
-
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    pin_frags(f1);
-    rotate_scales(f1, c_slot);
-    uint64_t t0 = 0, t1 = 0;
-    if constexpr (PROF) {
-      t0 = __builtin_readcyclecounter();
-      prof_body += t0 - prof_last;
-    }
-    // block b+1 (and any output stores): everything but the copies issued in step A
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kCopiesA) : "memory");
-    if constexpr (PROF) {
-      t1 = __builtin_readcyclecounter();
-      prof_vm += t1 - t0;
-    }
-    __builtin_amdgcn_s_barrier();
-    if constexpr (PROF) {
-      prof_last = __builtin_readcyclecounter();
-      prof_bar += prof_last - t1;
-    }
-    {
-      const uint32_t sbase = lds_base + (c_slot ^ 1) * kBlock32;
-      static_for<0, 16>([&](auto i_) {
-        constexpr int i = decltype(i_)::value;
-        mfma_one(f1, std::false_type{}, i_);
-#ifndef MX_ABL_NO_DMA
-        // copies kCopiesA .. 17, one per slot, every kSkipB-th slot left free
-        constexpr int j = kSkipB ? i - i / kSkipB : i;
-        constexpr bool skip = kSkipB && (i % kSkipB) == kSkipB - 1;
-        if constexpr (!skip && kCopiesA + j < 17) issue_piece(std::integral_constant<int, kCopiesA + j>{});
-#endif
-#ifndef MX_ABL_NO_READ
-        if constexpr (i < kReadSlotsB) {
-          constexpr int r0 = i * 18 / kReadSlotsB, r1 = (i + 1) * 18 / kReadSlotsB;
-          static_for<r0, r1>([&](auto r_) { read_piece(f0, sbase, std::integral_constant<int, 0>{}, r_); });
-        }
-#endif
-        __builtin_amdgcn_sched_barrier(0);
-      });
-      c_slot ^= 1;
-    }
-    // the fragments read in this step become ordinary values before the loader may open a
-    // new tile (a register the compiler moved or spilled while its read was still in
-    // flight would lose the data)
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    pin_frags(f0);
-    rotate_scales(f0, c_slot);
-    issue_advance();
-  };
-
-#else
-  // ---- MX_MFMA16: fragment sets, scale dwords
+  // ---- fragment sets, scale dwords
   // one b128 read of a fragment set: i = 2t + (0: K bytes [16 lj, +16), 1: [64 + 16 lj, +16)) of
   // sub-tile 4h + t
   auto read_set_piece = [&](v8i (&set)[4], uint32_t sbase, uint32_t delta, auto h_, auto i_) {
@@ -1080,15 +853,14 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     issue_advance();
   };
 
-#endif  // MX_MFMA16
-  // Output: a lane holds, per 32x32 sub-tile, row li and columns 8q + 4lj + 0..3.  The two
-  // lanes of a row (lj = 0, 1) trade halves with v_permlane32_swap so that each owns 8
-  // consecutive bf16; a 32-row x 64-column piece is then turned around in this wave's private
-  // LDS patch (the 28 KB the ring leaves free) so that 8 lanes store one full 128-byte line of
-  // a row -- stores that scatter 32-byte pieces over 32 rows back up the write path.
+  // Output: a lane holds, per 16x16 sub-tile, row li and columns 4lj + 0..3.  Lanes of
+  // neighbouring lane groups trade halves with v_permlane16_swap so that each owns 8 consecutive
+  // bf16 of a row; a 32-row x 64-column piece is then turned around in this wave's private LDS
+  // patch (the 26 KB the ring leaves free) so that 8 lanes store one full 128-byte line of a row
+  // -- stores that scatter 32-byte pieces over many rows back up the write path.
   // Buffer stores: one descriptor per tile bounds the rows, a 32-bit offset per lane, scalar
   // offsets per piece.  Requires N % 8 == 0 and ldd % 8 == 0 (checked on the host).
-  // (LDS accesses as assembly, for the reason given at read_piece.)
+  // (LDS accesses as assembly, for the reason given at the fragment reads.)
   constexpr int kPatchPitch = 144;  // bytes per staged row: 128 + 16, keeps b128 accesses spread
   const uint32_t patch = lds_base + kRing32 + wave * kPatch32;
   const uint32_t nan_mask = (MODE != kDense && poison) ? 0x7FC07FC0u : 0u;
@@ -1099,12 +871,8 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     // flight (s_waitcnt vmcnt(0)) at exactly the two places where those should keep running.
     uint32_t lane_e = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
     asm volatile("" : "+v"(lane_e));
-#if MX_MFMA16
     // + (m & 1) * 16 rows + (second sub-tile pair of the piece) * 64
     const uint32_t patch_w = patch + (lane_e & 15) * kPatchPitch + ((lane_e >> 4) & 1) * 32 + (lane_e >> 5) * 16;
-#else
-    const uint32_t patch_w = patch + (lane_e & 31) * kPatchPitch + (lane_e >> 5) * 16;   // + (n&1)*64 + h*32
-#endif
     const uint32_t patch_r = patch + (lane_e >> 3) * kPatchPitch + (lane_e & 7) * 16;  // + pass*8 rows
     const int64_t rows_valid = t.rows_a;
     const uint32_t cols_valid = (uint32_t)(t.rows_b < kT32 ? t.rows_b : kT32);
@@ -1114,7 +882,6 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       const uint32_t ld_b = (uint32_t)p.ldd * 4;
       const __amdgpu_buffer_rsrc_t rp = make_rsrc(t.d, rows_valid * ld_b);
       const uint32_t row_b = (wm * 128 + li) * ld_b;
-#if MX_MFMA16
       // (a lane holds row 16m + li, columns 16n + 4lj + 0..3 of sub-tile (m, n))
       static_for<0, 64>([&](auto i_) {
         constexpr int m = decltype(i_)::value >> 3, n = decltype(i_)::value & 7;
@@ -1125,21 +892,6 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
         __builtin_amdgcn_raw_buffer_store_b128(w, rp, v, m * 16 * ld_b, MX_STORE_AUX);
       });
       return;
-#else
-      static_for<0, 16>([&](auto i_) {
-        constexpr int m = decltype(i_)::value >> 2, n = decltype(i_)::value & 3;
-        const v16f a = acc[m][n];
-        static_for<0, 4>([&](auto q_) {
-          constexpr int q = decltype(q_)::value;
-          const uint32_t col = wn * 128 + n * 32 + 8 * q + 4 * lj;
-          const uint32_t v = col < cols_valid ? row_b + col * 4 : 0x80000000u;
-          const u32x4 w = {__float_as_uint(a[4 * q + 0]), __float_as_uint(a[4 * q + 1]),
-                           __float_as_uint(a[4 * q + 2]), __float_as_uint(a[4 * q + 3])};
-          __builtin_amdgcn_raw_buffer_store_b128(w, rp, v, m * 32 * ld_b, MX_STORE_AUX);
-        });
-      });
-      return;
-#endif
     }
     const uint32_t ldd_b = (uint32_t)p.ldd * 2;
     const __amdgpu_buffer_rsrc_t rd = make_rsrc(t.d, rows_valid * ldd_b);
@@ -1150,8 +902,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     // A wave's LDS instructions execute in order, so a piece's reads may follow its writes
     // without a wait, and the next piece's writes may follow those reads: the only waits are
     // for the read data, with the next piece's conversion and writes already under way.
-#if MX_MFMA16
-    // MX_MFMA16: a lane holds row 16m + li, columns 16n + 4lj + 0..3 of sub-tile (m, n).  Part k of
+    // a lane holds row 16m + li, columns 16n + 4lj + 0..3 of sub-tile (m, n).  Part k of
     // piece p covers 16 rows x 32 columns: sub-tiles (m, n) and (m, n + 1), m = 2(p / 2) + k / 2,
     // n = 4(p % 2) + 2(k % 2).  v_permlane16_swap trades the halves of two neighbouring lane
     // groups: the even groups end up with 8 consecutive columns of sub-tile n, the odd ones with
@@ -1177,33 +928,6 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       lds_write_b128_hidden<(m & 1) * 16 * kPatchPitch + (k & 1) * 64>(patch_w, w);
       __builtin_amdgcn_sched_barrier(0);
     };
-#else
-    auto stage_part = [&](auto p_, auto k_) {  // 32 rows x 16 columns: accumulators -> bf16 -> patch
-      constexpr int m = decltype(p_)::value >> 1, np = decltype(p_)::value & 1;
-      constexpr int n = 2 * np + (decltype(k_)::value >> 1), h = decltype(k_)::value & 1;
-      // the eight accumulator registers of this part, read here and now (left to the compiler, the
-      // reads of the whole tile are gathered at the top of the epilogue: 180 registers at once)
-      const v16f& c = acc[m][n];
-      const float a[8] = {acc_read<8 * h + 0>(c), acc_read<8 * h + 1>(c), acc_read<8 * h + 2>(c),
-                          acc_read<8 * h + 3>(c), acc_read<8 * h + 4>(c), acc_read<8 * h + 5>(c),
-                          acc_read<8 * h + 6>(c), acc_read<8 * h + 7>(c)};
-      uint32_t x0 = pack_bf16(a[0], a[1]), y0 = pack_bf16(a[2], a[3]);
-      uint32_t x1 = pack_bf16(a[4], a[5]), y1 = pack_bf16(a[6], a[7]);
-      if constexpr (MODE != kDense) {  // a broken group contract must not pass unnoticed: NaN
-        x0 |= nan_mask;
-        y0 |= nan_mask;
-        x1 |= nan_mask;
-        y1 |= nan_mask;
-      }
-      const u32x2 sx = __builtin_amdgcn_permlane32_swap(x0, x1, false, false);
-      const u32x2 sy = __builtin_amdgcn_permlane32_swap(y0, y1, false, false);
-      const v4i w = {(int)sx.x, (int)sy.x, (int)sx.y, (int)sy.y};
-      lds_write_b128_hidden<(n & 1) * 64 + h * 32>(patch_w, w);
-      // keep a part's reads, conversion and write together: left free, the scheduler reads many
-      // accumulator blocks ahead and the epilogue spreads over registers the K loop's constants sit in
-      __builtin_amdgcn_sched_barrier(0);
-    };
-#endif
     v4i r[2][4];
     static_for<0, 4>([&](auto k_) { stage_part(std::integral_constant<int, 0>{}, k_); });
     static_for<0, 8>([&](auto p_) {
@@ -1245,7 +969,6 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __builtin_amdgcn_s_barrier();
   issue_block();  // block 1: in flight when the first step starts
-#if MX_MFMA16
   Frags16 f;
   {
     using Z = std::integral_constant<int, 0>;
@@ -1260,13 +983,6 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     pin_set(f.b[0]);
     next_scales(f, 0);
   }
-#else
-  Frags32 f0, f1;
-  read_frags(f0, 0, std::integral_constant<int, 0>{});
-  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-  pin_frags(f0);
-  rotate_scales(f0, 0);
-#endif
   if constexpr (PROF) prof_last = __builtin_readcyclecounter();
 
   // ---- tiles; at the top of every tile f0 holds the fragments of its first half block (the
@@ -1278,7 +994,6 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       // PAIR: the loader walks both segments of the tile one after the other (same K for both);
       // for the compute stream they are one run of blocks
       const uint32_t nblocks = PAIR ? 2 * t.nblocks : t.nblocks;
-#if MX_MFMA16
       block_steps(f, std::true_type{});
       // two blocks per trip: a taken branch stalls the lone wave of a SIMD for longer than the
       // 32 cycles its last MFMA covers, and the trip's end has two of them
@@ -1293,15 +1008,6 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       pin_set(f.a[0]);
       pin_set(f.a[1]);
-#else
-      block_steps(f0, f1, std::true_type{});
-      for (uint32_t i = 1; i < nblocks; ++i) block_steps(f0, f1, std::false_type{});
-      // the next tile's first fragments were read in the last step: make them ordinary
-      // values before anything else runs (a register the compiler moved or spilled while
-      // its read was still in flight would lose the data)
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-      pin_frags(f0);
-#endif
       if constexpr (PROF) {
         const uint64_t e0 = __builtin_readcyclecounter();
         prof_body += e0 - prof_last;

@@ -61,6 +61,63 @@ typedef int y_v8i __attribute__((ext_vector_type(8)));
 typedef float y_v16f __attribute__((ext_vector_type(16)));
 typedef float y_v4f __attribute__((ext_vector_type(4)));
 
+// The same 64 MFMAs per iteration (8 x 8 sub-tiles of 16x16x128) in a fixed order, as assembly so
+// that the order is what runs.  HOLD = how many MFMAs in a row share one operand fragment:
+//   8: sub-tile row i meets all eight columns in a row (a[i] stays, b changes)
+//   4: the order of the GEMM's K loop: four quarters a0 x b0, a1 x b0, a1 x b1, a0 x b1 over halves
+//      of four fragments, the held operand changing sides from quarter to quarter
+//   1: along diagonals, both fragments change with every MFMA
+template <int HOLD>
+__global__ __launch_bounds__(256) void mfma_order_kernel(const y_v8i* __restrict__ src, float* __restrict__ dst,
+                                                         int iters) {
+  const int lane = threadIdx.x;
+  y_v8i a[8], b[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    a[i] = src[i * 256 + lane];
+    b[i] = src[(8 + i) * 256 + lane];
+  }
+  const int sc = 0x7f7f7f7f;
+  y_v4f acc[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[i][j] = y_v4f{0.f, 0.f, 0.f, 0.f};
+  auto one = [&](int i, int j) {
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %3 op_sel:[0,0,0] op_sel_hi:[0,0,0]"
+                 : "+a"(acc[i][j])
+                 : "v"(b[j]), "v"(a[i]), "v"(sc));
+  };
+  for (int it = 0; it < iters; ++it) {
+    if constexpr (HOLD == 8) {
+#pragma unroll
+      for (int k = 0; k < 64; ++k) one(k >> 3, k & 7);
+    } else if constexpr (HOLD == 4) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int ah = (q == 1 || q == 2) ? 1 : 0, bh = q >= 2 ? 1 : 0;
+        const bool amajor = q == 0 || q == 3;
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+          const int tm = amajor ? k >> 2 : k & 3, tn = amajor ? k & 3 : k >> 2;
+          one(4 * ah + tm, 4 * bh + tn);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < 64; ++k) one(k & 7, ((k & 7) + (k >> 3)) & 7);
+    }
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s += acc[i][j][e];
+  dst[blockIdx.x * 256 + lane] = s;
+}
+
 template <int SHAPE>
 __global__ __launch_bounds__(256) void mfma_only_kernel(const y_v8i* __restrict__ src, float* __restrict__ dst,
                                                         int iters) {
@@ -123,6 +180,18 @@ __global__ __launch_bounds__(256) void mfma_only_kernel(const y_v8i* __restrict_
 
 extern "C" int mx_debug_mfma_only(int shape, const void* operands, void* out, int workgroups, int iters,
                                   void* stream) {
+  if (shape == 1601 || shape == 1604 || shape == 1608) {  // 16x16x128 in a fixed order, see mfma_order_kernel
+    if (!operands || !out || workgroups <= 0 || iters <= 0 || ((uintptr_t)operands & 31)) return MX_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const dim3 g((unsigned)workgroups), b(256);
+    if (shape == 1601)
+      hipLaunchKernelGGL(mx::mfma_order_kernel<1>, g, b, 0, st, (const mx::y_v8i*)operands, (float*)out, iters);
+    else if (shape == 1604)
+      hipLaunchKernelGGL(mx::mfma_order_kernel<4>, g, b, 0, st, (const mx::y_v8i*)operands, (float*)out, iters);
+    else
+      hipLaunchKernelGGL(mx::mfma_order_kernel<8>, g, b, 0, st, (const mx::y_v8i*)operands, (float*)out, iters);
+    return hipGetLastError() == hipSuccess ? MX_OK : MX_ERR_LAUNCH;
+  }
   if ((shape != 16 && shape != 32) || !operands || !out || workgroups <= 0 || iters <= 0 ||
       ((uintptr_t)operands & 31))
     return MX_ERR_INVALID_ARG;
