@@ -267,6 +267,25 @@ int mx_gemm_nt_pair(const uint8_t* a_codes, const uint8_t* a_scales, const uint8
                     const uint8_t* b2_codes, const uint8_t* b2_scales, void* d, int64_t M,
                     int64_t N, int64_t K, int64_t ldd, void* stream);
 
+/* Two products that share an operand, in one launch of the persistent kernel: the output tiles
+ * of the second product are numbered behind those of the first, so the panels of the shared
+ * operand are fetched once for both, and the launch's fixed cost is paid once.
+ *   mx_gemm_nt_shared_a:  D = deq(A) deq(B)^T  and  D2 = deq(A) deq(B2)^T   (B, B2 [N,K]; D, D2 [M,N])
+ *     h1 = x W1^T and h3 = x W3^T of a SwiGLU block (torchtitan/models/common/feed_forward.py:61-62)
+ *   mx_gemm_nt_shared_b:  D = deq(A) deq(B)^T  and  D2 = deq(A2) deq(B)^T   (A, A2 [M,K])
+ *     the weight gradients dW1 = d(h1)^T x and dW3 = d(h3)^T x of the same block (its autograd)
+ * Every tile is computed exactly as by mx_gemm_nt: results are bit-identical to two calls.
+ * Both outputs share ldd.  Shapes the persistent kernel does not take (as for mx_gemm_nt_pair)
+ * return MX_ERR_UNSUPPORTED: the caller then runs two mx_gemm_nt calls. */
+int mx_gemm_nt_shared_a(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                        const uint8_t* b_scales, const uint8_t* b2_codes, const uint8_t* b2_scales,
+                        void* d, void* d2, int64_t M, int64_t N, int64_t K, int64_t ldd,
+                        void* stream);
+int mx_gemm_nt_shared_b(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* a2_codes,
+                        const uint8_t* a2_scales, const uint8_t* b_codes, const uint8_t* b_scales,
+                        void* d, void* d2, int64_t M, int64_t N, int64_t K, int64_t ldd,
+                        void* stream);
+
 /* Grouped GEMM, 2D x 3D: for group g with rows [offs[g-1], offs[g]) of A:
  * D[rows, :] = deq(A[rows, :]) * deq(B[g])^T.  a_codes [T,K]; b_codes [G,N,K];
  * b_scales G consecutive MFMA-order blocks, each for [N, K/32].
@@ -276,7 +295,7 @@ int mx_gemm_nt_pair(const uint8_t* a_codes, const uint8_t* a_scales, const uint8
  *   MX_SCALES_MFMA      MFMA order over the whole [T, K/32] matrix; every group must end at a
  *                       multiple of 32 rows (the alignment of the reference's padded token
  *                       groups, torchtitan/components/quantization/__init__.py:36),
- *                       T % 32 == 0, K % 128 == 0, N % 8 == 0, G <= 510: the persistent
+ *                       T % 32 == 0, K % 128 == 0, N % 8 == 0, G <= 510: the
  *                       persistent kernel (several times faster).  The group ends live on the
  *                       device, so they are checked there: a violation fills D with NaN.
  * Stands in for torch._grouped_mm(x, w^T, offs) in forward and dgrad
@@ -310,6 +329,24 @@ int mx_grouped_gemm_2d2d(const uint8_t* at_codes, const uint8_t* at_scales,
                          const uint8_t* bt_codes, const uint8_t* bt_scales, const int32_t* offs,
                          void* d, int64_t T, int64_t N, int64_t K, int64_t G, int scale_order,
                          void* stream);
+
+/* The grouped forms of mx_gemm_nt_shared_a / _shared_b, MFMA-order scales and the contracts of
+ * the MX_SCALES_MFMA forms above only:
+ *   mx_grouped_gemm_2d3d_shared_a:  D = A x B[g]^T and D2 = A x B2[g]^T per group -- the experts'
+ *     h1 and h3 from one pass over the routed tokens (torchtitan/models/common/moe/moe.py:68-73)
+ *   mx_grouped_gemm_2d2d_shared_b:  D[g] = A^T B^T' and D2[g] = A2^T B^T' over the tokens of group g
+ *     -- dW1 and dW3 of the experts from one pass over the column-wise form of the routed tokens
+ * Bit-identical to two calls of the plain forms. */
+int mx_grouped_gemm_2d3d_shared_a(const uint8_t* a_codes, const uint8_t* a_scales,
+                                  const uint8_t* b_codes, const uint8_t* b_scales,
+                                  const uint8_t* b2_codes, const uint8_t* b2_scales,
+                                  const int32_t* offs, void* d, void* d2, int64_t T, int64_t N,
+                                  int64_t K, int64_t G, int64_t ldd, void* stream);
+int mx_grouped_gemm_2d2d_shared_b(const uint8_t* at_codes, const uint8_t* at_scales,
+                                  const uint8_t* at2_codes, const uint8_t* at2_scales,
+                                  const uint8_t* bt_codes, const uint8_t* bt_scales,
+                                  const int32_t* offs, void* d, void* d2, int64_t T, int64_t N,
+                                  int64_t K, int64_t G, void* stream);
 
 /* Token-group padding: from per-(rank, expert) counts build
  *   m_sizes[e]   = round_up(max(sum_r counts[r*E+e], alignment), alignment)   int32 [E]

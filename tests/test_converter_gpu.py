@@ -286,7 +286,8 @@ def test_per_op_checkpoint_policy_keeps_grouped_gemm_outputs(device, fuse, monke
                 y = checkpoint(ex, xi, counts, use_reentrant=False,
                                context_fn=lambda: create_selective_checkpoint_contexts(policy))
             y.backward(dy)
-            runs[how] = (launches.count("mx_grouped_gemm_2d3d"),
+            # grouped 2D x 3D products computed (the launch for h1 and h3 together computes two)
+            runs[how] = (launches.count("mx_grouped_gemm_2d3d") + 2 * launches.count("mx_grouped_gemm_2d3d_shared_a"),
                          [y.detach(), xi.grad, ex.w1.grad.clone(), ex.w2.grad.clone(), ex.w3.grad.clone()])
         # forward 3; backward: d(g), and d(x) as two launches or as one of the paired form
         base = 4 if fuse else 6

@@ -338,3 +338,42 @@ def test_pair_gemm_is_one_gemm_over_the_concatenated_contraction(device, M, N, K
     err = rel_l2(_f32(bits_of(got)), ref)
     two = ops.mx_gemm_nt(a, b) + ops.mx_gemm_nt(a2, b2)
     assert err <= TOL and err <= rel_l2(_f32(bits_of(two)), ref) + 1e-5, err
+
+
+def _launch_names(fn):
+    """(result of fn(), names of the C-ABI entry points it called)."""
+    names = []
+    real_call = ops._call
+    ops._call = lambda name, *rest: (names.append(name), real_call(name, *rest))[1]
+    try:
+        return fn(), names
+    finally:
+        ops._call = real_call
+
+
+@pytest.mark.parametrize("M,N,K", [(512, 384, 256), (300, 264, 128), (2304, 1280, 512), (1024, 4096, 1024)])
+def test_two_products_sharing_an_operand_equal_two_gemms(device, M, N, K):
+    """One launch for A B^T and A B2^T (and for A B^T and A2 B^T): every tile is computed as by
+    mx_gemm_nt, so both outputs equal the separate calls bit for bit; and against the oracle."""
+    rng = np.random.default_rng(7 * M + N + K)
+    q = lambda rows, std: ops.to_mx_dim0(bf16_from_bits(randn_bits(rng, (rows, K), std=std), device), "rceil",
+                                         ops.MX_SCALES_MFMA)
+    a, a2, b, b2 = q(M, 1.0), q(M, 0.3), q(N, 0.02), q(N, 0.05)
+    (d, d2), names = _launch_names(lambda: ops.mx_gemm_nt_shared_a(a, b, b2))
+    assert names == ["mx_gemm_nt_shared_a"]
+    assert torch.equal(d, ops.mx_gemm_nt(a, b)) and torch.equal(d2, ops.mx_gemm_nt(a, b2))
+    (e, e2), names = _launch_names(lambda: ops.mx_gemm_nt_shared_b(a, a2, b))
+    assert names == ["mx_gemm_nt_shared_b"]
+    assert torch.equal(e, d) and torch.equal(e2, ops.mx_gemm_nt(a2, b))
+    un = lambda t: ops.scale_unlayout(t.scales, t.codes.shape[0], K // 32).cpu().numpy()
+    ref = mo.mx_matmul_q(a2.codes.cpu().numpy(), un(a2), b.codes.cpu().numpy(), un(b))
+    assert rel_l2(_f32(bits_of(e2)), _f32(ref)) <= TOL
+
+
+def test_two_products_fall_back_to_two_gemms_on_small_shapes(device):
+    rng = np.random.default_rng(5)
+    q = lambda rows: ops.to_mx_dim0(bf16_from_bits(randn_bits(rng, (rows, 96)), device), "rceil", ops.MX_SCALES_MFMA)
+    a, b, b2 = q(64), q(40), q(40)
+    (d, d2), names = _launch_names(lambda: ops.mx_gemm_nt_shared_a(a, b, b2))
+    assert names == ["mx_gemm_nt", "mx_gemm_nt"]
+    assert torch.equal(d, ops.mx_gemm_nt(a, b)) and torch.equal(d2, ops.mx_gemm_nt(a, b2))

@@ -437,3 +437,52 @@ def test_grouped_pair_gemm_matches_the_oracle_over_the_concatenated_contraction(
                          np.cumsum(sizes), mo.RCEIL)
     assert rel_l2(_f32(bits_of(y)), _f32(ref)) <= TOL
     assert np.all(bits_of(y)[sum(sizes):] == 0)
+
+
+def _launch_names(fn):
+    names = []
+    real_call = ops._call
+    ops._call = lambda name, *rest: (names.append(name), real_call(name, *rest))[1]
+    try:
+        return fn(), names
+    finally:
+        ops._call = real_call
+
+
+@pytest.mark.parametrize("sizes,N,K,tail", [([256, 0, 128, 640], 256, 256, 128), ([96, 160, 32, 0, 416, 288], 264, 384, 0),
+                                            ([128] * 9 + [1024, 0, 384], 768, 512, 256)])
+def test_grouped_forward_of_two_weight_stacks_in_one_launch(device, sizes, N, K, tail):
+    """x against w1[g] and w3[g] in one launch of the persistent kernel: both outputs bit-identical
+    to the two separate grouped GEMMs (ragged 32-aligned groups, rows behind the last group zero)."""
+    rng = np.random.default_rng(sum(sizes) + N + K + 1)
+    T, G = sum(sizes) + tail, len(sizes)
+    offs = _sizes_to_offs(sizes, device)
+    xq = ops.to_mx_dim0(bf16_from_bits(randn_bits(rng, (T, K), outliers=1e-3), device), "rceil", L)
+    w1 = ops.to_mx_dim0_batched(bf16_from_bits(randn_bits(rng, (G, N, K), std=0.02), device), "rceil", L)
+    w3 = ops.to_mx_dim0_batched(bf16_from_bits(randn_bits(rng, (G, N, K), std=0.05), device), "rceil", L)
+    (h1, h3), names = _launch_names(lambda: ops.mx_grouped_gemm_2d3d_shared_a(xq, w1, w3, offs))
+    assert names == ["mx_grouped_gemm_2d3d_shared_a"]
+    assert torch.equal(h1, ops.mx_grouped_gemm_2d3d(xq, w1, offs))
+    assert torch.equal(h3, ops.mx_grouped_gemm_2d3d(xq, w3, offs))
+    assert not h1[sum(sizes):].any() and not h3[sum(sizes):].any()
+    # a broken group end poisons both outputs
+    bad = offs.clone()
+    bad[0] += 8
+    p1, p3 = ops.mx_grouped_gemm_2d3d_shared_a(xq, w1, w3, bad)
+    assert p1.isnan().all() and p3.isnan().all()
+
+
+@pytest.mark.parametrize("sizes,N,K", [([256, 0, 128, 640], 256, 256), ([96, 160, 32, 0, 416, 288], 264, 384),
+                                       ([32 * (1 + (7 * g) % 11) for g in range(40)], 768, 512)])
+def test_grouped_wgrads_of_two_gradients_in_one_launch(device, sizes, N, K):
+    """da^T x and db^T x per group in one launch: bit-identical to the two separate 2D x 2D GEMMs,
+    also with enough groups for the dealing of tiles by group length."""
+    rng = np.random.default_rng(sum(sizes) * 3 + N + K)
+    T = -(-(sum(sizes) + 128) // 128) * 128
+    offs = _sizes_to_offs(sizes, device)
+    col = lambda cols, std: ops.to_mx_dim1(bf16_from_bits(randn_bits(rng, (T, cols), std=std), device), "rceil", L)
+    da, db, x = col(N, 1e-3), col(N, 3e-3), col(K, 1.0)
+    (dw1, dw3), names = _launch_names(lambda: ops.mx_grouped_gemm_2d2d_shared_b(da, db, x, offs))
+    assert names == ["mx_grouped_gemm_2d2d_shared_b"]
+    assert torch.equal(dw1, ops.mx_grouped_gemm_2d2d(da, x, offs))
+    assert torch.equal(dw3, ops.mx_grouped_gemm_2d2d(db, x, offs))

@@ -51,6 +51,10 @@ SIGNATURES = {
     "mx_gemm_nt_static_max_bytes": (_I, []),
     "mx_gemm_nt_static": (c_int, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "mx_gemm_nt_pair": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
+    "mx_gemm_nt_shared_a": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
+    "mx_gemm_nt_shared_b": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
+    "mx_grouped_gemm_2d3d_shared_a": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
+    "mx_grouped_gemm_2d2d_shared_b": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "mx_grouped_gemm_2d3d_pair": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "mx_grouped_gemm_2d3d": (c_int, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, c_int, _P]),
     "mx_grouped_gemm_2d2d": (c_int, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, c_int, _P]),

@@ -83,7 +83,15 @@ struct Gemm32Args {
   const uint8_t* a2_scales = nullptr;
   const uint8_t* b2_codes = nullptr;
   const uint8_t* b2_scales = nullptr;
+  // Two products that share one operand in one launch (not with PAIR).  kTwoB: D = A B^T and
+  // D2 = A B2^T, the tile columns of the second product numbered behind those of the first
+  // (h1 = x W1^T and h3 = x W3^T of a SwiGLU block: every A panel is fetched for both).  kTwoA:
+  // D = A B^T and D2 = A2 B^T, the tile rows of the second behind those of the first (the weight
+  // gradients dW1 = d(h1)^T x and dW3 = d(h3)^T x).
+  int32_t two = 0;
+  uint16_t* d2 = nullptr;
 };
+enum Gemm32Two { kTwoNone = 0, kTwoB = 1, kTwoA = 2 };
 
 // Where one 256x256 tile lives.
 struct Tile32 {
@@ -182,7 +190,11 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void_t*)smem;  // LDS byte address of the ring
   const uint32_t K = (uint32_t)p.K;  // bytes per operand row; a multiple of 128 for this kernel
   const uint32_t ks_n = K / kK32;    // 64-deep steps per 128-row scale group
-  const uint32_t tiles_n = MODE == kDense ? (uint32_t)((p.N + kT32 - 1) / kT32) : (uint32_t)p.tn_cnt;
+  // tile rows / columns of one product, and of the launch (p.two: the second product's tile
+  // columns or rows come behind the first's; grouped launches cover columns [tn0, tn0 + tn_cnt))
+  const uint32_t tiles_n1 = (uint32_t)((p.N + kT32 - 1) / kT32), tiles_m1 = (uint32_t)((p.M + kT32 - 1) / kT32);
+  const uint32_t tiles_n = MODE == kDense ? (p.two == kTwoB ? 2 * tiles_n1 : tiles_n1) : (uint32_t)p.tn_cnt;
+  const uint32_t tiles_m = p.two == kTwoA ? 2 * tiles_m1 : tiles_m1;
   const uint32_t tn0 = MODE == kDense ? 0u : (uint32_t)p.tn0;
   const uint32_t G = (uint32_t)p.G;
 
@@ -205,11 +217,11 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     return *flag != 0;
   };
   if constexpr (MODE == kDense) {
-    nb = (uint32_t)((p.M + kT32 - 1) / kT32) * tiles_n;
+    nb = tiles_m * tiles_n;
   } else if constexpr (MODE == kSplitK) {
-    nb = G * (uint32_t)((p.M + kT32 - 1) / kT32) * tiles_n;
+    nb = G * tiles_m * tiles_n;
   } else if constexpr (MODE == kGrouped2d2d) {
-    nb = G * (uint32_t)((p.M + kT32 - 1) / kT32) * tiles_n;
+    nb = G * tiles_m * tiles_n;
     // group lengths in K blocks, kept for the dealing below (up to kMaxDealt groups)
     uint16_t* g_blocks = reinterpret_cast<uint16_t*>(smem + kRing32 + kPatchUsed);
     int bad = 0;
@@ -265,7 +277,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     }
     __syncthreads();
     nb = first[G + 1];
-    if (poison) nb = (uint32_t)((p.M + kT32 - 1) / kT32) * tiles_n;  // then: NaN over all of D
+    if (poison) nb = tiles_m * tiles_n;  // then: NaN over all of D
   }
 
   // ---- this workgroup's tile list: XCD x (= blockIdx % 8) owns one contiguous run of tiles,
@@ -286,7 +298,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   auto snake = [](uint32_t band, uint32_t k, uint32_t width) -> uint32_t {
     return (band & 1) ? width - 1 - k : k;
   };
-  const uint32_t per_g2 = (uint32_t)((p.M + kT32 - 1) / kT32) * tiles_n;  // tiles of one group
+  const uint32_t per_g2 = tiles_m * tiles_n;  // tiles of one group
   if (MODE == kGrouped2d2d && dealt) {
     const uint32_t full = G / 8, rest = G % 8;
     const uint32_t groups_x = full + (snake(full, xcd, 8) < rest ? 1 : 0);
@@ -312,14 +324,34 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     r.rot = 0;
     r.head = 0;
     r.tail = 0;
-    const uint8_t* const a_codes = (PAIR && seg) ? p.a2_codes : p.a_codes;
-    const uint8_t* const a_scales = (PAIR && seg) ? p.a2_scales : p.a_scales;
-    const uint8_t* const b_codes = (PAIR && seg) ? p.b2_codes : p.b_codes;
-    const uint8_t* const b_scales = (PAIR && seg) ? p.b2_scales : p.b_scales;
+    const uint8_t* a_codes = (PAIR && seg) ? p.a2_codes : p.a_codes;
+    const uint8_t* a_scales = (PAIR && seg) ? p.a2_scales : p.a_scales;
+    const uint8_t* b_codes = (PAIR && seg) ? p.b2_codes : p.b_codes;
+    const uint8_t* b_scales = (PAIR && seg) ? p.b2_scales : p.b_scales;
+    uint16_t* d_base = p.d;
+    // p.two: a tile column / row of the second product becomes that product's own, with its
+    // operand and output in place of the first's
+    auto second_product = [&](uint32_t& tm, uint32_t& tn) {
+      if constexpr (!PAIR && (MODE == kDense || MODE == kGrouped2d3d || MODE == kGrouped2d2d)) {
+        if (p.two == kTwoB && tn >= tiles_n1) {
+          tn -= tiles_n1;
+          b_codes = p.b2_codes;
+          b_scales = p.b2_scales;
+          d_base = p.d2;
+        }
+        if (p.two == kTwoA && tm >= tiles_m1) {
+          tm -= tiles_m1;
+          a_codes = p.a2_codes;
+          a_scales = p.a2_scales;
+          d_base = p.d2;
+        }
+      }
+    };
     uint32_t tm, tn;
     if (MODE == kDense || (MODE == kGrouped2d3d && poison)) {
-      tile_coords(t, (uint32_t)((p.M + kT32 - 1) / kT32), tiles_n, tm, tn);
+      tile_coords(t, tiles_m, tiles_n, tm, tn);
       tn += tn0;
+      second_product(tm, tn);
 #if defined(MX_ABL_SAME_PANEL)  // timing ablation: every 8 x 4 round reads the same twelve operand panels
       r.a = a_codes + (int64_t)(tm & 7) * kT32 * K;
       r.b = b_codes + (int64_t)(tn & 3) * kT32 * K;
@@ -335,7 +367,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
 #endif
       r.sa = a_scales + (int64_t)(tm * 2) * ks_n * 256;
       r.sb = b_scales + (int64_t)(tn * 2) * ks_n * 256;
-      r.d = p.d + (int64_t)tm * kT32 * p.ldd + (int64_t)tn * kT32;
+      r.d = d_base + (int64_t)tm * kT32 * p.ldd + (int64_t)tn * kT32;
       r.rows_a = p.M - (int64_t)tm * kT32;
       r.rows_b = p.N - (int64_t)tn * kT32;
       r.nblocks = poison ? 1 : K / kKB;
@@ -351,6 +383,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       const uint32_t tiles_mg = (uint32_t)((hi - lo + kT32 - 1) / kT32);
       tile_coords(t - first[g], tiles_mg, tiles_n, tm, tn);
       tn += tn0;
+      second_product(tm, tn);
       const int64_t row0 = lo + (int64_t)tm * kT32;
       const uint32_t gb = g < G ? g : 0;  // the zero rows have no expert: any valid address
       r.a = a_codes + row0 * K;
@@ -358,14 +391,14 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       r.sa = a_scales + (row0 >> 7) * ks_n * 256;
       r.rot = (uint32_t)(row0 >> 5) & 3;
       r.sb = b_scales + ((int64_t)gb * ((p.N + 127) >> 7) + tn * 2) * ks_n * 256;
-      r.d = p.d + row0 * p.ldd + (int64_t)tn * kT32;
+      r.d = d_base + row0 * p.ldd + (int64_t)tn * kT32;
       r.rows_a = hi - row0;
       r.rows_b = p.N - (int64_t)tn * kT32;
       r.nblocks = g < G ? K / kKB : 1;
       r.empty = g >= G;
     } else if (MODE == kSplitK) {
       // slice g of the K blocks: ceil(blocks / G) each, the host picks G so that none is empty
-      const uint32_t tiles_m = (uint32_t)((p.M + kT32 - 1) / kT32), per_g = tiles_m * tiles_n;
+      const uint32_t per_g = tiles_m * tiles_n;
       const uint32_t g = t / per_g;
       tile_coords(t - g * per_g, tiles_m, tiles_n, tm, tn);
       const uint32_t blocks = K / kKB, per = (blocks + G - 1) / G;
@@ -383,7 +416,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       r.koff = lo;
       r.nblocks = b_hi - b_lo;
     } else {
-      const uint32_t tiles_m = (uint32_t)((p.M + kT32 - 1) / kT32), per_g = tiles_m * tiles_n;
+      const uint32_t per_g = tiles_m * tiles_n;
       uint32_t g = t / per_g, in_g = t - g * per_g;
       if (dealt) {  // t counts this workgroup's tiles: the i-th tile it was dealt
         const uint16_t* g_sorted = reinterpret_cast<const uint16_t*>(smem + kRing32 + kPatchUsed) + kMaxDealt;
@@ -394,6 +427,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       }
       tile_coords(in_g, tiles_m, tiles_n, tm, tn);
       tn += tn0;
+      second_product(tm, tn);
       const int64_t lo = poison ? 0 : (g ? p.offs[g - 1] : 0), hi = poison ? 0 : p.offs[g];
       // the K blocks keep to multiples of 128 (whole cache lines per operand row: a copy that
       // straddles two lines costs the texture path twice); a range that starts or ends inside
@@ -403,7 +437,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       r.b = b_codes + (int64_t)tn * kT32 * K + lo128;
       r.sa = a_scales + ((int64_t)(tm * 2) * ks_n + (lo128 >> 6)) * 256;
       r.sb = b_scales + ((int64_t)(tn * 2) * ks_n + (lo128 >> 6)) * 256;
-      r.d = p.d + ((int64_t)g * p.M + (int64_t)tm * kT32) * p.ldd + (int64_t)tn * kT32;
+      r.d = d_base + ((int64_t)g * p.M + (int64_t)tm * kT32) * p.ldd + (int64_t)tn * kT32;
       r.rows_a = p.M - (int64_t)tm * kT32;
       r.rows_b = p.N - (int64_t)tn * kT32;
       r.koff = (uint32_t)lo128;
@@ -1212,6 +1246,51 @@ int launch_grouped32_2d3d(const uint8_t* a_codes, const uint8_t* a_scales, const
   Gemm32Args p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, T, N, K, ldd, offs, G, 0, 0, debug_prof};
   // an upper bound of the tile rows: every group may add one partly filled tile
   return launch_grouped32<kGrouped2d3d>(p, (T + kT32 - 1) / kT32 + G + 1, (N + kT32 - 1) / kT32, st);
+}
+
+// D = A B^T and D2 = A B2^T in one launch (same shapes), dense and grouped 2D x 3D.
+int launch_gemm_nt32_two_b(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                           const uint8_t* b_scales, const uint8_t* b2_codes, const uint8_t* b2_scales,
+                           void* d, void* d2, int64_t M, int64_t N, int64_t K, int64_t ldd, hipStream_t st) {
+  Gemm32Args p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, M, N, K, ldd, nullptr, 0, 0, 0, nullptr};
+  p.b2_codes = b2_codes;
+  p.b2_scales = b2_scales;
+  p.two = kTwoB;
+  p.d2 = (uint16_t*)d2;
+  return launch32<kDense, false>(p, ((M + kT32 - 1) / kT32) * 2 * ((N + kT32 - 1) / kT32), st);
+}
+int launch_grouped32_2d3d_two_b(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                                const uint8_t* b_scales, const uint8_t* b2_codes, const uint8_t* b2_scales,
+                                const int32_t* offs, void* d, void* d2, int64_t T, int64_t N, int64_t K,
+                                int64_t G, int64_t ldd, hipStream_t st) {
+  Gemm32Args p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, T, N, K, ldd, offs, G, 0, 0, nullptr};
+  p.b2_codes = b2_codes;
+  p.b2_scales = b2_scales;
+  p.two = kTwoB;
+  p.d2 = (uint16_t*)d2;
+  return launch_grouped32<kGrouped2d3d>(p, (T + kT32 - 1) / kT32 + G + 1, 2 * ((N + kT32 - 1) / kT32), st);
+}
+// D = A B^T and D2 = A2 B^T in one launch (same shapes), dense and grouped 2D x 2D.
+int launch_gemm_nt32_two_a(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* a2_codes,
+                           const uint8_t* a2_scales, const uint8_t* b_codes, const uint8_t* b_scales,
+                           void* d, void* d2, int64_t M, int64_t N, int64_t K, int64_t ldd, hipStream_t st) {
+  Gemm32Args p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, M, N, K, ldd, nullptr, 0, 0, 0, nullptr};
+  p.a2_codes = a2_codes;
+  p.a2_scales = a2_scales;
+  p.two = kTwoA;
+  p.d2 = (uint16_t*)d2;
+  return launch32<kDense, false>(p, 2 * ((M + kT32 - 1) / kT32) * ((N + kT32 - 1) / kT32), st);
+}
+int launch_grouped32_2d2d_two_a(const uint8_t* at_codes, const uint8_t* at_scales, const uint8_t* at2_codes,
+                                const uint8_t* at2_scales, const uint8_t* bt_codes, const uint8_t* bt_scales,
+                                const int32_t* offs, void* d, void* d2, int64_t T, int64_t N, int64_t K,
+                                int64_t G, hipStream_t st) {
+  Gemm32Args p{at_codes, at_scales, bt_codes, bt_scales, (uint16_t*)d, N, K, T, K, offs, G, 0, 0, nullptr};
+  p.a2_codes = at2_codes;
+  p.a2_scales = at2_scales;
+  p.two = kTwoA;
+  p.d2 = (uint16_t*)d2;
+  return launch_grouped32<kGrouped2d2d>(p, (G + 7) / 8 * 8 * 2 * ((N + kT32 - 1) / kT32), (K + kT32 - 1) / kT32, st);
 }
 
 // D = A B^T + A2 B2^T (dense) and its grouped 2D x 3D form: both operand sets of the same shapes.

@@ -134,8 +134,7 @@ class _MXFeedForward(torch.autograd.Function):
         w1q0, w1q1 = _cast_weight(w1, mode, need_dx, cfg)
         w3q0, w3q1 = _cast_weight(w3, mode, need_dx, cfg)
         w2q0, w2q1 = _cast_weight(w2, mode, need_dx or need_dw, cfg)
-        h1 = ops.mx_gemm_nt(xq0, w1q0)
-        h3 = ops.mx_gemm_nt(xq0, w3q0)
+        h1, h3 = ops.mx_gemm_nt_shared_a(xq0, w1q0, w3q0)  # one launch: x's panels fetched once
         gq0, gq1, _ = ops.swiglu_to_mx_dim0_dim1(h1, h3, mode, MX_SCALES_MFMA)
         y = ops.mx_gemm_nt(gq0, w2q0)
         ctx.cfg, ctx.x_shape = cfg, x.shape
@@ -172,12 +171,15 @@ class _MXFeedForward(torch.autograd.Function):
         if ctx.need_dw:
             xq1, gq1 = take(), take()
             cast_back = lambda g, dt: g if g.dtype == dt else g.to(dt)
-            if ctx.needs_input_grad[1]:
+            if ctx.needs_input_grad[1] and ctx.needs_input_grad[3]:
+                dw1, dw3 = ops.mx_gemm_nt_shared_b(da1, db1, xq1)  # one launch over x's column-wise form
+                dw1, dw3 = cast_back(dw1, ctx.w_dtypes[0]), cast_back(dw3, ctx.w_dtypes[2])
+            elif ctx.needs_input_grad[1]:
                 dw1 = cast_back(ops.mx_gemm_nt(da1, xq1), ctx.w_dtypes[0])
+            elif ctx.needs_input_grad[3]:
+                dw3 = cast_back(ops.mx_gemm_nt(db1, xq1), ctx.w_dtypes[2])
             if ctx.needs_input_grad[2]:
                 dw2 = cast_back(ops.mx_gemm_nt(dyq1, gq1), ctx.w_dtypes[1])
-            if ctx.needs_input_grad[3]:
-                dw3 = cast_back(ops.mx_gemm_nt(db1, xq1), ctx.w_dtypes[2])
         dnw = None
         if ctx.need_dx:
             w1q1, w3q1 = take(), take()
@@ -359,8 +361,7 @@ class _MXGroupedFeedForward(torch.autograd.Function):
         w1q0, w1q1 = _cast_weight(w1, mode, need_dx, cfg)
         w3q0, w3q1 = _cast_weight(w3, mode, need_dx, cfg)
         w2q0, w2q1 = _cast_weight(w2, mode, need_dx or need_dw, cfg)
-        h1 = ops.mx_grouped_gemm_2d3d(xq0, w1q0, offs_p)
-        h3 = ops.mx_grouped_gemm_2d3d(xq0, w3q0, offs_p)
+        h1, h3 = ops.mx_grouped_gemm_2d3d_shared_a(xq0, w1q0, w3q0, offs_p)  # one pass over the routed tokens
         gq0, gq1, _ = ops.swiglu_to_mx_dim0_dim1(h1, h3, mode, order)
         y = _grouped_2d3d_padded(gq0, w2q0, offs_p, back)
         ctx.cfg, ctx.order, ctx.padded, ctx.D = cfg, order, plan is not None, D
@@ -397,12 +398,15 @@ class _MXGroupedFeedForward(torch.autograd.Function):
         if ctx.need_dw:
             xq1 = MXData(saved.pop(0), saved.pop(0), order)
             gq1 = MXData(saved.pop(0), saved.pop(0), order)
-            if ctx.needs_input_grad[1]:
+            if ctx.needs_input_grad[1] and ctx.needs_input_grad[3]:
+                dw1, dw3 = ops.mx_grouped_gemm_2d2d_shared_b(da1, db1, xq1, offs_p)
+                dw1, dw3 = cast_back(dw1, ctx.dtypes[1]), cast_back(dw3, ctx.dtypes[3])
+            elif ctx.needs_input_grad[1]:
                 dw1 = cast_back(ops.mx_grouped_gemm_2d2d(da1, xq1, offs_p), ctx.dtypes[1])
+            elif ctx.needs_input_grad[3]:
+                dw3 = cast_back(ops.mx_grouped_gemm_2d2d(db1, xq1, offs_p), ctx.dtypes[3])
             if ctx.needs_input_grad[2]:
                 dw2 = cast_back(ops.mx_grouped_gemm_2d2d(dyq1, gq1, offs_p), ctx.dtypes[2])
-            if ctx.needs_input_grad[3]:
-                dw3 = cast_back(ops.mx_grouped_gemm_2d2d(db1, xq1, offs_p), ctx.dtypes[3])
         if ctx.need_dx:
             w1q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
             w3q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
@@ -487,8 +491,7 @@ class _MXRoutedExperts(torch.autograd.Function):
         w1q0, w1q1 = _cast_weight(w1, mode, need_dx or need_ds, cfg)
         w3q0, w3q1 = _cast_weight(w3, mode, need_dx or need_ds, cfg)
         w2q0, w2q1 = _cast_weight(w2, mode, need_dg, cfg)
-        h1 = ops.mx_grouped_gemm_2d3d(xq0, w1q0, offs_p)
-        h3 = ops.mx_grouped_gemm_2d3d(xq0, w3q0, offs_p)
+        h1, h3 = ops.mx_grouped_gemm_2d3d_shared_a(xq0, w1q0, w3q0, offs_p)  # one pass over the routed tokens
         gq0, gq1, _ = ops.swiglu_to_mx_dim0_dim1(h1, h3, mode, order)
         yp = ops.mx_grouped_gemm_2d3d(gq0, w2q0, offs_p)
         out = ops.moe_combine(yp, pos, None if score_before else scores)
@@ -527,12 +530,15 @@ class _MXRoutedExperts(torch.autograd.Function):
         if need_dw:
             xq1 = MXData(saved.pop(0), saved.pop(0), order)
             gq1 = MXData(saved.pop(0), saved.pop(0), order)
-            if ctx.needs_input_grad[2]:
+            if ctx.needs_input_grad[2] and ctx.needs_input_grad[4]:
+                dw1, dw3 = ops.mx_grouped_gemm_2d2d_shared_b(da1, db1, xq1, offs_p)
+                dw1, dw3 = cast_back(dw1, ctx.dtypes[2]), cast_back(dw3, ctx.dtypes[4])
+            elif ctx.needs_input_grad[2]:
                 dw1 = cast_back(ops.mx_grouped_gemm_2d2d(da1, xq1, offs_p), ctx.dtypes[2])
+            elif ctx.needs_input_grad[4]:
+                dw3 = cast_back(ops.mx_grouped_gemm_2d2d(db1, xq1, offs_p), ctx.dtypes[4])
             if ctx.needs_input_grad[3]:
                 dw2 = cast_back(ops.mx_grouped_gemm_2d2d(dyq1, gq1, offs_p), ctx.dtypes[3])
-            if ctx.needs_input_grad[4]:
-                dw3 = cast_back(ops.mx_grouped_gemm_2d2d(db1, xq1, offs_p), ctx.dtypes[4])
         if need_dx or need_ds:
             w1q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
             w3q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
