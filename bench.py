@@ -616,7 +616,7 @@ def time_decoder_block(dev, recipe):
             h = x + self.attention(x, rope, self.attention_norm)
             ff = self.feed_forward
             w = (ff.w1.weight, ff.w2.weight, ff.w3.weight)
-            if norm_fusable(h, self.ffn_norm.weight, w[0], w[2]) and feed_forward_fusable(h, *w):
+            if norm_fusable(h, self.ffn_norm.weight, w[0], w[2], for_feed_forward=True) and feed_forward_fusable(h, *w):
                 return h + mx_norm_feed_forward(h, self.ffn_norm.weight, self.ffn_norm.eps, *w)
             return h + ff(self.ffn_norm(h))
 
@@ -969,7 +969,40 @@ def time_moe_grouped(dev, recipe_mode):
         torch.cuda.synchronize()
         sec = s.elapsed_time(e) * 1e-3 / 8
         out[name] = {"us": round(sec * 1e6, 1), "TFLOP/s": round(flops / sec / 1e12, 1)}
-    del x, w, dy, xq0, xq1, dyq0, dyq1, wq0, wq1, y, dx, dw
+    # the block's pairs of products that share an operand, one launch each: h1 | h3 from one pass over
+    # the routed tokens, dW1 | dW3 from one pass over their column-wise form (two products per launch)
+    w3 = (torch.randn((E, hid, dim), generator=g, device=dev, dtype=torch.float32) * 0.02).to(torch.bfloat16)
+    w3q0 = ops.to_mx_dim0_batched(w3, recipe_mode, L)
+    db = (torch.randn((max_len, hid), generator=g, device=dev, dtype=torch.float32) * 1e-3).to(torch.bfloat16)
+    dbq1 = ops.to_mx_dim1(db, recipe_mode, L)
+    for name, fn in (("fwd_2d3d_two_weight_stacks", lambda: ops.mx_grouped_gemm_2d3d_shared_a(xq0, wq0, w3q0, offs)),
+                     ("wgrad_2d2d_two_gradients", lambda: ops.mx_grouped_gemm_2d2d_shared_b(dyq1, dbq1, xq1, offs))):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(8):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        sec = s.elapsed_time(e) * 1e-3 / 8
+        out[name] = {"us": round(sec * 1e6, 1), "TFLOP/s": round(2 * flops / sec / 1e12, 1), "products": 2}
+    # both bounds of every pass: the matrix peak, and the bytes a launch has to move (operand codes
+    # and scales once, output once) against HBM
+    pad_rows = max_len
+    byts = {"fwd_2d3d": pad_rows * dim * 33 / 32 + E * hid * dim * 33 / 32 + pad_rows * hid * 2,
+            "dgrad_2d3d": pad_rows * hid * 33 / 32 + E * hid * dim * 33 / 32 + pad_rows * dim * 2,
+            "wgrad_2d2d": pad_rows * (hid + dim) * 33 / 32 + E * hid * dim * 2}
+    byts["fwd_2d3d_two_weight_stacks"] = byts["fwd_2d3d"] + E * hid * dim * 33 / 32 + pad_rows * hid * 2
+    byts["wgrad_2d2d_two_gradients"] = byts["wgrad_2d2d"] + pad_rows * hid * 33 / 32 + E * hid * dim * 2
+    for name, b in byts.items():
+        sec = out[name]["us"] * 1e-6
+        out[name]["frac_of_mfma_peak"] = round(out[name]["TFLOP/s"] / PEAK_MXFP8_TFLOPS, 3)
+        out[name]["algorithmic_MB"] = round(b / 1e6, 1)
+        out[name]["GB/s"] = round(b / sec / 1e9, 1)
+        out[name]["frac_of_hbm_peak"] = round(b / sec / 1e9 / PEAK_HBM_GBPS, 3)
+    del x, w, dy, xq0, xq1, dyq0, dyq1, wq0, wq1, y, dx, dw, w3, w3q0, db, dbq1
     out["expert_block"] = time_expert_block(dev, recipe_mode, counts)
     out["moe_layer"] = time_moe_layer(dev, recipe_mode)
     return out
@@ -1247,6 +1280,11 @@ def main():
         torch.cuda.empty_cache()
         line["yardsticks"] = time_yardsticks(dev)
         _casts_against_streams(line["casts"], line["yardsticks"])
+        copy_gbps = line["yardsticks"].get("stream_copy", {}).get("GB/s")
+        if copy_gbps:  # the memory bound as this box's plain copy delivers it, same run
+            for v in line["moe_grouped_gemms"].values():
+                if isinstance(v, dict) and "GB/s" in v:
+                    v["frac_of_stream_copy"] = round(v["GB/s"] / copy_gbps, 3)
         same = line["yardsticks"].get("this_gemm_kernel_on_constant_operands", {})
         if "frac_of_peak" in same:
             line["roofline"]["frac_on_constant_operands"] = same["frac_of_peak"]

@@ -52,16 +52,42 @@ def _count_fwd(gm):
 def test_converted_linear_traces_as_one_operator():
     lin = Linear.Config(bias=True).build(in_features=64, out_features=96)
     lin.weight = wrap_parameter(lin.weight, MXFP8Config("rceil"))
-    gm = _trace(lin, torch.randn(2, 32, 64))
+    gm = _trace(lin, torch.randn(2, 32, 64, requires_grad=True))
     assert _count_fwd(gm) == 1
     assert F.linear not in _targets(gm) and torch._C._nn.linear not in _targets(gm)
     # the operator's first output is what the module returns (plus the bias add)
     node = next(n for n in gm.graph.nodes if n.target in _FWD)
-    assert node.args[2] == ops.SCALE_MODES["rceil"]
+    assert node.args[2] == ops.SCALE_MODES["rceil"] and node.args[3:5] == (True, True)
     y, xc, xs, wc, ws = node.meta["example_value"]
     assert y.shape == (2, 32, 96) and y.dtype == torch.bfloat16
     assert xc.shape == (64, 64) and wc.shape == (64, 96) and xc.dtype == torch.uint8
     assert xs.numel() == ops.mfma_scale_bytes(64, 2) and ws.numel() == ops.mfma_scale_bytes(64, 3)
+
+
+def test_traced_linear_leaves_out_the_casts_no_gradient_needs():
+    """An input that needs no gradient: no column-wise form of W is made or kept; under no_grad
+    none of x either."""
+    lin = Linear.Config(bias=False).build(in_features=64, out_features=96)
+    lin.weight = wrap_parameter(lin.weight, MXFP8Config("rceil"))
+    gm = _trace(lin, torch.randn(32, 64))
+    node = next(n for n in gm.graph.nodes if n.target in _FWD)
+    assert node.args[3:5] == (False, True)
+    _, xc, xs, wc, ws = node.meta["example_value"]
+    assert xc.shape == (64, 32) and wc.numel() == 0 and ws.numel() == 0
+
+    class NoGrad(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.lin = lin
+
+        def forward(self, x):
+            with torch.no_grad():
+                return self.lin(x)
+
+    gm = _trace(NoGrad(), torch.randn(32, 64))
+    node = next(n for n in gm.graph.nodes if n.target in _FWD)
+    assert node.args[3:5] == (False, False)
+    assert all(t.numel() == 0 for t in node.meta["example_value"][1:])
 
 
 def test_feed_forward_block_traces_as_three_operators():
@@ -142,6 +168,49 @@ def test_grouped_fake_kernels_give_the_static_shapes(T, K, N, G, pad):
         assert dx.shape == (T, K) and dw.numel() == 0
         with pytest.raises(Exception):
             torch.ops.torchtitan_amd.mx_grouped_mm_fwd(torch.empty(T, 40), torch.empty(G, N, 40), offs, 1, pad)
+
+
+def test_fused_block_fake_kernels_give_the_shapes_the_backward_takes():
+    """The fused block operators (feed-forward, expert block, routed experts): fake forward
+    outputs feed the fake backward, with and without the parts no gradient asks for."""
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    A = torch.ops.torchtitan_amd
+    with FakeTensorMode():
+        x, w1, w2 = torch.empty(2, 64, 128, dtype=torch.bfloat16), torch.empty(256, 128), torch.empty(128, 256)
+        out = A.mx_ffn_fwd(x, w1, w2, w1, None, 0.0, 1, False, True, True)
+        assert len(out) == 15 and out[0].shape == (2, 64, 128) and out[1].shape == (2, 128, 256)
+        assert out[4].shape == (128, 128) and out[8].shape == (128, 256)
+        dx, dw13, dw2, dnw = A.mx_ffn_bwd(torch.empty(2, 64, 128), list(out[1:]), None, None, 1, True, True, True, True, False)
+        assert dx.shape == (128, 128) and dw13.shape == (2, 256, 128) and dw2.shape == (128, 256) and dnw.numel() == 0
+        out = A.mx_ffn_fwd(x, w1, w2, w1, None, 0.0, 1, False, False, False)
+        assert all(t.numel() == 0 for t in out[1:])
+        nw = torch.empty(128, dtype=torch.bfloat16)
+        out = A.mx_ffn_fwd(x, w1, w2, w1, nw, 1e-5, 1, False, True, True)
+        assert out[13].shape == (128,) and out[12].numel() == 0 and out[14].numel() == 0
+        dx, _, _, dnw = A.mx_ffn_bwd(torch.empty(2, 64, 128), list(out[1:]), x, nw, 1, True, True, True, True, True)
+        assert dx.shape == (128, 128) and dnw.shape == (128,)
+        with pytest.raises(Exception):
+            A.mx_ffn_fwd(torch.empty(40, 128), w1, w2, w1, None, 0.0, 1, False, True, True)
+
+        T, D, H, G, k = 96, 128, 256, 4, 2
+        xg, e1, e2 = torch.empty(T, D, dtype=torch.bfloat16), torch.empty(G, H, D), torch.empty(G, D, H)
+        offs = torch.empty(G, dtype=torch.int32)
+        Tp = -(-(T + 32 * G) // 128) * 128
+        out = A.mx_grouped_ffn_fwd(xg, e1, e2, e1, offs, 1, True, False, True, True)
+        assert out[0].shape == (T, D) and out[2].shape == (Tp,) and out[3].shape == (T,) and out[4].shape == (2, Tp, H)
+        dx, dw13, dw2 = A.mx_grouped_ffn_bwd(torch.empty(T, D), list(out[1:]), 1, ops.MX_SCALES_MFMA, True, True, True, False)
+        assert dx.shape == (T, D) and dw13.shape == (1, G, H, D) and dw2.shape == (G, D, H)
+
+        scores, order, counts = torch.empty(T, k), torch.empty(T * k, dtype=torch.int64), torch.empty(G, dtype=torch.int64)
+        Tp = -(-(T * k + 32 * G) // 128) * 128
+        for before in (True, False):
+            out = A.mx_routed_experts_fwd(xg, scores, e1, e2, e1, order, counts, before, 1, False, True, True, True)
+            assert len(out) == 18 and out[0].shape == (T, D) and out[4].shape == (T, k) and out[6].shape == (2, Tp, H)
+            assert out[17].shape == ((0,) if before else (Tp, D))
+            dx, ds, dw13, dw2 = A.mx_routed_experts_bwd(torch.empty(T, D), list(out[1:]), xg if before else None, 1,
+                                                        ops.MX_SCALES_MFMA, before, True, True, True, True, True)
+            assert dx.shape == (T, D) and ds.shape == (T, k) and ds.dtype == torch.float32 and dw13.shape == (2, G, H, D)
 
 
 def test_operators_have_no_cpu_kernel():

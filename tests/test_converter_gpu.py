@@ -325,7 +325,7 @@ class _NormedBlock(nn.Module):
             q, k, v = a.wq(h), a.wk(h), a.wv(h)
         mixed = q + torch.cat((k, v), dim=-1)[..., : q.shape[-1]]      # stands in for attention
         w = (ff.w1.weight, ff.w2.weight, ff.w3.weight)
-        if norm_fusable(mixed, self.ffn_norm.weight, w[0], w[2]) and feed_forward_fusable(mixed, *w):
+        if norm_fusable(mixed, self.ffn_norm.weight, w[0], w[2], for_feed_forward=True) and feed_forward_fusable(mixed, *w):
             return mixed + mx_norm_feed_forward(mixed, self.ffn_norm.weight, self.ffn_norm.eps, *w)
         return mixed + ff(self.ffn_norm(mixed))
 
@@ -706,13 +706,14 @@ def test_decoder_block_with_all_seven_linears_converted(device):
             assert rel_l2(pa.grad.float().cpu().numpy(), pb.grad.float().cpu().numpy()) < 0.15, n
 
 
-def test_decoder_block_under_torch_compile_equals_eager(device):
+@pytest.mark.parametrize("fuse", [False, True])
+def test_decoder_block_under_torch_compile_equals_eager(device, fuse):
     """The block wrapped as the reference wraps its transformer blocks
     (torchtitan/models/llama3/parallelize.py:271-284: ``torch.compile(block, fullgraph=True)``):
-    every converted linear enters the graph as one opaque operator, forward and backward run
-    without a graph break, and output and all gradients equal the eager run bit for bit.  The
-    eager side runs with the gate fusion off, i.e. the same sequence of kernels; the backend
-    replays the traced graph op by op, so no code generator for the glue ops is involved."""
+    every converted linear -- with the gate fusion on, the whole SwiGLU block -- enters the graph
+    as one opaque operator, forward and backward run without a graph break, and output and all
+    gradients equal the eager run of the same configuration bit for bit.  The backend replays the
+    traced graph op by op, so no code generator for the glue ops is involved."""
     import torch._dynamo
 
     torch.manual_seed(17)
@@ -720,7 +721,7 @@ def test_decoder_block_under_torch_compile_equals_eager(device):
     for m in blk.modules():
         if isinstance(m, nn.Linear):
             nn.init.normal_(m.weight, std=0.02)
-    _convert(blk, ["attention", "feed_forward"], fuse=False)
+    _convert(blk, ["attention", "feed_forward"], fuse=fuse)
     x = torch.randn(2, 128, 256, device=device, dtype=torch.bfloat16)
     dy = torch.randn_like(x) * 1e-2
 
@@ -735,7 +736,15 @@ def test_decoder_block_under_torch_compile_equals_eager(device):
     want = run(blk)
     torch._dynamo.reset()
     compiled_blk = torch.compile(blk, backend="aot_eager", fullgraph=True)
-    got = run(compiled_blk)
+    launches = []
+    real_call = ops._call
+    ops._call = lambda name, *a: (launches.append(name), real_call(name, *a))[1]
+    try:
+        got = run(compiled_blk)
+    finally:
+        ops._call = real_call
+    # with the fusion on the compiled block runs the gate kernels, not separate silu / product ops
+    assert ("mx_swiglu_cast_dim0_dim1" in launches) == fuse and ("mx_swiglu_bwd_cast_dim0_dim1" in launches) == fuse
     again = run(compiled_blk)  # the second call reuses the compiled graph
     assert len(got) == len(want)
     for g, a, w in zip(got, again, want):
@@ -743,9 +752,10 @@ def test_decoder_block_under_torch_compile_equals_eager(device):
     torch._dynamo.reset()
 
 
+@pytest.mark.parametrize("fuse", [False, True])
 @pytest.mark.parametrize("pad,align", [(True, 8), (False, 32)])
 @pytest.mark.parametrize("dim,hidden", [(128, 256), (96, 160)])
-def test_grouped_experts_under_torch_compile_equal_eager(device, pad, align, dim, hidden):
+def test_grouped_experts_under_torch_compile_equal_eager(device, pad, align, dim, hidden, fuse):
     """The expert block compiled as one graph (the reference compiles MoE blocks as well): each
     converted grouped GEMM is one opaque operator that holds the padding plan, the casts and the
     grouped kernels of the eager path, so output and all gradients equal the eager run bit for
@@ -761,7 +771,7 @@ def test_grouped_experts_under_torch_compile_equal_eager(device, pad, align, dim
         ex.init_weights(init_std=0.05)
         holder = nn.Module()
         holder.experts = ex
-        _convert(holder, ["experts"], pad=pad, fuse=False)
+        _convert(holder, ["experts"], pad=pad, fuse=fuse)
         counts = torch.tensor([5, 0, 33, 64, 1, 41], device=device)
         x = torch.randn(int(counts.sum()), dim, device=device, dtype=torch.bfloat16)
         dy = torch.randn_like(x) * 1e-2
@@ -786,19 +796,22 @@ def test_grouped_experts_under_torch_compile_equal_eager(device, pad, align, dim
         torch._dynamo.reset()
 
 
-def test_moe_layer_under_torch_compile_equals_eager(device):
+@pytest.mark.parametrize("fuse", [False, True])
+@pytest.mark.parametrize("score_before", [True, False])
+def test_moe_layer_under_torch_compile_equals_eager(device, fuse, score_before):
     """Router, reordering, converted experts, shared experts and the combine as one compiled
-    graph without a break; bit-identical to the eager layer built from the same unfused ops."""
+    graph without a break; bit-identical to the eager layer of the same configuration (fused: the
+    routed half is one operator with gather, score multiply and combine inside its kernels)."""
     import torch._dynamo
 
     torch.manual_seed(29)
     cfg = MoE.Config(num_experts=8, num_shared_experts=1, top_k=2, hidden_dim=128,
-                     score_before_experts=True, score_func="softmax", route_norm=True)
+                     score_before_experts=score_before, score_func="softmax", route_norm=True)
     moe = MoE(cfg, dim=256).to(device).to(torch.bfloat16)
     moe.init_weights(init_std=0.05, buffer_device=device)
     holder = nn.Module()
     holder.moe = moe
-    _convert(holder, ["experts"], fuse=False)
+    _convert(holder, ["experts"], fuse=fuse)
     x = torch.randn(2, 96, 256, device=device, dtype=torch.bfloat16)
     dy = torch.randn_like(x)
 
@@ -819,6 +832,82 @@ def test_moe_layer_under_torch_compile_equals_eager(device):
         for g, w in zip(got, want):
             assert torch.equal(g, w)
     finally:
+        torch._dynamo.reset()
+
+
+def test_norm_inside_the_feed_forward_cast_under_torch_compile_equals_eager(device):
+    """RMSNorm + SwiGLU block with the norm inside the cast (opt-in), compiled as one graph: the
+    block is one operator whose backward also returns the norm weight's gradient; bit-identical
+    to the eager function."""
+    import torch._dynamo
+    from torchtitan_amd.mx_blocks import feed_forward_fusable, mx_norm_feed_forward, norm_fusable
+
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.feed_forward = FeedForward.Config(hidden_dim=512).build(dim=256)
+            self.ffn_norm = nn.RMSNorm(256, eps=1e-5)
+
+        def forward(self, x):
+            w = (self.feed_forward.w1.weight, self.feed_forward.w2.weight, self.feed_forward.w3.weight)
+            assert norm_fusable(x, self.ffn_norm.weight, w[0], w[2], for_feed_forward=True) and feed_forward_fusable(x, *w)
+            return x + mx_norm_feed_forward(x, self.ffn_norm.weight, self.ffn_norm.eps, *w)
+
+    torch.manual_seed(37)
+    blk = Block().to(device).to(torch.bfloat16)
+    for lin in (blk.feed_forward.w1, blk.feed_forward.w2, blk.feed_forward.w3):
+        nn.init.normal_(lin.weight, std=0.05)
+    with torch.no_grad():
+        blk.ffn_norm.weight.add_(0.1 * torch.randn_like(blk.ffn_norm.weight))
+    _convert(blk, ["feed_forward"], norm=True)
+    x = torch.randn(2, 64, 256, device=device, dtype=torch.bfloat16)
+    dy = torch.randn_like(x)
+
+    def run(fn):
+        for p in blk.parameters():
+            p.grad = None
+        xi = x.clone().requires_grad_(True)
+        y = fn(xi)
+        y.backward(dy)
+        return [y.detach().clone(), xi.grad.clone()] + [p.grad.clone() for p in blk.parameters()]
+
+    try:
+        want = run(blk)
+        torch._dynamo.reset()
+        got = run(torch.compile(blk, backend="aot_eager", fullgraph=True))
+        assert len(got) == len(want) == 2 + 4
+        for g, w in zip(got, want):
+            assert torch.equal(g, w)
+    finally:
+        torch._dynamo.reset()
+
+
+def test_compiled_block_without_gradients_runs_the_row_wise_casts_only(device):
+    """Under no_grad the traced operators leave the column-wise casts out (nothing is kept for a
+    backward) and the output equals the eager one."""
+    import torch._dynamo
+
+    torch.manual_seed(41)
+    ff = FeedForward.Config(hidden_dim=512).build(dim=256).to(device).to(torch.bfloat16)
+    for lin in (ff.w1, ff.w2, ff.w3):
+        nn.init.normal_(lin.weight, std=0.05)
+    holder = nn.Module()
+    holder.ff = ff
+    _convert(holder, ["ff"], fuse=False)
+    x = torch.randn(256, 256, device=device, dtype=torch.bfloat16)
+    launches = []
+    real_call = ops._call
+    try:
+        with torch.no_grad():
+            want = ff(x)
+            torch._dynamo.reset()
+            fn = torch.compile(ff, backend="aot_eager", fullgraph=True)
+            ops._call = lambda name, *a: (launches.append(name), real_call(name, *a))[1]
+            got = fn(x)
+        assert torch.equal(got, want)
+        assert launches.count("mx_cast_dim0") == 6 and "mx_cast_dim0_dim1" not in launches and "mx_cast_dim1" not in launches
+    finally:
+        ops._call = real_call
         torch._dynamo.reset()
 
 

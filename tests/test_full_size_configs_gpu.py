@@ -168,7 +168,7 @@ class _Block(nn.Module):
     def ffn(self, h):
         ff = self.feed_forward
         w = (ff.w1.weight, ff.w2.weight, ff.w3.weight)
-        if norm_fusable(h, self.ffn_norm.weight, w[0], w[2]) and feed_forward_fusable(h, *w):
+        if norm_fusable(h, self.ffn_norm.weight, w[0], w[2], for_feed_forward=True) and feed_forward_fusable(h, *w):
             return mx_norm_feed_forward(h, self.ffn_norm.weight, self.ffn_norm.eps, *w)
         return ff(self.ffn_norm(h))
 

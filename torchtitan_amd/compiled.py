@@ -8,8 +8,7 @@ The eager path of this package calls the HIP library through ``ctypes`` inside
 backward operator registered with ``torch.library`` (schemas, fake kernels for shape
 propagation, an autograd formula), whose bodies run the same casts and GEMMs as the eager
 functions.  A compiled block therefore holds the MXFP8 linears as single nodes with no graph
-break, and its results equal the eager ones bit for bit when the eager path runs the same
-unfused sequence (``fuse_swiglu_cast=False``; the fused block functions are eager-only).
+break, and its results equal the eager ones bit for bit.
 
 ``torch._grouped_mm`` on a converted 3-D weight traces the same way (the reference compiles MoE
 blocks too, torchtitan/models/llama4/parallelize.py ``apply_compile``): one forward and one
@@ -18,10 +17,15 @@ output shapes that depend on the static sizes only (the padded token axis is the
 round_up(T + 32 G), never the routed counts), and the index fill of the token-group padding
 wrapper is a third operator.
 
+The fused block functions (SwiGLU feed-forward block with the gate inside the casts, optionally
+with the RMSNorm in front of it; the expert block; the routed half of an MoE layer) are operators
+of the same kind further down: a compiled block runs the kernel sequence the eager path runs.
 What the traced form does not do: share one cast of an activation between sibling linears
-(w1 / w3, wq / wk / wv), fuse the SwiGLU gate or the RMSNorm into the casts, or reuse cached
-weight casts -- those stay eager features.  Dense shapes need tokens, in_features and
-out_features that are multiples of 32; grouped shapes need K and N multiples of 32.
+outside those blocks (wq / wk / wv), or fuse the RMSNorm in front of them (`mx_norm_linears`).
+Without gradients (``torch.no_grad()``, inputs that need none) the column-wise casts are left
+out; weights converted with ``cache_weight_casts`` take their casts from the cache.  Dense
+shapes need tokens, in_features and out_features that are multiples of 32; grouped shapes need
+K and N multiples of 32.
 """
 from __future__ import annotations
 
@@ -42,30 +46,42 @@ def _dims(x: torch.Tensor, weight: torch.Tensor):
 
 
 @torch.library.custom_op("torchtitan_amd::mx_linear_fwd", mutates_args=())
-def mx_linear_fwd(x: torch.Tensor, weight: torch.Tensor, mode: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+def mx_linear_fwd(x: torch.Tensor, weight: torch.Tensor, mode: int, need_dx: bool = True, need_dw: bool = True,
+                  cache_w: bool = False) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """y = x W^T in MXFP8 plus what the backward needs: the column-wise MXFP8 forms of x
-    (codes [K, M], MFMA-order scales) and of W (codes [K, N], MFMA-order scales)."""
+    (codes [K, M], MFMA-order scales; empty unless `need_dw`) and of W (codes [K, N], MFMA-order
+    scales; empty unless `need_dx`).  Without gradients only the row-wise casts run.  `cache_w`:
+    the weight's casts come from, and go to, the cache of unchanged weights."""
+    from .mx_tensor import _cast_weight
+
     M, K, N = _dims(x, weight)
     name = _MODE_NAMES[mode]
     x2 = x.reshape(M, K)
     if x2.dtype != torch.bfloat16:
         x2 = x2.to(torch.bfloat16)
-    w = (weight if weight.dtype == torch.bfloat16 else weight.to(torch.bfloat16)).contiguous()
-    xq0, xq1 = ops.to_mx_dim0_dim1(x2.contiguous(), name, MX_SCALES_MFMA)
-    wq0, wq1 = ops.to_mx_dim0_dim1(w, name, MX_SCALES_MFMA)
+    x2 = x2.contiguous()
+    if need_dw:
+        xq0, xq1 = ops.to_mx_dim0_dim1(x2, name, MX_SCALES_MFMA)
+    else:
+        xq0, xq1 = ops.to_mx_dim0(x2, name, MX_SCALES_MFMA), None
+    wq0, wq1 = _cast_weight(weight, name, need_dx, _block_cfg(mode, cache_w))
     y = ops.mx_gemm_nt(xq0, wq0).view(*x.shape[:-1], N)
-    return y, xq1.codes, xq1.scales, wq1.codes, wq1.scales
+    if cache_w and wq1 is not None:  # an operator's outputs are its own: not the cache's tensors
+        wq1 = MXData(wq1.codes.clone(), wq1.scales.clone(), MX_SCALES_MFMA)
+    e = lambda: _empty(x.device)
+    return (y, xq1.codes if need_dw else e(), xq1.scales if need_dw else e(),
+            wq1.codes if need_dx else e(), wq1.scales if need_dx else e())
 
 
 @mx_linear_fwd.register_fake
-def _(x, weight, mode):
+def _(x, weight, mode, need_dx=True, need_dw=True, cache_w=False):
     M, K, N = _dims(x, weight)
     torch._check(K % 32 == 0 and N % 32 == 0, lambda: "the traced MXFP8 linear needs in_features and out_features % 32 == 0")
     torch._check(M % 32 == 0, lambda: "the traced MXFP8 linear needs a multiple of 32 tokens")
-    u8 = dict(dtype=torch.uint8, device=x.device)
+    dev = x.device
     return (x.new_empty((*x.shape[:-1], N), dtype=torch.bfloat16),
-            torch.empty((K, M), **u8), torch.empty((ops.mfma_scale_bytes(K, M // 32),), **u8),
-            torch.empty((K, N), **u8), torch.empty((ops.mfma_scale_bytes(K, N // 32),), **u8))
+            _u8((K, M), dev) if need_dw else _empty(dev), _mfma(K, M // 32, dev) if need_dw else _empty(dev),
+            _u8((K, N), dev) if need_dx else _empty(dev), _mfma(K, N // 32, dev) if need_dx else _empty(dev))
 
 
 @torch.library.custom_op("torchtitan_amd::mx_linear_bwd", mutates_args=())
@@ -100,7 +116,7 @@ def _(dy, x_codes_t, x_scales_t, w_codes_t, w_scales_t, mode, need_dx, need_dw):
 
 
 def _setup_context(ctx, inputs, output):
-    x, weight, mode = inputs
+    x, weight, mode = inputs[:3]
     _, xc, xs, wc, ws = output
     ctx.save_for_backward(xc, xs, wc, ws)
     ctx.mode = mode
@@ -113,16 +129,19 @@ def _backward(ctx, gy, *unused):
     dx, dw = torch.ops.torchtitan_amd.mx_linear_bwd(gy, xc, xs, wc, ws, ctx.mode, need_dx, need_dw)
     gx = dx.view(ctx.x_shape).to(ctx.x_dtype) if need_dx else None
     gw = dw.to(ctx.w_dtype) if need_dw else None
-    return gx, gw, None
+    return gx, gw, None, None, None, None
 
 
 mx_linear_fwd.register_autograd(_backward, setup_context=_setup_context)
 
 
-def mx_linear_traced(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, scale_mode: str):
+def mx_linear_traced(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, scale_mode: str,
+                     cache_w: bool = False):
     """``F.linear`` on a converted weight while a graph is being traced.  `weight` and `bias` may
     still be the wrapper subclass: the caller has switched its ``__torch_function__`` off."""
-    y = torch.ops.torchtitan_amd.mx_linear_fwd(x, weight, ops.SCALE_MODES[scale_mode])[0]
+    grads = torch.is_grad_enabled()
+    y = torch.ops.torchtitan_amd.mx_linear_fwd(x, weight, ops.SCALE_MODES[scale_mode], grads and x.requires_grad,
+                                               grads and weight.requires_grad, cache_w)[0]
     if y.dtype != x.dtype:
         y = y.to(x.dtype)
     if bias is not None:
@@ -264,3 +283,393 @@ def _(counts, experts_per_rank, num_ranks, max_len, alignment):
     i32 = dict(dtype=torch.int32, device=counts.device)
     return (torch.empty((max_len,), dtype=torch.int64, device=counts.device),
             torch.empty((experts_per_rank,), **i32), torch.empty((experts_per_rank,), **i32))
+
+
+# ----------------------------------------------------------------------------- fused blocks
+# The SwiGLU feed-forward block, the expert block and the routed half of an MoE layer as single
+# operators: their bodies are the very functions the eager autograd functions run
+# (mx_blocks.ffn_forward / ffn_backward and their grouped and routed counterparts), so a compiled
+# block keeps the eager kernel sequence -- one cast of x for w1 and w3, the gate and its backward
+# inside the casts, the gather, score multiply and combine of the routed tokens inside theirs,
+# cached weight casts -- and equals it bit for bit.  A forward operator returns its output
+# followed by a fixed number of tensors for the backward, empty where the eager function keeps
+# nothing; tensors that are inputs (x, the norm weight) are kept by the autograd wrapper itself,
+# since an operator's outputs may not alias its inputs.
+def _empty(dev):
+    return torch.empty((0,), dtype=torch.uint8, device=dev)
+
+
+def _filled(saved, dev, skip=()):
+    return [(_empty(dev) if (t is None or i in skip) else t) for i, t in enumerate(saved)]
+
+
+def _restored(saved):
+    return [(t if t.numel() else None) for t in saved]
+
+
+def _block_cfg(mode: int, cache_w: bool, pad: bool = True):
+    from .mx_tensor import MXFP8Config
+
+    return MXFP8Config(scale_mode=_MODE_NAMES[mode], pad_token_groups_for_grouped_mm=pad, cache_weight_casts=cache_w)
+
+
+def _pack_pair(g1, g3, dev):
+    """dW1 and dW3 as ONE operator output (the two halves of one launch's output share their
+    storage, and an operator's outputs may not alias each other): [2, ...] when both exist,
+    [1, ...] for one, empty for none."""
+    if g1 is not None and g3 is not None:
+        base = g1._base
+        if base is not None and base is g3._base and base.shape[0] == 2:
+            return base
+        return torch.stack((g1, g3))
+    one = g1 if g1 is not None else g3
+    return one.unsqueeze(0) if one is not None else torch.empty((0,), dtype=torch.bfloat16, device=dev)
+
+
+def _unpack_pair(pack, need1: bool, need3: bool):
+    if need1 and need3:
+        return pack[0], pack[1]
+    return (pack[0] if need1 else None), (pack[0] if need3 else None)
+
+
+def _pair_shape(shape, need1: bool, need3: bool):
+    n = int(need1) + int(need3)
+    return (n, *shape) if n else (0,)
+
+
+def _u8(shape, dev):
+    return torch.empty(shape, dtype=torch.uint8, device=dev)
+
+
+def _mfma(rows: int, nblk: int, dev):
+    return _u8((ops.mfma_scale_bytes(rows, nblk),), dev)
+
+
+_T3 = tuple[(torch.Tensor,) * 3]
+_T4 = tuple[(torch.Tensor,) * 4]
+_T5 = tuple[(torch.Tensor,) * 5]
+_T15 = tuple[(torch.Tensor,) * 15]
+_T18 = tuple[(torch.Tensor,) * 18]
+
+
+@torch.library.custom_op("torchtitan_amd::mx_ffn_fwd", mutates_args=())
+def mx_ffn_fwd(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, w3: torch.Tensor, norm_weight: torch.Tensor | None,
+               eps: float, mode: int, cache_w: bool, need_dx: bool, need_dw: bool) -> _T15:
+    """(y, 14 tensors for the backward) of the SwiGLU block w2(silu(w1 x) * w3 x), RMSNorm in front
+    when `norm_weight` is given."""
+    from . import mx_blocks
+
+    D = x.shape[-1]
+    x2 = x.reshape(-1, D)
+    if x2.dtype != torch.bfloat16:
+        x2 = x2.to(torch.bfloat16)
+    y, saved = mx_blocks.ffn_forward(x2, None, w1, w2, w3, _block_cfg(mode, cache_w), need_dx, need_dw, norm_weight, eps)
+    return (y.view(*x.shape[:-1], w2.shape[0]), *_filled(saved, x.device, skip=(11, 13)))
+
+
+@mx_ffn_fwd.register_fake
+def _(x, w1, w2, w3, norm_weight, eps, mode, cache_w, need_dx, need_dw):
+    D, H, O = x.shape[-1], w1.shape[0], w2.shape[0]
+    M = x.numel() // D
+    torch._check(D % 32 == 0 and H % 32 == 0 and O % 32 == 0 and M % 32 == 0,
+                 lambda: "the traced SwiGLU block needs tokens and sizes that are multiples of 32")
+    dev = x.device
+    s = [_empty(dev) for _ in range(14)]
+    if need_dx or need_dw:
+        s[0:3] = [torch.empty((2, M, H), dtype=torch.bfloat16, device=dev), _u8((H, O), dev), _mfma(H, O // 32, dev)]
+    if need_dw:
+        s[3:7] = [_u8((D, M), dev), _mfma(D, M // 32, dev), _u8((H, M), dev), _mfma(H, M // 32, dev)]
+    if need_dx:
+        s[7:11] = [_u8((D, H), dev), _mfma(D, H // 32, dev), _u8((D, H), dev), _mfma(D, H // 32, dev)]
+        if norm_weight is not None:
+            s[12] = torch.empty((M,), dtype=torch.float32, device=dev)
+    return (x.new_empty((*x.shape[:-1], O), dtype=torch.bfloat16), *s)
+
+
+@torch.library.custom_op("torchtitan_amd::mx_ffn_bwd", mutates_args=())
+def mx_ffn_bwd(dy: torch.Tensor, saved: list[torch.Tensor], x: torch.Tensor | None, norm_weight: torch.Tensor | None,
+               mode: int, need_x: bool, need_dw1: bool, need_dw2: bool, need_dw3: bool, need_dnw: bool) -> _T4:
+    """(dx [M, in], dW1 and dW3 stacked, dW2, d norm weight) in bf16, empty where not asked for."""
+    from . import mx_blocks
+
+    s = _restored(saved)
+    if norm_weight is not None:
+        s[11], s[13] = x.reshape(-1, x.shape[-1]).contiguous(), norm_weight
+    dy2 = dy.reshape(-1, dy.shape[-1])
+    if dy2.dtype != torch.bfloat16:
+        dy2 = dy2.to(torch.bfloat16)
+    dx, dw1, dw2, dw3, dnw = mx_blocks.ffn_backward(dy2.contiguous(), s, _block_cfg(mode, False), need_x, need_dw1,
+                                                    need_dw2, need_dw3, need_dnw)
+    none = lambda: torch.empty((0,), dtype=torch.bfloat16, device=dy.device)
+    return (dx if (dx is not None and need_x) else none(), _pack_pair(dw1, dw3, dy.device),
+            dw2 if dw2 is not None else none(), dnw if dnw is not None else none())
+
+
+@mx_ffn_bwd.register_fake
+def _(dy, saved, x, norm_weight, mode, need_x, need_dw1, need_dw2, need_dw3, need_dnw):
+    dev = dy.device
+    bf = lambda shape, on: torch.empty(shape if on else (0,), dtype=torch.bfloat16, device=dev)
+    M = dy.numel() // dy.shape[-1]
+    H = saved[0].shape[2]
+    D = saved[7].shape[0] if saved[7].numel() else (saved[3].shape[0] if saved[3].numel() else 0)
+    O = dy.shape[-1]
+    dx = bf((M, D), need_x)
+    if norm_weight is not None and need_x:
+        dx = torch.empty((M, D), dtype=x.dtype, device=dev)
+    dnw = torch.empty(norm_weight.shape if (norm_weight is not None and need_dnw) else (0,),
+                      dtype=norm_weight.dtype if norm_weight is not None else torch.bfloat16, device=dev)
+    return (dx, bf(_pair_shape((H, D), need_dw1, need_dw3), True), bf((O, H), need_dw2), dnw)
+
+
+def _ffn_setup(ctx, inputs, output):
+    x, w1, w2, w3, norm_weight, eps, mode, cache_w, need_dx, need_dw = inputs
+    ctx.normed = norm_weight is not None
+    ctx.save_for_backward(*output[1:], *((x, norm_weight) if ctx.normed else ()))
+    ctx.mode, ctx.x_shape = mode, x.shape
+    ctx.dtypes = (x.dtype, w1.dtype, w2.dtype, w3.dtype)
+
+
+def _ffn_backward(ctx, gy, *unused):
+    saved = list(ctx.saved_tensors)
+    x, nw = (saved[14], saved[15]) if ctx.normed else (None, None)
+    need = ctx.needs_input_grad
+    dx, dw13, dw2, dnw = torch.ops.torchtitan_amd.mx_ffn_bwd(gy, saved[:14], x, nw, ctx.mode, need[0], need[1],
+                                                           need[2], need[3], bool(ctx.normed and need[4]))
+    dw1, dw3 = _unpack_pair(dw13, need[1], need[3])
+    back = lambda g, on, dt: g.to(dt) if on else None
+    return (back(dx, need[0], ctx.dtypes[0]).view(ctx.x_shape) if need[0] else None, back(dw1, need[1], ctx.dtypes[1]),
+            back(dw2, need[2], ctx.dtypes[2]), back(dw3, need[3], ctx.dtypes[3]),
+            (dnw if (ctx.normed and need[4]) else None), None, None, None, None, None)
+
+
+mx_ffn_fwd.register_autograd(_ffn_backward, setup_context=_ffn_setup)
+
+
+def _wants_grad(*tensors) -> bool:
+    return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
+
+
+def mx_feed_forward_traced(x, w1, w2, w3, bias2, norm_weight=None, eps: float = 0.0):
+    """The fused SwiGLU block while a graph is being traced; the weights may still be the wrapper
+    subclass (the caller has switched its ``__torch_function__`` off)."""
+    cfg = w2.mx_config
+    need_dx = _wants_grad(x, norm_weight)
+    need_dw = _wants_grad(w1, w2, w3)
+    y = torch.ops.torchtitan_amd.mx_ffn_fwd(x, w1, w2, w3, norm_weight, float(eps), ops.SCALE_MODES[cfg.scale_mode],
+                                            cfg.cache_weight_casts, need_dx, need_dw)[0]
+    if bias2 is not None:
+        y = y + bias2.to(y.dtype)
+    return y
+
+
+# ---- the expert block
+@torch.library.custom_op("torchtitan_amd::mx_grouped_ffn_fwd", mutates_args=())
+def mx_grouped_ffn_fwd(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, w3: torch.Tensor, offs: torch.Tensor,
+                       mode: int, pad: bool, cache_w: bool, need_dx: bool, need_dw: bool) -> _T15:
+    """(y [T, D] bf16, 14 tensors for the backward) of grouped_mm(silu(grouped_mm(x, w1)) * grouped_mm(x, w3), w2)."""
+    from . import mx_blocks
+
+    xb = x if x.dtype == torch.bfloat16 else x.to(torch.bfloat16)
+    y, saved = mx_blocks.grouped_ffn_forward(xb, w1, w2, w3, offs, _block_cfg(mode, cache_w, pad), need_dx, need_dw)
+    if saved[0] is offs:
+        saved[0] = offs.clone()
+    return (y, *_filled(saved, x.device))
+
+
+def _grouped_ffn_sizes(T, D, H, G, pad):
+    from . import mx_blocks
+
+    order, multiple, fast = mx_blocks.grouped_layout(D, H, G)
+    padded = pad or fast
+    step = max(ops.BLOCK, multiple)
+    Tp = -(-(T + ops.BLOCK * G) // step) * step if padded else T
+    return order, padded, Tp
+
+
+@mx_grouped_ffn_fwd.register_fake
+def _(x, w1, w2, w3, offs, mode, pad, cache_w, need_dx, need_dw):
+    T, D = x.shape
+    G, H, _ = w1.shape
+    torch._check(D % 32 == 0 and H % 32 == 0, lambda: "the traced expert block needs sizes that are multiples of 32")
+    order, padded, Tp = _grouped_ffn_sizes(T, D, H, G, pad)
+    dev = x.device
+    s = [_empty(dev) for _ in range(14)]
+    s[0] = torch.empty((G,), dtype=torch.int32, device=dev)
+    if padded:
+        s[1] = torch.empty((Tp,), dtype=torch.int64, device=dev)
+        s[2] = torch.empty((T,), dtype=torch.int64, device=dev)
+    if need_dx or need_dw:
+        s[3:6] = [torch.empty((2, Tp, H), dtype=torch.bfloat16, device=dev), _u8((G, H, D), dev),
+                  _u8((G * ops.mfma_scale_bytes(H, D // 32),), dev)]
+    if need_dw:
+        s[6:10] = [_u8((D, Tp), dev), _fake_scales(D, Tp // 32, order, dev), _u8((H, Tp), dev),
+                   _fake_scales(H, Tp // 32, order, dev)]
+    if need_dx:
+        wq = lambda: [_u8((G, D, H), dev), _u8((G * ops.mfma_scale_bytes(D, H // 32),), dev)]
+        s[10:14] = wq() + wq()
+    return (torch.empty((T, D), dtype=torch.bfloat16, device=dev), *s)
+
+
+@torch.library.custom_op("torchtitan_amd::mx_grouped_ffn_bwd", mutates_args=())
+def mx_grouped_ffn_bwd(dy: torch.Tensor, saved: list[torch.Tensor], mode: int, order: int, need_dx: bool, need_dw1: bool,
+                       need_dw2: bool, need_dw3: bool) -> _T3:
+    """(dx [T, D], dW1 and dW3 stacked, dW2) in bf16, empty where not asked for."""
+    from . import mx_blocks
+
+    dyb = (dy if dy.dtype == torch.bfloat16 else dy.to(torch.bfloat16)).contiguous()
+    dx, dw1, dw2, dw3 = mx_blocks.grouped_ffn_backward(dyb, _restored(saved), _block_cfg(mode, False), order, need_dx,
+                                                       need_dw1, need_dw2, need_dw3)
+    none = lambda: torch.empty((0,), dtype=torch.bfloat16, device=dy.device)
+    return (dx if dx is not None else none(), _pack_pair(dw1, dw3, dy.device), dw2 if dw2 is not None else none())
+
+
+@mx_grouped_ffn_bwd.register_fake
+def _(dy, saved, mode, order, need_dx, need_dw1, need_dw2, need_dw3):
+    dev = dy.device
+    bf = lambda shape, on: torch.empty(shape if on else (0,), dtype=torch.bfloat16, device=dev)
+    T, D = dy.shape
+    G, H = saved[4].shape[0], saved[4].shape[1]
+    return (bf((T, D), need_dx), bf(_pair_shape((G, H, D), need_dw1, need_dw3), True), bf((G, D, H), need_dw2))
+
+
+def _grouped_ffn_setup(ctx, inputs, output):
+    x, w1, w2, w3, offs, mode, pad, cache_w, need_dx, need_dw = inputs
+    ctx.save_for_backward(*output[1:])
+    ctx.mode = mode
+    ctx.order = _grouped_ffn_sizes(x.shape[0], x.shape[1], w1.shape[1], w1.shape[0], pad)[0]
+    ctx.dtypes = (x.dtype, w1.dtype, w2.dtype, w3.dtype)
+
+
+def _grouped_ffn_backward(ctx, gy, *unused):
+    need = ctx.needs_input_grad
+    dx, dw13, dw2 = torch.ops.torchtitan_amd.mx_grouped_ffn_bwd(gy, list(ctx.saved_tensors), ctx.mode, ctx.order, need[0],
+                                                              need[1], need[2], need[3])
+    dw1, dw3 = _unpack_pair(dw13, need[1], need[3])
+    grads = (dx, dw1, dw2, dw3)
+    return (*(g.to(dt) if on else None for g, dt, on in zip(grads, ctx.dtypes, need[:4])), None, None, None, None, None, None)
+
+
+mx_grouped_ffn_fwd.register_autograd(_grouped_ffn_backward, setup_context=_grouped_ffn_setup)
+
+
+def mx_grouped_feed_forward_traced(x, w1, w2, w3, offs):
+    """The fused expert block while a graph is being traced (weights as for the dense block)."""
+    cfg = w2.mx_config
+    return torch.ops.torchtitan_amd.mx_grouped_ffn_fwd(
+        x, w1, w2, w3, offs.to(torch.int32), ops.SCALE_MODES[cfg.scale_mode], cfg.pad_token_groups_for_grouped_mm,
+        cfg.cache_weight_casts, _wants_grad(x), _wants_grad(w1, w2, w3))[0]
+
+
+# ---- the routed half of an MoE layer
+@torch.library.custom_op("torchtitan_amd::mx_routed_experts_fwd", mutates_args=())
+def mx_routed_experts_fwd(x: torch.Tensor, top_scores: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, w3: torch.Tensor,
+                          tok_sorted: torch.Tensor, counts: torch.Tensor, score_before: bool, mode: int, cache_w: bool,
+                          need_dx: bool, need_ds: bool, need_dw: bool) -> _T18:
+    """(out [T, D] bf16, 17 tensors for the backward) of the routed experts with gather, score
+    multiply and combine inside the cast / combine kernels."""
+    from . import mx_blocks
+
+    xb = (x if x.dtype == torch.bfloat16 else x.to(torch.bfloat16)).contiguous()
+    out, saved = mx_blocks.routed_forward(xb, top_scores, w1, w2, w3, tok_sorted, counts, score_before,
+                                          _block_cfg(mode, cache_w), need_dx, need_ds, need_dw)
+    if saved[4].data_ptr() == top_scores.data_ptr():
+        saved[4] = saved[4].clone()
+    skip = (16,) if score_before else ()  # x itself: kept by the autograd wrapper
+    return (out, *_filled(saved, x.device, skip=skip))
+
+
+@mx_routed_experts_fwd.register_fake
+def _(x, top_scores, w1, w2, w3, tok_sorted, counts, score_before, mode, cache_w, need_dx, need_ds, need_dw):
+    from . import mx_blocks
+
+    T, D = x.shape
+    k = top_scores.shape[1]
+    G, H, _ = w1.shape
+    torch._check(D % 32 == 0 and H % 32 == 0, lambda: "the traced routed experts need sizes that are multiples of 32")
+    order, multiple, _ = mx_blocks.grouped_layout(D, H, G)
+    step = max(ops.BLOCK, multiple)
+    Tp = -(-(T * k + ops.BLOCK * G) // step) * step
+    dev = x.device
+    s = [_empty(dev) for _ in range(17)]
+    s[0] = torch.empty((G,), dtype=torch.int32, device=dev)
+    s[1] = torch.empty((Tp,), dtype=torch.int64, device=dev)
+    s[2] = torch.empty((Tp,), dtype=torch.float32, device=dev)
+    s[3] = torch.empty((T, k), dtype=torch.int64, device=dev)
+    s[4] = torch.empty((T, k), dtype=torch.float32, device=dev)
+    if need_dx or need_ds or need_dw:
+        s[5:8] = [torch.empty((2, Tp, H), dtype=torch.bfloat16, device=dev), _u8((G, H, D), dev),
+                  _u8((G * ops.mfma_scale_bytes(H, D // 32),), dev)]
+    if need_dw:
+        s[8:12] = [_u8((D, Tp), dev), _fake_scales(D, Tp // 32, order, dev), _u8((H, Tp), dev),
+                   _fake_scales(H, Tp // 32, order, dev)]
+    if need_dx or need_ds:
+        wq = lambda: [_u8((G, D, H), dev), _u8((G * ops.mfma_scale_bytes(D, H // 32),), dev)]
+        s[12:16] = wq() + wq()
+    if need_ds and not score_before:
+        s[16] = torch.empty((Tp, D), dtype=torch.bfloat16, device=dev)
+    return (torch.empty((T, D), dtype=torch.bfloat16, device=dev), *s)
+
+
+@torch.library.custom_op("torchtitan_amd::mx_routed_experts_bwd", mutates_args=())
+def mx_routed_experts_bwd(dout: torch.Tensor, saved: list[torch.Tensor], x: torch.Tensor | None, mode: int, order: int,
+                          score_before: bool, need_dx: bool, need_ds: bool, need_dw1: bool, need_dw2: bool,
+                          need_dw3: bool) -> _T4:
+    """(dx [T, D] bf16, d scores [T, k] float32, dW1 and dW3 stacked, dW2 bf16), empty where not
+    asked for."""
+    from . import mx_blocks
+
+    s = _restored(saved)
+    if x is not None:
+        s[16] = (x if x.dtype == torch.bfloat16 else x.to(torch.bfloat16)).contiguous()
+    dob = (dout if dout.dtype == torch.bfloat16 else dout.to(torch.bfloat16)).contiguous()
+    dx, ds, dw1, dw2, dw3 = mx_blocks.routed_backward(dob, s, _block_cfg(mode, False), order, score_before, need_dx,
+                                                      need_ds, need_dw1, need_dw2, need_dw3)
+    none = lambda dt=torch.bfloat16: torch.empty((0,), dtype=dt, device=dout.device)
+    return (dx if dx is not None else none(), ds if ds is not None else none(torch.float32),
+            _pack_pair(dw1, dw3, dout.device), dw2 if dw2 is not None else none())
+
+
+@mx_routed_experts_bwd.register_fake
+def _(dout, saved, x, mode, order, score_before, need_dx, need_ds, need_dw1, need_dw2, need_dw3):
+    dev = dout.device
+    mk = lambda shape, on, dt=torch.bfloat16: torch.empty(shape if on else (0,), dtype=dt, device=dev)
+    T, D = dout.shape
+    k = saved[3].shape[1]
+    G, H = saved[6].shape[0], saved[6].shape[1]
+    return (mk((T, D), need_dx), mk((T, k), need_ds, torch.float32), mk(_pair_shape((G, H, D), need_dw1, need_dw3), True),
+            mk((G, D, H), need_dw2))
+
+
+def _routed_setup(ctx, inputs, output):
+    x, top_scores, w1, w2, w3, tok_sorted, counts, score_before, mode, cache_w, need_dx, need_ds, need_dw = inputs
+    ctx.keep_x = bool(score_before and need_ds)
+    ctx.save_for_backward(*output[1:], *((x,) if ctx.keep_x else ()))
+    from . import mx_blocks
+
+    ctx.mode, ctx.score_before = mode, score_before
+    ctx.order = mx_blocks.grouped_layout(x.shape[1], w1.shape[1], w1.shape[0])[0]
+    ctx.dtypes = (x.dtype, top_scores.dtype, w1.dtype, w2.dtype, w3.dtype)
+
+
+def _routed_backward(ctx, gout, *unused):
+    saved = list(ctx.saved_tensors)
+    x = saved[17] if ctx.keep_x else None
+    need = ctx.needs_input_grad
+    dx, ds, dw13, dw2 = torch.ops.torchtitan_amd.mx_routed_experts_bwd(gout, saved[:17], x, ctx.mode, ctx.order,
+                                                                     ctx.score_before, need[0], need[1], need[2], need[3],
+                                                                     need[4])
+    dw1, dw3 = _unpack_pair(dw13, need[2], need[4])
+    grads = (dx, ds, dw1, dw2, dw3)
+    return (*(g.to(dt) if on else None for g, dt, on in zip(grads, ctx.dtypes, need[:5])),
+            None, None, None, None, None, None, None, None)
+
+
+mx_routed_experts_fwd.register_autograd(_routed_backward, setup_context=_routed_setup)
+
+
+def mx_routed_experts_traced(x, top_scores, w1, w2, w3, tok_sorted, counts, score_before: bool):
+    """The fused routed half of an MoE layer while a graph is being traced."""
+    cfg = w2.mx_config
+    return torch.ops.torchtitan_amd.mx_routed_experts_fwd(
+        x, top_scores, w1, w2, w3, tok_sorted, counts, bool(score_before), ops.SCALE_MODES[cfg.scale_mode],
+        cfg.cache_weight_casts, _wants_grad(x), _wants_grad(top_scores), _wants_grad(w1, w2, w3))[0]

@@ -616,6 +616,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   // piece 0..15 = unit pairs (A unit, B unit alternating), 16 = scales, then advance.
   auto issue_piece = [&](auto i_) {
     constexpr int i = decltype(i_)::value;
+
     const uint32_t sbase = lds_base + ld_slot * kBlock32;
     if constexpr (i < 16) {
       constexpr int q = i >> 1;

@@ -109,6 +109,82 @@ def _bf16(t: torch.Tensor) -> torch.Tensor:
     return t if t.dtype == torch.bfloat16 else t.to(torch.bfloat16)
 
 
+def _take(saved, i):
+    """MXData (MFMA-order scales) from two neighbouring slots of a saved list."""
+    return MXData(saved[i], saved[i + 1], MX_SCALES_MFMA)
+
+
+# What the SwiGLU block keeps for its backward, by slot (None where a gradient is not needed):
+#   0 h1 and h3 stacked [2, M, H]    1, 2 column-wise W2       3, 4 column-wise x     5, 6 column-wise g
+#   7, 8 column-wise W1              9, 10 column-wise W3      11 x, 12 rstd, 13 norm weight (norm in front)
+FFN_SAVED = 14
+
+
+def ffn_forward(x2, x_src, w1, w2, w3, cfg: MXFP8Config, need_dx: bool, need_dw: bool, norm_weight=None,
+                eps: float = 0.0):
+    """Forward of the SwiGLU block on a 2-D bf16 activation: (y [M, out], the FFN_SAVED slots).
+    `x_src` is the tensor the activation-cast cache is keyed on (None: no sharing of x's cast
+    with sibling linears).  The eager autograd function and the traced operator both run this."""
+    mode = cfg.scale_mode
+    rstd = None
+    if norm_weight is not None:  # RMSNorm in front: normalised inside the cast, rstd kept for its backward
+        x2 = x2.contiguous()
+        xq0, xq1, rstd, _ = ops.rms_norm_to_mx(x2, _bf16(norm_weight), eps, mode, MX_SCALES_MFMA)
+    elif x_src is not None:
+        xq0, xq1 = _cast_activation(x2, x_src, mode, need_cols=need_dw)
+    elif need_dw:
+        xq0, xq1 = ops.to_mx_dim0_dim1(x2.contiguous(), mode, MX_SCALES_MFMA)
+    else:
+        xq0, xq1 = ops.to_mx_dim0(x2.contiguous(), mode, MX_SCALES_MFMA), None
+    w1q0, w1q1 = _cast_weight(w1, mode, need_dx, cfg)
+    w3q0, w3q1 = _cast_weight(w3, mode, need_dx, cfg)
+    w2q0, w2q1 = _cast_weight(w2, mode, need_dx or need_dw, cfg)
+    h13 = ops.mx_gemm_nt_shared_a(xq0, w1q0, w3q0)  # one launch: x's panels fetched once for both
+    gq0, gq1, _ = ops.swiglu_to_mx_dim0_dim1(h13[0], h13[1], mode, MX_SCALES_MFMA)
+    y = ops.mx_gemm_nt(gq0, w2q0)
+    saved = [None] * FFN_SAVED
+    if need_dx or need_dw:
+        saved[0:3] = [h13, w2q1.codes, w2q1.scales]
+    if need_dw:
+        saved[3:7] = [xq1.codes, xq1.scales, gq1.codes, gq1.scales]
+    if need_dx:
+        saved[7:11] = [w1q1.codes, w1q1.scales, w3q1.codes, w3q1.scales]
+        if norm_weight is not None:
+            saved[11:14] = [x2, rstd, norm_weight]
+    return y, saved
+
+
+def ffn_backward(dy2, saved, cfg: MXFP8Config, need_x: bool, need_dw1: bool, need_dw2: bool, need_dw3: bool,
+                 need_dnw: bool = False):
+    """(dx [M, in], dW1, dW2, dW3, d norm weight), bf16, None where not asked for."""
+    mode = cfg.scale_mode
+    h13 = saved[0]
+    w2q1 = _take(saved, 1)
+    if need_dw2:
+        dyq0, dyq1 = ops.to_mx_dim0_dim1(dy2, mode, MX_SCALES_MFMA)
+    else:
+        dyq0, dyq1 = ops.to_mx_dim0(dy2, mode, MX_SCALES_MFMA), None
+    dg = ops.mx_gemm_nt(dyq0, w2q1)
+    (da0, da1), (db0, db1), _ = ops.swiglu_bwd_to_mx_dim0_dim1(dg, h13[0], h13[1], mode, MX_SCALES_MFMA)
+    dx = dw1 = dw2 = dw3 = dnw = None
+    if need_dw1 or need_dw2 or need_dw3:
+        xq1, gq1 = _take(saved, 3), _take(saved, 5)
+        if need_dw1 and need_dw3:
+            dw1, dw3 = ops.mx_gemm_nt_shared_b(da1, db1, xq1).unbind(0)  # one launch over x's column-wise form
+        elif need_dw1:
+            dw1 = ops.mx_gemm_nt(da1, xq1)
+        elif need_dw3:
+            dw3 = ops.mx_gemm_nt(db1, xq1)
+        if need_dw2:
+            dw2 = ops.mx_gemm_nt(dyq1, gq1)
+    if need_x or need_dnw:
+        # dx = d(h1) W1 + d(h3) W3 as one GEMM: summed in float32, rounded once
+        dx = ops.mx_gemm_nt_pair(da0, _take(saved, 7), db0, _take(saved, 9))
+        if saved[11] is not None:
+            dx, dnw = _rms_norm_backward(dx, saved[11], saved[12], saved[13], need_x, need_dnw)
+    return dx, dw1, dw2, dw3, dnw
+
+
 class _MXFeedForward(torch.autograd.Function):
     """y = (silu(x W1^T) * (x W3^T)) W2^T with every elementwise step folded into a cast kernel.
 
@@ -120,83 +196,31 @@ class _MXFeedForward(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, w1, w2, w3, cfg: MXFP8Config, norm_weight=None, eps: float = 0.0):
-        mode = cfg.scale_mode
-        D, H = x.shape[-1], w1.shape[0]
-        x2 = x.reshape(-1, D)
         need_dx = ctx.needs_input_grad[0] or ctx.needs_input_grad[5]
         need_dw = any(ctx.needs_input_grad[1:4])
-        ctx.normed = norm_weight is not None
-        if ctx.normed:  # RMSNorm in front: normalised inside the cast, rstd kept for its backward
-            x2 = x2.contiguous()
-            xq0, xq1, rstd, _ = ops.rms_norm_to_mx(x2, _bf16(norm_weight), eps, mode, MX_SCALES_MFMA)
-        else:
-            xq0, xq1 = _cast_activation(x2, x, mode, need_cols=need_dw)
-        w1q0, w1q1 = _cast_weight(w1, mode, need_dx, cfg)
-        w3q0, w3q1 = _cast_weight(w3, mode, need_dx, cfg)
-        w2q0, w2q1 = _cast_weight(w2, mode, need_dx or need_dw, cfg)
-        h1, h3 = ops.mx_gemm_nt_shared_a(xq0, w1q0, w3q0)  # one launch: x's panels fetched once
-        gq0, gq1, _ = ops.swiglu_to_mx_dim0_dim1(h1, h3, mode, MX_SCALES_MFMA)
-        y = ops.mx_gemm_nt(gq0, w2q0)
+        y, saved = ffn_forward(x.reshape(-1, x.shape[-1]), x, w1, w2, w3, cfg, need_dx, need_dw, norm_weight, eps)
         ctx.cfg, ctx.x_shape = cfg, x.shape
         ctx.w_dtypes = (w1.dtype, w2.dtype, w3.dtype)
-        ctx.need_dx, ctx.need_dw = need_dx, need_dw
-        saved = []
-        if need_dx or need_dw:
-            saved += [h1, h3, w2q1.codes, w2q1.scales]
-        if need_dw:
-            saved += [xq1.codes, xq1.scales, gq1.codes, gq1.scales]
-        if need_dx:
-            saved += [w1q1.codes, w1q1.scales, w3q1.codes, w3q1.scales]
-            if ctx.normed:
-                saved += [x2, rstd, norm_weight]
         ctx.save_for_backward(*saved)
         return y.view(*x.shape[:-1], w2.shape[0])
 
     @staticmethod
     def backward(ctx, dy):
         _cast_cache.clear()  # the forward that shared x's cast with a sibling is over
-        mode = ctx.cfg.scale_mode
-        saved = list(ctx.saved_tensors)
-        take = lambda: MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
-        h1, h3 = saved.pop(0), saved.pop(0)
-        w2q1 = take()
+        need = ctx.needs_input_grad
         dy2 = _bf16(dy.reshape(-1, dy.shape[-1])).contiguous()
-        if ctx.needs_input_grad[2]:
-            dyq0, dyq1 = ops.to_mx_dim0_dim1(dy2, mode, MX_SCALES_MFMA)
-        else:
-            dyq0, dyq1 = ops.to_mx_dim0(dy2, mode, MX_SCALES_MFMA), None
-        dg = ops.mx_gemm_nt(dyq0, w2q1)
-        (da0, da1), (db0, db1), _ = ops.swiglu_bwd_to_mx_dim0_dim1(dg, h1, h3, mode, MX_SCALES_MFMA)
-        dx = dw1 = dw2 = dw3 = None
-        if ctx.need_dw:
-            xq1, gq1 = take(), take()
-            cast_back = lambda g, dt: g if g.dtype == dt else g.to(dt)
-            if ctx.needs_input_grad[1] and ctx.needs_input_grad[3]:
-                dw1, dw3 = ops.mx_gemm_nt_shared_b(da1, db1, xq1)  # one launch over x's column-wise form
-                dw1, dw3 = cast_back(dw1, ctx.w_dtypes[0]), cast_back(dw3, ctx.w_dtypes[2])
-            elif ctx.needs_input_grad[1]:
-                dw1 = cast_back(ops.mx_gemm_nt(da1, xq1), ctx.w_dtypes[0])
-            elif ctx.needs_input_grad[3]:
-                dw3 = cast_back(ops.mx_gemm_nt(db1, xq1), ctx.w_dtypes[2])
-            if ctx.needs_input_grad[2]:
-                dw2 = cast_back(ops.mx_gemm_nt(dyq1, gq1), ctx.w_dtypes[1])
-        dnw = None
-        if ctx.need_dx:
-            w1q1, w3q1 = take(), take()
-            # dx = d(h1) W1 + d(h3) W3 as one GEMM: summed in float32, rounded once
-            dx = ops.mx_gemm_nt_pair(da0, w1q1, db0, w3q1)
-            if ctx.normed:
-                dx, dnw = _rms_norm_backward(dx, *saved[:3], ctx.needs_input_grad[0], ctx.needs_input_grad[5])
-            if dx is not None:
-                dx = dx.view(ctx.x_shape)
-        return dx, dw1, dw2, dw3, None, dnw, None
+        dx, dw1, dw2, dw3, dnw = ffn_backward(dy2, list(ctx.saved_tensors), ctx.cfg, need[0], need[1], need[2],
+                                              need[3], need[5])
+        cast_back = lambda g, dt: g if g is None or g.dtype == dt else g.to(dt)
+        if dx is not None:
+            dx = dx.view(ctx.x_shape)
+        return (dx, cast_back(dw1, ctx.w_dtypes[0]), cast_back(dw2, ctx.w_dtypes[1]), cast_back(dw3, ctx.w_dtypes[2]),
+                None, dnw, None)
 
 
 def feed_forward_fusable(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, w3: torch.Tensor) -> bool:
     """The whole-block function needs all three weights converted with gate fusion on, a bf16
     GPU activation and 32-aligned token, model and hidden sizes."""
-    if torch.compiler.is_compiling():  # the fused block functions are eager-only
-        return False
     ws = (w1, w2, w3)
     if not all(isinstance(w, MXFP8TrainingWeight) and w.mx_config.fuse_swiglu_cast for w in ws):
         return False
@@ -212,6 +236,11 @@ def mx_feed_forward(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, w3: tor
                     bias2: torch.Tensor | None = None):
     """``F.linear(F.silu(F.linear(x, w1)) * F.linear(x, w3), w2, bias2)`` for converted weights.
     Callers check `feed_forward_fusable` first."""
+    if torch.compiler.is_compiling():  # the same function as one node of the graph (compiled.py)
+        from .compiled import mx_feed_forward_traced
+
+        with torch._C.DisableTorchFunctionSubclass():
+            return mx_feed_forward_traced(x, w1, w2, w3, bias2)
     y = _MXFeedForward.apply(x, _unwrap(w1), _unwrap(w2), _unwrap(w3), w2.mx_config, None, 0.0)
     if bias2 is not None:
         y = y + _unwrap(bias2).to(y.dtype)
@@ -288,12 +317,15 @@ class _MXNormLinears(torch.autograd.Function):
         return (dx, dnw, None, None, *dws)
 
 
-def norm_fusable(x: torch.Tensor, norm_weight: torch.Tensor | None, *weights: torch.Tensor) -> bool:
+def norm_fusable(x: torch.Tensor, norm_weight: torch.Tensor | None, *weights: torch.Tensor,
+                 for_feed_forward: bool = False) -> bool:
     """RMSNorm can move into the cast when the converter was built with `fuse_rmsnorm_cast`, the
     norm has a bf16 weight, every linear behind it is converted with in_features % 32 == 0 and
-    out_features % 32 == 0, and x is a bf16 GPU tensor with a multiple of 32 tokens."""
-    if torch.compiler.is_compiling():  # the fused block functions are eager-only
-        return False
+    out_features % 32 == 0, and x is a bf16 GPU tensor with a multiple of 32 tokens.
+    `for_feed_forward`: the caller is about to use `mx_norm_feed_forward`, which also exists as a
+    traced operator; `mx_norm_linears` is an eager function only."""
+    if torch.compiler.is_compiling() and not for_feed_forward:
+        return False  # of the two norm fusions only the feed-forward block has a traced operator
     if norm_weight is None or norm_weight.dtype != torch.bfloat16 or not weights:
         return False
     if not all(isinstance(w, MXFP8TrainingWeight) and w.mx_config.fuse_rmsnorm_cast and w.dim() == 2 for w in weights):
@@ -323,11 +355,97 @@ def mx_norm_feed_forward(x: torch.Tensor, norm_weight: torch.Tensor, eps: float 
                          w2: torch.Tensor, w3: torch.Tensor, bias2: torch.Tensor | None = None):
     """The SwiGLU block applied to ``F.rms_norm(x, (dim,), norm_weight, eps)``, norm inside the
     cast.  Callers check `norm_fusable(x, norm_weight, w1, w3)` and `feed_forward_fusable`."""
+    if torch.compiler.is_compiling():
+        from .compiled import mx_feed_forward_traced
+
+        with torch._C.DisableTorchFunctionSubclass():
+            return mx_feed_forward_traced(x, w1, w2, w3, bias2, norm_weight, _norm_eps(x, eps))
     y = _MXFeedForward.apply(x, _unwrap(w1), _unwrap(w2), _unwrap(w3), w2.mx_config, norm_weight,
                              _norm_eps(x, eps))
     if bias2 is not None:
         y = y + _unwrap(bias2).to(y.dtype)
     return y
+
+
+def grouped_layout(D: int, H: int, G: int):
+    """(scale order of the activations, multiple the padded token axis is rounded up to) for an
+    expert block of model size D and hidden size H: the persistent kernel with MFMA-order scales
+    where it takes the shape, the general grouped kernels with row-major scales otherwise."""
+    fast = D % 128 == 0 and H % 128 == 0 and G <= ops.FAST_MAX_GROUPS
+    return (MX_SCALES_MFMA if fast else MX_SCALES_ROWMAJOR), (ops.FAST_LENGTH_MULTIPLE if fast else 1), fast
+
+
+# What the expert block keeps for its backward, by slot (None where not needed):
+#   0 padded group ends   1 gather indices, 2 rows' places in the padded layout (groups moved)
+#   3 h1 and h3 stacked [2, Tp, H]   4, 5 column-wise W2   6, 7 column-wise x   8, 9 column-wise g
+#   10, 11 column-wise W1            12, 13 column-wise W3
+GROUPED_FFN_SAVED = 14
+
+
+def grouped_ffn_forward(x, w1, w2, w3, offs, cfg: MXFP8Config, need_dx: bool, need_dw: bool):
+    """Forward of the expert block on x [T, D] (bf16): (y [T, D], the GROUPED_FFN_SAVED slots)."""
+    mode = cfg.scale_mode
+    T, D = x.shape
+    G, H, _ = w1.shape
+    order, multiple, fast = grouped_layout(D, H, G)
+    perm = back = None
+    if cfg.pad_token_groups_for_grouped_mm or fast:
+        perm, offs_p, back = _pad_plan(offs, T, ops.BLOCK, multiple)
+    else:
+        offs_p = offs
+        if T % ops.BLOCK:
+            raise ValueError("without padding the token dimension must be a multiple of 32")
+    xq0, xq1 = _cast_into_groups(x.contiguous(), perm, mode, order, need_dw)
+    w1q0, w1q1 = _cast_weight(w1, mode, need_dx, cfg)
+    w3q0, w3q1 = _cast_weight(w3, mode, need_dx, cfg)
+    w2q0, w2q1 = _cast_weight(w2, mode, need_dx or need_dw, cfg)
+    h13 = ops.mx_grouped_gemm_2d3d_shared_a(xq0, w1q0, w3q0, offs_p)  # one pass over the routed tokens
+    gq0, gq1, _ = ops.swiglu_to_mx_dim0_dim1(h13[0], h13[1], mode, order)
+    y = _grouped_2d3d_padded(gq0, w2q0, offs_p, back)
+    saved = [None] * GROUPED_FFN_SAVED
+    saved[0:3] = [offs_p, perm, back]
+    if need_dx or need_dw:
+        saved[3:6] = [h13, w2q1.codes, w2q1.scales]
+    if need_dw:
+        saved[6:10] = [xq1.codes, xq1.scales, gq1.codes, gq1.scales]
+    if need_dx:
+        saved[10:14] = [w1q1.codes, w1q1.scales, w3q1.codes, w3q1.scales]
+    return y, saved
+
+
+def grouped_ffn_backward(dy, saved, cfg: MXFP8Config, order: int, need_dx: bool, need_dw1: bool, need_dw2: bool,
+                         need_dw3: bool):
+    """(dx [T, D], dW1, dW2, dW3), bf16, None where not asked for; dy [T, D] bf16 contiguous."""
+    mode = cfg.scale_mode
+    offs_p, perm, back, h13 = saved[0:4]
+    w2q1 = _take(saved, 4)
+    dyq0, dyq1 = _cast_into_groups(dy, perm, mode, order, need_dw2)
+    dg = ops.mx_grouped_gemm_2d3d(dyq0, w2q1, offs_p)
+    (da0, da1), (db0, db1), _ = ops.swiglu_bwd_to_mx_dim0_dim1(dg, h13[0], h13[1], mode, order)
+    dx = dw1 = dw2 = dw3 = None
+    if need_dw1 or need_dw2 or need_dw3:
+        xq1, gq1 = MXData(saved[6], saved[7], order), MXData(saved[8], saved[9], order)
+        if need_dw1 and need_dw3:
+            dw1, dw3 = ops.mx_grouped_gemm_2d2d_shared_b(da1, db1, xq1, offs_p).unbind(0)
+        elif need_dw1:
+            dw1 = ops.mx_grouped_gemm_2d2d(da1, xq1, offs_p)
+        elif need_dw3:
+            dw3 = ops.mx_grouped_gemm_2d2d(db1, xq1, offs_p)
+        if need_dw2:
+            dw2 = ops.mx_grouped_gemm_2d2d(dyq1, gq1, offs_p)
+    if need_dx:
+        w1q1, w3q1 = _take(saved, 10), _take(saved, 12)
+        # d(h1) W1[g] + d(h3) W3[g] as one grouped GEMM (summed in float32, rounded once); the
+        # spare zero row behind it serves rows that belong to no group
+        Tp, D = da0.codes.shape[0], w1q1.codes.shape[1]
+        if back is None:
+            dx = ops.mx_grouped_gemm_2d3d_pair(da0, w1q1, db0, w3q1, offs_p)
+        else:
+            buf = torch.empty((Tp + 1, D), dtype=torch.bfloat16, device=da0.codes.device)
+            buf[Tp].zero_()
+            ops.mx_grouped_gemm_2d3d_pair(da0, w1q1, db0, w3q1, offs_p, buf[:Tp])
+            dx = buf[back]
+    return dx, dw1, dw2, dw3
 
 
 class _MXGroupedFeedForward(torch.autograd.Function):
@@ -339,88 +457,21 @@ class _MXGroupedFeedForward(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, w1, w2, w3, offs, cfg: MXFP8Config):
-        mode = cfg.scale_mode
-        T, D = x.shape
-        G, H, _ = w1.shape
-        xb = _bf16(x)
-        pad = cfg.pad_token_groups_for_grouped_mm
-        fast = D % 128 == 0 and H % 128 == 0 and G <= ops.FAST_MAX_GROUPS  # persistent kernel
-        order = MX_SCALES_MFMA if fast else MX_SCALES_ROWMAJOR
-        plan = perm = back = None
-        if pad or fast:
-            plan = _pad_plan(offs, T, ops.BLOCK, ops.FAST_LENGTH_MULTIPLE if fast else 1)
-            perm, offs_p, back = plan
-        else:
-            offs_p = offs
-            if T % ops.BLOCK:
-                raise ValueError("without padding the token dimension must be a multiple of 32")
-        xb = xb.contiguous()
         need_dx = ctx.needs_input_grad[0]
         need_dw = any(ctx.needs_input_grad[1:4])
-        xq0, xq1 = _cast_into_groups(xb, perm, mode, order, need_dw)
-        w1q0, w1q1 = _cast_weight(w1, mode, need_dx, cfg)
-        w3q0, w3q1 = _cast_weight(w3, mode, need_dx, cfg)
-        w2q0, w2q1 = _cast_weight(w2, mode, need_dx or need_dw, cfg)
-        h1, h3 = ops.mx_grouped_gemm_2d3d_shared_a(xq0, w1q0, w3q0, offs_p)  # one pass over the routed tokens
-        gq0, gq1, _ = ops.swiglu_to_mx_dim0_dim1(h1, h3, mode, order)
-        y = _grouped_2d3d_padded(gq0, w2q0, offs_p, back)
-        ctx.cfg, ctx.order, ctx.padded, ctx.D = cfg, order, plan is not None, D
+        y, saved = grouped_ffn_forward(_bf16(x), w1, w2, w3, offs, cfg, need_dx, need_dw)
+        ctx.cfg = cfg
+        ctx.order = grouped_layout(x.shape[1], w1.shape[1], w1.shape[0])[0]
         ctx.dtypes = (x.dtype, w1.dtype, w2.dtype, w3.dtype)
-        ctx.need_dx, ctx.need_dw = need_dx, need_dw
-        saved = [offs_p]
-        if plan is not None:
-            saved += [plan[0], plan[2]]
-        if need_dx or need_dw:
-            saved += [h1, h3, w2q1.codes, w2q1.scales]
-        if need_dw:
-            saved += [xq1.codes, xq1.scales, gq1.codes, gq1.scales]
-        if need_dx:
-            saved += [w1q1.codes, w1q1.scales, w3q1.codes, w3q1.scales]
         ctx.save_for_backward(*saved)
         return y
 
     @staticmethod
     def backward(ctx, dy):
-        mode, order = ctx.cfg.scale_mode, ctx.order
-        saved = list(ctx.saved_tensors)
-        offs_p = saved.pop(0)
-        dyb = _bf16(dy).contiguous()
-        perm = back = None
-        if ctx.padded:
-            perm, back = saved.pop(0), saved.pop(0)
-        h1, h3 = saved.pop(0), saved.pop(0)
-        w2q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
-        dyq0, dyq1 = _cast_into_groups(dyb, perm, mode, order, ctx.needs_input_grad[2])
-        dg = ops.mx_grouped_gemm_2d3d(dyq0, w2q1, offs_p)
-        (da0, da1), (db0, db1), _ = ops.swiglu_bwd_to_mx_dim0_dim1(dg, h1, h3, mode, order)
-        dx = dw1 = dw2 = dw3 = None
-        cast_back = lambda g, dt: g if g.dtype == dt else g.to(dt)
-        if ctx.need_dw:
-            xq1 = MXData(saved.pop(0), saved.pop(0), order)
-            gq1 = MXData(saved.pop(0), saved.pop(0), order)
-            if ctx.needs_input_grad[1] and ctx.needs_input_grad[3]:
-                dw1, dw3 = ops.mx_grouped_gemm_2d2d_shared_b(da1, db1, xq1, offs_p)
-                dw1, dw3 = cast_back(dw1, ctx.dtypes[1]), cast_back(dw3, ctx.dtypes[3])
-            elif ctx.needs_input_grad[1]:
-                dw1 = cast_back(ops.mx_grouped_gemm_2d2d(da1, xq1, offs_p), ctx.dtypes[1])
-            elif ctx.needs_input_grad[3]:
-                dw3 = cast_back(ops.mx_grouped_gemm_2d2d(db1, xq1, offs_p), ctx.dtypes[3])
-            if ctx.needs_input_grad[2]:
-                dw2 = cast_back(ops.mx_grouped_gemm_2d2d(dyq1, gq1, offs_p), ctx.dtypes[2])
-        if ctx.need_dx:
-            w1q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
-            w3q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
-            # d(h1) W1[g] + d(h3) W3[g] as one grouped GEMM (summed in float32, rounded once); the
-            # spare zero row behind it serves rows that belong to no group
-            Tp, D = da0.codes.shape[0], w1q1.codes.shape[1]
-            if back is None:
-                dx = ops.mx_grouped_gemm_2d3d_pair(da0, w1q1, db0, w3q1, offs_p)
-            else:
-                buf = torch.empty((Tp + 1, D), dtype=torch.bfloat16, device=da0.codes.device)
-                buf[Tp].zero_()
-                ops.mx_grouped_gemm_2d3d_pair(da0, w1q1, db0, w3q1, offs_p, buf[:Tp])
-                dx = buf[back]
-            dx = cast_back(dx, ctx.dtypes[0])
+        need = ctx.needs_input_grad
+        grads = grouped_ffn_backward(_bf16(dy).contiguous(), list(ctx.saved_tensors), ctx.cfg, ctx.order, need[0],
+                                     need[1], need[2], need[3])
+        dx, dw1, dw2, dw3 = (g if g is None or g.dtype == dt else g.to(dt) for g, dt in zip(grads, ctx.dtypes))
         return dx, dw1, dw2, dw3, None, None
 
 
@@ -435,8 +486,6 @@ def grouped_feed_forward_fusable(x: torch.Tensor, w1: torch.Tensor, w2: torch.Te
                                  w3: torch.Tensor) -> bool:
     """All three expert parameters converted with gate fusion on, a 2-D GPU activation, model
     and hidden sizes multiples of 32."""
-    if torch.compiler.is_compiling():  # the fused block functions are eager-only
-        return False
     ws = (w1, w2, w3)
     if not all(isinstance(w, MXFP8TrainingWeight) and w.mx_config.fuse_swiglu_cast and w.dim() == 3 for w in ws):
         return False
@@ -452,8 +501,96 @@ def mx_grouped_feed_forward(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
     """The SwiGLU expert block for converted 3-D parameters w1, w3 [G, hidden, dim] and
     w2 [G, dim, hidden]; offs = inclusive cumulative group sizes.  Returns bf16.
     Callers check `grouped_feed_forward_fusable` first."""
+    if torch.compiler.is_compiling():
+        from .compiled import mx_grouped_feed_forward_traced
+
+        with torch._C.DisableTorchFunctionSubclass():
+            return mx_grouped_feed_forward_traced(x, w1, w2, w3, offs)
     return _MXGroupedFeedForward.apply(x, _unwrap(w1), _unwrap(w2), _unwrap(w3), offs.to(torch.int32),
                                        w2.mx_config)
+
+
+# What the routed half of an MoE layer keeps for its backward, by slot (None where not needed):
+#   0 padded group ends   1 token of every padded row   2 score of every padded row   3 padded row of every
+#   (token, choice) pair [T, k]   4 scores (float32)   5 h1 and h3 stacked   6, 7 column-wise W2
+#   8, 9 column-wise x    10, 11 column-wise g    12, 13 column-wise W1    14, 15 column-wise W3
+#   16 x (scores in front of the experts) or the padded expert outputs (scores behind them)
+ROUTED_SAVED = 17
+
+
+def routed_forward(x, top_scores, w1, w2, w3, tok_sorted, counts, score_before: bool, cfg: MXFP8Config,
+                   need_dx: bool, need_ds: bool, need_dw: bool):
+    """Forward of the routed half on x [T, D] (bf16 contiguous): (out [T, D], the ROUTED_SAVED slots)."""
+    mode = cfg.scale_mode
+    T, D = x.shape
+    k = top_scores.shape[1]
+    G, H, _ = w1.shape
+    scores = top_scores.float().contiguous()
+    order, multiple, _ = grouped_layout(D, H, G)
+    # aligned group layout and the maps between padded rows, tokens and (token, j) pairs
+    offs_p, src_row, row_score, pos = ops.moe_route_plan(counts, tok_sorted, scores.view(-1), k, ops.BLOCK, multiple)
+    pos = pos.view(T, k)
+    xq0, xq1 = ops.to_mx_rows_gathered(x, src_row, mode, order, need_dw, row_score if score_before else None)
+    need_dg = need_dx or need_ds or need_dw
+    w1q0, w1q1 = _cast_weight(w1, mode, need_dx or need_ds, cfg)
+    w3q0, w3q1 = _cast_weight(w3, mode, need_dx or need_ds, cfg)
+    w2q0, w2q1 = _cast_weight(w2, mode, need_dg, cfg)
+    h13 = ops.mx_grouped_gemm_2d3d_shared_a(xq0, w1q0, w3q0, offs_p)  # one pass over the routed tokens
+    gq0, gq1, _ = ops.swiglu_to_mx_dim0_dim1(h13[0], h13[1], mode, order)
+    yp = ops.mx_grouped_gemm_2d3d(gq0, w2q0, offs_p)
+    out = ops.moe_combine(yp, pos, None if score_before else scores)
+    saved = [None] * ROUTED_SAVED
+    saved[0:5] = [offs_p, src_row, row_score, pos, scores]
+    if need_dg:
+        saved[5:8] = [h13, w2q1.codes, w2q1.scales]
+    if need_dw:
+        saved[8:12] = [xq1.codes, xq1.scales, gq1.codes, gq1.scales]
+    if need_dx or need_ds:
+        saved[12:16] = [w1q1.codes, w1q1.scales, w3q1.codes, w3q1.scales]
+    if need_ds:
+        saved[16] = x if score_before else yp
+    return out, saved
+
+
+def routed_backward(dout, saved, cfg: MXFP8Config, order: int, score_before: bool, need_dx: bool, need_ds: bool,
+                    need_dw1: bool, need_dw2: bool, need_dw3: bool):
+    """(dx [T, D] bf16, d scores [T, k] float32, dW1, dW2, dW3 bf16), None where not asked for."""
+    mode = cfg.scale_mode
+    offs_p, src_row, row_score, pos, scores, h13 = saved[0:6]
+    T, k = pos.shape
+    w2q1 = _take(saved, 6)
+    # gradient of the padded expert outputs: dout of the row's token (times its score)
+    dyq0, dyq1 = ops.to_mx_rows_gathered(dout, src_row, mode, order, need_dw2, None if score_before else row_score)
+    dg = ops.mx_grouped_gemm_2d3d(dyq0, w2q1, offs_p)
+    (da0, da1), (db0, db1), _ = ops.swiglu_bwd_to_mx_dim0_dim1(dg, h13[0], h13[1], mode, order)
+    dx = ds = dw1 = dw2 = dw3 = None
+    if need_dw1 or need_dw2 or need_dw3:
+        xq1, gq1 = MXData(saved[8], saved[9], order), MXData(saved[10], saved[11], order)
+        if need_dw1 and need_dw3:
+            dw1, dw3 = ops.mx_grouped_gemm_2d2d_shared_b(da1, db1, xq1, offs_p).unbind(0)
+        elif need_dw1:
+            dw1 = ops.mx_grouped_gemm_2d2d(da1, xq1, offs_p)
+        elif need_dw3:
+            dw3 = ops.mx_grouped_gemm_2d2d(db1, xq1, offs_p)
+        if need_dw2:
+            dw2 = ops.mx_grouped_gemm_2d2d(dyq1, gq1, offs_p)
+    if need_dx or need_ds:
+        w1q1, w3q1 = _take(saved, 12), _take(saved, 14)
+        if need_dx or (need_ds and score_before):
+            # gradient of the (scaled) routed inputs, padded layout: the halves from w1 and
+            # w3 summed inside one grouped GEMM (float32, one rounding)
+            dxp = ops.mx_grouped_gemm_2d3d_pair(da0, w1q1, db0, w3q1, offs_p)
+        if need_dx:
+            dx = ops.moe_combine(dxp, pos, scores if score_before else None)
+        if need_ds:
+            other = saved[16]  # x (scores in front of the experts) or the expert outputs
+            token = torch.arange(T * k, device=pos.device, dtype=torch.int64).div_(k, rounding_mode="floor")
+            if score_before:
+                ds = ops.moe_row_dot(dxp, pos.view(-1), other, token)
+            else:
+                ds = ops.moe_row_dot(other, pos.view(-1), dout, token)
+            ds = ds.view(T, k)
+    return dx, ds, dw1, dw2, dw3
 
 
 class _MXRoutedExperts(torch.autograd.Function):
@@ -469,94 +606,22 @@ class _MXRoutedExperts(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, top_scores, w1, w2, w3, tok_sorted, counts, score_before: bool, cfg: MXFP8Config):
-        mode = cfg.scale_mode
-        T, D = x.shape
-        k = top_scores.shape[1]
-        R = T * k
-        G, H, _ = w1.shape
-        xb = _bf16(x).contiguous()
-        scores = top_scores.float().contiguous()
-        fast = D % 128 == 0 and H % 128 == 0 and G <= ops.FAST_MAX_GROUPS
-        order = MX_SCALES_MFMA if fast else MX_SCALES_ROWMAJOR
-        # aligned group layout and the maps between padded rows, tokens and (token, j) pairs
-        offs_p, src_row, row_score, pos = ops.moe_route_plan(counts, tok_sorted, scores.view(-1), k,
-                                                             ops.BLOCK, ops.FAST_LENGTH_MULTIPLE if fast else 1)
-        pos = pos.view(T, k)
-        need_dx = ctx.needs_input_grad[0]
-        need_ds = ctx.needs_input_grad[1]
+        need_dx, need_ds = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         need_dw = any(ctx.needs_input_grad[2:5])
-        xq0, xq1 = ops.to_mx_rows_gathered(xb, src_row, mode, order, need_dw,
-                                           row_score if score_before else None)
-        need_dg = need_dx or need_ds or need_dw
-        w1q0, w1q1 = _cast_weight(w1, mode, need_dx or need_ds, cfg)
-        w3q0, w3q1 = _cast_weight(w3, mode, need_dx or need_ds, cfg)
-        w2q0, w2q1 = _cast_weight(w2, mode, need_dg, cfg)
-        h1, h3 = ops.mx_grouped_gemm_2d3d_shared_a(xq0, w1q0, w3q0, offs_p)  # one pass over the routed tokens
-        gq0, gq1, _ = ops.swiglu_to_mx_dim0_dim1(h1, h3, mode, order)
-        yp = ops.mx_grouped_gemm_2d3d(gq0, w2q0, offs_p)
-        out = ops.moe_combine(yp, pos, None if score_before else scores)
-        ctx.cfg, ctx.order, ctx.score_before = cfg, order, score_before
+        out, saved = routed_forward(_bf16(x).contiguous(), top_scores, w1, w2, w3, tok_sorted, counts, score_before,
+                                    cfg, need_dx, need_ds, need_dw)
+        ctx.cfg, ctx.score_before = cfg, score_before
+        ctx.order = grouped_layout(x.shape[1], w1.shape[1], w1.shape[0])[0]
         ctx.dtypes = (x.dtype, top_scores.dtype, w1.dtype, w2.dtype, w3.dtype)
-        ctx.flags = (need_dx, need_ds, need_dw)
-        saved = [offs_p, src_row, row_score, pos, scores]
-        if need_dg:
-            saved += [h1, h3, w2q1.codes, w2q1.scales]
-        if need_dw:
-            saved += [xq1.codes, xq1.scales, gq1.codes, gq1.scales]
-        if need_dx or need_ds:
-            saved += [w1q1.codes, w1q1.scales, w3q1.codes, w3q1.scales]
-        if need_ds:
-            saved += [xb if score_before else yp]
         ctx.save_for_backward(*saved)
         return out
 
     @staticmethod
     def backward(ctx, dout):
-        mode, order, score_before = ctx.cfg.scale_mode, ctx.order, ctx.score_before
-        need_dx, need_ds, need_dw = ctx.flags
-        saved = list(ctx.saved_tensors)
-        offs_p, src_row, row_score, pos, scores = (saved.pop(0) for _ in range(5))
-        T, k = pos.shape
-        dob = _bf16(dout).contiguous()
-        h1, h3 = saved.pop(0), saved.pop(0)
-        w2q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
-        # gradient of the padded expert outputs: dout of the row's token (times its score)
-        dyq0, dyq1 = ops.to_mx_rows_gathered(dob, src_row, mode, order, ctx.needs_input_grad[3],
-                                             None if score_before else row_score)
-        dg = ops.mx_grouped_gemm_2d3d(dyq0, w2q1, offs_p)
-        (da0, da1), (db0, db1), _ = ops.swiglu_bwd_to_mx_dim0_dim1(dg, h1, h3, mode, order)
-        dx = ds = dw1 = dw2 = dw3 = None
-        cast_back = lambda g, dt: g if g.dtype == dt else g.to(dt)
-        if need_dw:
-            xq1 = MXData(saved.pop(0), saved.pop(0), order)
-            gq1 = MXData(saved.pop(0), saved.pop(0), order)
-            if ctx.needs_input_grad[2] and ctx.needs_input_grad[4]:
-                dw1, dw3 = ops.mx_grouped_gemm_2d2d_shared_b(da1, db1, xq1, offs_p)
-                dw1, dw3 = cast_back(dw1, ctx.dtypes[2]), cast_back(dw3, ctx.dtypes[4])
-            elif ctx.needs_input_grad[2]:
-                dw1 = cast_back(ops.mx_grouped_gemm_2d2d(da1, xq1, offs_p), ctx.dtypes[2])
-            elif ctx.needs_input_grad[4]:
-                dw3 = cast_back(ops.mx_grouped_gemm_2d2d(db1, xq1, offs_p), ctx.dtypes[4])
-            if ctx.needs_input_grad[3]:
-                dw2 = cast_back(ops.mx_grouped_gemm_2d2d(dyq1, gq1, offs_p), ctx.dtypes[3])
-        if need_dx or need_ds:
-            w1q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
-            w3q1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
-            need_dxp = need_dx or (need_ds and score_before)
-            if need_dxp:
-                # gradient of the (scaled) routed inputs, padded layout: the halves from w1 and
-                # w3 summed inside one grouped GEMM (float32, one rounding)
-                dxp = ops.mx_grouped_gemm_2d3d_pair(da0, w1q1, db0, w3q1, offs_p)
-            if need_dx:
-                dx = cast_back(ops.moe_combine(dxp, pos, scores if score_before else None), ctx.dtypes[0])
-            if need_ds:
-                other = saved.pop(0)  # x (scores in front of the experts) or the expert outputs
-                token = torch.arange(T * k, device=pos.device, dtype=torch.int64).div_(k, rounding_mode="floor")
-                if score_before:
-                    ds = ops.moe_row_dot(dxp, pos.view(-1), other, token)
-                else:
-                    ds = ops.moe_row_dot(other, pos.view(-1), dob, token)
-                ds = cast_back(ds.view(T, k), ctx.dtypes[1])
+        need = ctx.needs_input_grad
+        grads = routed_backward(_bf16(dout).contiguous(), list(ctx.saved_tensors), ctx.cfg, ctx.order,
+                                ctx.score_before, need[0], need[1], need[2], need[3], need[4])
+        dx, ds, dw1, dw2, dw3 = (g if g is None or g.dtype == dt else g.to(dt) for g, dt in zip(grads, ctx.dtypes))
         return dx, ds, dw1, dw2, dw3, None, None, None, None
 
 
@@ -566,6 +631,12 @@ def mx_routed_experts(x: torch.Tensor, top_scores: torch.Tensor, w1: torch.Tenso
     """Gather, score, run the SwiGLU experts and combine, for converted expert parameters.
     x [T, dim] bf16, top_scores [T, top_k]; the index tensor is the stable argsort of the
     flattened expert choices.  Callers check `grouped_feed_forward_fusable` first."""
+    if torch.compiler.is_compiling():
+        from .compiled import mx_routed_experts_traced
+
+        with torch._C.DisableTorchFunctionSubclass():
+            return mx_routed_experts_traced(x, top_scores, w1, w2, w3, token_indices_experts_sorted,
+                                            num_tokens_per_expert, score_before_experts)
     return _MXRoutedExperts.apply(x, top_scores, _unwrap(w1), _unwrap(w2), _unwrap(w3),
                                   token_indices_experts_sorted, num_tokens_per_expert,
                                   bool(score_before_experts), w2.mx_config)

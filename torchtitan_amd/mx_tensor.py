@@ -485,7 +485,7 @@ class MXFP8TrainingWeight(torch.Tensor):
                     from .compiled import mx_linear_traced
 
                     with torch._C.DisableTorchFunctionSubclass():
-                        return mx_linear_traced(x, w, b, w.mx_config.scale_mode)
+                        return mx_linear_traced(x, w, b, w.mx_config.scale_mode, w.mx_config.cache_weight_casts)
                 return mx_linear(x, _unwrap(w), _unwrap(b), w.mx_config)
         elif func in _GROUPED_FUNCS:
             a, b = args[0], args[1]

@@ -541,37 +541,43 @@ def _persistent_shape(M: int, N: int, K: int) -> bool:
     return M > 128 and N > 128 and K % 128 == 0 and N % 8 == 0
 
 
-def mx_gemm_nt_shared_a(a: MXData, b: MXData, b2: MXData):
-    """(deq(a) @ deq(b)^T, deq(a) @ deq(b2)^T), both bf16 [M, N]: one launch in which the panels of
-    `a` are fetched once for both products where the persistent kernel takes the shape, otherwise
-    two GEMMs; bit-identical either way."""
+def mx_gemm_nt_shared_a(a: MXData, b: MXData, b2: MXData) -> torch.Tensor:
+    """bf16 [2, M, N]: deq(a) @ deq(b)^T and deq(a) @ deq(b2)^T.  One launch in which the panels
+    of `a` are fetched once for both products where the persistent kernel takes the shape,
+    otherwise two GEMMs; bit-identical either way."""
     M, K = a.codes.shape
     N = b.codes.shape[0]
     if b2.codes.shape != b.codes.shape or b.codes.shape[1] != K:
         raise ValueError("both second operands must have the same shape")
-    if not _persistent_shape(M, N, K) or _watched():
-        return mx_gemm_nt(a, b), mx_gemm_nt(a, b2)
+    if _watched():  # as dispatcher ops, so that a per-op checkpoint policy can keep the outputs
+        return torch.stack((mx_gemm_nt(a, b), mx_gemm_nt(a, b2)))
     out = torch.empty((2, M, N), dtype=torch.bfloat16, device=a.codes.device)
+    if not _persistent_shape(M, N, K):
+        mx_gemm_nt(a, b, out[0])
+        mx_gemm_nt(a, b2, out[1])
+        return out
     sa, sb, sb2 = _as_mfma(a), _as_mfma(b), _as_mfma(b2)
     _call("mx_gemm_nt_shared_a", "gemm_nt_shared_a", out.device, _ptr(a.codes), _ptr(sa), _ptr(b.codes), _ptr(sb),
           _ptr(b2.codes), _ptr(sb2), _ptr(out[0]), _ptr(out[1]), M, N, K, N, _stream(out))
-    return out[0], out[1]
+    return out
 
 
-def mx_gemm_nt_shared_b(a: MXData, a2: MXData, b: MXData):
-    """(deq(a) @ deq(b)^T, deq(a2) @ deq(b)^T), both bf16 [M, N], as `mx_gemm_nt_shared_a` with the
+def mx_gemm_nt_shared_b(a: MXData, a2: MXData, b: MXData) -> torch.Tensor:
+    """bf16 [2, M, N]: deq(a) @ deq(b)^T and deq(a2) @ deq(b)^T, as `mx_gemm_nt_shared_a` with the
     roles of the operands swapped."""
     M, K = a.codes.shape
     N = b.codes.shape[0]
     if a2.codes.shape != a.codes.shape or b.codes.shape[1] != K:
         raise ValueError("both first operands must have the same shape")
-    if not _persistent_shape(M, N, K) or _watched():
-        return mx_gemm_nt(a, b), mx_gemm_nt(a2, b)
     out = torch.empty((2, M, N), dtype=torch.bfloat16, device=a.codes.device)
+    if not _persistent_shape(M, N, K):
+        mx_gemm_nt(a, b, out[0])
+        mx_gemm_nt(a2, b, out[1])
+        return out
     sa, sa2, sb = _as_mfma(a), _as_mfma(a2), _as_mfma(b)
     _call("mx_gemm_nt_shared_b", "gemm_nt_shared_b", out.device, _ptr(a.codes), _ptr(sa), _ptr(a2.codes), _ptr(sa2),
           _ptr(b.codes), _ptr(sb), _ptr(out[0]), _ptr(out[1]), M, N, K, N, _stream(out))
-    return out[0], out[1]
+    return out
 
 
 # --------------------------------------------------------------------------- 3-D weights
@@ -686,43 +692,49 @@ def mx_grouped_gemm_2d3d_pair(a: MXData, b: MXData, a2: MXData, b2: MXData, offs
     return out
 
 
-def mx_grouped_gemm_2d3d_shared_a(a: MXData, b: MXData, b2: MXData, offs: torch.Tensor):
-    """(grouped a x b[g]^T, grouped a x b2[g]^T), both bf16 [T, N]: one launch of the persistent
+def mx_grouped_gemm_2d3d_shared_a(a: MXData, b: MXData, b2: MXData, offs: torch.Tensor) -> torch.Tensor:
+    """bf16 [2, T, N]: grouped a x b[g]^T and grouped a x b2[g]^T.  One launch of the persistent
     kernel over both products when every scale buffer is in MFMA order (32-aligned groups),
     otherwise two grouped GEMMs; bit-identical either way."""
     T, K = a.codes.shape
     G, N, _ = b.codes.shape
     if b2.codes.shape != b.codes.shape:
         raise ValueError("both weight stacks must have the same shape")
-    fast = all(d.scale_order == MX_SCALES_MFMA for d in (a, b, b2))
-    if not fast or K % 128 or N % 8 or T % 32 or G > FAST_MAX_GROUPS or _watched():
-        return mx_grouped_gemm_2d3d(a, b, offs), mx_grouped_gemm_2d3d(a, b2, offs)
     if offs.dtype != torch.int32 or offs.numel() != G:
         raise ValueError("offs must be int32 with one entry per group")
+    if _watched():  # as dispatcher ops, so that a per-op checkpoint policy can keep the outputs
+        return torch.stack((mx_grouped_gemm_2d3d(a, b, offs), mx_grouped_gemm_2d3d(a, b2, offs)))
     out = torch.empty((2, T, N), dtype=torch.bfloat16, device=a.codes.device)
+    fast = all(d.scale_order == MX_SCALES_MFMA for d in (a, b, b2))
+    if not fast or K % 128 or N % 8 or T % 32 or G > FAST_MAX_GROUPS:
+        mx_grouped_gemm_2d3d(a, b, offs, out[0])
+        mx_grouped_gemm_2d3d(a, b2, offs, out[1])
+        return out
     _call("mx_grouped_gemm_2d3d_shared_a", "grouped_gemm_2d3d_shared_a", out.device, _ptr(a.codes), _ptr(a.scales),
           _ptr(b.codes), _ptr(b.scales), _ptr(b2.codes), _ptr(b2.scales), _ptr(offs), _ptr(out[0]), _ptr(out[1]),
           T, N, K, G, N, _stream(out))
-    return out[0], out[1]
+    return out
 
 
-def mx_grouped_gemm_2d2d_shared_b(at: MXData, at2: MXData, bt: MXData, offs: torch.Tensor):
-    """(out[g] = at[:, tokens of g] x bt[:, tokens of g]^T, the same with at2), both bf16
-    [G, N, K]: one launch of the persistent kernel when the scales are in MFMA order, otherwise
-    two grouped GEMMs; bit-identical either way."""
+def mx_grouped_gemm_2d2d_shared_b(at: MXData, at2: MXData, bt: MXData, offs: torch.Tensor) -> torch.Tensor:
+    """bf16 [2, G, N, K]: out[0][g] = at[:, tokens of g] x bt[:, tokens of g]^T and out[1][g] the
+    same with at2.  One launch of the persistent kernel when the scales are in MFMA order,
+    otherwise two grouped GEMMs; bit-identical either way."""
     N, T = at.codes.shape
     K = bt.codes.shape[0]
     if at2.codes.shape != at.codes.shape or bt.codes.shape[1] != T:
         raise ValueError("operand shapes do not match")
     G = offs.numel()
+    out = torch.empty((2, G, N, K), dtype=torch.bfloat16, device=at.codes.device)
     fast = all(d.scale_order == MX_SCALES_MFMA for d in (at, at2, bt))
     if not fast or T == 0 or T % 128 or K % 8:
-        return mx_grouped_gemm_2d2d(at, bt, offs), mx_grouped_gemm_2d2d(at2, bt, offs)
-    out = torch.empty((2, G, N, K), dtype=torch.bfloat16, device=at.codes.device)
+        mx_grouped_gemm_2d2d(at, bt, offs, out[0])
+        mx_grouped_gemm_2d2d(at2, bt, offs, out[1])
+        return out
     _call("mx_grouped_gemm_2d2d_shared_b", "grouped_gemm_2d2d_shared_b", out.device, _ptr(at.codes), _ptr(at.scales),
           _ptr(at2.codes), _ptr(at2.scales), _ptr(bt.codes), _ptr(bt.scales), _ptr(offs), _ptr(out[0]), _ptr(out[1]),
           T, N, K, G, _stream(out))
-    return out[0], out[1]
+    return out
 
 
 def mx_grouped_gemm_2d2d(at: MXData, bt: MXData, offs: torch.Tensor,
