@@ -667,6 +667,44 @@ def time_decoder_block(dev, recipe):
     return out
 
 
+def _time_compiled(module, run, eager_step, reps=5):
+    """ms per forward + backward of `module` wrapped as the reference wraps its blocks
+    (torch.compile(block, fullgraph=True), torchtitan/models/llama3/parallelize.py:278-280): the
+    converted block enters the graph as the package's operators.  `eager_step` clears the
+    gradients between runs (its own forward + backward is not timed here)."""
+    import torch
+    import torch._dynamo
+
+    try:
+        import triton  # noqa: F401
+        backend = "inductor"
+    except ImportError:
+        backend = "aot_eager"
+    torch._dynamo.reset()
+    fn = torch.compile(module, backend=backend, fullgraph=True)
+
+    def step():
+        for p in module.parameters():
+            p.grad = None
+        run(fn)
+
+    try:
+        for _ in range(3):
+            step()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(reps):
+            step()
+        e.record()
+        torch.cuda.synchronize()
+        return {"ms": round(s.elapsed_time(e) / reps, 3), "backend": backend}
+    except Exception as ex:  # a backend that cannot build here must not take the benchmark down
+        return {"error": f"{type(ex).__name__}: {str(ex)[:200]}", "backend": backend}
+    finally:
+        torch._dynamo.reset()
+
+
 def time_graph_replay(step, reps=5):
     """Capture `step` (forward + backward on static tensors) in a HIP graph after a warm-up on a
     side stream and return the mean replay time in ms: the same kernels without the host in
@@ -740,6 +778,7 @@ def time_ffn_block(dev, recipe):
         out[name] = {"ms": round(ms, 3), "TFLOP/s": round(18.0 * M * DIM * HIDDEN / ms / 1e9, 1)}
         if fuse:
             out[name]["ms_replayed_from_a_hip_graph"] = round(time_graph_replay(step), 3)
+            out[name]["ms_under_torch_compile"] = _time_compiled(ff, lambda fn: fn(x).backward(dy), step)
         del ff, holder
     el = M * HIDDEN
     a = torch.randn((M, HIDDEN), device=dev, dtype=torch.bfloat16)
@@ -1104,6 +1143,8 @@ def time_expert_block(dev, recipe_mode, counts):
         torch.cuda.synchronize()
         ms = s.elapsed_time(e) / 5
         out[name] = {"ms": round(ms, 3), "TFLOP/s": round(18.0 * routed * dim * hid / ms / 1e9, 1)}
+        if fuse:
+            out[name]["ms_under_torch_compile"] = _time_compiled(ex, lambda fn: fn(x, counts).backward(dy), step)
         del ex, holder
     return out
 

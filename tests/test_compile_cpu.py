@@ -90,6 +90,20 @@ def test_traced_linear_leaves_out_the_casts_no_gradient_needs():
     assert all(t.numel() == 0 for t in node.meta["example_value"][1:])
 
 
+def test_weights_converted_before_the_dtype_change_still_trace():
+    """The reference converts first and moves / casts the model afterwards
+    (torchtitan/trainer.py:272-276 then :399-418): ``module.to(dtype)`` swaps the data of the
+    converted parameter in place, and nothing of the parameter may keep the old dtype (a tracer
+    compares a tensor and its base with their fake twins)."""
+    lin = Linear.Config().build(in_features=64, out_features=96)
+    lin.weight = wrap_parameter(lin.weight, MXFP8Config("rceil"))
+    assert isinstance(lin.weight, nn.Parameter) and lin.weight._base is None
+    lin.to(torch.bfloat16)
+    assert lin.weight.dtype == torch.bfloat16 and isinstance(lin.weight, MXFP8TrainingWeight)
+    gm = _trace(lin, torch.randn(32, 64, dtype=torch.bfloat16))
+    assert _count_fwd(gm) == 1
+
+
 def test_feed_forward_block_traces_as_three_operators():
     """Under a tracer the block takes the three-linears route (the fused block functions are
     eager-only), silu and the product stay ordinary graph nodes."""

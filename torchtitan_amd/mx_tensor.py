@@ -519,15 +519,28 @@ class MXFP8TrainingWeight(torch.Tensor):
         data = self.as_subclass(torch.Tensor).detach().clone(memory_format=torch.preserve_format)
         out = MXFP8TrainingWeight(data, self.mx_config)
         if getattr(self, "_is_param", False):
-            out = torch.nn.Parameter(out, requires_grad=self.requires_grad)
+            out = _as_parameter(data, self.mx_config, self.requires_grad)
         else:
             out.requires_grad_(self.requires_grad)
         memo[id(self)] = out
         return out
 
 
+def _as_parameter(data: torch.Tensor, cfg: MXFP8Config, requires_grad: bool) -> "MXFP8TrainingWeight":
+    """A converted weight that is an ``nn.Parameter`` (``isinstance`` holds through the
+    ``_is_param`` mark ``nn.Parameter`` itself puts on tensor subclasses), sharing `data`'s
+    storage.  Built directly rather than through ``nn.Parameter(wrapper)``: that detaches the
+    wrapper, and the result is a view whose base keeps the dtype and device of conversion time
+    when ``module.to(...)`` later swaps the parameter's data -- a tracer that checks a tensor's
+    base against its fake twin then refuses the parameter."""
+    t = torch.Tensor._make_subclass(MXFP8TrainingWeight, data, requires_grad)
+    t.mx_config = cfg
+    t._is_param = True
+    return t
+
+
 def _rebuild_parameter(data: torch.Tensor, cfg: MXFP8Config, requires_grad: bool):
-    return torch.nn.Parameter(MXFP8TrainingWeight(data, cfg), requires_grad=requires_grad)
+    return _as_parameter(data, cfg, requires_grad)
 
 
 # views, casts, detach and clone of a weight are still that weight, and so is the storage that
@@ -566,4 +579,4 @@ def wrap_parameter(param: torch.nn.Parameter, cfg: MXFP8Config) -> torch.nn.Para
     """A Parameter of type MXFP8TrainingWeight sharing `param`'s storage."""
     if isinstance(param.data, MXFP8TrainingWeight) or isinstance(param, MXFP8TrainingWeight):
         return param
-    return torch.nn.Parameter(MXFP8TrainingWeight(param.data, cfg), requires_grad=param.requires_grad)
+    return _as_parameter(param.data, cfg, param.requires_grad)
