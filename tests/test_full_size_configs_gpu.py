@@ -6,7 +6,10 @@
 * One layer of the 1.7B Qwen3-style policy (torchtitan/models/qwen3/__init__.py:120-150): dim 2048,
   16 heads / 8 KV heads of 128, FFN 6144, over the 147 456 packed tokens of a policy step, then
   the MXFP8 hand-over of a 28-layer stack of those weights, and the token log-probabilities at the
-  real vocabulary over more rows than one backward launch covers.
+  real vocabulary over more rows than one backward launch covers; and the policy step composed:
+  packed sequences of uneven lengths through two such layers and the language-model head into the
+  policy-gradient loss (torchtitan/experiments/rl/unified/actors/utils.py:56-147), backward, an
+  optimizer step and the hand-over.
 
 No CPU pass can follow these sizes, so each result is checked three ways: (1) row blocks of the
 output equal the same kernels run on the slice alone, bit for bit (every row of a cast or a GEMM
@@ -123,12 +126,15 @@ def test_llama3_8b_block_linears_at_seq_8192(device, name):
 
 # ---- the whole block ---------------------------------------------------------------------------
 class _Attention(nn.Module):
-    def __init__(self, dim, heads, kv_heads):
+    def __init__(self, dim, heads, kv_heads, qk_norm_eps=None):
         super().__init__()
         self.dim, self.heads, self.kv_heads, self.hd = dim, heads, kv_heads, dim // heads
         mk = lambda i, o: Linear.Config().build(in_features=i, out_features=o)
         self.wq, self.wo = mk(dim, dim), mk(dim, dim)
         self.wk, self.wv = mk(dim, kv_heads * self.hd), mk(dim, kv_heads * self.hd)
+        # Qwen3 normalises q and k per head in front of the rotation (torchtitan/models/qwen3/__init__.py:120-150)
+        self.q_norm = nn.RMSNorm(self.hd, eps=qk_norm_eps) if qk_norm_eps is not None else None
+        self.k_norm = nn.RMSNorm(self.hd, eps=qk_norm_eps) if qk_norm_eps is not None else None
 
     def qkv(self, x, norm):
         qkv_w = (self.wq.weight, self.wk.weight, self.wv.weight)
@@ -141,6 +147,8 @@ class _Attention(nn.Module):
         B, S, _ = q.shape
         q = q.view(B, S, self.heads, self.hd)
         k, v = k.view(B, S, self.kv_heads, self.hd), v.view(B, S, self.kv_heads, self.hd)
+        if self.q_norm is not None:
+            q, k = self.q_norm(q), self.k_norm(k)
         cos, sin = rope
 
         def rot(t):  # rotate pairs (even, odd) of the head dimension
@@ -158,9 +166,9 @@ class _Attention(nn.Module):
 
 
 class _Block(nn.Module):
-    def __init__(self, dim, heads, kv_heads, ffn, eps):
+    def __init__(self, dim, heads, kv_heads, ffn, eps, qk_norm=False):
         super().__init__()
-        self.attention = _Attention(dim, heads, kv_heads)
+        self.attention = _Attention(dim, heads, kv_heads, eps if qk_norm else None)
         self.feed_forward = FeedForward.Config(hidden_dim=ffn).build(dim=dim)
         self.attention_norm = nn.RMSNorm(dim, eps=eps)
         self.ffn_norm = nn.RMSNorm(dim, eps=eps)
@@ -265,6 +273,8 @@ def test_llama3_8b_block_at_seq_8192(device, norms_in_casts):
         # the whole block
         want = ref(xd[:, :head], rope_head)
         errs["block"] = err(y.detach()[:, :head], want)
+        # and without the residual stream, which carries most of the output's norm
+        errs["block_minus_input"] = err(y.detach()[:, :head] - xd[:, :head], want - xd[:, :head])
         print(f"rel-L2 against the block built from oracle linears: {errs}", flush=True)
         assert errs["block"] <= 8e-2, errs
 
@@ -373,3 +383,153 @@ def test_token_log_probs_at_the_real_vocabulary_over_many_rows(device):
     assert bool((mags[g != 0] > 0).all())
     # sum_v dlogits[r, v] = g[r] (1 - sum softmax) ~ 0 up to the bf16 rounding of 151 936 entries
     assert float((sums.abs() / g.abs().clamp_min(1e-3)).max()) < 0.05
+
+
+def test_policy_step_composed_at_real_layer_shapes(device):
+    """BASELINE configs[4] composed, at the real layer shapes on two layers: 16 sequences (2 prompts
+    x 8 samples) of uneven lengths uniform in [256, 2048] with random token ids below 151 936,
+    each through embedding -> two Qwen3-1.7B-shaped layers (dim 2048, 16 heads / 8 KV heads of
+    128 with q/k norms, FFN 6144, all seven linears MXFP8, the SwiGLU block fused) -> norm ->
+    language-model head at the full vocabulary -> fused token log-probabilities, into
+    `compute_policy_gradient_loss` with advantages = reward - group mean; backward; an optimizer
+    step; the MXFP8 hand-over of the updated weights.
+
+    Checked: the loss and its metrics against the float64 oracle on the model's own log-probs; one
+    sequence's log-probs against the oracle's log-softmax of the same logits; on the first 256
+    tokens of the longest sequence every stage of both layers against the same stage built from
+    oracle linears on identical inputs (as for the Llama block above); every gradient finite and
+    non-zero and the same from a second run; the payload of sampled weights bit-exact against the
+    oracle's cast of the updated weight."""
+    import math
+
+    from torchtitan_amd.rl import compute_policy_gradient_loss, token_log_probs
+
+    dim, heads, kv_heads, ffn, vocab, eps, head = 2048, 16, 8, 6144, 151936, 1e-6, 256
+
+    class PolicyLM(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.tok_embeddings = nn.Embedding(vocab, dim)
+            self.layers = nn.ModuleList([_Block(dim, heads, kv_heads, ffn, eps, qk_norm=True) for _ in range(2)])
+            self.norm = nn.RMSNorm(dim, eps=eps)
+            self.output = Linear.Config().build(in_features=dim, out_features=vocab)
+            self.hidden = None  # inputs of the layers of the last forward, for the stage checks
+
+        def forward(self, tokens, attention_masks=None):
+            h = self.tok_embeddings(tokens)
+            S = h.shape[1]
+            pad = -S % 32  # the MXFP8 linears take multiples of 32 tokens; causal: real positions do not see the padding
+            if pad:
+                h = torch.cat((h, h.new_zeros((1, pad, dim))), dim=1)
+            rope = _rope(S + pad, dim // heads, 1000000.0, h.device)
+            self.hidden = []
+            for layer in self.layers:
+                self.hidden.append(h.detach())
+                h = layer(h, rope)
+            return self.output(self.norm(h[:, :S]))
+
+    torch.manual_seed(15)
+    model = PolicyLM()
+    box = ModelConvertersContainer.Config(
+        converters=[MXFP8Converter.Config(fqns=["attention", "feed_forward"], recipe_name="mxfp8_rceil")]
+    ).build(parallel_dims=None, model_compile_enabled=False)
+    box.convert(model)
+    model.to(device).to(torch.bfloat16)
+    with torch.no_grad():
+        for m in model.modules():
+            if isinstance(m, nn.Linear):
+                m.weight.normal_(0.0, 0.02)
+        model.tok_embeddings.weight.normal_(0.0, 1.0)
+    converted = {n: p for n, p in model.named_parameters() if isinstance(p, MXFP8TrainingWeight)}
+    assert len(converted) == 14 and "output.weight" not in converted
+
+    rng = np.random.default_rng(21)
+    total_len = rng.integers(256, 2049, 16)
+    total_len[3] = 2048  # one sequence at the upper end, one that needs padding to 32
+    total_len[5] = 333
+    prompts, gens = [], []
+    for i, L in enumerate(total_len):
+        p_len = int(rng.integers(16, 65)) if i % 8 else 32  # samples of a group share a prompt length
+        ids = rng.integers(0, vocab, int(L)).tolist()
+        prompts.append(ids[:p_len])
+        gens.append(ids[p_len:])
+    rewards = torch.tensor(rng.standard_normal(16), dtype=torch.float32)
+    adv = (rewards.view(2, 8) - rewards.view(2, 8).mean(dim=1, keepdim=True)).view(-1)
+
+    with torch.no_grad():  # the reference policy's log-probs: the same model, shifted a little
+        ref = []
+        for i, (p, g) in enumerate(zip(prompts, gens)):
+            logits = model(torch.tensor([p + g], device=device))[0, len(p) - 1:len(p) - 1 + len(g)]
+            tgt = torch.tensor(g, device=device)
+            lp = token_log_probs(logits, tgt)
+            ref.append(lp + 0.05 * torch.randn(lp.shape, device=device, generator=None))
+            if i == 5:  # one sequence against the oracle's float64 log-softmax of the same logits (sampled rows)
+                rows = np.sort(rng.choice(len(g), size=24, replace=False))
+                want, _ = mo.token_log_probs(bits_of(logits[torch.from_numpy(rows).to(device)]), np.array(g)[rows])
+                assert np.abs(lp[torch.from_numpy(rows).to(device)].cpu().numpy() - want).max() <= 1e-5
+
+    def step():
+        for p in model.parameters():
+            p.grad = None
+        total, metrics, lps = compute_policy_gradient_loss(model, gens, prompts, adv, ref)
+        total.backward()
+        return total, metrics, lps
+
+    total, metrics, lps = step()
+    o_total, o_m = mo.policy_gradient_loss([l.detach().cpu().numpy() for l in lps], [r.cpu().numpy() for r in ref],
+                                           adv.numpy())
+    assert math.isclose(total.item(), o_total, rel_tol=1e-4, abs_tol=1e-5)
+    for k in ("pg_loss", "entropy", "kl_div", "ratio_mean"):
+        assert math.isclose(metrics[k], o_m[k], rel_tol=1e-3, abs_tol=1e-5), k
+    grads = {n: p.grad.clone() for n, p in model.named_parameters()}
+    for n, gr in grads.items():
+        assert torch.isfinite(gr).all() and float(gr.abs().max()) > 0, n
+    total2, _, _ = step()
+    assert total2.item() == total.item()
+    for n, p in model.named_parameters():
+        assert torch.equal(p.grad, grads[n]), n
+
+    # stage by stage on the first 256 tokens of the longest sequence, inputs as the model produced them
+    with torch.no_grad():
+        i = 3
+        model(torch.tensor([prompts[i] + gens[i]], device=device))
+        rope = _rope(2048, dim // heads, 1000000.0, device)
+        rope_head = (rope[0][:, :head], rope[1][:, :head])
+        err = lambda got, want: rel_l2(got.float().cpu().numpy(), want.float().cpu().numpy())
+        for li, (blk, xd) in enumerate(zip(model.layers, model.hidden)):
+            ref_blk = _Block(dim, heads, kv_heads, ffn, eps, qk_norm=True).to(device).to(torch.bfloat16)
+            ref_blk.load_state_dict(blk.state_dict())
+            for parent, names in ((ref_blk.attention, ("wq", "wk", "wv", "wo")), (ref_blk.feed_forward, ("w1", "w2", "w3"))):
+                for nme in names:
+                    setattr(parent, nme, _OracleLinear(getattr(parent, nme).weight.detach()))
+            errs = {}
+            for name, got, want in zip(("wq", "wk", "wv"), blk.attention.qkv(xd, blk.attention_norm),
+                                       ref_blk.attention.qkv(xd[:, :head], ref_blk.attention_norm)):
+                errs[name] = err(got[:, :head], want)
+                assert errs[name] <= TOL, (li, name, errs)
+            o = blk.attention.attend(*blk.attention.qkv(xd, blk.attention_norm), rope)
+            errs["wo"] = err(blk.attention.wo(o)[:, :head], ref_blk.attention.wo(o[:, :head]))
+            assert errs["wo"] <= TOL, (li, errs)
+            h = xd + blk.attention.wo(o)
+            errs["ffn"] = err(blk.ffn(h)[:, :head], ref_blk.ffn(h[:, :head]))
+            assert errs["ffn"] <= 6e-3, (li, errs)
+            # the layer without its residual stream (which would hide everything else)
+            errs["layer_minus_input"] = err(blk(xd, rope)[:, :head] - xd[:, :head], ref_blk(xd[:, :head], rope_head) - xd[:, :head])
+            print(f"layer {li}: rel-L2 against the stages built from oracle linears: {errs}", flush=True)
+            assert errs["layer_minus_input"] <= 3e-2, (li, errs)
+            del ref_blk
+
+    # optimizer step, then the hand-over of the updated weights
+    with torch.no_grad():
+        for p in model.parameters():
+            p.add_(p.grad, alpha=-1.0)
+    box.post_optimizer_hook(model)
+    payload = export_mxfp8_state_dict(model)
+    for name in ("layers.0.attention.wk.weight", "layers.1.feed_forward.w2.weight", "layers.1.feed_forward.w1.weight"):
+        p = converted[name]
+        plain = p.detach().as_subclass(torch.Tensor)
+        pick = torch.from_numpy(np.sort(rng.choice(p.shape[0], size=16, replace=False))).to(device)
+        c, s_ = mo.cast_dim0(bits_of(plain[pick]), mo.RCEIL)
+        assert np.array_equal(payload[name]["codes"][pick].cpu().numpy(), c), name
+        assert np.array_equal(payload[name]["scales"][pick].cpu().numpy(), s_), name
+    assert set(payload) >= set(converted)
