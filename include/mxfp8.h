@@ -79,6 +79,18 @@ int mx_cast_dim0_dim1(const void* x, int64_t rows, int64_t cols, int64_t ldx, ui
                       uint8_t* scales, uint8_t* codes_t, uint8_t* scales_t, int scale_mode,
                       int scale_order, void* stream);
 
+/* mx_cast_dim0_dim1 with a row pitch for each code matrix: row r of the row-wise codes starts at
+ * codes + r * ld_codes (ld_codes >= cols), row c of the column-wise codes at
+ * codes_t + c * ld_codes_t (ld_codes_t >= rows); both multiples of 16, the bytes between the
+ * rows are left alone.  Scales as ever.  Why: codes whose rows lie a multiple of 4 KB apart put
+ * the lines a GEMM fetches together (one K block of many rows) on few channels of the L2; a
+ * pitch of row length + 128 spreads them.  Inputs the tile kernel does not take (x not 16-byte
+ * aligned, cols % 8, ldx % 8) return MX_ERR_UNSUPPORTED: the caller then casts densely.  Same
+ * reference anchors as mx_cast_dim0 / mx_cast_dim1. */
+int mx_cast_dim0_dim1_ld(const void* x, int64_t rows, int64_t cols, int64_t ldx, uint8_t* codes,
+                         int64_t ld_codes, uint8_t* scales, uint8_t* codes_t, int64_t ld_codes_t,
+                         uint8_t* scales_t, int scale_mode, int scale_order, void* stream);
+
 /* Batched forms for 3-D expert weights x [batch, rows, cols] (dense, matrix stride rows*ldx):
  * every matrix is cast on its own; outputs are [batch, cols, rows] codes (and [batch, rows,
  * cols] for the fused form) with one scale block per matrix, each laid out as for the
@@ -234,6 +246,13 @@ int64_t mx_gemm_nt_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int mx_gemm_nt_ws(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                   const uint8_t* b_scales, void* d, int64_t M, int64_t N, int64_t K, int64_t ldd,
                   void* workspace, int64_t workspace_bytes, void* stream);
+
+/* mx_gemm_nt / mx_gemm_nt_ws for operands whose rows lie `ldk` >= K bytes apart (a multiple of 16;
+ * of 128 for the persistent kernel), e.g. the codes mx_cast_dim0_dim1_ld writes.  workspace may be
+ * NULL (then as mx_gemm_nt).  Same reference anchor as mx_gemm_nt. */
+int mx_gemm_nt_ld(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                  const uint8_t* b_scales, void* d, int64_t M, int64_t N, int64_t K, int64_t ldk,
+                  int64_t ldd, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* mx_gemm_nt_ws for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The

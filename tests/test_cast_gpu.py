@@ -5,7 +5,7 @@ import torch
 
 from oracle import mx_oracle as mo
 from tests.helpers import bf16_from_bits, bits_of, randn_bits, u8
-from torchtitan_amd import ops
+from torchtitan_amd import _lib, ops
 
 pytestmark = pytest.mark.gpu
 
@@ -434,3 +434,30 @@ def test_rms_norm_fused_cast(device, mode_name, mode, shape):
         assert np.array_equal(u8(q1.codes), c1) and np.array_equal(u8(q1.scales).reshape(-1), s1.reshape(-1))
         p0, p1, _, none = ops.rms_norm_to_mx(x, w, 1e-5, mode_name, order)
         assert none is None and torch.equal(p0.codes, q0.codes) and torch.equal(p1.scales, q1.scales)
+
+
+@pytest.mark.parametrize("R,C,pad", [(128, 256, 128), (4096, 4096, 128), (96, 160, 16), (1024, 14336, 384)])
+def test_fused_cast_with_row_pitches_writes_the_same_codes(device, R, C, pad):
+    """Codes whose rows lie `pad` bytes further apart than they are long: every row equals the
+    dense cast's, the bytes between the rows are left alone, scales are unchanged."""
+    torch.manual_seed(R + C)
+    x = torch.randn(R, C, device=device, dtype=torch.bfloat16)
+    x[3, 5] = 300.0
+    for mode in ("floor", "rceil"):
+        want0, want1 = ops.to_mx_dim0_dim1(x, mode, ops.MX_SCALES_MFMA)
+        got0, got1 = ops.to_mx_dim0_dim1(x, mode, ops.MX_SCALES_MFMA, pitch_pad=pad)
+        assert got0.codes.stride(0) == C + pad and got1.codes.stride(0) == R + pad
+        assert torch.equal(got0.codes, want0.codes) and torch.equal(got1.codes, want1.codes)
+        assert torch.equal(got0.scales, want0.scales) and torch.equal(got1.scales, want1.scales)
+    # between the rows: untouched
+    lib = _lib.load()
+    base0 = torch.full((R, C + pad), 0xAB, dtype=torch.uint8, device=device)
+    base1 = torch.full((C, R + pad), 0xCD, dtype=torch.uint8, device=device)
+    s0 = torch.empty_like(want0.scales)
+    s1 = torch.empty_like(want1.scales)
+    with torch.cuda.device(device):
+        st = lib.mx_cast_dim0_dim1_ld(ops._ptr(x), R, C, x.stride(0), ops._ptr(base0), C + pad, ops._ptr(s0),
+                                      ops._ptr(base1), R + pad, ops._ptr(s1), 1, ops.MX_SCALES_MFMA, ops._stream(x))
+    assert st == 0
+    assert bool((base0[:, C:] == 0xAB).all()) and bool((base1[:, R:] == 0xCD).all())
+    assert torch.equal(base0[:, :C], want0.codes) and torch.equal(base1[:, :R], want1.codes)

@@ -239,7 +239,8 @@ def test_per_op_checkpoint_policy_can_keep_gemm_outputs(device, fuse, monkeypatc
             y = checkpoint(ff, xi, use_reentrant=False,
                            context_fn=lambda: create_selective_checkpoint_contexts(policy))
         y.backward(dy)
-        runs[how] = (launches.count("mx_gemm_nt"),
+        # (mx_gemm_nt_ld: the same GEMM on operands whose rows carry the dense linear's pitch)
+        runs[how] = (launches.count("mx_gemm_nt") + launches.count("mx_gemm_nt_ld"),
                      [y.detach(), xi.grad] + [p.grad.clone() for p in ff.parameters()])
     assert [runs[h][0] for h in ("plain", "full", "per_op")] == [9, 12, 9]
     for how in ("full", "per_op"):

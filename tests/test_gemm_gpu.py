@@ -5,7 +5,7 @@ import torch
 
 from oracle import mx_oracle as mo
 from tests.helpers import bf16_from_bits, bits_of, randn_bits, rel_l2, u8
-from torchtitan_amd import ops
+from torchtitan_amd import _lib, ops
 
 pytestmark = pytest.mark.gpu
 
@@ -377,3 +377,32 @@ def test_two_products_fall_back_to_two_gemms_on_small_shapes(device):
     (d, d2), names = _launch_names(lambda: ops.mx_gemm_nt_shared_a(a, b, b2))
     assert names == ["mx_gemm_nt", "mx_gemm_nt"]
     assert torch.equal(d, ops.mx_gemm_nt(a, b)) and torch.equal(d2, ops.mx_gemm_nt(a, b2))
+
+
+@pytest.mark.parametrize("M,N,K", [(512, 384, 256), (300, 264, 128), (96, 64, 160), (2048, 1024, 4096), (768, 256, 16384)])
+def test_gemm_on_operands_with_a_row_pitch_equals_the_dense_gemm(device, M, N, K):
+    """Operand rows 128 bytes further apart than they are long (what the fused cast writes for the
+    dense linear): the same kernels on the same values, so bit-identical to dense operands, on the
+    persistent kernel, its split form and the small-shape tile kernels alike; operands whose
+    pitches differ are brought to one."""
+    rng = np.random.default_rng(M + N + K)
+    a = ops.to_mx_dim0(bf16_from_bits(randn_bits(rng, (M, K), outliers=1e-3), device), "rceil", ops.MX_SCALES_MFMA)
+    b = ops.to_mx_dim0(bf16_from_bits(randn_bits(rng, (N, K), std=0.02), device), "rceil", ops.MX_SCALES_MFMA)
+    want = ops.mx_gemm_nt(a, b)
+
+    def pitched(d, pad):
+        buf = torch.full((d.codes.shape[0], K + pad), 0x7F, dtype=torch.uint8, device=device)  # NaN codes between the rows
+        buf[:, :K] = d.codes
+        return ops.MXData(buf[:, :K], d.scales, d.scale_order)
+
+    (got, names) = _launch_names(lambda: ops.mx_gemm_nt(pitched(a, 128), pitched(b, 128)))
+    assert names == ["mx_gemm_nt_ld"] and torch.equal(got, want)
+    assert torch.equal(ops.mx_gemm_nt(pitched(a, 128), b), want)  # differing pitches: copies, then dense
+    # a pitch that is not a multiple of 128: the tile kernel, which never splits the contraction
+    odd = ops.mx_gemm_nt(pitched(a, 16), pitched(b, 16))
+    with torch.cuda.device(device):
+        split = int(_lib.load().mx_gemm_nt_workspace_bytes(M, N, K)) > 0
+    if split:
+        assert rel_l2(odd.float().cpu().numpy(), want.float().cpu().numpy()) <= 3e-4
+    else:
+        assert torch.equal(odd, want)

@@ -31,6 +31,7 @@ SIGNATURES = {
     "mx_cast_dim0": (c_int, [_P, _I, _I, _I, _P, _P, c_int, c_int, _P]),
     "mx_cast_dim1": (c_int, [_P, _I, _I, _I, _P, _P, c_int, c_int, _P]),
     "mx_cast_dim0_dim1": (c_int, [_P, _I, _I, _I, _P, _P, _P, _P, c_int, c_int, _P]),
+    "mx_cast_dim0_dim1_ld": (c_int, [_P, _I, _I, _I, _P, _I, _P, _P, _I, _P, c_int, c_int, _P]),
     "mx_cast_dim1_batched": (c_int, [_P, _I, _I, _I, _I, _P, _P, c_int, c_int, _P]),
     "mx_cast_dim0_dim1_batched": (c_int, [_P, _I, _I, _I, _I, _P, _P, _P, _P, c_int, c_int, _P]),
     "mx_cast_rows_gathered": (c_int, [_P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P, c_int, c_int, _P]),
@@ -48,6 +49,7 @@ SIGNATURES = {
     "mx_gemm_nt": (c_int, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "mx_gemm_nt_workspace_bytes": (_I, [_I, _I, _I]),
     "mx_gemm_nt_ws": (c_int, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _I, _P]),
+    "mx_gemm_nt_ld": (c_int, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _I, _P]),
     "mx_gemm_nt_static_max_bytes": (_I, []),
     "mx_gemm_nt_static": (c_int, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "mx_gemm_nt_pair": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),

@@ -516,7 +516,8 @@ __device__ __forceinline__ void emit_tile(
     uint8_t* __restrict__ codes_t, uint8_t* __restrict__ scales_t, uint8_t* lds_codes,
     uint8_t* lds_st, uint8_t* lds_sr, int64_t rows, int64_t cols, int64_t nblk, int64_t ks_n,
     int64_t nblk_t, int64_t ks_n_t, int64_t r0, int64_t c0, int64_t c, int rl0, int rows_left,
-    bool col_ok, int tid, int wave, int lane) {
+    bool col_ok, int tid, int wave, int lane, int64_t ldc, int64_t ldct) {
+  // ldc / ldct: bytes between rows of the row-wise / column-wise codes (>= cols / rows)
   constexpr int TR = 32 * WAVES, TC = 128, PITCH = TR + 16;
   // block maxima first: they also tell whether the wave holds any Inf / NaN
   uint32_t mr[8] = {0, 0, 0, 0, 0, 0, 0, 0}, mc[4] = {0, 0, 0, 0};
@@ -552,13 +553,13 @@ __device__ __forceinline__ void emit_tile(
       top = max(t & 0xFFFFu, t >> 16);
     }
   }
-  uint8_t* codes_row = ROW ? codes + (r0 + rl0) * cols + c : nullptr;
+  uint8_t* codes_row = ROW ? codes + (r0 + rl0) * ldc + c : nullptr;
   if (__builtin_amdgcn_ballot_w64(top >= 0x7F80u) == 0)
-    quantize_patch<MODE, ORDER, ROW, COL, WAVES, true>(v, mr, mc, codes_row, cols, rows_left,
+    quantize_patch<MODE, ORDER, ROW, COL, WAVES, true>(v, mr, mc, codes_row, ldc, rows_left,
                                                        col_ok, lds_codes, lds_st, lds_sr, wave,
                                                        lane, rl0);
   else
-    quantize_patch<MODE, ORDER, ROW, COL, WAVES, false>(v, mr, mc, codes_row, cols, rows_left,
+    quantize_patch<MODE, ORDER, ROW, COL, WAVES, false>(v, mr, mc, codes_row, ldc, rows_left,
                                                         col_ok, lds_codes, lds_st, lds_sr, wave,
                                                         lane, rl0);
   __syncthreads();
@@ -589,7 +590,7 @@ __device__ __forceinline__ void emit_tile(
       if (c0 + o < cols && r0 + seg * 16 < rows) {
         const u32x4 t = *reinterpret_cast<const u32x4*>(lds_codes + o * PITCH + seg * 16);
         __builtin_nontemporal_store(
-            t, reinterpret_cast<u32x4*>(codes_t + (c0 + o) * rows + r0 + seg * 16));
+            t, reinterpret_cast<u32x4*>(codes_t + (c0 + o) * ldct + r0 + seg * 16));
       }
     }
     if (ORDER == MX_SCALES_MFMA) {
@@ -652,6 +653,7 @@ struct TileExtras {
   int64_t src_rows = 0;
   uint32_t batch = 1;  // stacked independent matrices
   const float* row_scale = nullptr;  // GATHER: optional multiplier of every output row; GATE 3: rstd
+  int64_t ldc = 0, ldct = 0;  // bytes between rows of the row-wise / column-wise codes (0: dense)
 };
 
 // The gate-backward variant is bound by vector ALU work: four workgroups per CU (128 VGPRs).
@@ -682,13 +684,14 @@ __global__ __launch_bounds__(64 * WAVES, GATE == 2 ? 4 : 1) void cast_tile_kerne
   const uint32_t by_all = (sup / spr) * BY + in % BY;
   if (bx >= gx || by_all >= gy_all) return;
   const uint32_t bz = by_all / gy, by = by_all - bz * gy;
+  const int64_t ldc = ex.ldc ? ex.ldc : cols, ldct = ex.ldct ? ex.ldct : rows;
   x += bz * x_bstride;
   if (ROW) {
-    codes += bz * rows * cols;
+    codes += bz * rows * ldc;
     scales += bz * s_bstride;
   }
   if (COL) {
-    codes_t += bz * rows * cols;
+    codes_t += bz * cols * ldct;
     scales_t += bz * st_bstride;
   }
 
@@ -761,20 +764,20 @@ __global__ __launch_bounds__(64 * WAVES, GATE == 2 ? 4 : 1) void cast_tile_kerne
     }
     emit_tile<MODE, ORDER, ROW, COL, WAVES>(w, codes, scales, codes_t, scales_t, lds_codes, lds_st,
                                             lds_sr, rows, cols, nblk, ks_n, nblk_t, ks_n_t, r0, c0,
-                                            c, rl0, rows_left, col_ok, tid, wave, lane);
+                                            c, rl0, rows_left, col_ok, tid, wave, lane, ldc, ldct);
     __syncthreads();  // the staging buffers are reused by the second output
     if (ROW) {
-      codes += rows * cols;
+      codes += rows * ldc;
       scales += s_bstride;
     }
     if (COL) {
-      codes_t += rows * cols;
+      codes_t += cols * ldct;
       scales_t += st_bstride;
     }
   }
   emit_tile<MODE, ORDER, ROW, COL, WAVES>(v, codes, scales, codes_t, scales_t, lds_codes, lds_st,
                                           lds_sr, rows, cols, nblk, ks_n, nblk_t, ks_n_t, r0, c0, c,
-                                          rl0, rows_left, col_ok, tid, wave, lane);
+                                          rl0, rows_left, col_ok, tid, wave, lane, ldc, ldct);
 }
 
 // ------------------------------------------------------------------------------------
@@ -1013,6 +1016,39 @@ extern "C" int mx_cast_dim0_dim1_batched(const void* x, int64_t batch, int64_t r
   MX_DISPATCH_MODE_ORDER(cast_dim0_dim1_kernel, (const uint16_t*)x, rows, cols, ldx, codes,
                          scales, nblk, ks_n, codes_t, scales_t, nblk_t, ks_n_t, rows * ldx, s_b,
                          st_b);
+  return launch_status();
+}
+
+// The fused cast with a row pitch for each of its code outputs (scales are laid out as ever): rows of
+// codes that start at different positions within a 4 KB span of addresses spread the lines a GEMM
+// fetches together (the same K block of many rows) over the channels of the L2.
+extern "C" int mx_cast_dim0_dim1_ld(const void* x, int64_t rows, int64_t cols, int64_t ldx,
+                                    uint8_t* codes, int64_t ld_codes, uint8_t* scales,
+                                    uint8_t* codes_t, int64_t ld_codes_t, uint8_t* scales_t,
+                                    int scale_mode, int scale_order, void* stream) {
+  if (rows < 0 || cols < 0 || ldx < cols || ld_codes < cols || ld_codes_t < rows || bad_enums(scale_mode, scale_order))
+    return MX_ERR_INVALID_ARG;
+  if (rows == 0 || cols == 0) return MX_OK;
+  if (ld_codes == cols && ld_codes_t == rows)
+    return mx_cast_dim0_dim1_batched(x, 1, rows, cols, ldx, codes, scales, codes_t, scales_t, scale_mode,
+                                     scale_order, stream);
+  if (!x || !codes || !scales || !codes_t || !scales_t) return MX_ERR_INVALID_ARG;
+  if (rows % 32 || cols % 32 || ld_codes % 16 || ld_codes_t % 16 || ((uintptr_t)codes & 15) ||
+      ((uintptr_t)codes_t & 15) || ((uintptr_t)scales & 3) || ((uintptr_t)scales_t & 3))
+    return MX_ERR_ALIGNMENT;
+  const int64_t nblk = cols / 32, ks_n = (nblk + 1) / 2;
+  const int64_t nblk_t = rows / 32, ks_n_t = (nblk_t + 1) / 2;
+  const int64_t gx = (cols + kT - 1) / kT, tgy = (rows + kTileRows - 1) / kTileRows;
+  // only the tile kernel knows pitches: inputs it does not take are the caller's dense cast
+  if (!tile_ok(x, cols, ldx) || tile_grid_x(gx, tgy, true) > 0x7FFFFFFF) return MX_ERR_UNSUPPORTED;
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid = tile_grid(gx, tgy, 1, true), block(64 * MX_CAST_WAVES);
+  TileExtras ex = tile_batch(1);
+  ex.ldc = ld_codes;
+  ex.ldct = ld_codes_t;
+  MX_DISPATCH_TILE(true, true, 0, false, (const uint16_t*)x, rows, cols, ldx, codes, scales, nblk, ks_n,
+                   codes_t, scales_t, nblk_t, ks_n_t, rows * ldx, scale_bytes(rows, nblk, scale_order),
+                   scale_bytes(cols, nblk_t, scale_order), (uint32_t)gx, (uint32_t)tgy, ex);
   return launch_status();
 }
 

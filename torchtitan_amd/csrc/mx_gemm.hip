@@ -12,6 +12,7 @@ struct DenseArgs {
   const uint8_t* b_scales;
   uint16_t* d;
   int64_t M, N, K, ldd;
+  int64_t ldk;  // bytes between operand rows (>= K)
 };
 
 template <int BM, int BN>
@@ -22,9 +23,9 @@ __global__ __launch_bounds__(256, 1) void gemm_nt_kernel(DenseArgs p) {
   int64_t tm, tn;
   if (!map_tile(tiles_m, tiles_n, tm, tn)) return;
   const int64_t ks_n = (p.K / 32 + 1) / 2;
-  Operand A{p.a_codes + tm * BM * p.K, p.K, p.M - tm * BM,
+  Operand A{p.a_codes + tm * BM * p.ldk, p.ldk, p.M - tm * BM,
             p.a_scales + tm * (BM / 128) * ks_n * 256, ks_n};
-  Operand B{p.b_codes + tn * BN * p.K, p.K, p.N - tn * BN,
+  Operand B{p.b_codes + tn * BN * p.ldk, p.ldk, p.N - tn * BN,
             p.b_scales + tn * (BN / 128) * ks_n * 256, ks_n};
   Tile::run(smem, A, B, 0, p.K, p.d + tm * BM * p.ldd + tn * BN, p.ldd);
 }
@@ -49,13 +50,13 @@ using namespace mx;
 namespace mx {
 int launch_gemm_nt32(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                      const uint8_t* b_scales, void* d, int64_t M, int64_t N, int64_t K,
-                     int64_t ldd, hipStream_t st);
+                     int64_t ldk, int64_t ldd, hipStream_t st);
 }
 namespace mx {
 int splitk_slices(int64_t M, int64_t N, int64_t K);
 int launch_gemm_nt32_splitk(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                             const uint8_t* b_scales, void* d, int64_t M, int64_t N, int64_t K,
-                            int64_t ldd, int slices, void* workspace, hipStream_t st);
+                            int64_t ldk, int64_t ldd, int slices, void* workspace, hipStream_t st);
 }
 // Test hooks (include/mxfp8_debug.h), process-wide.
 // 0: pick by shape; 1 / 2: the 16x16x128 tile kernel with 256x256 / 128x128 tiles for every
@@ -85,17 +86,22 @@ static int check_dense(const uint8_t* a_codes, const uint8_t* a_scales, const ui
 }
 
 // What the persistent kernel (mx_gemm32.hip) needs beyond the general checks.
-static bool persistent_ok(const void* d, int64_t N, int64_t K, int64_t ldd) {
-  return !(K % 128 || (uint64_t)K * 256 > 0x7FFFFFFFull || N % 8 || ldd % 8 || ((uintptr_t)d & 15) ||
+static bool persistent_ok(const void* d, int64_t N, int64_t K, int64_t ldd, int64_t ldk = 0) {
+  if (ldk == 0) ldk = K;
+  return !(K % 128 || ldk % 128 || (uint64_t)ldk * 256 > 0x7FFFFFFFull || N % 8 || ldd % 8 || ((uintptr_t)d & 15) ||
            (uint64_t)ldd * 512 > 0x7FFFFFFFull);
 }
 
-extern "C" int mx_gemm_nt(const uint8_t* a_codes, const uint8_t* a_scales,
-                          const uint8_t* b_codes, const uint8_t* b_scales, void* d, int64_t M,
-                          int64_t N, int64_t K, int64_t ldd, void* stream) {
+// mx_gemm_nt with operand rows `ldk` bytes apart (ldk >= K, a multiple of 16).
+static int gemm_nt_pitched(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                           const uint8_t* b_scales, void* d, int64_t M, int64_t N, int64_t K, int64_t ldk,
+                           int64_t ldd, void* stream) {
   const int rc = check_dense(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd);
   if (rc != MX_OK || M == 0 || N == 0) return rc;
-  DenseArgs p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, M, N, K, ldd};
+  if (ldk < K) return MX_ERR_INVALID_ARG;
+  if (ldk % 16) return MX_ERR_ALIGNMENT;
+  if (256 * ldk > 0x7FFFFFFFll) return MX_ERR_UNSUPPORTED;
+  DenseArgs p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, M, N, K, ldd, ldk};
   hipStream_t st = (hipStream_t)stream;
   if (M <= 128 || N <= 128 || force_kernel == 2) return launch_dense<128, 128>(p, st);
   // Few 256x256 tiles leave most CUs of the persistent kernel idle when the contraction is not
@@ -105,8 +111,14 @@ extern "C" int mx_gemm_nt(const uint8_t* a_codes, const uint8_t* a_scales,
   if (num_cus == 0) num_cus = 256;
   const int64_t tiles256 = ((M + 255) / 256) * ((N + 255) / 256);
   if (force_kernel == 0 && tiles256 * 8 <= (int64_t)num_cus * 3) return launch_dense<128, 128>(p, st);
-  if (force_kernel == 1 || !persistent_ok(d, N, K, ldd)) return launch_dense<256, 256>(p, st);
-  return launch_gemm_nt32(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd, st);
+  if (force_kernel == 1 || !persistent_ok(d, N, K, ldd, ldk)) return launch_dense<256, 256>(p, st);
+  return launch_gemm_nt32(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldk, ldd, st);
+}
+
+extern "C" int mx_gemm_nt(const uint8_t* a_codes, const uint8_t* a_scales,
+                          const uint8_t* b_codes, const uint8_t* b_scales, void* d, int64_t M,
+                          int64_t N, int64_t K, int64_t ldd, void* stream) {
+  return gemm_nt_pitched(a_codes, a_scales, b_codes, b_scales, d, M, N, K, K, ldd, stream);
 }
 
 namespace mx {
@@ -178,18 +190,27 @@ extern "C" int64_t mx_gemm_nt_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   return s > 1 ? (int64_t)s * M * N * 4 : 0;
 }
 
+extern "C" int mx_gemm_nt_ld(const uint8_t* a_codes, const uint8_t* a_scales,
+                             const uint8_t* b_codes, const uint8_t* b_scales, void* d, int64_t M,
+                             int64_t N, int64_t K, int64_t ldk, int64_t ldd, void* workspace,
+                             int64_t workspace_bytes, void* stream) {
+  const int rc = check_dense(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd);
+  if (rc != MX_OK || M == 0 || N == 0) return rc;
+  if (ldk < K) return MX_ERR_INVALID_ARG;
+  const int64_t need = force_kernel == 0 ? mx_gemm_nt_workspace_bytes(M, N, K) : 0;
+  if (need == 0 || !workspace || workspace_bytes < need || ((uintptr_t)workspace & 15) ||
+      !persistent_ok(d, N, K, ldd, ldk))
+    return gemm_nt_pitched(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldk, ldd, stream);
+  return launch_gemm_nt32_splitk(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldk, ldd,
+                                 (int)(need / (M * N * 4)), workspace, (hipStream_t)stream);
+}
+
 extern "C" int mx_gemm_nt_ws(const uint8_t* a_codes, const uint8_t* a_scales,
                              const uint8_t* b_codes, const uint8_t* b_scales, void* d, int64_t M,
                              int64_t N, int64_t K, int64_t ldd, void* workspace,
                              int64_t workspace_bytes, void* stream) {
-  const int rc = check_dense(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd);
-  if (rc != MX_OK || M == 0 || N == 0) return rc;
-  const int64_t need = force_kernel == 0 ? mx_gemm_nt_workspace_bytes(M, N, K) : 0;
-  if (need == 0 || !workspace || workspace_bytes < need || ((uintptr_t)workspace & 15) ||
-      !persistent_ok(d, N, K, ldd))
-    return mx_gemm_nt(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd, stream);
-  return launch_gemm_nt32_splitk(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd,
-                                 (int)(need / (M * N * 4)), workspace, (hipStream_t)stream);
+  return mx_gemm_nt_ld(a_codes, a_scales, b_codes, b_scales, d, M, N, K, K, ldd, workspace, workspace_bytes,
+                       stream);
 }
 
 // ---- the split GEMM for callers that cannot allocate -------------------------------------------
@@ -229,6 +250,6 @@ extern "C" int mx_gemm_nt_static(const uint8_t* a_codes, const uint8_t* a_scales
     return mx_gemm_nt(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd, stream);
   void* ws = scratch_of_current_device();
   if (!ws) return MX_ERR_LAUNCH;
-  return launch_gemm_nt32_splitk(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd,
+  return launch_gemm_nt32_splitk(a_codes, a_scales, b_codes, b_scales, d, M, N, K, K, ldd,
                                  (int)(need / (M * N * 4)), ws, (hipStream_t)stream);
 }

@@ -90,6 +90,9 @@ struct Gemm32Args {
   // gradients dW1 = d(h1)^T x and dW3 = d(h3)^T x).
   int32_t two = 0;
   uint16_t* d2 = nullptr;
+  // kDense, kSplitK: bytes between the rows of A and of B (both operands' rows are K bytes long
+  // and may lie further apart, by a multiple of 128); 0 = K
+  int64_t ldk = 0;
 };
 enum Gemm32Two { kTwoNone = 0, kTwoB = 1, kTwoA = 2 };
 
@@ -189,6 +192,13 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   const int li = lane & 15, lj = lane >> 4;
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void_t*)smem;  // LDS byte address of the ring
   const uint32_t K = (uint32_t)p.K;  // bytes per operand row; a multiple of 128 for this kernel
+#ifndef MX_ABL_ROW_PAD  // timing ablation: the rows of a tile are read this many bytes further apart than they lie
+#define MX_ABL_ROW_PAD 0
+#endif
+  // Kp: bytes from one operand row to the next.  A pitch that is not a multiple of 4 KB spreads the
+  // lines a block's copies fetch together (one K block of 512 rows) over the channels of the L2.
+  const uint32_t Kp = ((MODE == kDense || MODE == kSplitK) && p.ldk ? (uint32_t)p.ldk : K) + MX_ABL_ROW_PAD;
+  const int64_t Kt = (MODE == kDense || MODE == kSplitK) && p.ldk ? p.ldk : p.K;  // ... as the tile origins use it
   const uint32_t ks_n = K / kK32;    // 64-deep steps per 128-row scale group
   // tile rows / columns of one product, and of the launch (p.two: the second product's tile
   // columns or rows come behind the first's; grouped launches cover columns [tn0, tn0 + tn_cnt))
@@ -362,8 +372,8 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       r.a = a_codes + (int64_t)tm * kT32 * K;
       r.b = b_codes + (int64_t)(tn & 3) * kT32 * K;
 #else
-      r.a = a_codes + (int64_t)tm * kT32 * K;
-      r.b = b_codes + (int64_t)tn * kT32 * K;
+      r.a = a_codes + (int64_t)tm * kT32 * Kt;
+      r.b = b_codes + (int64_t)tn * kT32 * Kt;
 #endif
       r.sa = a_scales + (int64_t)(tm * 2) * ks_n * 256;
       r.sb = b_scales + (int64_t)(tn * 2) * ks_n * 256;
@@ -404,8 +414,8 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       const uint32_t blocks = K / kKB, per = (blocks + G - 1) / G;
       const uint32_t b_lo = g * per, b_hi = b_lo + per < blocks ? b_lo + per : blocks;
       const uint32_t lo = b_lo * kKB;
-      r.a = a_codes + (int64_t)tm * kT32 * K + lo;
-      r.b = b_codes + (int64_t)tn * kT32 * K + lo;
+      r.a = a_codes + (int64_t)tm * kT32 * Kt + lo;
+      r.b = b_codes + (int64_t)tn * kT32 * Kt + lo;
       r.sa = a_scales + ((int64_t)(tm * 2) * ks_n + (lo >> 6)) * 256;
       r.sb = b_scales + ((int64_t)(tn * 2) * ks_n + (lo >> 6)) * 256;
       float* part = reinterpret_cast<float*>(p.d) +
@@ -523,10 +533,6 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   // chunk that belongs at physical chunk l%8 of that row:
   // c = (l%8) ^ ((row & 2) | ((row & 8) >> 1)), see the fragment reads
   const uint32_t c_even = (lane & 7) ^ ((lane >> 3) & 2);
-#ifndef MX_ABL_ROW_PAD  // timing ablation: the rows of a tile are read this many bytes further apart than they lie
-#define MX_ABL_ROW_PAD 0
-#endif
-  const uint32_t Kp = K + MX_ABL_ROW_PAD;
   const uint32_t v_even = (uint32_t)(lane >> 3) * Kp + c_even * 16;
   // (odd units: v_even ^ 64 -- K is a multiple of 128, so bit 6 belongs to the chunk alone)
   // LDS -> VGPR: lane (li = l & 15, lj = l >> 4) of a 16-row sub-tile reads chunks lj and lj + 4 of
@@ -586,8 +592,8 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       //  the K range is exact because nblocks is.)  A tile without a K range reads nothing:
       // its one block arrives as zeros, scales included.
       const bool none = MODE != kDense && t.empty;
-      ra = make_rsrc(t.a, none ? 0 : t.rows_a * K - t.koff);
-      rb = make_rsrc(t.b, none ? 0 : t.rows_b * K - t.koff);
+      ra = make_rsrc(t.a, none ? 0 : t.rows_a * (int64_t)Kp - t.koff);
+      rb = make_rsrc(t.b, none ? 0 : t.rows_b * (int64_t)Kp - t.koff);
       // wave 0 copies the scales of A's two 128-row groups, wave 2 those of B's (one copy per
       // block each: lanes 0-31 fetch group 0, lanes 32-63 group 1); a group beyond the operand
       // is cut off by the range and arrives as zeros
@@ -1115,8 +1121,9 @@ void set_debug_prof(uint64_t* buf) { debug_prof = buf; }
 
 int launch_gemm_nt32(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                      const uint8_t* b_scales, void* d, int64_t M, int64_t N, int64_t K,
-                     int64_t ldd, hipStream_t st) {
+                     int64_t ldk, int64_t ldd, hipStream_t st) {
   Gemm32Args p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, M, N, K, ldd, nullptr, 0, 0, 0, debug_prof};
+  p.ldk = ldk;
   const int64_t nb = ((M + kT32 - 1) / kT32) * ((N + kT32 - 1) / kT32);
 #ifdef MX_TIMING_BUILD
   if (debug_prof) return launch32<kDense, true>(p, nb, st);
@@ -1195,10 +1202,11 @@ int splitk_slices(int64_t M, int64_t N, int64_t K) {
 // D = sum over slices, through `workspace` (S * M * N floats).
 int launch_gemm_nt32_splitk(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                             const uint8_t* b_scales, void* d, int64_t M, int64_t N, int64_t K,
-                            int64_t ldd, int slices, void* workspace, hipStream_t st) {
+                            int64_t ldk, int64_t ldd, int slices, void* workspace, hipStream_t st) {
   const int64_t tiles_n = (N + kT32 - 1) / kT32, tiles = ((M + kT32 - 1) / kT32) * tiles_n;
   Gemm32Args p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)workspace, M, N, K, N, nullptr,
                slices, 0, (int32_t)tiles_n, nullptr};
+  p.ldk = ldk;
   const int rc = launch32<kSplitK, false>(p, tiles * slices, st);
   if (rc != MX_OK) return rc;
   const int64_t threads = M * (N / 8);

@@ -102,16 +102,18 @@ def clear_cast_cache() -> None:
     _cast_cache.clear()
 
 
-def _cast_activation(x2: torch.Tensor, src: torch.Tensor, mode: str, need_cols: bool):
-    """(row-wise, column-wise or None) MXFP8 forms of the 2-D bf16 activation `x2`."""
-    hit = _cast_cache.get(src, mode)
+def _cast_activation(x2: torch.Tensor, src: torch.Tensor, mode: str, need_cols: bool, pitch_pad: int = 0):
+    """(row-wise, column-wise or None) MXFP8 forms of the 2-D bf16 activation `x2`.  `pitch_pad`:
+    see `ops.to_mx_dim0_dim1`; callers that feed anything but `ops.mx_gemm_nt` leave it 0."""
+    key = (mode, pitch_pad)
+    hit = _cast_cache.get(src, key)
     if hit is not None and (hit[1] is not None or not need_cols):
         return hit
     if need_cols and x2.shape[0] % ops.BLOCK == 0:
-        rows, cols = ops.to_mx_dim0_dim1(x2, mode, MX_SCALES_MFMA)
+        rows, cols = ops.to_mx_dim0_dim1(x2, mode, MX_SCALES_MFMA, pitch_pad)
     else:
         rows, cols = ops.to_mx_dim0(x2, mode, MX_SCALES_MFMA), None
-    _cast_cache.put(src, mode, (rows, cols))
+    _cast_cache.put(src, key, (rows, cols))
     return rows, cols
 
 
@@ -160,23 +162,29 @@ class _WeightCastCache:
 _weight_cache = _WeightCastCache()
 
 
-def _cast_weight(w: torch.Tensor, mode: str, need_cols: bool, cfg: MXFP8Config):
+def _cast_weight(w: torch.Tensor, mode: str, need_cols: bool, cfg: MXFP8Config, pitch_pad: int = 0):
     """(row-wise, column-wise or None) MXFP8 forms of a weight [N, K] or stacked [G, N, K], MFMA
-    scale order.  The column-wise form exists when asked for and N is a multiple of 32."""
+    scale order.  The column-wise form exists when asked for and N is a multiple of 32.
+    `pitch_pad` (2-D weights, both forms asked for): see `ops.to_mx_dim0_dim1`."""
     cached = cfg.cache_weight_casts
+    mode_key = mode
+    if pitch_pad:
+        mode = (mode, pitch_pad)  # the cache keeps padded and dense casts apart
     if cached:
         hit = _weight_cache.get(w, mode)
         if hit is not None and (hit[1] is not None or not need_cols or w.shape[-2] % ops.BLOCK):
             return hit
         need_cols = True  # cast once in full, whoever asks first
+    key, mode = mode, mode_key
     wb = (w if w.dtype == torch.bfloat16 else w.to(torch.bfloat16)).contiguous()
     both = need_cols and wb.shape[-2] % ops.BLOCK == 0
     if wb.dim() == 3:
         q = ops.to_mx_dim0_dim1_batched(wb, mode, MX_SCALES_MFMA) if both else (_cast_w_rows(wb, mode), None)
     else:
-        q = ops.to_mx_dim0_dim1(wb, mode, MX_SCALES_MFMA) if both else (ops.to_mx_dim0(wb, mode, MX_SCALES_MFMA), None)
+        q = (ops.to_mx_dim0_dim1(wb, mode, MX_SCALES_MFMA, pitch_pad) if both
+             else (ops.to_mx_dim0(wb, mode, MX_SCALES_MFMA), None))
     if cached:
-        _weight_cache.put(w, mode, q[0], q[1])
+        _weight_cache.put(w, key, q[0], q[1])
     return q
 
 
@@ -193,8 +201,11 @@ class _MXLinear(torch.autograd.Function):
         w = weight if weight.dtype == torch.bfloat16 else weight.to(torch.bfloat16)
         needs_bwd = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
         M = x2.shape[0]
-        xq0, xq1 = _cast_activation(x2, x, mode, need_cols=ctx.needs_input_grad[1])
-        wq0, wq1 = _cast_weight(weight, mode, needs_bwd and ctx.needs_input_grad[0], cfg)
+        # operands of mx_gemm_nt only: their rows may lie further apart than they are long (not with
+        # cached weight casts, which the fused blocks and the hand-over share in their dense form)
+        pad = 0 if cfg.cache_weight_casts else ops.CODE_PITCH_PAD
+        xq0, xq1 = _cast_activation(x2, x, mode, need_cols=ctx.needs_input_grad[1], pitch_pad=pad)
+        wq0, wq1 = _cast_weight(weight, mode, needs_bwd and ctx.needs_input_grad[0], cfg, pitch_pad=pad)
         y = ops.mx_gemm_nt(xq0, wq0)
         ctx.cfg = cfg
         ctx.x_shape = x.shape
@@ -235,7 +246,8 @@ class _MXLinear(torch.autograd.Function):
                 wq1 = _cast_cols_padded(saved.pop(0), mode)
         dyq0 = dyq1 = None
         if need_dx and need_dw and M % ops.BLOCK == 0 and N % ops.BLOCK == 0:
-            dyq0, dyq1 = ops.to_mx_dim0_dim1(dy2, mode, MX_SCALES_MFMA)
+            dyq0, dyq1 = ops.to_mx_dim0_dim1(dy2, mode, MX_SCALES_MFMA,
+                                             0 if ctx.cfg.cache_weight_casts else ops.CODE_PITCH_PAD)
         else:
             if need_dx:
                 dyq0 = _cast_rows_padded(dy2, mode)
