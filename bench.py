@@ -155,8 +155,11 @@ def time_casts(dev, recipe_mode, also_floor=False):
         # the plain stream kernels over exactly this tensor's bytes, same rotation of buffers: a
         # launch's fixed cost weighs three times as much on 134 MB as on the 512 MiB yardsticks
         same_size = _streams_of_size(dev, bufs)
+        # dim0_dim1_pitched: the fused cast as the converted linears call it, code rows 128 bytes
+        # further apart than they are long (the same bytes written; see ops.CODE_PITCH_PAD)
+        pitched = lambda t, mode, order: ops.to_mx_dim0_dim1(t, mode, order, ops.CODE_PITCH_PAD)
         for kind, fn, bpe in (("dim0", ops.to_mx_dim0, 3.03125), ("dim1", ops.to_mx_dim1, 3.03125),
-                              ("dim0_dim1", ops.to_mx_dim0_dim1, 4.0625)):
+                              ("dim0_dim1", ops.to_mx_dim0_dim1, 4.0625), ("dim0_dim1_pitched", pitched, 4.0625)):
             for b in bufs[:2]:
                 fn(b, recipe_mode, L)
             torch.cuda.synchronize()
@@ -170,7 +173,7 @@ def time_casts(dev, recipe_mode, also_floor=False):
             sec = s.elapsed_time(e) * 1e-3 / reps
             out[f"{kind}:{name}"] = {"us": round(sec * 1e6, 1), "GB/s": round(el * bpe / sec / 1e9, 1),
                                      "frac_hbm": round(el * bpe / sec / 1e9 / PEAK_HBM_GBPS, 3)}
-            ref = same_size["stream_copy" if kind == "dim0_dim1" else "stream_2to1"]
+            ref = same_size["stream_copy" if kind.startswith("dim0_dim1") else "stream_2to1"]
             out[f"{kind}:{name}"]["same_size_stream_us"] = ref["us"]
             out[f"{kind}:{name}"]["frac_of_same_size_stream"] = round(el * bpe / sec / 1e9 / ref["GB/s"], 3)
         del bufs
@@ -361,13 +364,18 @@ def _casts_against_streams(casts, yardsticks):
 def cast_table(dev, recipe_mode):
     """The HBM yardsticks and then the casts, in a fixed order (see --cast-table): one JSON line of
     HIP-event times; under rocprofv3 --pmc the dispatches appear in the same order."""
-    per_tensor = lambda t: [f"stream_copy_of_size:{t}", f"stream_2to1_of_size:{t}", f"dim0:{t}", f"dim1:{t}", f"dim0_dim1:{t}"]
+    per_tensor = lambda t: [f"stream_copy_of_size:{t}", f"stream_2to1_of_size:{t}", f"dim0:{t}", f"dim1:{t}", f"dim0_dim1:{t}",
+                            f"dim0_dim1_pitched:{t}"]
     out = {"order": ["stream_copy", "stream_read", "stream_write", "stream_2to1"] + per_tensor("x") + per_tensor("dy") + per_tensor("w"),
            "launches_per_kernel": "2 warm-up + 8 timed (casts and the streams of a tensor's size: 2 + 3 x buffers, "
                                   "x and w 6 buffers, dy 3)"}
     out["yardsticks"] = _stream_yardsticks(dev)
     out["casts"] = time_casts(dev, recipe_mode)
     _casts_against_streams(out["casts"], out["yardsticks"])
+    # then the casts with the gate, its backward and the norm folded in, 2 warm-up + 10 (12) launches each
+    out["order"] += ["swiglu_cast_dim0_dim1", "swiglu_bwd_cast_dim0_dim1", "rmsnorm_cast_dim0_dim1", "torch_rms_norm_then_cast"]
+    recipe = {"rceil": "mxfp8_rceil", "floor": "mxfp8_floor"}[recipe_mode]
+    out["gate_and_norm_casts"] = time_gate_casts(dev, recipe)
     return out
 
 
@@ -470,6 +478,8 @@ def mfma_ceiling(dev, recipe_mode, launches=500, kinds=None, shapes=(32, 16)):
     st = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
     out = {"workgroups": cus, "waves_per_simd": 1}
     for shape in shapes:
+        # 1601 / 1604 / 1608: the 16x16x128 form in a fixed order in which 1 / 4 (the GEMM's K loop) / 8
+        # MFMAs in a row share an operand fragment
         iters = 2400 if shape == 32 else 1200
         flop = iters * 16 * 2.0 * 32 * 32 * 64 * 4 * cus * (1 if shape == 32 else 2)
         for name, buf in operands.items():
@@ -780,6 +790,18 @@ def time_ffn_block(dev, recipe):
             out[name]["ms_replayed_from_a_hip_graph"] = round(time_graph_replay(step), 3)
             out[name]["ms_under_torch_compile"] = _time_compiled(ff, lambda fn: fn(x).backward(dy), step)
         del ff, holder
+    out.update(time_gate_casts(dev, recipe))
+    return out
+
+
+def time_gate_casts(dev, recipe):
+    """The cast kernels with the SwiGLU gate, its backward and the RMSNorm folded in, alone, at the
+    benchmark sizes (16384 x 14336 for the gate, 16384 x 4096 for the norm)."""
+    import torch
+
+    from torchtitan_amd import ops
+
+    out = {}
     el = M * HIDDEN
     a = torch.randn((M, HIDDEN), device=dev, dtype=torch.bfloat16)
     b = torch.randn((M, HIDDEN), device=dev, dtype=torch.bfloat16)
@@ -1226,7 +1248,7 @@ def main():
         print(json.dumps(clock_table(dev, recipe_mode)))
         return
     if args.mfma_ceiling:
-        print(json.dumps(mfma_ceiling(dev, recipe_mode)))
+        print(json.dumps(mfma_ceiling(dev, recipe_mode, shapes=(32, 16, 1608, 1604, 1601))))
         return
     if args.gemm_ablation:
         print(json.dumps(gemm_ablation(dev, recipe_mode)))
