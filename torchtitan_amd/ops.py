@@ -6,6 +6,7 @@ call into libmxfp8_gfx950.so.  There is no fallback path: CPU tensors are reject
 from __future__ import annotations
 
 import ctypes
+import os
 from typing import NamedTuple
 
 import torch
@@ -147,7 +148,8 @@ def to_mx_dim1(x: torch.Tensor, mode="floor", order: int = MX_SCALES_ROWMAJOR) -
 # 16384 ...) put the lines a GEMM fetches together -- one 128-byte K block of 512 rows -- on few
 # channels of the L2; 128 bytes between the end of a row and the start of the next spread them
 # (measured on the dense GEMM inside the benchmark step: 2.4 % less time per launch).
-CODE_PITCH_PAD = 128
+# (MXFP8_CODE_PITCH_PAD in the environment: another multiple of 128, 0 = dense codes; for measurements.)
+CODE_PITCH_PAD = int(os.environ.get("MXFP8_CODE_PITCH_PAD", "128"))
 
 
 def to_mx_dim0_dim1(x: torch.Tensor, mode="floor", order: int = MX_SCALES_ROWMAJOR, pitch_pad: int = 0):
