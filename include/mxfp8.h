@@ -335,6 +335,24 @@ int mx_grouped_gemm_2d3d_pair(const uint8_t* a_codes, const uint8_t* a_scales,
                               const int32_t* offs, void* d, int64_t T, int64_t N, int64_t K,
                               int64_t G, int64_t ldd, void* stream);
 
+/* The grouped 2D x 3D GEMM (one product, or with a2_codes .. b2_scales non-null the sum of two as
+ * mx_grouped_gemm_2d3d_pair) over operands whose groups are padded to multiples of 32 rows, with
+ * the padding left out of the output: the first out_offs[g] - out_offs[g-1] rows of group g are
+ * written to rows [out_offs[g-1], out_offs[g]) of d [out_rows, ldd] (out_offs: int32 [G]
+ * inclusive ends, on the device); rows from out_offs[G-1] on are written as zeros as far as A
+ * has rows behind its last group (out_rows - out_offs[G-1] <= T - offs[G-1] is the caller's
+ * side of the contract; whatever the arrays hold, no row outside d is written).  Takes the
+ * place of the grouped GEMM followed by the gather that moves the rows back
+ * (`_unpermute`, torchtitan/models/common/moe/utils.py:85-89, called at :116).  MFMA-order scales
+ * and the contract of the MX_SCALES_MFMA form of mx_grouped_gemm_2d3d only; out_rows <= T. */
+int mx_grouped_gemm_2d3d_rows_out(const uint8_t* a_codes, const uint8_t* a_scales,
+                                  const uint8_t* b_codes, const uint8_t* b_scales,
+                                  const uint8_t* a2_codes, const uint8_t* a2_scales,
+                                  const uint8_t* b2_codes, const uint8_t* b2_scales,
+                                  const int32_t* offs, const int32_t* out_offs, void* d, int64_t T,
+                                  int64_t out_rows, int64_t N, int64_t K, int64_t G, int64_t ldd,
+                                  void* stream);
+
 /* Grouped GEMM, 2D x 2D (wgrad): D[g][N,K] = deq(A^T[:, rows_g]) * deq(B^T[:, rows_g])^T,
  * contracting over the tokens of group g.  at_codes [N,T] and bt_codes [K,T] are the
  * column-wise casts; scale_order says how both scale buffers are laid out:

@@ -170,7 +170,9 @@ def test_grouped_fake_kernels_give_the_static_shapes(T, K, N, G, pad):
         x, w, offs = torch.empty(T, K), torch.empty(G, N, K), torch.empty(G, dtype=torch.int32)
         y, offs_p, perm, back, xc, xs, wc, ws = torch.ops.torchtitan_amd.mx_grouped_mm_fwd(x, w, offs, 1, pad)
         assert y.shape == (T, N) and y.dtype == torch.bfloat16 and offs_p.shape == (G,)
-        assert perm.shape == ((Tp,) if padded else (0,)) and back.shape == ((T,) if padded else (0,))
+        assert perm.shape == ((Tp,) if padded else (0,))
+        # the way back: the unpadded group ends where the GEMM writes unpadded rows, else a gather
+        assert (back.shape, back.dtype) == (((G,), torch.int32) if fast else ((T,) if padded else (0,), torch.int64))
         assert xc.shape == (K, Tp) and wc.shape == (G, K, N)
         assert xs.shape == ((ops.mfma_scale_bytes(K, Tp // 32),) if fast else (K, Tp // 32))
         assert ws.numel() == G * ops.mfma_scale_bytes(K, N // 32)
@@ -212,7 +214,8 @@ def test_fused_block_fake_kernels_give_the_shapes_the_backward_takes():
         offs = torch.empty(G, dtype=torch.int32)
         Tp = -(-(T + 32 * G) // 128) * 128
         out = A.mx_grouped_ffn_fwd(xg, e1, e2, e1, offs, 1, True, False, True, True)
-        assert out[0].shape == (T, D) and out[2].shape == (Tp,) and out[3].shape == (T,) and out[4].shape == (2, Tp, H)
+        assert out[0].shape == (T, D) and out[2].shape == (Tp,) and out[4].shape == (2, Tp, H)
+        assert out[3].shape == (G,) and out[3].dtype == torch.int32  # the unpadded group ends: the GEMMs write unpadded rows
         dx, dw13, dw2 = A.mx_grouped_ffn_bwd(torch.empty(T, D), list(out[1:]), 1, ops.MX_SCALES_MFMA, True, True, True, False)
         assert dx.shape == (T, D) and dw13.shape == (1, G, H, D) and dw2.shape == (G, D, H)
 

@@ -261,7 +261,9 @@ def test_per_op_checkpoint_policy_keeps_grouped_gemm_outputs(device, fuse, monke
 
     launches = []
     real_call = ops._call
-    monkeypatch.setattr(ops, "_call", lambda name, *a: (launches.append(name), real_call(name, *a))[1])
+    # (the form that writes unpadded rows serves one product or, with a second operand set, a sum of two)
+    tag = lambda name, a: name + ("_sum_of_two" if name == "mx_grouped_gemm_2d3d_rows_out" and a[6] is not None else "")
+    monkeypatch.setattr(ops, "_call", lambda name, *a: (launches.append(tag(name, a)), real_call(name, *a))[1])
     torch.manual_seed(29)
     moe_mod.set_token_group_alignment_size_m(32)
     try:
@@ -288,7 +290,8 @@ def test_per_op_checkpoint_policy_keeps_grouped_gemm_outputs(device, fuse, monke
                                context_fn=lambda: create_selective_checkpoint_contexts(policy))
             y.backward(dy)
             # grouped 2D x 3D products computed (the launch for h1 and h3 together computes two)
-            runs[how] = (launches.count("mx_grouped_gemm_2d3d") + 2 * launches.count("mx_grouped_gemm_2d3d_shared_a"),
+            runs[how] = (launches.count("mx_grouped_gemm_2d3d") + launches.count("mx_grouped_gemm_2d3d_rows_out")
+                         + 2 * launches.count("mx_grouped_gemm_2d3d_shared_a"),
                          [y.detach(), xi.grad, ex.w1.grad.clone(), ex.w2.grad.clone(), ex.w3.grad.clone()])
         # forward 3; backward: d(g), and d(x) as two launches or as one of the paired form
         base = 4 if fuse else 6

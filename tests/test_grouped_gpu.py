@@ -486,3 +486,68 @@ def test_grouped_wgrads_of_two_gradients_in_one_launch(device, sizes, N, K):
     assert names == ["mx_grouped_gemm_2d2d_shared_b"]
     assert torch.equal(dw1, ops.mx_grouped_gemm_2d2d(da, x, offs))
     assert torch.equal(dw3, ops.mx_grouped_gemm_2d2d(db, x, offs))
+
+
+@pytest.mark.parametrize("real,N,K,tail_p,tail_out,two", [
+    ([250, 0, 97, 640, 1], 256, 256, 128, 0, False),     # ragged real sizes, an empty group, a one-row group
+    ([250, 0, 97, 640, 1], 264, 384, 128, 5, True),      # rows that belong to no group: zeros
+    ([300] * 3 + [31, 33, 1000, 0, 511], 768, 512, 256, 0, True),  # groups over several tiles
+])
+def test_grouped_gemm_leaves_the_padding_out_of_its_output(device, real, N, K, tail_p, tail_out, two):
+    """mx_grouped_gemm_2d3d_rows_out (one product and the sum of two): bit-identical to the grouped
+    GEMM over the padded groups followed by the gather of the real rows; rows of the output behind
+    the last group are zero, a row next to the output is not touched, and a broken (padded) group
+    end poisons exactly the output's rows."""
+    rng = np.random.default_rng(sum(real) + N + K + int(two))
+    G = len(real)
+    padded = [-(-r // 32) * 32 if r else 32 * (g % 2) for g, r in enumerate(real)]  # some empty groups get a block
+    Tp = sum(padded) + tail_p
+    T = sum(real) + tail_out
+    offs_p = _sizes_to_offs(padded, device)
+    offs = _sizes_to_offs(real, device)
+    q = lambda std: ops.to_mx_dim0(bf16_from_bits(randn_bits(rng, (Tp, K), std=std, outliers=1e-3), device), "rceil", L)
+    qb = lambda std: ops.to_mx_dim0_batched(bf16_from_bits(randn_bits(rng, (G, N, K), std=std), device), "rceil", L)
+    a, b = q(1.0), qb(0.02)
+    a2, b2 = (q(0.3), qb(0.05)) if two else (None, None)
+    full = ops.mx_grouped_gemm_2d3d_pair(a, b, a2, b2, offs_p) if two else ops.mx_grouped_gemm_2d3d(a, b, offs_p)
+    # the rows a gather would take: the first real[g] rows of padded group g, then zero rows
+    starts_p = np.cumsum([0] + padded[:-1])
+    rows = np.concatenate([np.arange(s, s + r) for s, r in zip(starts_p, real)] + [np.full(tail_out, -1)]).astype(np.int64)
+    idx = torch.from_numpy(rows).to(device)
+    want = torch.where((idx >= 0)[:, None], full[idx.clamp_min(0)], torch.zeros((), dtype=full.dtype, device=device))
+    got, names = _launch_names(lambda: ops.mx_grouped_gemm_2d3d_rows_out(a, b, offs_p, offs, T, a2, b2))
+    assert names == ["mx_grouped_gemm_2d3d_rows_out"]
+    assert got.shape == (T, N) and torch.equal(got, want)
+    # through the C ABI into a buffer with a guard row on each side and a wider row pitch
+    from torchtitan_amd import _lib
+    ld = N + 8
+    buf = torch.full((T + 2, ld), 7.0, dtype=torch.bfloat16, device=device)
+    second = [ops._ptr(t) for t in (a2.codes, a2.scales, b2.codes, b2.scales)] if two else [None] * 4
+    st = _lib.load().mx_grouped_gemm_2d3d_rows_out(
+        ops._ptr(a.codes), ops._ptr(a.scales), ops._ptr(b.codes), ops._ptr(b.scales), *second, ops._ptr(offs_p),
+        ops._ptr(offs), ops._ptr(buf[1]), Tp, T, N, K, G, ld, ops._stream(buf))
+    assert st == 0
+    assert torch.equal(buf[1:T + 1, :N], want)
+    assert (buf[0] == 7).all() and (buf[T + 1] == 7).all() and (buf[:, N:] == 7).all()
+    # a padded group end that is no multiple of 32: NaN over the output, nothing beyond it
+    bad = offs_p.clone()
+    bad[0] += 8
+    buf.fill_(7.0)
+    st = _lib.load().mx_grouped_gemm_2d3d_rows_out(
+        ops._ptr(a.codes), ops._ptr(a.scales), ops._ptr(b.codes), ops._ptr(b.scales), *second, ops._ptr(bad),
+        ops._ptr(offs), ops._ptr(buf[1]), Tp, T, N, K, G, ld, ops._stream(buf))
+    assert st == 0
+    assert buf[1:T + 1, :N].isnan().all()
+    assert (buf[0] == 7).all() and (buf[T + 1] == 7).all() and (buf[:, N:] == 7).all()
+    # unpadded group ends that make no sense never reach outside the output
+    wild = torch.tensor([-5, 10 ** 6] + [T // 2] * (G - 2), dtype=torch.int32, device=device)[:G]
+    buf.fill_(7.0)
+    st = _lib.load().mx_grouped_gemm_2d3d_rows_out(
+        ops._ptr(a.codes), ops._ptr(a.scales), ops._ptr(b.codes), ops._ptr(b.scales), *second, ops._ptr(offs_p),
+        ops._ptr(wild), ops._ptr(buf[1]), Tp, T, N, K, G, ld, ops._stream(buf))
+    assert st == 0
+    assert (buf[0] == 7).all() and (buf[T + 1] == 7).all() and (buf[:, N:] == 7).all()
+    # bad arguments
+    assert _lib.load().mx_grouped_gemm_2d3d_rows_out(
+        ops._ptr(a.codes), ops._ptr(a.scales), ops._ptr(b.codes), ops._ptr(b.scales), *second, ops._ptr(offs_p),
+        ops._ptr(offs), ops._ptr(buf[1]), Tp, Tp + 1, N, K, G, ld, ops._stream(buf)) != 0

@@ -57,6 +57,7 @@ SIGNATURES = {
     "mx_gemm_nt_shared_b": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "mx_grouped_gemm_2d3d_shared_a": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "mx_grouped_gemm_2d2d_shared_b": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
+    "mx_grouped_gemm_2d3d_rows_out": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
     "mx_grouped_gemm_2d3d_pair": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "mx_grouped_gemm_2d3d": (c_int, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, c_int, _P]),
     "mx_grouped_gemm_2d2d": (c_int, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, c_int, _P]),

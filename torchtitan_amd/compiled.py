@@ -170,7 +170,8 @@ def _fake_scales(rows: int, nblk: int, order: int, device):
 def mx_grouped_mm_fwd(x: torch.Tensor, weight: torch.Tensor, offs: torch.Tensor, mode: int, pad: bool) -> tuple[
         torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """y[rows of g] = x[rows of g] W[g]^T for x [T, K], W [G, N, K], offs = inclusive int32 group
-    ends; also the plan (padded offsets, gather indices, rows' places in the padded layout; the
+    ends; also the plan (padded offsets, gather indices, the way back -- rows' places in the
+    padded layout, or the unpadded group ends as int32 where the GEMM writes unpadded rows; the
     last two empty when the groups stay where they are) and the column-wise MXFP8 forms of the
     padded x (codes [K, Tp]) and of W (codes [G, K, N]) for the backward."""
     T, K = x.shape
@@ -180,13 +181,13 @@ def mx_grouped_mm_fwd(x: torch.Tensor, weight: torch.Tensor, offs: torch.Tensor,
     xb = (x if x.dtype == torch.bfloat16 else x.to(torch.bfloat16)).contiguous()
     w = (weight if weight.dtype == torch.bfloat16 else weight.to(torch.bfloat16)).contiguous()
     if padded:
-        perm, offs_p, back = _pad_plan(offs, T, ops.BLOCK, multiple)
+        perm, offs_p, back = _pad_plan(offs, T, ops.BLOCK, multiple, direct=order == MX_SCALES_MFMA)
     else:
         perm = back = None
         offs_p = offs.clone()
     xq0, xq1 = _cast_into_groups(xb, perm, name, order, True)
     wq0, wq1 = ops.to_mx_dim0_dim1_batched(w, name, MX_SCALES_MFMA)
-    y = _grouped_2d3d_padded(xq0, wq0, offs_p, back)
+    y = _grouped_2d3d_padded(xq0, wq0, offs_p, back, T)
     none = torch.empty((0,), dtype=torch.int64, device=x.device)
     return (y, offs_p, perm if padded else none, back if padded else none.clone(),
             xq1.codes, xq1.scales, wq1.codes, wq1.scales)
@@ -203,7 +204,9 @@ def _(x, weight, offs, mode, pad):
     i64 = dict(dtype=torch.int64, device=dev)
     return (torch.empty((T, N), dtype=torch.bfloat16, device=dev),
             torch.empty((G,), dtype=torch.int32, device=dev),
-            torch.empty((Tp if padded else 0,), **i64), torch.empty((T if padded else 0,), **i64),
+            torch.empty((Tp if padded else 0,), **i64),
+            (torch.empty((G,), dtype=torch.int32, device=dev) if padded and order == MX_SCALES_MFMA
+             else torch.empty((T if padded else 0,), **i64)),
             torch.empty((K, Tp), dtype=torch.uint8, device=dev), _fake_scales(K, Tp // 32, order, dev),
             torch.empty((G, K, N), dtype=torch.uint8, device=dev),
             torch.empty((G * ops.mfma_scale_bytes(K, N // 32),), dtype=torch.uint8, device=dev))
@@ -229,7 +232,7 @@ def mx_grouped_mm_bwd(dy: torch.Tensor, offs_p: torch.Tensor, perm: torch.Tensor
         dyq1 = ops.to_mx_dim1(dyb, name, order) if need_dw else None
     dx = dw = empty
     if need_dx:
-        dx = _grouped_2d3d_padded(dyq0, MXData(w_codes_t, w_scales_t, MX_SCALES_MFMA), offs_p, back if padded else None)
+        dx = _grouped_2d3d_padded(dyq0, MXData(w_codes_t, w_scales_t, MX_SCALES_MFMA), offs_p, back if padded else None, T)
     if need_dw:
         dw = ops.mx_grouped_gemm_2d2d(dyq1, MXData(x_codes_t, x_scales_t, order), offs_p)
     return dx, dw
@@ -497,7 +500,10 @@ def _(x, w1, w2, w3, offs, mode, pad, cache_w, need_dx, need_dw):
     s[0] = torch.empty((G,), dtype=torch.int32, device=dev)
     if padded:
         s[1] = torch.empty((Tp,), dtype=torch.int64, device=dev)
-        s[2] = torch.empty((T,), dtype=torch.int64, device=dev)
+        from . import mx_blocks
+
+        fast = mx_blocks.grouped_layout(D, H, G)[2]
+        s[2] = torch.empty((G,) if fast else (T,), dtype=torch.int32 if fast else torch.int64, device=dev)
     if need_dx or need_dw:
         s[3:6] = [torch.empty((2, Tp, H), dtype=torch.bfloat16, device=dev), _u8((G, H, D), dev),
                   _u8((G * ops.mfma_scale_bytes(H, D // 32),), dev)]

@@ -589,8 +589,13 @@ __device__ __forceinline__ void emit_tile(
       const int o = p * 32 + tid / SEGS;
       if (c0 + o < cols && r0 + seg * 16 < rows) {
         const u32x4 t = *reinterpret_cast<const u32x4*>(lds_codes + o * PITCH + seg * 16);
+#ifdef MX_ABL_COL_UNTRANSPOSED  // timing ablation: the column-wise codes go out as rows of the input
+        __builtin_nontemporal_store(
+            t, reinterpret_cast<u32x4*>(codes_t + (r0 + o) * cols + c0 + seg * 16));
+#else
         __builtin_nontemporal_store(
             t, reinterpret_cast<u32x4*>(codes_t + (c0 + o) * ldct + r0 + seg * 16));
+#endif
       }
     }
     if (ORDER == MX_SCALES_MFMA) {

@@ -36,7 +36,9 @@
 // read the same twelve operand panels (MX_ABL_SAME_A / MX_ABL_SAME_B: the same A / B panels only), so
 // that every read beyond the L2 finds its line in the memory-side cache; MX_ABL_ROW_PAD=n reads the
 // rows of a tile n bytes further apart than they lie (what a padded row pitch would do to the
-// spread of a block's lines over the cache channels).  Results are then meaningless.
+// spread of a block's lines over the cache channels); MX_ABL_TR_READ issues every fragment read as
+// two ds_read_b64_tr_b8 (what a K loop over operands stored K-strided would issue).  Results are
+// then meaningless.
 #include "mx_gemm_tile.h"
 
 namespace mx {
@@ -93,6 +95,12 @@ struct Gemm32Args {
   // kDense, kSplitK: bytes between the rows of A and of B (both operands' rows are K bytes long
   // and may lie further apart, by a multiple of 128); 0 = K
   int64_t ldk = 0;
+  // kGrouped2d3d: output rows without the groups' padding.  Group g's first d_offs[g] -
+  // d_offs[g-1] rows are written to rows [d_offs[g-1], d_offs[g]) of D (inclusive ends, on the
+  // device), the rest of its rows nowhere; rows [d_offs[G-1], d_rows) of D are written as zeros
+  // as far as A has rows behind its last group.  nullptr: D has A's rows.
+  const int32_t* d_offs = nullptr;
+  int64_t d_rows = 0;
 };
 enum Gemm32Two { kTwoNone = 0, kTwoB = 1, kTwoA = 2 };
 
@@ -102,6 +110,7 @@ struct Tile32 {
   const uint8_t *sa, *sb;  // scales of the tile's first 128-row group at its first 64-deep step
   uint16_t* d;
   int64_t rows_a, rows_b;  // valid rows from the tile's origin (may exceed 256; <= 0: none)
+  int32_t rows_d;          // Gemm32Args::d_offs given: rows of the tile that D has (0..256)
   uint32_t koff;           // first K byte of the range inside an operand row (kGrouped2d2d)
   uint32_t nblocks;        // 128-deep K blocks, at least 1
   bool empty;              // no K range (an empty group, rows behind the last group, or poison):
@@ -331,6 +340,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     r.poison = poison;
     r.koff = 0;
     r.empty = false;
+    r.rows_d = 0;
     r.rot = 0;
     r.head = 0;
     r.tail = 0;
@@ -380,6 +390,10 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       r.d = d_base + (int64_t)tm * kT32 * p.ldd + (int64_t)tn * kT32;
       r.rows_a = p.M - (int64_t)tm * kT32;
       r.rows_b = p.N - (int64_t)tn * kT32;
+      if (MODE == kGrouped2d3d && p.d_offs) {
+        const int64_t left = p.d_rows - (int64_t)tm * kT32;
+        r.rows_d = (int32_t)(left < 0 ? 0 : (left > kT32 ? kT32 : left));
+      }
       r.nblocks = poison ? 1 : K / kKB;
       r.empty = poison;
     } else if (MODE == kGrouped2d3d) {
@@ -404,6 +418,14 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       r.d = d_base + row0 * p.ldd + (int64_t)tn * kT32;
       r.rows_a = hi - row0;
       r.rows_b = p.N - (int64_t)tn * kT32;
+      if (p.d_offs) {  // the group's rows in D, both ends kept inside D whatever the array holds
+        int64_t lo_d = g ? p.d_offs[g - 1] : 0, hi_d = g < G ? (int64_t)p.d_offs[g] : p.d_rows;
+        lo_d = lo_d < 0 ? 0 : (lo_d > p.d_rows ? p.d_rows : lo_d);
+        hi_d = hi_d < lo_d ? lo_d : (hi_d > p.d_rows ? p.d_rows : hi_d);
+        const int64_t left = hi_d - lo_d - (int64_t)tm * kT32;
+        r.rows_d = (int32_t)(left < 0 ? 0 : (left > kT32 ? kT32 : left));
+        r.d = d_base + (lo_d + (int64_t)tm * kT32) * p.ldd + (int64_t)tn * kT32;
+      }
       r.nblocks = g < G ? K / kKB : 1;
       r.empty = g >= G;
     } else if (MODE == kSplitK) {
@@ -486,7 +508,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       w[2] = (int32_t)t.nblocks;
       w[3] = (int32_t)t.koff;
       w[4] = t.empty ? 1 : 0;
-      w[5] = (int32_t)(t.rot | (t.tail << 8) | (t.head << 16));
+      w[5] = (int32_t)(t.rot | (t.tail << 8) | (t.head << 16) | ((uint32_t)t.rows_d << 20));
     }
     __syncthreads();
   }
@@ -523,6 +545,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
       t.rot = rt & 3;
       t.tail = (rt >> 8) & 3;
       t.head = (rt >> 16) & 3;
+      t.rows_d = (int32_t)(rt >> 20);
       t.poison = poison;
       return t;
     }
@@ -669,10 +692,24 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
   // has landed (vmcnt(0)) and the prefetch distance collapses.  The reads are therefore
   // invisible to its wait-count tracking; `pin_set` / `landed` (after an explicit lgkmcnt wait)
   // are what the MFMAs depend on.
+#ifdef MX_ABL_TR_READ
+  constexpr int kReadsPerPiece = 2;
+#else
+  constexpr int kReadsPerPiece = 1;
+#endif
   auto lds_b128 = [&](uint32_t addr, auto off_) -> v4i {
     constexpr int off = decltype(off_)::value;
     v4i v;
+#ifdef MX_ABL_TR_READ  // timing ablation: the 16 bytes come as two transposing 8-byte reads
+    typedef int v2i_t __attribute__((ext_vector_type(2)));
+    v2i_t lo, hi;
+    const uint32_t first = addr + ((lane & 16) >> 1);  // each 32-lane pass still covers all banks
+    asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(lo) : "v"(first), "n"(off));
+    asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(hi) : "v"(first ^ 8u), "n"(off));
+    v = v4i{lo.x, lo.y, hi.x, hi.y};
+#else
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(off));
+#endif
     return v;
   };
   // ---- fragment sets, scale dwords
@@ -793,7 +830,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     });
   };
   auto landed = [&](auto n_, v8i& frag) {  // all LDS reads but the n youngest have landed
-    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(decltype(n_)::value) : "memory");
+    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(kReadsPerPiece * decltype(n_)::value > 15 ? 15 : kReadsPerPiece * decltype(n_)::value) : "memory");
     asm volatile("" : "+v"(frag));
   };
   auto block_steps = [&](Frags16& f, auto first_) {
@@ -887,7 +924,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     c_slot ^= 1;
     // the next block's first MFMAs need its b[0], its scales and the first sub-tile of its
     // a[0]: everything but the eight reads issued since
-    asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
+    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(kReadsPerPiece * 8 > 15 ? 15 : kReadsPerPiece * 8) : "memory");
     pin_set(f.b[0]);
     asm volatile("" : "+v"(f.a[0][0]));
     next_scales(f, c_slot);
@@ -915,7 +952,7 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     // + (m & 1) * 16 rows + (second sub-tile pair of the piece) * 64
     const uint32_t patch_w = patch + (lane_e & 15) * kPatchPitch + ((lane_e >> 4) & 1) * 32 + (lane_e >> 5) * 16;
     const uint32_t patch_r = patch + (lane_e >> 3) * kPatchPitch + (lane_e & 7) * 16;  // + pass*8 rows
-    const int64_t rows_valid = t.rows_a;
+    const int64_t rows_valid = (MODE == kGrouped2d3d && p.d_offs) ? (int64_t)t.rows_d : t.rows_a;
     const uint32_t cols_valid = (uint32_t)(t.rows_b < kT32 ? t.rows_b : kT32);
     if constexpr (MODE == kSplitK) {
       // float32 partial sums straight from the accumulators: a lane stores 16 bytes of row li
@@ -1321,6 +1358,23 @@ int launch_grouped32_2d3d_pair(const uint8_t* a_codes, const uint8_t* a_scales, 
   Gemm32Args p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, T, N, K, ldd, offs, G, 0, 0, nullptr,
                a2_codes, a2_scales, b2_codes, b2_scales};
   return launch_grouped32<kGrouped2d3d, true>(p, (T + kT32 - 1) / kT32 + G + 1, (N + kT32 - 1) / kT32, st);
+}
+
+// Grouped 2D x 3D (one product, or with a2_codes the sum of two) whose output leaves the groups'
+// padding out: see Gemm32Args::d_offs.
+int launch_grouped32_2d3d_rows_out(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                                   const uint8_t* b_scales, const uint8_t* a2_codes,
+                                   const uint8_t* a2_scales, const uint8_t* b2_codes,
+                                   const uint8_t* b2_scales, const int32_t* offs, const int32_t* d_offs,
+                                   void* d, int64_t T, int64_t d_rows, int64_t N, int64_t K, int64_t G,
+                                   int64_t ldd, hipStream_t st) {
+  Gemm32Args p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, T, N, K, ldd, offs, G, 0, 0, nullptr,
+               a2_codes, a2_scales, b2_codes, b2_scales};
+  p.d_offs = d_offs;
+  p.d_rows = d_rows;
+  const int64_t tile_rows = (T + kT32 - 1) / kT32 + G + 1, tiles_n = (N + kT32 - 1) / kT32;
+  if (a2_codes) return launch_grouped32<kGrouped2d3d, true>(p, tile_rows, tiles_n, st);
+  return launch_grouped32<kGrouped2d3d>(p, tile_rows, tiles_n, st);
 }
 
 // D[g][N, K] = A^T[N, lo:hi] B^T[K, lo:hi]^T; operand rows are T long.

@@ -140,6 +140,12 @@ int launch_grouped32_2d3d_pair(const uint8_t* a_codes, const uint8_t* a_scales, 
                                const uint8_t* a2_scales, const uint8_t* b2_codes,
                                const uint8_t* b2_scales, const int32_t* offs, void* d, int64_t T,
                                int64_t N, int64_t K, int64_t G, int64_t ldd, hipStream_t st);
+int launch_grouped32_2d3d_rows_out(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                                   const uint8_t* b_scales, const uint8_t* a2_codes,
+                                   const uint8_t* a2_scales, const uint8_t* b2_codes,
+                                   const uint8_t* b2_scales, const int32_t* offs, const int32_t* d_offs,
+                                   void* d, int64_t T, int64_t d_rows, int64_t N, int64_t K, int64_t G,
+                                   int64_t ldd, hipStream_t st);
 int launch_grouped32_2d3d_two_b(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                                 const uint8_t* b_scales, const uint8_t* b2_codes, const uint8_t* b2_scales,
                                 const int32_t* offs, void* d, void* d2, int64_t T, int64_t N, int64_t K,
@@ -189,6 +195,33 @@ extern "C" int mx_grouped_gemm_2d2d_shared_b(const uint8_t* at_codes, const uint
   if (256 * T > 0x7FFFFFFFll || K * 512 > 0x7FFFFFFFll) return MX_ERR_UNSUPPORTED;
   return launch_grouped32_2d2d_two_a(at_codes, at_scales, at2_codes, at2_scales, bt_codes, bt_scales, offs,
                                      d, d2, T, N, K, G, (hipStream_t)stream);
+}
+
+extern "C" int mx_grouped_gemm_2d3d_rows_out(const uint8_t* a_codes, const uint8_t* a_scales,
+                                             const uint8_t* b_codes, const uint8_t* b_scales,
+                                             const uint8_t* a2_codes, const uint8_t* a2_scales,
+                                             const uint8_t* b2_codes, const uint8_t* b2_scales,
+                                             const int32_t* offs, const int32_t* out_offs, void* d,
+                                             int64_t T, int64_t out_rows, int64_t N, int64_t K,
+                                             int64_t G, int64_t ldd, void* stream) {
+  if (T < 0 || out_rows < 0 || out_rows > T || N < 0 || K < 0 || G <= 0 || ldd < N)
+    return MX_ERR_INVALID_ARG;
+  if (out_rows == 0 || N == 0) return MX_OK;
+  if (!a_codes || !a_scales || !b_codes || !b_scales || !offs || !out_offs || !d)
+    return MX_ERR_INVALID_ARG;
+  const bool two = a2_codes || a2_scales || b2_codes || b2_scales;
+  if (two && (!a2_codes || !a2_scales || !b2_codes || !b2_scales)) return MX_ERR_INVALID_ARG;
+  if (K == 0 || K % 128 || N % 8 || ldd % 8 || T % 32) return MX_ERR_ALIGNMENT;
+  if (((uintptr_t)a_codes & 15) || ((uintptr_t)b_codes & 15) || ((uintptr_t)a_scales & 3) ||
+      ((uintptr_t)b_scales & 3) || ((uintptr_t)d & 15))
+    return MX_ERR_ALIGNMENT;
+  if (two && (((uintptr_t)a2_codes & 15) || ((uintptr_t)b2_codes & 15) || ((uintptr_t)a2_scales & 3) ||
+              ((uintptr_t)b2_scales & 3)))
+    return MX_ERR_ALIGNMENT;
+  if (256 * K > 0x7FFFFFFFll || G > 510 || ldd * 512 > 0x7FFFFFFFll) return MX_ERR_UNSUPPORTED;
+  return launch_grouped32_2d3d_rows_out(a_codes, a_scales, b_codes, b_scales, a2_codes, a2_scales,
+                                        b2_codes, b2_scales, offs, out_offs, d, T, out_rows, N, K, G,
+                                        ldd, (hipStream_t)stream);
 }
 
 extern "C" int mx_grouped_gemm_2d3d_pair(const uint8_t* a_codes, const uint8_t* a_scales,

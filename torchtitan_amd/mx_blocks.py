@@ -376,7 +376,8 @@ def grouped_layout(D: int, H: int, G: int):
 
 
 # What the expert block keeps for its backward, by slot (None where not needed):
-#   0 padded group ends   1 gather indices, 2 rows' places in the padded layout (groups moved)
+#   0 padded group ends   1 gather indices, 2 the way back (`_pad_plan`: rows' places in the padded
+#   layout, int64 [T], or the unpadded group ends, int32 [G], when the GEMMs write unpadded rows)
 #   3 h1 and h3 stacked [2, Tp, H]   4, 5 column-wise W2   6, 7 column-wise x   8, 9 column-wise g
 #   10, 11 column-wise W1            12, 13 column-wise W3
 GROUPED_FFN_SAVED = 14
@@ -390,7 +391,7 @@ def grouped_ffn_forward(x, w1, w2, w3, offs, cfg: MXFP8Config, need_dx: bool, ne
     order, multiple, fast = grouped_layout(D, H, G)
     perm = back = None
     if cfg.pad_token_groups_for_grouped_mm or fast:
-        perm, offs_p, back = _pad_plan(offs, T, ops.BLOCK, multiple)
+        perm, offs_p, back = _pad_plan(offs, T, ops.BLOCK, multiple, direct=fast)
     else:
         offs_p = offs
         if T % ops.BLOCK:
@@ -401,7 +402,7 @@ def grouped_ffn_forward(x, w1, w2, w3, offs, cfg: MXFP8Config, need_dx: bool, ne
     w2q0, w2q1 = _cast_weight(w2, mode, need_dx or need_dw, cfg)
     h13 = ops.mx_grouped_gemm_2d3d_shared_a(xq0, w1q0, w3q0, offs_p)  # one pass over the routed tokens
     gq0, gq1, _ = ops.swiglu_to_mx_dim0_dim1(h13[0], h13[1], mode, order)
-    y = _grouped_2d3d_padded(gq0, w2q0, offs_p, back)
+    y = _grouped_2d3d_padded(gq0, w2q0, offs_p, back, T)
     saved = [None] * GROUPED_FFN_SAVED
     saved[0:3] = [offs_p, perm, back]
     if need_dx or need_dw:
@@ -435,16 +436,8 @@ def grouped_ffn_backward(dy, saved, cfg: MXFP8Config, order: int, need_dx: bool,
             dw2 = ops.mx_grouped_gemm_2d2d(dyq1, gq1, offs_p)
     if need_dx:
         w1q1, w3q1 = _take(saved, 10), _take(saved, 12)
-        # d(h1) W1[g] + d(h3) W3[g] as one grouped GEMM (summed in float32, rounded once); the
-        # spare zero row behind it serves rows that belong to no group
-        Tp, D = da0.codes.shape[0], w1q1.codes.shape[1]
-        if back is None:
-            dx = ops.mx_grouped_gemm_2d3d_pair(da0, w1q1, db0, w3q1, offs_p)
-        else:
-            buf = torch.empty((Tp + 1, D), dtype=torch.bfloat16, device=da0.codes.device)
-            buf[Tp].zero_()
-            ops.mx_grouped_gemm_2d3d_pair(da0, w1q1, db0, w3q1, offs_p, buf[:Tp])
-            dx = buf[back]
+        # d(h1) W1[g] + d(h3) W3[g] as one grouped GEMM (summed in float32, rounded once)
+        dx = _grouped_2d3d_padded(da0, w1q1, offs_p, back, dy.shape[0], db0, w3q1)
     return dx, dw1, dw2, dw3
 
 

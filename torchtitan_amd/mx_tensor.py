@@ -300,11 +300,13 @@ def mx_linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, 
 
 
 # ----------------------------------------------------------------------------- grouped GEMM
-def _pad_plan(offs: torch.Tensor, T: int, align: int = 32, length_multiple: int = 1):
+def _pad_plan(offs: torch.Tensor, T: int, align: int = 32, length_multiple: int = 1, direct: bool = False):
     """Device-side plan that moves rows of variable-size groups into `align`-aligned groups.
 
     Returns (gather indices into [x; 0-row] for the padded layout, padded inclusive offsets,
-    for every original row its row in the padded layout or the index of an appended zero row).
+    the way back).  The way back is, for every original row, its row in the padded layout or the
+    index of an appended zero row (int64 [T]: a gather) -- or, with `direct`, a copy of the
+    unpadded group ends (int32 [G]) for a grouped GEMM that writes the unpadded rows itself.
     No host synchronisation: the padded length is the static bound round_up(T + align G, align),
     rounded up further to `length_multiple` (a multiple of align) when one is given.
     """
@@ -313,6 +315,8 @@ def _pad_plan(offs: torch.Tensor, T: int, align: int = 32, length_multiple: int 
     step = max(align, length_multiple)
     max_len = -(-(T + align * G) // step) * step
     perm, _, m_offsets = ops.group_offsets_pad(sizes, G, 1, max_len, align)
+    if direct:
+        return perm, m_offsets, offs.to(torch.int32).clone()
     back = torch.full((T + 1,), max_len, dtype=torch.int64, device=offs.device)
     back[perm] = torch.arange(max_len, device=offs.device)  # perm == -1 writes the spare slot T
     return perm, m_offsets, back[:T]
@@ -328,18 +332,27 @@ def _cast_into_groups(t: torch.Tensor, perm, mode: str, order: int, want_cols: b
     return ops.to_mx_dim0(t, mode, order), None
 
 
-def _grouped_2d3d_padded(a: MXData, b: MXData, offs_p: torch.Tensor, back):
-    """Grouped GEMM in the padded layout, result moved back to the original row order.  One
-    spare zero row behind the GEMM's output serves rows that belong to no group."""
+def _grouped_2d3d_padded(a: MXData, b: MXData, offs_p: torch.Tensor, back, out_rows: int,
+                         a2: MXData | None = None, b2: MXData | None = None):
+    """Grouped GEMM (with a2, b2: the sum of two) in the padded layout, result in the original
+    row order [out_rows, N]; `back` as `_pad_plan` returns it (None: nothing was padded).  On
+    the gather path one spare zero row behind the GEMM's output serves rows that belong to no
+    group."""
     Tp, N = a.codes.shape[0], b.codes.shape[1]
+    two = a2 is not None
+    if back is not None and back.dtype == torch.int32:  # the GEMM leaves the padding out itself
+        return ops.mx_grouped_gemm_2d3d_rows_out(a, b, offs_p, back, out_rows, a2, b2)
     if back is None:
-        return ops.mx_grouped_gemm_2d3d(a, b, offs_p)
-    if ops._watched():  # the dispatcher form of the GEMM allocates its own output
+        return ops.mx_grouped_gemm_2d3d_pair(a, b, a2, b2, offs_p) if two else ops.mx_grouped_gemm_2d3d(a, b, offs_p)
+    if ops._watched() and not two:  # the dispatcher form of the GEMM allocates its own output
         y = ops.mx_grouped_gemm_2d3d(a, b, offs_p)
         return torch.cat((y, y.new_zeros(1, N)))[back]
     buf = torch.empty((Tp + 1, N), dtype=torch.bfloat16, device=a.codes.device)
     buf[Tp].zero_()
-    ops.mx_grouped_gemm_2d3d(a, b, offs_p, buf[:Tp])
+    if two:
+        ops.mx_grouped_gemm_2d3d_pair(a, b, a2, b2, offs_p, buf[:Tp])
+    else:
+        ops.mx_grouped_gemm_2d3d(a, b, offs_p, buf[:Tp])
     return buf[back]
 
 
@@ -361,7 +374,7 @@ class _MXGroupedMM(torch.autograd.Function):
         order = MX_SCALES_MFMA if fast else MX_SCALES_ROWMAJOR
         perm = back = None
         if cfg.pad_token_groups_for_grouped_mm or fast:
-            plan = _pad_plan(offs, T, ops.BLOCK, ops.FAST_LENGTH_MULTIPLE if fast else 1)
+            plan = _pad_plan(offs, T, ops.BLOCK, ops.FAST_LENGTH_MULTIPLE if fast else 1, direct=fast)
             perm, offs_p, back = plan
         else:
             offs_p = offs
@@ -371,7 +384,7 @@ class _MXGroupedMM(torch.autograd.Function):
         need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         xq0, xq1 = _cast_into_groups(xb, perm, mode, order, need_dw)
         wq0, wq1 = _cast_weight(weight, mode, need_dx, cfg)
-        y = _grouped_2d3d_padded(xq0, wq0, offs_p, back)
+        y = _grouped_2d3d_padded(xq0, wq0, offs_p, back, T)
         ctx.cfg = cfg
         ctx.dims = (T, K, N, G)
         ctx.dtypes = (x.dtype, weight.dtype)
@@ -412,7 +425,7 @@ class _MXGroupedMM(torch.autograd.Function):
                 wq1 = MXData(saved.pop(0), saved.pop(0), MX_SCALES_MFMA)
             else:
                 wq1 = ops.to_mx_dim1_batched(saved.pop(0), mode, MX_SCALES_MFMA)
-            dx = _grouped_2d3d_padded(dyq0, wq1, offs_p, back)
+            dx = _grouped_2d3d_padded(dyq0, wq1, offs_p, back, T)
             if dx.dtype != ctx.dtypes[0]:
                 dx = dx.to(ctx.dtypes[0])
         if need_dw:

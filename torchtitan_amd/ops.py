@@ -509,6 +509,17 @@ def _grouped_2d3d_op(a_codes, a_scales, a_order, b_codes, b_scales, offs):
     return _grouped_2d3d_into(a_codes, a_scales, a_order, b_codes, b_scales, offs, out)
 
 
+def _grouped_2d3d_rows_out_op(a_codes, a_scales, b_codes, b_scales, offs, out_offs, out_rows, second=None):
+    T, K = a_codes.shape
+    G, N, _ = b_codes.shape
+    out = torch.empty((out_rows, N), dtype=torch.bfloat16, device=a_codes.device)
+    extra = [_ptr(t) for t in second] if second is not None else [None] * 4
+    _call("mx_grouped_gemm_2d3d_rows_out", "grouped_gemm_2d3d_rows_out", out.device, _ptr(a_codes), _ptr(a_scales),
+          _ptr(b_codes), _ptr(b_scales), *extra, _ptr(offs), _ptr(out_offs), _ptr(out), T, out_rows, N, K, G, N,
+          _stream(out))
+    return out
+
+
 # The GEMMs whose output a forward pass hands on are also registered with torch's dispatcher, so
 # that a per-op activation-checkpoint policy (torch.utils.checkpoint's selective contexts, which
 # watch dispatched ops) can name them and keep their outputs instead of running them again in
@@ -518,8 +529,11 @@ _dispatcher_ops = torch.library.Library("torchtitan_amd", "DEF")
 _dispatcher_ops.define("mx_gemm_nt(Tensor a_codes, Tensor a_scales, Tensor b_codes, Tensor b_scales) -> Tensor")
 _dispatcher_ops.define("mx_grouped_gemm_2d3d(Tensor a_codes, Tensor a_scales, int a_order, Tensor b_codes, "
                        "Tensor b_scales, Tensor offs) -> Tensor")
+_dispatcher_ops.define("mx_grouped_gemm_2d3d_rows_out(Tensor a_codes, Tensor a_scales, Tensor b_codes, "
+                       "Tensor b_scales, Tensor offs, Tensor out_offs, int out_rows) -> Tensor")
 _dispatcher_ops.impl("mx_gemm_nt", _gemm_nt_op, "CUDA")
 _dispatcher_ops.impl("mx_grouped_gemm_2d3d", _grouped_2d3d_op, "CUDA")
+_dispatcher_ops.impl("mx_grouped_gemm_2d3d_rows_out", _grouped_2d3d_rows_out_op, "CUDA")
 
 
 _dispatch_depth = getattr(torch._C, "_len_torch_dispatch_stack", None)
@@ -536,7 +550,8 @@ def op_sac_save_list() -> set:
     (torchtitan/models/llama3/parallelize.py:44-60) to keep MXFP8 GEMM outputs through the
     recomputation, as the bf16 path keeps its `aten.mm` outputs.  Casts stay recomputed."""
     return {torch.ops.torchtitan_amd.mx_gemm_nt.default,
-            torch.ops.torchtitan_amd.mx_grouped_gemm_2d3d.default}
+            torch.ops.torchtitan_amd.mx_grouped_gemm_2d3d.default,
+            torch.ops.torchtitan_amd.mx_grouped_gemm_2d3d_rows_out.default}
 
 
 def mx_gemm_nt(a: MXData, b: MXData, out: torch.Tensor | None = None) -> torch.Tensor:
@@ -725,6 +740,46 @@ def mx_grouped_gemm_2d3d_pair(a: MXData, b: MXData, a2: MXData, b2: MXData, offs
           _ptr(b.codes), _ptr(b.scales), _ptr(a2.codes), _ptr(a2.scales), _ptr(b2.codes), _ptr(b2.scales),
           _ptr(offs), _ptr(out), T, N, K, G, out.stride(0), _stream(out))
     return out
+
+
+def mx_grouped_gemm_2d3d_rows_out(a: MXData, b: MXData, offs: torch.Tensor, out_offs: torch.Tensor,
+                                  out_rows: int, a2: MXData | None = None,
+                                  b2: MXData | None = None) -> torch.Tensor:
+    """bf16 [out_rows, N]: the grouped product (with a2, b2: the sum of two, as
+    `mx_grouped_gemm_2d3d_pair`) of operands whose groups are padded, written without the padding:
+    the first out_offs[g] - out_offs[g-1] rows of group g go to rows [out_offs[g-1], out_offs[g])
+    (out_offs: int32 [G] inclusive ends on the device), rows from out_offs[-1] on are zero.
+
+    Takes the place of the grouped GEMM followed by a gather of the unpadded rows (the second
+    half of the padding wrapper, torchtitan/models/common/moe/utils.py:85-89 and :116).  MFMA-order scales and 32-aligned
+    padded groups only (the persistent kernel); `rows_out_supported` tells.  The zero rows need
+    a.codes to have at least as many rows behind its last group as the output has."""
+    T, K = a.codes.shape
+    G, N, _ = b.codes.shape
+    if not rows_out_supported(a, b, a2, b2):
+        raise ValueError("unpadded output needs MFMA-order scales, K % 128 == 0, N % 8 == 0, T % 32 == 0")
+    for o in (offs, out_offs):
+        if o.dtype != torch.int32 or o.numel() != G:
+            raise ValueError("offs and out_offs must be int32 with one entry per group")
+    if not 0 <= out_rows <= T:
+        raise ValueError("the output cannot have more rows than the padded operand")
+    if a2 is None:
+        if _watched():  # as a dispatcher op: a forward GEMM whose output a checkpoint policy may keep
+            return torch.ops.torchtitan_amd.mx_grouped_gemm_2d3d_rows_out(a.codes, a.scales, b.codes, b.scales,
+                                                                          offs, out_offs, out_rows)
+        return _grouped_2d3d_rows_out_op(a.codes, a.scales, b.codes, b.scales, offs, out_offs, out_rows)
+    if a2.codes.shape != a.codes.shape or b2.codes.shape != b.codes.shape:
+        raise ValueError("both operand sets must have the same shapes")
+    return _grouped_2d3d_rows_out_op(a.codes, a.scales, b.codes, b.scales, offs, out_offs, out_rows,
+                                     (a2.codes, a2.scales, b2.codes, b2.scales))
+
+
+def rows_out_supported(a: MXData, b: MXData, a2: MXData | None = None, b2: MXData | None = None) -> bool:
+    T, K = a.codes.shape
+    G, N, _ = b.codes.shape
+    every = [d for d in (a, b, a2, b2) if d is not None]
+    return (len(every) in (2, 4) and all(d.scale_order == MX_SCALES_MFMA for d in every)
+            and K % 128 == 0 and N % 8 == 0 and T % 32 == 0 and G <= FAST_MAX_GROUPS)
 
 
 def mx_grouped_gemm_2d3d_shared_a(a: MXData, b: MXData, b2: MXData, offs: torch.Tensor) -> torch.Tensor:
