@@ -195,6 +195,28 @@ int mx_swiglu_bwd_cast_dim0_dim1(const void* dg, const void* a, const void* b, i
                                  uint8_t* scales_t, void* dab, int scale_mode, int scale_order,
                                  void* stream);
 
+/* The three casts above with a row pitch for their codes, as mx_cast_dim0_dim1_ld has it:
+ * rows of `codes` ld_codes bytes apart (>= cols), rows of `codes_t` ld_codes_t bytes apart
+ * (>= rows), both multiples of 16 with 16-byte aligned buffers; 0 stands for dense rows.  The
+ * two halves of the backward cast's outputs lie rows * ld_codes and cols * ld_codes_t bytes
+ * apart.  Scales, every other argument and the results are those of the dense forms, which
+ * forward here.  (The pitched operands of the fused SwiGLU block's GEMMs: see mx_gemm_nt_ld.) */
+int mx_swiglu_cast_dim0_dim1_ld(const void* a, const void* b, int64_t rows, int64_t cols,
+                                int64_t lda, int64_t ldb, uint8_t* codes, int64_t ld_codes,
+                                uint8_t* scales, uint8_t* codes_t, int64_t ld_codes_t,
+                                uint8_t* scales_t, void* g, int scale_mode, int scale_order,
+                                void* stream);
+int mx_rmsnorm_cast_dim0_dim1_ld(const void* x, const void* weight, float eps, int64_t rows,
+                                 int64_t cols, int64_t ldx, float* rstd, void* y, uint8_t* codes,
+                                 int64_t ld_codes, uint8_t* scales, uint8_t* codes_t,
+                                 int64_t ld_codes_t, uint8_t* scales_t, int scale_mode,
+                                 int scale_order, void* stream);
+int mx_swiglu_bwd_cast_dim0_dim1_ld(const void* dg, const void* a, const void* b, int64_t rows,
+                                    int64_t cols, int64_t lddg, int64_t lda, int64_t ldb,
+                                    uint8_t* codes, int64_t ld_codes, uint8_t* scales,
+                                    uint8_t* codes_t, int64_t ld_codes_t, uint8_t* scales_t,
+                                    void* dab, int scale_mode, int scale_order, void* stream);
+
 /* MXFP8 -> bf16: out[r, c] = e4m3(codes[r, c]) * 2^(scale of row r, block c / 32 - 127) rounded
  * to bf16 (exact above bf16's subnormal range); a scale byte 255 gives NaN.  codes uint8
  * [rows, cols] dense (16-byte aligned, cols % 32 == 0), scales in either order, out bf16
@@ -304,6 +326,22 @@ int mx_gemm_nt_shared_b(const uint8_t* a_codes, const uint8_t* a_scales, const u
                         const uint8_t* a2_scales, const uint8_t* b_codes, const uint8_t* b_scales,
                         void* d, void* d2, int64_t M, int64_t N, int64_t K, int64_t ldd,
                         void* stream);
+
+/* mx_gemm_nt_pair / _shared_a / _shared_b on operands whose rows lie ldk bytes apart (every code
+ * matrix of the call with the same pitch, ldk >= K and a multiple of 128, as for mx_gemm_nt_ld);
+ * the dense forms forward here with ldk = K.  Same results. */
+int mx_gemm_nt_pair_ld(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                       const uint8_t* b_scales, const uint8_t* a2_codes, const uint8_t* a2_scales,
+                       const uint8_t* b2_codes, const uint8_t* b2_scales, void* d, int64_t M,
+                       int64_t N, int64_t K, int64_t ldk, int64_t ldd, void* stream);
+int mx_gemm_nt_shared_a_ld(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                           const uint8_t* b_scales, const uint8_t* b2_codes, const uint8_t* b2_scales,
+                           void* d, void* d2, int64_t M, int64_t N, int64_t K, int64_t ldk,
+                           int64_t ldd, void* stream);
+int mx_gemm_nt_shared_b_ld(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* a2_codes,
+                           const uint8_t* a2_scales, const uint8_t* b_codes, const uint8_t* b_scales,
+                           void* d, void* d2, int64_t M, int64_t N, int64_t K, int64_t ldk,
+                           int64_t ldd, void* stream);
 
 /* Grouped GEMM, 2D x 3D: for group g with rows [offs[g-1], offs[g]) of A:
  * D[rows, :] = deq(A[rows, :]) * deq(B[g])^T.  a_codes [T,K]; b_codes [G,N,K];

@@ -461,3 +461,48 @@ def test_fused_cast_with_row_pitches_writes_the_same_codes(device, R, C, pad):
     assert st == 0
     assert bool((base0[:, C:] == 0xAB).all()) and bool((base1[:, R:] == 0xCD).all())
     assert torch.equal(base0[:, :C], want0.codes) and torch.equal(base1[:, :R], want1.codes)
+
+
+@pytest.mark.parametrize("R,C,pad", [(160, 224, 128), (1024, 768, 128), (96, 160, 16)])
+def test_gate_and_norm_casts_with_row_pitches_write_the_same_codes(device, R, C, pad):
+    """The SwiGLU forward and backward casts and the RMSNorm cast with a row pitch: codes, scales
+    and optional bf16 outputs equal those of the dense forms; through the C ABI the bytes between
+    the rows (and between the two halves of the backward cast) are left alone."""
+    torch.manual_seed(R * 3 + C)
+    a, b, dg = (torch.randn(R, C, device=device, dtype=torch.bfloat16) * s for s in (2.0, 1.0, 0.5))
+    w = (1 + 0.2 * torch.randn(C, device=device)).to(torch.bfloat16)
+    L = ops.MX_SCALES_MFMA
+    eq = lambda p, q: (p.codes.stride(0) == q.codes.shape[1] + pad and torch.equal(p.codes, q.codes)
+                       and torch.equal(p.scales, q.scales))
+    for mode in ("floor", "rceil"):
+        d0, d1, dgate = ops.swiglu_to_mx_dim0_dim1(a, b, mode, L, want_g=True)
+        p0, p1, pgate = ops.swiglu_to_mx_dim0_dim1(a, b, mode, L, want_g=True, pitch_pad=pad)
+        assert eq(p0, d0) and eq(p1, d1) and torch.equal(pgate, dgate)
+        (da0, da1), (db0, db1), dgr = ops.swiglu_bwd_to_mx_dim0_dim1(dg, a, b, mode, L, want_grads=True)
+        (pa0, pa1), (pb0, pb1), pgr = ops.swiglu_bwd_to_mx_dim0_dim1(dg, a, b, mode, L, want_grads=True, pitch_pad=pad)
+        assert eq(pa0, da0) and eq(pa1, da1) and eq(pb0, db0) and eq(pb1, db1) and torch.equal(pgr, dgr)
+        n0, n1, rstd, y = ops.rms_norm_to_mx(a, w, 1e-5, mode, L, want_y=True)
+        q0, q1, prstd, py = ops.rms_norm_to_mx(a, w, 1e-5, mode, L, want_y=True, pitch_pad=pad)
+        assert eq(q0, n0) and eq(q1, n1) and torch.equal(prstd, rstd) and torch.equal(py, y)
+    # the backward cast through the C ABI into buffers filled with a marker
+    lib = _lib.load()
+    (da0, da1), (db0, db1), _ = ops.swiglu_bwd_to_mx_dim0_dim1(dg, a, b, "rceil", L)
+    c = torch.full((2, R, C + pad), 0xAB, dtype=torch.uint8, device=device)
+    ct = torch.full((2, C, R + pad), 0xCD, dtype=torch.uint8, device=device)
+    s = torch.empty(2 * da0.scales.numel(), dtype=torch.uint8, device=device)
+    st_ = torch.empty(2 * da1.scales.numel(), dtype=torch.uint8, device=device)
+    with torch.cuda.device(device):
+        rc = lib.mx_swiglu_bwd_cast_dim0_dim1_ld(ops._ptr(dg), ops._ptr(a), ops._ptr(b), R, C, C, C, C, ops._ptr(c), C + pad,
+                                                 ops._ptr(s), ops._ptr(ct), R + pad, ops._ptr(st_), None, 1, L,
+                                                 ops._stream(a))
+    assert rc == 0
+    assert bool((c[:, :, C:] == 0xAB).all()) and bool((ct[:, :, R:] == 0xCD).all())
+    assert torch.equal(c[0, :, :C], da0.codes) and torch.equal(c[1, :, :C], db0.codes)
+    assert torch.equal(ct[0, :, :R], da1.codes) and torch.equal(ct[1, :, :R], db1.codes)
+    assert torch.equal(s[:da0.scales.numel()], da0.scales.reshape(-1)) and torch.equal(st_[da1.scales.numel():], db1.scales.reshape(-1))
+    # pitches that are too small or not multiples of 16 are refused
+    with torch.cuda.device(device):
+        assert lib.mx_swiglu_cast_dim0_dim1_ld(ops._ptr(a), ops._ptr(b), R, C, C, C, ops._ptr(c), C - 16, ops._ptr(s),
+                                               ops._ptr(ct), R + pad, ops._ptr(st_), None, 1, L, ops._stream(a)) != 0
+        assert lib.mx_swiglu_cast_dim0_dim1_ld(ops._ptr(a), ops._ptr(b), R, C, C, C, ops._ptr(c), C + 8, ops._ptr(s),
+                                               ops._ptr(ct), R + pad, ops._ptr(st_), None, 1, L, ops._stream(a)) != 0

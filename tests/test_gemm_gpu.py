@@ -334,7 +334,7 @@ def test_pair_gemm_is_one_gemm_over_the_concatenated_contraction(device, M, N, K
         got = ops.mx_gemm_nt_pair(a, b, a2, b2)
     finally:
         ops._call = real_call
-    assert launches.count("mx_gemm_nt_pair") == 1 and "mx_gemm_nt" not in launches
+    assert launches.count("mx_gemm_nt_pair_ld") == 1 and "mx_gemm_nt" not in launches
     err = rel_l2(_f32(bits_of(got)), ref)
     two = ops.mx_gemm_nt(a, b) + ops.mx_gemm_nt(a2, b2)
     assert err <= TOL and err <= rel_l2(_f32(bits_of(two)), ref) + 1e-5, err
@@ -360,11 +360,25 @@ def test_two_products_sharing_an_operand_equal_two_gemms(device, M, N, K):
                                          ops.MX_SCALES_MFMA)
     a, a2, b, b2 = q(M, 1.0), q(M, 0.3), q(N, 0.02), q(N, 0.05)
     (d, d2), names = _launch_names(lambda: ops.mx_gemm_nt_shared_a(a, b, b2))
-    assert names == ["mx_gemm_nt_shared_a"]
+    assert names == ["mx_gemm_nt_shared_a_ld"]
     assert torch.equal(d, ops.mx_gemm_nt(a, b)) and torch.equal(d2, ops.mx_gemm_nt(a, b2))
     (e, e2), names = _launch_names(lambda: ops.mx_gemm_nt_shared_b(a, a2, b))
-    assert names == ["mx_gemm_nt_shared_b"]
+    assert names == ["mx_gemm_nt_shared_b_ld"]
     assert torch.equal(e, d) and torch.equal(e2, ops.mx_gemm_nt(a2, b))
+    # the same on operands whose rows lie 128 bytes further apart (NaN codes between the rows), and the
+    # sum of two products likewise: bit-identical; one operand with another pitch: copies, then dense
+    def pitched(t, pad=128):
+        buf = torch.full((t.codes.shape[0], K + pad), 0x7F, dtype=torch.uint8, device=device)
+        buf[:, :K] = t.codes
+        return ops.MXData(buf[:, :K], t.scales, t.scale_order)
+
+    pa, pa2, pb, pb2 = pitched(a), pitched(a2), pitched(b), pitched(b2)
+    assert torch.equal(ops.mx_gemm_nt_shared_a(pa, pb, pb2), torch.stack((d, d2)))
+    assert torch.equal(ops.mx_gemm_nt_shared_b(pa, pa2, pb), torch.stack((e, e2)))
+    assert torch.equal(ops.mx_gemm_nt_shared_a(pa, pb, b2), torch.stack((d, d2)))
+    both = ops.mx_gemm_nt_pair(a, b, a2, b2)
+    assert torch.equal(ops.mx_gemm_nt_pair(pa, pb, pa2, pb2), both)
+    assert torch.equal(ops.mx_gemm_nt_pair(pa, pb, pa2, pitched(b2, 256)), both)
     un = lambda t: ops.scale_unlayout(t.scales, t.codes.shape[0], K // 32).cpu().numpy()
     ref = mo.mx_matmul_q(a2.codes.cpu().numpy(), un(a2), b.codes.cpu().numpy(), un(b))
     assert rel_l2(_f32(bits_of(e2)), _f32(ref)) <= TOL

@@ -42,6 +42,9 @@ SIGNATURES = {
     "mx_moe_combine": (c_int, [_P, _P, _I, _I, _P, _P, _I, _I, _I, _P, _I, _P]),
     "mx_moe_row_dot": (c_int, [_P, _P, _I, _I, _P, _P, _I, _I, _P, _I, _I, _P, _P]),
     "mx_rmsnorm_cast_dim0_dim1": (c_int, [_P, _P, ctypes.c_float, _I, _I, _I, _P, _P, _P, _P, _P, _P, c_int, c_int, _P]),
+    "mx_rmsnorm_cast_dim0_dim1_ld": (c_int, [_P, _P, ctypes.c_float, _I, _I, _I, _P, _P, _P, _I, _P, _P, _I, _P, c_int, c_int, _P]),
+    "mx_swiglu_cast_dim0_dim1_ld": (c_int, [_P, _P, _I, _I, _I, _I, _P, _I, _P, _P, _I, _P, _P, c_int, c_int, _P]),
+    "mx_swiglu_bwd_cast_dim0_dim1_ld": (c_int, [_P, _P, _P, _I, _I, _I, _I, _I, _P, _I, _P, _P, _I, _P, _P, c_int, c_int, _P]),
     "mx_swiglu_cast_dim0_dim1": (c_int, [_P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, c_int, c_int, _P]),
     "mx_swiglu_bwd_cast_dim0_dim1": (c_int, [_P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, c_int, c_int, _P]),
     "mx_scale_layout": (c_int, [_P, _I, _I, _P, _P]),
@@ -53,6 +56,9 @@ SIGNATURES = {
     "mx_gemm_nt_static_max_bytes": (_I, []),
     "mx_gemm_nt_static": (c_int, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "mx_gemm_nt_pair": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
+    "mx_gemm_nt_pair_ld": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
+    "mx_gemm_nt_shared_a_ld": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
+    "mx_gemm_nt_shared_b_ld": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "mx_gemm_nt_shared_a": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "mx_gemm_nt_shared_b": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "mx_grouped_gemm_2d3d_shared_a": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),

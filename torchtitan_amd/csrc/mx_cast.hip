@@ -1157,13 +1157,24 @@ __global__ __launch_bounds__(256) void rms_rstd_kernel(const uint16_t* __restric
 }
 }  // namespace mx
 
-extern "C" int mx_rmsnorm_cast_dim0_dim1(const void* x, const void* weight, float eps, int64_t rows,
-                                         int64_t cols, int64_t ldx, float* rstd, void* y,
-                                         uint8_t* codes, uint8_t* scales, uint8_t* codes_t,
-                                         uint8_t* scales_t, int scale_mode, int scale_order,
-                                         void* stream) {
-  if (rows < 0 || cols < 0 || ldx < cols || bad_enums(scale_mode, scale_order)) return MX_ERR_INVALID_ARG;
+// A code pitch of 0 stands for dense rows; a pitch must keep every row 16-byte aligned.
+static inline bool bad_pitches(int64_t ld_codes, int64_t cols, int64_t ld_codes_t, int64_t rows) {
+  return (ld_codes && ld_codes < cols) || (ld_codes_t && ld_codes_t < rows);
+}
+static inline bool misaligned_pitches(int64_t ld_codes, int64_t ld_codes_t, const void* codes) {
+  return (ld_codes % 16) || (ld_codes_t % 16) || ((ld_codes || ld_codes_t) && ((uintptr_t)codes & 15));
+}
+
+extern "C" int mx_rmsnorm_cast_dim0_dim1_ld(const void* x, const void* weight, float eps, int64_t rows,
+                                            int64_t cols, int64_t ldx, float* rstd, void* y,
+                                            uint8_t* codes, int64_t ld_codes, uint8_t* scales,
+                                            uint8_t* codes_t, int64_t ld_codes_t, uint8_t* scales_t,
+                                            int scale_mode, int scale_order, void* stream) {
+  if (rows < 0 || cols < 0 || ldx < cols || bad_enums(scale_mode, scale_order) ||
+      bad_pitches(ld_codes, cols, ld_codes_t, rows))
+    return MX_ERR_INVALID_ARG;
   if (rows == 0 || cols == 0) return MX_OK;
+  if (misaligned_pitches(ld_codes, ld_codes_t, codes)) return MX_ERR_ALIGNMENT;
   if (!x || !weight || !rstd || !codes || !scales || !codes_t || !scales_t) return MX_ERR_INVALID_ARG;
   if (rows % 32 || cols % 32 || ldx % 8 || ((uintptr_t)x & 15) || ((uintptr_t)weight & 15) ||
       ((uintptr_t)y & 15) || ((uintptr_t)rstd & 3) || ((uintptr_t)codes & 7) ||
@@ -1181,19 +1192,33 @@ extern "C" int mx_rmsnorm_cast_dim0_dim1(const void* x, const void* weight, floa
   ex.x3 = (const uint16_t*)weight;
   ex.g_out = (uint16_t*)y;
   ex.row_scale = rstd;
+  ex.ldc = ld_codes;
+  ex.ldct = ld_codes_t;
   MX_DISPATCH_TILE(true, true, 3, false, (const uint16_t*)x, rows, cols, ldx, codes, scales, nblk, ks_n,
                    codes_t, scales_t, nblk_t, ks_n_t, (int64_t)0, (int64_t)0, (int64_t)0,
                    (uint32_t)gx, (uint32_t)tgy, ex);
   return launch_status();
 }
 
-extern "C" int mx_swiglu_cast_dim0_dim1(const void* a, const void* b, int64_t rows, int64_t cols,
-                                        int64_t lda, int64_t ldb, uint8_t* codes, uint8_t* scales,
-                                        uint8_t* codes_t, uint8_t* scales_t, void* g,
-                                        int scale_mode, int scale_order, void* stream) {
-  if (rows < 0 || cols < 0 || lda < cols || ldb < cols || bad_enums(scale_mode, scale_order))
+extern "C" int mx_rmsnorm_cast_dim0_dim1(const void* x, const void* weight, float eps, int64_t rows,
+                                         int64_t cols, int64_t ldx, float* rstd, void* y,
+                                         uint8_t* codes, uint8_t* scales, uint8_t* codes_t,
+                                         uint8_t* scales_t, int scale_mode, int scale_order,
+                                         void* stream) {
+  return mx_rmsnorm_cast_dim0_dim1_ld(x, weight, eps, rows, cols, ldx, rstd, y, codes, 0, scales, codes_t, 0,
+                                      scales_t, scale_mode, scale_order, stream);
+}
+
+extern "C" int mx_swiglu_cast_dim0_dim1_ld(const void* a, const void* b, int64_t rows, int64_t cols,
+                                           int64_t lda, int64_t ldb, uint8_t* codes, int64_t ld_codes,
+                                           uint8_t* scales, uint8_t* codes_t, int64_t ld_codes_t,
+                                           uint8_t* scales_t, void* g, int scale_mode,
+                                           int scale_order, void* stream) {
+  if (rows < 0 || cols < 0 || lda < cols || ldb < cols || bad_enums(scale_mode, scale_order) ||
+      bad_pitches(ld_codes, cols, ld_codes_t, rows))
     return MX_ERR_INVALID_ARG;
   if (rows == 0 || cols == 0) return MX_OK;
+  if (misaligned_pitches(ld_codes, ld_codes_t, codes)) return MX_ERR_ALIGNMENT;
   if (!a || !b || !codes || !scales || !codes_t || !scales_t) return MX_ERR_INVALID_ARG;
   if (rows % 32 || cols % 32 || lda % 8 || ldb % 8 || ((uintptr_t)a & 15) || ((uintptr_t)b & 15) ||
       ((uintptr_t)codes & 7) || ((uintptr_t)codes_t & 15) || ((uintptr_t)scales & 3) ||
@@ -1205,22 +1230,34 @@ extern "C" int mx_swiglu_cast_dim0_dim1(const void* a, const void* b, int64_t ro
   if (tile_grid_x(gx, tgy, true) > 0x7FFFFFFF) return MX_ERR_UNSUPPORTED;
   hipStream_t st = (hipStream_t)stream;
   dim3 grid = tile_grid(gx, tgy, 1, true), block(64 * MX_CAST_WAVES);
+  TileExtras ex{(const uint16_t*)b, ldb, (uint16_t*)g, nullptr, 0, nullptr, 0};
+  ex.ldc = ld_codes;
+  ex.ldct = ld_codes_t;
   MX_DISPATCH_TILE(true, true, 1, false, (const uint16_t*)a, rows, cols, lda, codes, scales, nblk, ks_n,
                    codes_t, scales_t, nblk_t, ks_n_t, (int64_t)0, (int64_t)0, (int64_t)0,
-                   (uint32_t)gx, (uint32_t)tgy,
-                   TileExtras{(const uint16_t*)b, ldb, (uint16_t*)g, nullptr, 0, nullptr, 0});
+                   (uint32_t)gx, (uint32_t)tgy, ex);
   return launch_status();
 }
 
-extern "C" int mx_swiglu_bwd_cast_dim0_dim1(const void* dg, const void* a, const void* b,
-                                            int64_t rows, int64_t cols, int64_t lddg, int64_t lda,
-                                            int64_t ldb, uint8_t* codes, uint8_t* scales,
-                                            uint8_t* codes_t, uint8_t* scales_t, void* dab,
-                                            int scale_mode, int scale_order, void* stream) {
+extern "C" int mx_swiglu_cast_dim0_dim1(const void* a, const void* b, int64_t rows, int64_t cols,
+                                        int64_t lda, int64_t ldb, uint8_t* codes, uint8_t* scales,
+                                        uint8_t* codes_t, uint8_t* scales_t, void* g,
+                                        int scale_mode, int scale_order, void* stream) {
+  return mx_swiglu_cast_dim0_dim1_ld(a, b, rows, cols, lda, ldb, codes, 0, scales, codes_t, 0, scales_t, g,
+                                     scale_mode, scale_order, stream);
+}
+
+extern "C" int mx_swiglu_bwd_cast_dim0_dim1_ld(const void* dg, const void* a, const void* b,
+                                               int64_t rows, int64_t cols, int64_t lddg, int64_t lda,
+                                               int64_t ldb, uint8_t* codes, int64_t ld_codes,
+                                               uint8_t* scales, uint8_t* codes_t, int64_t ld_codes_t,
+                                               uint8_t* scales_t, void* dab, int scale_mode,
+                                               int scale_order, void* stream) {
   if (rows < 0 || cols < 0 || lddg < cols || lda < cols || ldb < cols ||
-      bad_enums(scale_mode, scale_order))
+      bad_enums(scale_mode, scale_order) || bad_pitches(ld_codes, cols, ld_codes_t, rows))
     return MX_ERR_INVALID_ARG;
   if (rows == 0 || cols == 0) return MX_OK;
+  if (misaligned_pitches(ld_codes, ld_codes_t, codes)) return MX_ERR_ALIGNMENT;
   if (!dg || !a || !b || !codes || !scales || !codes_t || !scales_t) return MX_ERR_INVALID_ARG;
   if (rows % 32 || cols % 32 || lddg % 8 || lda % 8 || ldb % 8 || ((uintptr_t)dg & 15) ||
       ((uintptr_t)a & 15) || ((uintptr_t)b & 15) || ((uintptr_t)codes & 7) ||
@@ -1236,9 +1273,20 @@ extern "C" int mx_swiglu_bwd_cast_dim0_dim1(const void* dg, const void* a, const
   if (tile_grid_x(gx, tgy, true) > 0x7FFFFFFF) return MX_ERR_UNSUPPORTED;
   hipStream_t st = (hipStream_t)stream;
   dim3 grid = tile_grid(gx, tgy, 1, true), block(64 * MX_CAST_WAVES);
+  TileExtras ex{(const uint16_t*)b, ldb, (uint16_t*)dab, (const uint16_t*)dg, lddg, nullptr, 0};
+  ex.ldc = ld_codes;
+  ex.ldct = ld_codes_t;
   MX_DISPATCH_TILE(true, true, 2, false, (const uint16_t*)a, rows, cols, lda, codes, scales, nblk, ks_n,
                    codes_t, scales_t, nblk_t, ks_n_t, (int64_t)0, s_b, st_b, (uint32_t)gx,
-                   (uint32_t)tgy,
-                   TileExtras{(const uint16_t*)b, ldb, (uint16_t*)dab, (const uint16_t*)dg, lddg, nullptr, 0});
+                   (uint32_t)tgy, ex);
   return launch_status();
+}
+
+extern "C" int mx_swiglu_bwd_cast_dim0_dim1(const void* dg, const void* a, const void* b,
+                                            int64_t rows, int64_t cols, int64_t lddg, int64_t lda,
+                                            int64_t ldb, uint8_t* codes, uint8_t* scales,
+                                            uint8_t* codes_t, uint8_t* scales_t, void* dab,
+                                            int scale_mode, int scale_order, void* stream) {
+  return mx_swiglu_bwd_cast_dim0_dim1_ld(dg, a, b, rows, cols, lddg, lda, ldb, codes, 0, scales, codes_t, 0,
+                                         scales_t, dab, scale_mode, scale_order, stream);
 }

@@ -125,7 +125,25 @@ namespace mx {
 int launch_gemm_nt32_pair(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                           const uint8_t* b_scales, const uint8_t* a2_codes, const uint8_t* a2_scales,
                           const uint8_t* b2_codes, const uint8_t* b2_scales, void* d, int64_t M,
-                          int64_t N, int64_t K, int64_t ldd, hipStream_t st);
+                          int64_t N, int64_t K, int64_t ldk, int64_t ldd, hipStream_t st);
+}
+
+// The forms over two operand sets exist for the persistent kernel only, dense rows (ldk == K) or
+// pitched: other shapes are the caller's two GEMMs (and an add).
+extern "C" int mx_gemm_nt_pair_ld(const uint8_t* a_codes, const uint8_t* a_scales,
+                                  const uint8_t* b_codes, const uint8_t* b_scales,
+                                  const uint8_t* a2_codes, const uint8_t* a2_scales,
+                                  const uint8_t* b2_codes, const uint8_t* b2_scales, void* d,
+                                  int64_t M, int64_t N, int64_t K, int64_t ldk, int64_t ldd,
+                                  void* stream) {
+  int rc = check_dense(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd);
+  if (rc == MX_OK) rc = check_dense(a2_codes, a2_scales, b2_codes, b2_scales, d, M, N, K, ldd);
+  if (rc != MX_OK || M == 0 || N == 0) return rc;
+  if (ldk < K) return MX_ERR_INVALID_ARG;
+  if (M <= 128 || N <= 128 || !persistent_ok(d, N, K, ldd, ldk) || force_kernel == 1 || force_kernel == 2)
+    return MX_ERR_UNSUPPORTED;
+  return launch_gemm_nt32_pair(a_codes, a_scales, b_codes, b_scales, a2_codes, a2_scales, b2_codes,
+                               b2_scales, d, M, N, K, ldk, ldd, (hipStream_t)stream);
 }
 
 extern "C" int mx_gemm_nt_pair(const uint8_t* a_codes, const uint8_t* a_scales,
@@ -133,40 +151,62 @@ extern "C" int mx_gemm_nt_pair(const uint8_t* a_codes, const uint8_t* a_scales,
                                const uint8_t* a2_codes, const uint8_t* a2_scales,
                                const uint8_t* b2_codes, const uint8_t* b2_scales, void* d,
                                int64_t M, int64_t N, int64_t K, int64_t ldd, void* stream) {
-  int rc = check_dense(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd);
-  if (rc == MX_OK) rc = check_dense(a2_codes, a2_scales, b2_codes, b2_scales, d, M, N, K, ldd);
-  if (rc != MX_OK || M == 0 || N == 0) return rc;
-  // the persistent kernel only: other shapes are the caller's two GEMMs and an add
-  if (M <= 128 || N <= 128 || !persistent_ok(d, N, K, ldd) || force_kernel == 1 || force_kernel == 2)
-    return MX_ERR_UNSUPPORTED;
-  return launch_gemm_nt32_pair(a_codes, a_scales, b_codes, b_scales, a2_codes, a2_scales, b2_codes,
-                               b2_scales, d, M, N, K, ldd, (hipStream_t)stream);
+  return mx_gemm_nt_pair_ld(a_codes, a_scales, b_codes, b_scales, a2_codes, a2_scales, b2_codes, b2_scales, d,
+                            M, N, K, K, ldd, stream);
 }
 
 namespace mx {
 int launch_gemm_nt32_two_b(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                            const uint8_t* b_scales, const uint8_t* b2_codes, const uint8_t* b2_scales,
-                           void* d, void* d2, int64_t M, int64_t N, int64_t K, int64_t ldd, hipStream_t st);
+                           void* d, void* d2, int64_t M, int64_t N, int64_t K, int64_t ldk, int64_t ldd,
+                           hipStream_t st);
 int launch_gemm_nt32_two_a(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* a2_codes,
                            const uint8_t* a2_scales, const uint8_t* b_codes, const uint8_t* b_scales,
-                           void* d, void* d2, int64_t M, int64_t N, int64_t K, int64_t ldd, hipStream_t st);
+                           void* d, void* d2, int64_t M, int64_t N, int64_t K, int64_t ldk, int64_t ldd,
+                           hipStream_t st);
 }
 
 // Two products that share an operand, one launch of the persistent kernel; other shapes are the
 // caller's two mx_gemm_nt calls.
+extern "C" int mx_gemm_nt_shared_a_ld(const uint8_t* a_codes, const uint8_t* a_scales,
+                                      const uint8_t* b_codes, const uint8_t* b_scales,
+                                      const uint8_t* b2_codes, const uint8_t* b2_scales, void* d,
+                                      void* d2, int64_t M, int64_t N, int64_t K, int64_t ldk,
+                                      int64_t ldd, void* stream) {
+  int rc = check_dense(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd);
+  if (rc == MX_OK) rc = check_dense(a_codes, a_scales, b2_codes, b2_scales, d2, M, N, K, ldd);
+  if (rc != MX_OK || M == 0 || N == 0) return rc;
+  if (ldk < K) return MX_ERR_INVALID_ARG;
+  if (M <= 128 || N <= 128 || !persistent_ok(d, N, K, ldd, ldk) || !persistent_ok(d2, N, K, ldd, ldk) ||
+      force_kernel == 1 || force_kernel == 2)
+    return MX_ERR_UNSUPPORTED;
+  return launch_gemm_nt32_two_b(a_codes, a_scales, b_codes, b_scales, b2_codes, b2_scales, d, d2, M, N,
+                                K, ldk, ldd, (hipStream_t)stream);
+}
+
 extern "C" int mx_gemm_nt_shared_a(const uint8_t* a_codes, const uint8_t* a_scales,
                                    const uint8_t* b_codes, const uint8_t* b_scales,
                                    const uint8_t* b2_codes, const uint8_t* b2_scales, void* d,
                                    void* d2, int64_t M, int64_t N, int64_t K, int64_t ldd,
                                    void* stream) {
+  return mx_gemm_nt_shared_a_ld(a_codes, a_scales, b_codes, b_scales, b2_codes, b2_scales, d, d2, M, N, K, K,
+                                ldd, stream);
+}
+
+extern "C" int mx_gemm_nt_shared_b_ld(const uint8_t* a_codes, const uint8_t* a_scales,
+                                      const uint8_t* a2_codes, const uint8_t* a2_scales,
+                                      const uint8_t* b_codes, const uint8_t* b_scales, void* d,
+                                      void* d2, int64_t M, int64_t N, int64_t K, int64_t ldk,
+                                      int64_t ldd, void* stream) {
   int rc = check_dense(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd);
-  if (rc == MX_OK) rc = check_dense(a_codes, a_scales, b2_codes, b2_scales, d2, M, N, K, ldd);
+  if (rc == MX_OK) rc = check_dense(a2_codes, a2_scales, b_codes, b_scales, d2, M, N, K, ldd);
   if (rc != MX_OK || M == 0 || N == 0) return rc;
-  if (M <= 128 || N <= 128 || !persistent_ok(d, N, K, ldd) || !persistent_ok(d2, N, K, ldd) ||
+  if (ldk < K) return MX_ERR_INVALID_ARG;
+  if (M <= 128 || N <= 128 || !persistent_ok(d, N, K, ldd, ldk) || !persistent_ok(d2, N, K, ldd, ldk) ||
       force_kernel == 1 || force_kernel == 2)
     return MX_ERR_UNSUPPORTED;
-  return launch_gemm_nt32_two_b(a_codes, a_scales, b_codes, b_scales, b2_codes, b2_scales, d, d2, M, N,
-                                K, ldd, (hipStream_t)stream);
+  return launch_gemm_nt32_two_a(a_codes, a_scales, a2_codes, a2_scales, b_codes, b_scales, d, d2, M, N,
+                                K, ldk, ldd, (hipStream_t)stream);
 }
 
 extern "C" int mx_gemm_nt_shared_b(const uint8_t* a_codes, const uint8_t* a_scales,
@@ -174,14 +214,8 @@ extern "C" int mx_gemm_nt_shared_b(const uint8_t* a_codes, const uint8_t* a_scal
                                    const uint8_t* b_codes, const uint8_t* b_scales, void* d,
                                    void* d2, int64_t M, int64_t N, int64_t K, int64_t ldd,
                                    void* stream) {
-  int rc = check_dense(a_codes, a_scales, b_codes, b_scales, d, M, N, K, ldd);
-  if (rc == MX_OK) rc = check_dense(a2_codes, a2_scales, b_codes, b_scales, d2, M, N, K, ldd);
-  if (rc != MX_OK || M == 0 || N == 0) return rc;
-  if (M <= 128 || N <= 128 || !persistent_ok(d, N, K, ldd) || !persistent_ok(d2, N, K, ldd) ||
-      force_kernel == 1 || force_kernel == 2)
-    return MX_ERR_UNSUPPORTED;
-  return launch_gemm_nt32_two_a(a_codes, a_scales, a2_codes, a2_scales, b_codes, b_scales, d, d2, M, N,
-                                K, ldd, (hipStream_t)stream);
+  return mx_gemm_nt_shared_b_ld(a_codes, a_scales, a2_codes, a2_scales, b_codes, b_scales, d, d2, M, N, K, K,
+                                ldd, stream);
 }
 
 extern "C" int64_t mx_gemm_nt_workspace_bytes(int64_t M, int64_t N, int64_t K) {

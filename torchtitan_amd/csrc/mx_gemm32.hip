@@ -1297,12 +1297,14 @@ int launch_grouped32_2d3d(const uint8_t* a_codes, const uint8_t* a_scales, const
 // D = A B^T and D2 = A B2^T in one launch (same shapes), dense and grouped 2D x 3D.
 int launch_gemm_nt32_two_b(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                            const uint8_t* b_scales, const uint8_t* b2_codes, const uint8_t* b2_scales,
-                           void* d, void* d2, int64_t M, int64_t N, int64_t K, int64_t ldd, hipStream_t st) {
+                           void* d, void* d2, int64_t M, int64_t N, int64_t K, int64_t ldk, int64_t ldd,
+                           hipStream_t st) {
   Gemm32Args p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, M, N, K, ldd, nullptr, 0, 0, 0, nullptr};
   p.b2_codes = b2_codes;
   p.b2_scales = b2_scales;
   p.two = kTwoB;
   p.d2 = (uint16_t*)d2;
+  p.ldk = ldk;
   return launch32<kDense, false>(p, ((M + kT32 - 1) / kT32) * 2 * ((N + kT32 - 1) / kT32), st);
 }
 int launch_grouped32_2d3d_two_b(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
@@ -1319,12 +1321,14 @@ int launch_grouped32_2d3d_two_b(const uint8_t* a_codes, const uint8_t* a_scales,
 // D = A B^T and D2 = A2 B^T in one launch (same shapes), dense and grouped 2D x 2D.
 int launch_gemm_nt32_two_a(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* a2_codes,
                            const uint8_t* a2_scales, const uint8_t* b_codes, const uint8_t* b_scales,
-                           void* d, void* d2, int64_t M, int64_t N, int64_t K, int64_t ldd, hipStream_t st) {
+                           void* d, void* d2, int64_t M, int64_t N, int64_t K, int64_t ldk, int64_t ldd,
+                           hipStream_t st) {
   Gemm32Args p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, M, N, K, ldd, nullptr, 0, 0, 0, nullptr};
   p.a2_codes = a2_codes;
   p.a2_scales = a2_scales;
   p.two = kTwoA;
   p.d2 = (uint16_t*)d2;
+  p.ldk = ldk;
   return launch32<kDense, false>(p, 2 * ((M + kT32 - 1) / kT32) * ((N + kT32 - 1) / kT32), st);
 }
 int launch_grouped32_2d2d_two_a(const uint8_t* at_codes, const uint8_t* at_scales, const uint8_t* at2_codes,
@@ -1343,9 +1347,10 @@ int launch_grouped32_2d2d_two_a(const uint8_t* at_codes, const uint8_t* at_scale
 int launch_gemm_nt32_pair(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                           const uint8_t* b_scales, const uint8_t* a2_codes, const uint8_t* a2_scales,
                           const uint8_t* b2_codes, const uint8_t* b2_scales, void* d, int64_t M,
-                          int64_t N, int64_t K, int64_t ldd, hipStream_t st) {
+                          int64_t N, int64_t K, int64_t ldk, int64_t ldd, hipStream_t st) {
   Gemm32Args p{a_codes, a_scales, b_codes, b_scales, (uint16_t*)d, M, N, K, ldd, nullptr, 0, 0, 0, nullptr,
                a2_codes, a2_scales, b2_codes, b2_scales};
+  p.ldk = ldk;
   const int64_t nb = ((M + kT32 - 1) / kT32) * ((N + kT32 - 1) / kT32);
   return launch32<kDense, false, true>(p, nb, st);
 }

@@ -120,27 +120,35 @@ def _take(saved, i):
 FFN_SAVED = 14
 
 
+def block_pitch_pad(cfg: MXFP8Config, need_dx: bool, need_dw: bool) -> int:
+    """Bytes the eager SwiGLU block leaves between the rows of its MXFP8 codes: ops.CODE_PITCH_PAD
+    in a training step (every operand is then cast both ways by the kernels that know pitches);
+    none with cached weight casts, whose entries other callers read as dense codes."""
+    return ops.CODE_PITCH_PAD if need_dx and need_dw and not cfg.cache_weight_casts else 0
+
+
 def ffn_forward(x2, x_src, w1, w2, w3, cfg: MXFP8Config, need_dx: bool, need_dw: bool, norm_weight=None,
-                eps: float = 0.0):
+                eps: float = 0.0, pad: int = 0):
     """Forward of the SwiGLU block on a 2-D bf16 activation: (y [M, out], the FFN_SAVED slots).
     `x_src` is the tensor the activation-cast cache is keyed on (None: no sharing of x's cast
-    with sibling linears).  The eager autograd function and the traced operator both run this."""
+    with sibling linears); `pad`: the row pitch padding of every code matrix (the saved ones
+    carry it into the backward).  The eager autograd function and the traced operator both run this."""
     mode = cfg.scale_mode
     rstd = None
     if norm_weight is not None:  # RMSNorm in front: normalised inside the cast, rstd kept for its backward
         x2 = x2.contiguous()
-        xq0, xq1, rstd, _ = ops.rms_norm_to_mx(x2, _bf16(norm_weight), eps, mode, MX_SCALES_MFMA)
+        xq0, xq1, rstd, _ = ops.rms_norm_to_mx(x2, _bf16(norm_weight), eps, mode, MX_SCALES_MFMA, pitch_pad=pad)
     elif x_src is not None:
-        xq0, xq1 = _cast_activation(x2, x_src, mode, need_cols=need_dw)
+        xq0, xq1 = _cast_activation(x2, x_src, mode, need_cols=need_dw, pitch_pad=pad)
     elif need_dw:
-        xq0, xq1 = ops.to_mx_dim0_dim1(x2.contiguous(), mode, MX_SCALES_MFMA)
+        xq0, xq1 = ops.to_mx_dim0_dim1(x2.contiguous(), mode, MX_SCALES_MFMA, pitch_pad=pad)
     else:
         xq0, xq1 = ops.to_mx_dim0(x2.contiguous(), mode, MX_SCALES_MFMA), None
-    w1q0, w1q1 = _cast_weight(w1, mode, need_dx, cfg)
-    w3q0, w3q1 = _cast_weight(w3, mode, need_dx, cfg)
-    w2q0, w2q1 = _cast_weight(w2, mode, need_dx or need_dw, cfg)
+    w1q0, w1q1 = _cast_weight(w1, mode, need_dx, cfg, pitch_pad=pad)
+    w3q0, w3q1 = _cast_weight(w3, mode, need_dx, cfg, pitch_pad=pad)
+    w2q0, w2q1 = _cast_weight(w2, mode, need_dx or need_dw, cfg, pitch_pad=pad)
     h13 = ops.mx_gemm_nt_shared_a(xq0, w1q0, w3q0)  # one launch: x's panels fetched once for both
-    gq0, gq1, _ = ops.swiglu_to_mx_dim0_dim1(h13[0], h13[1], mode, MX_SCALES_MFMA)
+    gq0, gq1, _ = ops.swiglu_to_mx_dim0_dim1(h13[0], h13[1], mode, MX_SCALES_MFMA, pitch_pad=pad)
     y = ops.mx_gemm_nt(gq0, w2q0)
     saved = [None] * FFN_SAVED
     if need_dx or need_dw:
@@ -155,17 +163,18 @@ def ffn_forward(x2, x_src, w1, w2, w3, cfg: MXFP8Config, need_dx: bool, need_dw:
 
 
 def ffn_backward(dy2, saved, cfg: MXFP8Config, need_x: bool, need_dw1: bool, need_dw2: bool, need_dw3: bool,
-                 need_dnw: bool = False):
-    """(dx [M, in], dW1, dW2, dW3, d norm weight), bf16, None where not asked for."""
+                 need_dnw: bool = False, pad: int = 0):
+    """(dx [M, in], dW1, dW2, dW3, d norm weight), bf16, None where not asked for; `pad` as the
+    forward's."""
     mode = cfg.scale_mode
     h13 = saved[0]
     w2q1 = _take(saved, 1)
     if need_dw2:
-        dyq0, dyq1 = ops.to_mx_dim0_dim1(dy2, mode, MX_SCALES_MFMA)
+        dyq0, dyq1 = ops.to_mx_dim0_dim1(dy2, mode, MX_SCALES_MFMA, pitch_pad=pad)
     else:
         dyq0, dyq1 = ops.to_mx_dim0(dy2, mode, MX_SCALES_MFMA), None
     dg = ops.mx_gemm_nt(dyq0, w2q1)
-    (da0, da1), (db0, db1), _ = ops.swiglu_bwd_to_mx_dim0_dim1(dg, h13[0], h13[1], mode, MX_SCALES_MFMA)
+    (da0, da1), (db0, db1), _ = ops.swiglu_bwd_to_mx_dim0_dim1(dg, h13[0], h13[1], mode, MX_SCALES_MFMA, pitch_pad=pad)
     dx = dw1 = dw2 = dw3 = dnw = None
     if need_dw1 or need_dw2 or need_dw3:
         xq1, gq1 = _take(saved, 3), _take(saved, 5)
@@ -198,7 +207,9 @@ class _MXFeedForward(torch.autograd.Function):
     def forward(ctx, x, w1, w2, w3, cfg: MXFP8Config, norm_weight=None, eps: float = 0.0):
         need_dx = ctx.needs_input_grad[0] or ctx.needs_input_grad[5]
         need_dw = any(ctx.needs_input_grad[1:4])
-        y, saved = ffn_forward(x.reshape(-1, x.shape[-1]), x, w1, w2, w3, cfg, need_dx, need_dw, norm_weight, eps)
+        ctx.pad = block_pitch_pad(cfg, need_dx, need_dw)
+        y, saved = ffn_forward(x.reshape(-1, x.shape[-1]), x, w1, w2, w3, cfg, need_dx, need_dw, norm_weight, eps,
+                               pad=ctx.pad)
         ctx.cfg, ctx.x_shape = cfg, x.shape
         ctx.w_dtypes = (w1.dtype, w2.dtype, w3.dtype)
         ctx.save_for_backward(*saved)
@@ -210,7 +221,7 @@ class _MXFeedForward(torch.autograd.Function):
         need = ctx.needs_input_grad
         dy2 = _bf16(dy.reshape(-1, dy.shape[-1])).contiguous()
         dx, dw1, dw2, dw3, dnw = ffn_backward(dy2, list(ctx.saved_tensors), ctx.cfg, need[0], need[1], need[2],
-                                              need[3], need[5])
+                                              need[3], need[5], pad=ctx.pad)
         cast_back = lambda g, dt: g if g is None or g.dtype == dt else g.to(dt)
         if dx is not None:
             dx = dx.view(ctx.x_shape)

@@ -152,6 +152,17 @@ def to_mx_dim1(x: torch.Tensor, mode="floor", order: int = MX_SCALES_ROWMAJOR) -
 CODE_PITCH_PAD = int(os.environ.get("MXFP8_CODE_PITCH_PAD", "128"))
 
 
+def _code_rows(rows: int, cols: int, pad: int, device, stack: int = 0) -> torch.Tensor:
+    """uint8 [rows, cols] (or [stack, rows, cols]) whose rows lie cols + pad bytes apart."""
+    shape = (rows, cols + pad) if not stack else (stack, rows, cols + pad)
+    return torch.empty(shape, dtype=torch.uint8, device=device)[..., :cols]
+
+
+def _pitch_ok(pad: int) -> int:
+    """The row pitch padding the tile casts take: a multiple of 16 bytes (else none)."""
+    return pad if pad > 0 and pad % 16 == 0 else 0
+
+
 def to_mx_dim0_dim1(x: torch.Tensor, mode="floor", order: int = MX_SCALES_ROWMAJOR, pitch_pad: int = 0):
     """Both casts from one read of x; returns (row-wise MXData, column-wise MXData).  With
     `pitch_pad` the rows of both code matrices lie that many bytes further apart than they are
@@ -354,10 +365,10 @@ def token_logprob_bwd(logits: torch.Tensor, target: torch.Tensor, lse: torch.Ten
 
 
 def rms_norm_to_mx(x: torch.Tensor, weight: torch.Tensor, eps: float, mode="floor",
-                   order: int = MX_SCALES_ROWMAJOR, want_y: bool = False):
+                   order: int = MX_SCALES_ROWMAJOR, want_y: bool = False, pitch_pad: int = 0):
     """Both casts of y = rms_norm(x) * weight (float32 arithmetic, one rounding to bf16) without
     y passing through memory; returns (row-wise MXData, column-wise MXData, rstd float32 [rows],
-    y or None)."""
+    y or None).  `pitch_pad`: as for `to_mx_dim0_dim1`."""
     x = _check_hp(x)
     if weight.dtype != torch.bfloat16 or weight.shape != (x.shape[1],) or weight.device != x.device:
         raise TypeError("the norm weight must be bf16 [cols] on x's device")
@@ -365,36 +376,40 @@ def rms_norm_to_mx(x: torch.Tensor, weight: torch.Tensor, eps: float, mode="floo
     R, C = x.shape
     if R % BLOCK or C % BLOCK:
         raise ValueError(f"both dims of {tuple(x.shape)} must be multiples of {BLOCK}")
-    codes = torch.empty((R, C), dtype=torch.uint8, device=x.device)
+    pad = _pitch_ok(pitch_pad)
+    codes = _code_rows(R, C, pad, x.device)
     scales = _alloc_scales(R, C // BLOCK, order, x.device)
-    codes_t = torch.empty((C, R), dtype=torch.uint8, device=x.device)
+    codes_t = _code_rows(C, R, pad, x.device)
     scales_t = _alloc_scales(C, R // BLOCK, order, x.device)
     rstd = torch.empty(R, dtype=torch.float32, device=x.device)
     y = torch.empty((R, C), dtype=torch.bfloat16, device=x.device) if want_y else None
-    _call("mx_rmsnorm_cast_dim0_dim1", "rmsnorm_cast_dim0_dim1", x.device, _ptr(x), _ptr(weight),
+    _call("mx_rmsnorm_cast_dim0_dim1_ld", "rmsnorm_cast_dim0_dim1", x.device, _ptr(x), _ptr(weight),
           ctypes.c_float(eps), R, C, x.stride(0), _ptr(rstd), _ptr(y) if y is not None else None,
-          _ptr(codes), _ptr(scales), _ptr(codes_t), _ptr(scales_t), _mode(mode), order, _stream(x))
+          _ptr(codes), codes.stride(0), _ptr(scales), _ptr(codes_t), codes_t.stride(0), _ptr(scales_t),
+          _mode(mode), order, _stream(x))
     return MXData(codes, scales, order), MXData(codes_t, scales_t, order), rstd, y
 
 
 def swiglu_to_mx_dim0_dim1(a: torch.Tensor, b: torch.Tensor, mode="floor",
-                           order: int = MX_SCALES_ROWMAJOR, want_g: bool = False):
+                           order: int = MX_SCALES_ROWMAJOR, want_g: bool = False, pitch_pad: int = 0):
     """Both casts of g = silu(a) * b (bf16, every step rounded to bf16) without g passing through
-    memory; returns (row-wise MXData, column-wise MXData, g or None)."""
+    memory; returns (row-wise MXData, column-wise MXData, g or None).  `pitch_pad`: as for
+    `to_mx_dim0_dim1`."""
     a, b = _check_hp(a), _check_hp(b)
     if a.shape != b.shape:
         raise ValueError(f"shape mismatch: {tuple(a.shape)} vs {tuple(b.shape)}")
     R, C = a.shape
     if R % BLOCK or C % BLOCK:
         raise ValueError(f"both dims of {tuple(a.shape)} must be multiples of {BLOCK}")
-    codes = torch.empty((R, C), dtype=torch.uint8, device=a.device)
+    pad = _pitch_ok(pitch_pad)
+    codes = _code_rows(R, C, pad, a.device)
     scales = _alloc_scales(R, C // BLOCK, order, a.device)
-    codes_t = torch.empty((C, R), dtype=torch.uint8, device=a.device)
+    codes_t = _code_rows(C, R, pad, a.device)
     scales_t = _alloc_scales(C, R // BLOCK, order, a.device)
     g = torch.empty((R, C), dtype=torch.bfloat16, device=a.device) if want_g else None
-    _call("mx_swiglu_cast_dim0_dim1", "swiglu_cast_dim0_dim1", a.device, _ptr(a), _ptr(b), R, C,
-          a.stride(0), b.stride(0), _ptr(codes), _ptr(scales), _ptr(codes_t), _ptr(scales_t),
-          _ptr(g) if g is not None else None, _mode(mode), order, _stream(a))
+    _call("mx_swiglu_cast_dim0_dim1_ld", "swiglu_cast_dim0_dim1", a.device, _ptr(a), _ptr(b), R, C,
+          a.stride(0), b.stride(0), _ptr(codes), codes.stride(0), _ptr(scales), _ptr(codes_t), codes_t.stride(0),
+          _ptr(scales_t), _ptr(g) if g is not None else None, _mode(mode), order, _stream(a))
     return MXData(codes, scales, order), MXData(codes_t, scales_t, order), g
 
 
@@ -403,11 +418,12 @@ def _scale_count(rows: int, nblk: int, order: int) -> int:
 
 
 def swiglu_bwd_to_mx_dim0_dim1(dg: torch.Tensor, a: torch.Tensor, b: torch.Tensor, mode="floor",
-                               order: int = MX_SCALES_ROWMAJOR, want_grads: bool = False):
+                               order: int = MX_SCALES_ROWMAJOR, want_grads: bool = False, pitch_pad: int = 0):
     """Backward of g = silu(a) * b with both casts of each gradient from one pass over dg, a, b.
 
     Returns ((da row-wise, da column-wise), (db row-wise, db column-wise), stacked bf16 [2, R, C]
-    gradients or None).  The two row-wise (column-wise) results are the halves of one buffer."""
+    gradients or None).  The two row-wise (column-wise) results are the halves of one buffer.
+    `pitch_pad`: as for `to_mx_dim0_dim1`."""
     dg, a, b = _check_hp(dg), _check_hp(a), _check_hp(b)
     if a.shape != b.shape or a.shape != dg.shape:
         raise ValueError(f"shape mismatch: {tuple(dg.shape)}, {tuple(a.shape)}, {tuple(b.shape)}")
@@ -416,14 +432,15 @@ def swiglu_bwd_to_mx_dim0_dim1(dg: torch.Tensor, a: torch.Tensor, b: torch.Tenso
         raise ValueError(f"both dims of {tuple(a.shape)} must be multiples of {BLOCK}")
     dev = a.device
     n_s, n_st = _scale_count(R, C // BLOCK, order), _scale_count(C, R // BLOCK, order)
-    codes = torch.empty((2, R, C), dtype=torch.uint8, device=dev)
-    codes_t = torch.empty((2, C, R), dtype=torch.uint8, device=dev)
+    pad = _pitch_ok(pitch_pad)
+    codes = _code_rows(R, C, pad, dev, stack=2)
+    codes_t = _code_rows(C, R, pad, dev, stack=2)
     scales = torch.empty(2 * n_s, dtype=torch.uint8, device=dev)
     scales_t = torch.empty(2 * n_st, dtype=torch.uint8, device=dev)
     dab = torch.empty((2, R, C), dtype=torch.bfloat16, device=dev) if want_grads else None
-    _call("mx_swiglu_bwd_cast_dim0_dim1", "swiglu_bwd_cast_dim0_dim1", dev, _ptr(dg), _ptr(a), _ptr(b),
-          R, C, dg.stride(0), a.stride(0), b.stride(0), _ptr(codes), _ptr(scales), _ptr(codes_t),
-          _ptr(scales_t), _ptr(dab) if dab is not None else None, _mode(mode), order, _stream(a))
+    _call("mx_swiglu_bwd_cast_dim0_dim1_ld", "swiglu_bwd_cast_dim0_dim1", dev, _ptr(dg), _ptr(a), _ptr(b),
+          R, C, dg.stride(0), a.stride(0), b.stride(0), _ptr(codes), codes.stride(1), _ptr(scales), _ptr(codes_t),
+          codes_t.stride(1), _ptr(scales_t), _ptr(dab) if dab is not None else None, _mode(mode), order, _stream(a))
 
     def half(i):
         s, st = scales[i * n_s:(i + 1) * n_s], scales_t[i * n_st:(i + 1) * n_st]
@@ -456,18 +473,22 @@ def _as_mfma(d: MXData) -> torch.Tensor:
 _gemm_workspace: dict = {}  # (device index, M, N, K) -> bytes the library would split with
 
 
-def _same_pitch(a_codes, b_codes):
-    """(a_codes, b_codes, bytes between their rows): both operands of a GEMM as the kernels take
-    them, i.e. unit inner stride and one common row pitch (copies are made where they differ)."""
-    if a_codes.stride(1) != 1 or b_codes.stride(1) != 1 or a_codes.stride(0) != b_codes.stride(0):
-        a_codes, b_codes = a_codes.contiguous(), b_codes.contiguous()
-    return a_codes, b_codes, a_codes.stride(0)
+def _common_pitch(*codes, multiple: int = 128):
+    """(the code matrices as the kernels take them, bytes between their rows): unit inner stride
+    and one row pitch for all of them, a multiple of `multiple` where it is not the row length
+    (copies are made where they differ)."""
+    pitch = codes[0].stride(0)
+    K = codes[0].shape[1]
+    if any(c.stride(1) != 1 or c.stride(0) != pitch for c in codes) or (pitch != K and pitch % multiple):
+        codes = tuple(c.contiguous() for c in codes)
+        pitch = K
+    return codes, pitch
 
 
 def _gemm_nt_into(a_codes, a_scales, b_codes, b_scales, out):
     M, K = a_codes.shape
     N = b_codes.shape[0]
-    a_codes, b_codes, ldk = _same_pitch(a_codes, b_codes)
+    (a_codes, b_codes), ldk = _common_pitch(a_codes, b_codes, multiple=16)  # (the tile kernels take any such pitch)
     key = (out.device.index, M, N, K)
     need = _gemm_workspace.get(key)
     if need is None:
@@ -582,8 +603,9 @@ def mx_gemm_nt_pair(a: MXData, b: MXData, a2: MXData, b2: MXData) -> torch.Tenso
         return mx_gemm_nt(a, b) + mx_gemm_nt(a2, b2)
     out = torch.empty((M, N), dtype=torch.bfloat16, device=a.codes.device)
     sa, sb, sa2, sb2 = _as_mfma(a), _as_mfma(b), _as_mfma(a2), _as_mfma(b2)  # kept alive over the launch
-    _call("mx_gemm_nt_pair", "gemm_nt_pair", out.device, _ptr(a.codes), _ptr(sa), _ptr(b.codes), _ptr(sb),
-          _ptr(a2.codes), _ptr(sa2), _ptr(b2.codes), _ptr(sb2), _ptr(out), M, N, K, N, _stream(out))
+    (ac, bc, a2c, b2c), ldk = _common_pitch(a.codes, b.codes, a2.codes, b2.codes)
+    _call("mx_gemm_nt_pair_ld", "gemm_nt_pair", out.device, _ptr(ac), _ptr(sa), _ptr(bc), _ptr(sb),
+          _ptr(a2c), _ptr(sa2), _ptr(b2c), _ptr(sb2), _ptr(out), M, N, K, ldk, N, _stream(out))
     return out
 
 
@@ -607,8 +629,9 @@ def mx_gemm_nt_shared_a(a: MXData, b: MXData, b2: MXData) -> torch.Tensor:
         mx_gemm_nt(a, b2, out[1])
         return out
     sa, sb, sb2 = _as_mfma(a), _as_mfma(b), _as_mfma(b2)
-    _call("mx_gemm_nt_shared_a", "gemm_nt_shared_a", out.device, _ptr(a.codes), _ptr(sa), _ptr(b.codes), _ptr(sb),
-          _ptr(b2.codes), _ptr(sb2), _ptr(out[0]), _ptr(out[1]), M, N, K, N, _stream(out))
+    (ac, bc, b2c), ldk = _common_pitch(a.codes, b.codes, b2.codes)
+    _call("mx_gemm_nt_shared_a_ld", "gemm_nt_shared_a", out.device, _ptr(ac), _ptr(sa), _ptr(bc), _ptr(sb),
+          _ptr(b2c), _ptr(sb2), _ptr(out[0]), _ptr(out[1]), M, N, K, ldk, N, _stream(out))
     return out
 
 
@@ -625,8 +648,9 @@ def mx_gemm_nt_shared_b(a: MXData, a2: MXData, b: MXData) -> torch.Tensor:
         mx_gemm_nt(a2, b, out[1])
         return out
     sa, sa2, sb = _as_mfma(a), _as_mfma(a2), _as_mfma(b)
-    _call("mx_gemm_nt_shared_b", "gemm_nt_shared_b", out.device, _ptr(a.codes), _ptr(sa), _ptr(a2.codes), _ptr(sa2),
-          _ptr(b.codes), _ptr(sb), _ptr(out[0]), _ptr(out[1]), M, N, K, N, _stream(out))
+    (ac, a2c, bc), ldk = _common_pitch(a.codes, a2.codes, b.codes)
+    _call("mx_gemm_nt_shared_b_ld", "gemm_nt_shared_b", out.device, _ptr(ac), _ptr(sa), _ptr(a2c), _ptr(sa2),
+          _ptr(bc), _ptr(sb), _ptr(out[0]), _ptr(out[1]), M, N, K, ldk, N, _stream(out))
     return out
 
 
