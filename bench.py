@@ -74,16 +74,21 @@ def parse():
                     help="also run 4 elementwise passes over a 512 MiB tensor (reads 512 MiB, writes 512 MiB "
                          "each): the known-size kernel that scales FETCH_SIZE / WRITE_SIZE counter readings")
     ap.add_argument("--cast-table", action="store_true",
-                    help="instead of the benchmark: the HBM yardsticks (copy, read, write) and the three casts on "
-                         "X [16384, 4096] and dY [16384, 14336], 8 launches each in that order on rotating buffers "
-                         "(for rocprofv3 --pmc runs of the memory-path counters)")
+                    help="instead of the benchmark: the HBM yardsticks (copy, read, write, 2:1), then per tensor "
+                         "(X [16384, 4096], dY [16384, 14336], W [14336, 4096]) the streams over its bytes and its "
+                         "casts (row-wise, column-wise, fused, fused with a row pitch), then the SwiGLU and RMSNorm "
+                         "casts, in that order on rotating buffers (for rocprofv3 --pmc runs of the memory path)")
+    ap.add_argument("--expert-block", action="store_true",
+                    help="instead of the benchmark: only the fused expert block of the MoE config, 2 warm-up + 5 "
+                         "timed forward + backward passes (for a rocprofv3 kernel trace of that block alone)")
     ap.add_argument("--clock-table", action="store_true",
                     help="instead of the benchmark: the GEMM kernel at the benchmark shape on random data, on "
                          "constant operands and on half of the CUs, and the vendor library's fp8 GEMM, 8 launches "
                          "each in that order (for a rocprofv3 --pmc run: active cycles / time = shader clock)")
     ap.add_argument("--mfma-ceiling", action="store_true",
-                    help="only time the MFMA-only yardstick (both MFMA shapes, three kinds of operand bits) and "
-                         "print its JSON line: what the power limit leaves of the matrix peak")
+                    help="only time the MFMA-only yardstick (both MFMA shapes and three issue orders of the "
+                         "16x16x128 one, three kinds of operand bits) and print its JSON line: what the power limit "
+                         "leaves of the matrix peak")
     ap.add_argument("--gemm-ablation", action="store_true",
                     help="instead of the benchmark: the dense GEMM at the benchmark shape and the three grouped "
                          "GEMMs of the MoE config (equal groups and the skewed routing), timed with whatever build "
@@ -986,6 +991,16 @@ def time_policy_loss(dev):
     return out
 
 
+def _routed_counts(dev, g, E=128, tokens=16384, topk=8):
+    """Tokens per expert (int32 [E]) of a top-k routing from softmax over seeded Gumbel-perturbed logits."""
+    import torch
+
+    logits = torch.randn((tokens, E), generator=g, device=dev) + 0.5 * torch.randn((1, E), generator=g, device=dev)
+    gumbel = -torch.log(-torch.log(torch.rand((tokens, E), generator=g, device=dev).clamp_min(1e-9)))
+    top = torch.topk(torch.softmax(logits + gumbel, dim=-1), topk, dim=-1).indices
+    return torch.bincount(top.flatten(), minlength=E).to(torch.int32)
+
+
 def time_moe_grouped(dev, recipe_mode):
     """BASELINE configs[3] GEMMs (not the headline): 128 experts, hidden 2048, expert FFN 768,
     top-8 routing of 16384 tokens from softmax over seeded Gumbel-perturbed logits (uneven
@@ -997,10 +1012,7 @@ def time_moe_grouped(dev, recipe_mode):
 
     E, dim, hid, tokens, topk = 128, 2048, 768, 16384, 8
     g = torch.Generator(device=dev).manual_seed(3)
-    logits = torch.randn((tokens, E), generator=g, device=dev) + 0.5 * torch.randn((1, E), generator=g, device=dev)
-    gumbel = -torch.log(-torch.log(torch.rand((tokens, E), generator=g, device=dev).clamp_min(1e-9)))
-    top = torch.topk(torch.softmax(logits + gumbel, dim=-1), topk, dim=-1).indices
-    counts = torch.bincount(top.flatten(), minlength=E).to(torch.int32)
+    counts = _routed_counts(dev, g, E, tokens, topk)
     routed = tokens * topk
     max_len = -(-(routed + 32 * E) // 128) * 128
     _, m_sizes, offs = ops.group_offsets_pad(counts, E, 1, max_len, 32)
@@ -1121,7 +1133,7 @@ def time_moe_layer(dev, recipe_mode):
     return out
 
 
-def time_expert_block(dev, recipe_mode, counts):
+def time_expert_block(dev, recipe_mode, counts, compiled=True, unfused=True):
     """The whole expert SwiGLU block (three grouped GEMMs forward, six backward, padding, casts,
     gate) through the converted module on the routed rows in expert order: as one fused function
     and as separate grouped GEMMs around bf16 silu / product ops.  Bit-identical results."""
@@ -1138,7 +1150,7 @@ def time_expert_block(dev, recipe_mode, counts):
     x = torch.randn((routed, dim), device=dev, dtype=torch.bfloat16).requires_grad_(True)
     dy = torch.randn((routed, dim), device=dev, dtype=torch.bfloat16) * 1e-3
     out = {}
-    for name, fuse in (("fused", True), ("separate_ops", False)):
+    for name, fuse in (("fused", True), ("separate_ops", False))[:2 if unfused else 1]:
         ex = GroupedExperts(dim=dim, hidden_dim=hid, num_experts=E, use_grouped_mm=True)
         holder = nn.Module()
         holder.experts = ex
@@ -1165,7 +1177,7 @@ def time_expert_block(dev, recipe_mode, counts):
         torch.cuda.synchronize()
         ms = s.elapsed_time(e) / 5
         out[name] = {"ms": round(ms, 3), "TFLOP/s": round(18.0 * routed * dim * hid / ms / 1e9, 1)}
-        if fuse:
+        if fuse and compiled:
             out[name]["ms_under_torch_compile"] = _time_compiled(ex, lambda fn: fn(x, counts).backward(dy), step)
         del ex, holder
     return out
@@ -1255,6 +1267,10 @@ def main():
         return
     if args.cast_table:
         print(json.dumps(cast_table(dev, recipe_mode)))
+        return
+    if args.expert_block:
+        counts = _routed_counts(dev, torch.Generator(device=dev).manual_seed(3))
+        print(json.dumps(time_expert_block(dev, recipe_mode, counts, compiled=False, unfused=False)))
         return
     ffn, x, h, dy_h, dy_o = build_linears(dev, args.recipe)
     x.requires_grad_(True)
