@@ -239,10 +239,28 @@ def test_llama3_8b_block_at_seq_8192(device, norms_in_casts):
     x = emb(tokens).detach().requires_grad_(True)
     rope = _rope(seq, dim // heads, 500000.0, device)
     y = blk(x, rope)
-    y.backward(torch.randn_like(y) * 1e-3)
+    dy = torch.randn_like(y) * 1e-3
+    y.backward(dy)
     assert torch.isfinite(y).all() and torch.isfinite(x.grad).all()
     for n, p in blk.named_parameters():
         assert p.grad is not None and torch.isfinite(p.grad).all() and float(p.grad.abs().max()) > 0, n
+
+    # the backward as a whole: every gradient against the same block in plain bf16 (torch's linears
+    # and autograd) on the same input and output gradient.  The two differ by the MXFP8 rounding of
+    # every GEMM operand (about 3 % per operand, partly averaged out over the contraction), so a
+    # wiring mistake (a missing term, a transposed operand, a wrong cast direction) is an order of
+    # magnitude outside the bound
+    plain = _Block(dim, heads, kv_heads, ffn, 1e-5).to(device).to(torch.bfloat16)
+    plain.load_state_dict({k: v.detach().clone() for k, v in blk.state_dict().items()})
+    xb = x.detach().clone().requires_grad_(True)
+    plain(xb, rope).backward(dy)
+    g_errs = {"x": rel_l2(x.grad.float().cpu().numpy(), xb.grad.float().cpu().numpy())}
+    plain_grads = dict(plain.named_parameters())
+    for n, p in blk.named_parameters():
+        g_errs[n] = rel_l2(p.grad.float().cpu().numpy(), plain_grads[n].grad.float().cpu().numpy())
+    print(f"rel-L2 of the gradients against the bf16 block: {g_errs}", flush=True)
+    assert max(g_errs.values()) <= 0.2, g_errs  # observed: 0.07 (x, feed-forward weights) to 0.13 (attention weights)
+    del plain, plain_grads, xb
 
     ref = _Block(dim, heads, kv_heads, ffn, 1e-5).to(device).to(torch.bfloat16)
     ref.load_state_dict(blk.state_dict())
@@ -276,7 +294,7 @@ def test_llama3_8b_block_at_seq_8192(device, norms_in_casts):
         # and without the residual stream, which carries most of the output's norm
         errs["block_minus_input"] = err(y.detach()[:, :head] - xd[:, :head], want - xd[:, :head])
         print(f"rel-L2 against the block built from oracle linears: {errs}", flush=True)
-        assert errs["block"] <= 8e-2, errs
+        assert errs["block"] <= 6e-2 and errs["block_minus_input"] <= 7e-2, errs  # observed 0.031 / 0.034
 
 
 # ---- the policy step -------------------------------------------------------------------------

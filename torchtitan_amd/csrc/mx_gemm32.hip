@@ -37,8 +37,9 @@
 // that every read beyond the L2 finds its line in the memory-side cache; MX_ABL_ROW_PAD=n reads the
 // rows of a tile n bytes further apart than they lie (what a padded row pitch would do to the
 // spread of a block's lines over the cache channels); MX_ABL_TR_READ issues every fragment read as
-// two ds_read_b64_tr_b8 (what a K loop over operands stored K-strided would issue).  Results are
-// then meaningless.
+// two ds_read_b64_tr_b8 (what a K loop over operands stored K-strided would issue); MX_ABL_DMA_OOB
+// issues every copy with all lanes out of range (the instructions and their LDS writes stay, the
+// fetches go).  Results are then meaningless.
 #include "mx_gemm_tile.h"
 
 namespace mx {
@@ -641,10 +642,16 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
     }
     set_block_offsets();
   };
+#ifndef MX_LOAD_AUX  // cache policy bits of the operand copies (0: default)
+#define MX_LOAD_AUX 0
+#endif
   // The 17 copies of a block are issued one at a time, between MFMAs (see block_steps):
   // piece 0..15 = unit pairs (A unit, B unit alternating), 16 = scales, then advance.
   auto issue_piece = [&](auto i_) {
     constexpr int i = decltype(i_)::value;
+#ifdef MX_ABL_DMA_OOB  // timing ablation: every copy is issued with all lanes out of range (zeros land in LDS, nothing is fetched)
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.a_codes, 0), rb = ra, rs = ra;
+#endif
 
     const uint32_t sbase = lds_base + ld_slot * kBlock32;
     if constexpr (i < 16) {
@@ -654,10 +661,10 @@ __global__ __launch_bounds__(256, 1) void gemm_nt32_kernel(Gemm32Args p) {
                                               : ((q & 1) ? (v_even ^ 64) : v_even);
       const uint32_t so = (uint32_t)(unit * 8) * Kp + ld_kb * kKB;
       if constexpr ((i & 1) == 0)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void_t*)(uintptr_t)(sbase + unit * 1024), 16, v, so, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void_t*)(uintptr_t)(sbase + unit * 1024), 16, v, so, 0, MX_LOAD_AUX);
       else
         __builtin_amdgcn_raw_ptr_buffer_load_lds(
-            rb, (lds_void_t*)(uintptr_t)(sbase + kOperand32 + unit * 1024), 16, v, so, 0, 0);
+            rb, (lds_void_t*)(uintptr_t)(sbase + kOperand32 + unit * 1024), 16, v, so, 0, MX_LOAD_AUX);
     } else {
       // scales: a group's two 64-deep steps are 512 contiguous bytes, the two groups land behind
       // one another, which is the order the fragment reads expect.  Waves 0 and 2 copy A's and
