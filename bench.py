@@ -145,7 +145,7 @@ def one_step(ffn, x, h, dy_h, dy_o):
 
 def time_casts(dev, recipe_mode, also_floor=False):
     """to_mx GB/s per direction on cold inputs (rotating buffers > last-level cache).  With
-    `also_floor`, X is also cast with FLOOR scales (the mode BASELINE configs[0] names; it adds a
+    `also_floor`, X is also cast with FLOOR scales (the mode benchmark configs[0] names; it adds a
     clamp per element on the finite path), keys suffixed ":floor"."""
     import torch
 
@@ -514,7 +514,7 @@ def mfma_ceiling(dev, recipe_mode, launches=500, kinds=None, shapes=(32, 16)):
 def clock_table(dev, recipe_mode):
     """Evidence for what bounds the dense GEMM: the same kernel, same shape (M 16384, N 14336,
     K 4096), 8 launches per case, cases in a fixed order so that a counter run can tell them apart:
-      0 random BASELINE data (x ~ N(0,1), w ~ N(0,0.02))      4 the vendor library's tensor-scaled fp8 GEMM,
+      0 random benchmark data (x ~ N(0,1), w ~ N(0,0.02))      4 the vendor library's tensor-scaled fp8 GEMM,
       1 all-ones operands                                        random data, through torch._scaled_mm
       2 all-zero operands
       3 random data on half of the CUs (128 workgroups)
@@ -573,7 +573,7 @@ def clock_table(dev, recipe_mode):
 
 
 def time_decoder_block(dev, recipe):
-    """BASELINE configs[2] for scale (not the headline): one Llama-3-8B-style decoder block (dim
+    """benchmark configs[2] for scale (not the headline): one Llama-3-8B-style decoder block (dim
     4096, 32 heads / 8 KV heads, FFN 14336, RMSNorm eps 1e-5, RoPE theta 5e5, init N(0, 0.02)),
     forward + backward at batch 1 x seq 8192, with all seven linears converted to MXFP8
     (attention itself in bf16 through torch's SDPA), the same with the two RMSNorms inside the casts
@@ -886,7 +886,7 @@ def time_split_k(dev, recipe_mode):
 
 
 def time_policy_layer_linears(dev, recipe):
-    """BASELINE configs[4] for scale (not the headline): the seven linears of one layer of the
+    """benchmark configs[4] for scale (not the headline): the seven linears of one layer of the
     Qwen3-1.7B-shaped policy (dim 2048, 16 heads / 8 KV heads of 128, FFN 6144) over the packed
     tokens of one policy step (128 sequences, lengths uniform in [256, 2048]: 147 456 tokens),
     each forward + backward through a converted module on inputs of the config's distributions,
@@ -1002,7 +1002,7 @@ def _routed_counts(dev, g, E=128, tokens=16384, topk=8):
 
 
 def time_moe_grouped(dev, recipe_mode):
-    """BASELINE configs[3] GEMMs (not the headline): 128 experts, hidden 2048, expert FFN 768,
+    """benchmark configs[3] GEMMs (not the headline): 128 experts, hidden 2048, expert FFN 768,
     top-8 routing of 16384 tokens from softmax over seeded Gumbel-perturbed logits (uneven
     groups), groups padded to multiples of 32 rows as the config says (the token axis to a
     multiple of 128).  TFLOP/s counts the unpadded routed rows only."""
@@ -1184,7 +1184,7 @@ def time_expert_block(dev, recipe_mode, counts, compiled=True, unfused=True):
 
 
 def cpu_baseline(recipe_mode_int, target_s=15.0):
-    """CPU oracle on a bounded sample of the benchmark workload (BASELINE configs[1], the w1
+    """CPU oracle on a bounded sample of the benchmark workload (benchmark configs[1], the w1
     linear): the emulated MX linear forward (to_mx of X and W along K, dequantize, fp32 matmul,
     bf16 round) plus the column-wise casts the backward needs, with X ~ N(0,1) and W ~ N(0,0.02)
     as in the GPU run, at N=14336, K=4096 and as many rows M as fit about `target_s` seconds

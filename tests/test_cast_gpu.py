@@ -136,7 +136,7 @@ def test_empty_and_errors(device):
 
 
 def test_full_size_properties(device):
-    """BASELINE-size tensor: properties that need no CPU oracle pass over the whole tensor."""
+    """Benchmark-size tensor: properties that need no CPU oracle pass over the whole tensor."""
     torch.manual_seed(0)
     x = torch.randn((16384, 4096), device=device, dtype=torch.bfloat16)
     r, c = ops.to_mx_dim0_dim1(x, "floor")

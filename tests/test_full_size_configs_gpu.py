@@ -404,7 +404,7 @@ def test_token_log_probs_at_the_real_vocabulary_over_many_rows(device):
 
 
 def test_policy_step_composed_at_real_layer_shapes(device):
-    """BASELINE configs[4] composed, at the real layer shapes on two layers: 16 sequences (2 prompts
+    """benchmark configs[4] composed, at the real layer shapes on two layers: 16 sequences (2 prompts
     x 8 samples) of uneven lengths uniform in [256, 2048] with random token ids below 151 936,
     each through embedding -> two Qwen3-1.7B-shaped layers (dim 2048, 16 heads / 8 KV heads of
     128 with q/k norms, FFN 6144, all seven linears MXFP8, the SwiGLU block fused) -> norm ->

@@ -96,7 +96,7 @@ def test_policy_gradient_loss_fused_vs_oracle(device):
 
 
 def test_policy_step_on_a_small_converted_model_then_weight_hand_over(device):
-    """BASELINE configs[4] in small: a dense decoder-only model with MXFP8 linears, packed
+    """benchmark configs[4] in small: a dense decoder-only model with MXFP8 linears, packed
     prompts / completions of different lengths, the policy-gradient loss on fused log-probs,
     backward, an optimizer step, then the re-cast of all converted weights for the hand-over."""
     from tests.test_converter_gpu import _MiniDecoderBlock
